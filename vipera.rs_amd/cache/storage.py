@@ -1,0 +1,71 @@
+"""Device memory of the caches: paged keys and values per cache-owning layer entry, and state slots.
+
+Layout of a paged tensor: ``[pages + 1, kv_heads, block_size, head_dim]``; the last page is a
+scratch page that is never handed out, which padding tokens of a captured step write to.  A state
+tensor is ``[slots, *shape]``.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Sequence
+
+import torch
+
+from ..errors import InvalidArgumentError
+from .manager import CacheGroupSpec
+
+
+@dataclass
+class PagedKV:
+    k: torch.Tensor
+    v: torch.Tensor
+    group: int
+    block_size: int
+
+
+def plan_groups(needs, block_size: int, num_blocks: int) -> List[CacheGroupSpec]:
+    """One group per distinct retention rule among the run order's attention entries."""
+    windows: List[int] = []
+    for need in needs:
+        if need.kv is not None and need.kv.window not in windows:
+            windows.append(need.kv.window)
+    return [CacheGroupSpec(block_size, num_blocks, window) for window in windows]
+
+
+class CacheStorage:
+    def __init__(self, needs, groups: Sequence[CacheGroupSpec], num_slots: int, runtime):
+        self.kv: List[Optional[PagedKV]] = [None] * len(needs)
+        self.state: List[Optional[torch.Tensor]] = [None] * len(needs)
+        self.groups = list(groups)
+        self.bytes = 0
+        for index, need in enumerate(needs):
+            if need.owner != index:
+                continue
+            if need.kv is not None:
+                group = next((g for g, spec in enumerate(self.groups) if spec.window == need.kv.window), None)
+                if group is None:
+                    raise InvalidArgumentError(f"no cache group keeps a window of {need.kv.window}")
+                spec = self.groups[group]
+                shape = (spec.num_blocks + 1, need.kv.kv_heads, spec.block_size, need.kv.head_dim)
+                k = runtime.zeros(shape)
+                v = runtime.zeros(shape)
+                self.kv[index] = PagedKV(k, v, group, spec.block_size)
+                self.bytes += 2 * k.numel() * k.element_size()
+            if need.state is not None:
+                tensor = torch.zeros((num_slots,) + tuple(need.state.shape), dtype=need.state.dtype,
+                                     device=runtime.device)
+                self.state[index] = tensor
+                self.bytes += tensor.numel() * tensor.element_size()
+        for index, need in enumerate(needs):
+            if need.owner != index:
+                self.kv[index] = self.kv[need.owner]
+                self.state[index] = self.state[need.owner]
+
+    def bytes_per_token(self) -> int:
+        total = 0
+        seen = set()
+        for entry in self.kv:
+            if entry is not None and id(entry) not in seen:
+                seen.add(id(entry))
+                total += 2 * entry.k.shape[1] * entry.k.shape[3] * entry.k.element_size()
+        return total

@@ -1,0 +1,203 @@
+// Row-wise and element-wise kernels: embedding gather, RMSNorm, rotary + cache write,
+// gated activation, and a counter-based normal fill for random weights.
+//
+// Formulas as the reference computes them:
+//   embedding   x = table[token, :]                                  crates/vipera-backend-cpu/src/model.rs:607-616
+//   RMSNorm     inv = 1/sqrt(mean(x^2) + eps); out = (x*inv)*w       model.rs:4282-4288
+//   rotary      pairs (i, i + half): lo*c - hi*s, lo*s + hi*c        model.rs:4225-4251
+//   cache write K (after rotation) and V at table[pos / bs], pos % bs model.rs:1495-1542
+//   SwiGLU      up * gate / (1 + exp(-gate))                          model.rs:4368-4374
+#include "common.h"
+
+// ---------------------------------------------------------------------------------------------
+template <typename TW>
+__global__ void embed_gather_kernel(const TW* __restrict__ table, const int* __restrict__ tokens,
+                                    float* __restrict__ out, int width) {
+  const int t = blockIdx.x;
+  const TW* row = table + (size_t)tokens[t] * width;
+  float* dst = out + (size_t)t * width;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) dst[i] = to_float<TW>(row[i]);
+}
+
+extern "C" int vk_embed_gather(const void* table, int table_dtype, const int* tokens, float* out,
+                               int num_tokens, int width, void* stream) {
+  if (num_tokens <= 0) return 0;
+  if (width <= 0) return VK_BAD_ARGUMENT;
+  hipStream_t s = (hipStream_t)stream;
+  if (table_dtype == DT_F32)
+    embed_gather_kernel<float><<<num_tokens, 256, 0, s>>>((const float*)table, tokens, out, width);
+  else if (table_dtype == DT_BF16)
+    embed_gather_kernel<bf16_t><<<num_tokens, 256, 0, s>>>((const bf16_t*)table, tokens, out, width);
+  else
+    return VK_BAD_ARGUMENT;
+  VK_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------------
+// One block per output row. `rows` (may be null) picks the input row of each output row.
+template <typename TO>
+__global__ void rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ weight,
+                               const int* __restrict__ rows, TO* __restrict__ out, int width, float eps) {
+  __shared__ float scratch[16];
+  const int r = blockIdx.x;
+  const float* src = x + (size_t)(rows ? rows[r] : r) * width;
+  float sum = 0.f;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    const float v = src[i];
+    sum += v * v;
+  }
+  sum = block_sum(sum, scratch);
+  const float inv = 1.0f / sqrtf(sum / (float)width + eps);
+  TO* dst = out + (size_t)r * width;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) dst[i] = from_float<TO>(src[i] * inv * weight[i]);
+}
+
+extern "C" int vk_rmsnorm(const float* x, const float* weight, const int* rows, void* out, int out_dtype,
+                          int num_rows, int width, float eps, void* stream) {
+  if (num_rows <= 0) return 0;
+  if (width <= 0) return VK_BAD_ARGUMENT;
+  hipStream_t s = (hipStream_t)stream;
+  if (out_dtype == DT_F32)
+    rmsnorm_kernel<float><<<num_rows, 256, 0, s>>>(x, weight, rows, (float*)out, width, eps);
+  else if (out_dtype == DT_BF16)
+    rmsnorm_kernel<bf16_t><<<num_rows, 256, 0, s>>>(x, weight, rows, (bf16_t*)out, width, eps);
+  else
+    return VK_BAD_ARGUMENT;
+  VK_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------------
+// One block per token. `qkv` row layout: [heads*hd | kv_heads*hd | kv_heads*hd].
+// The first `rotary_dim` dims of every q and k head are rotated in place (angles in 32-bit:
+// float(pos) * inv_freq[i]); then the token's K and V rows go to the paged cache, whose layout is
+// [page, kv_head, slot, hd]. A token whose page id is negative writes nothing to the cache.
+template <typename T>
+__global__ void rope_kvwrite_kernel(T* __restrict__ qkv, const int* __restrict__ positions,
+                                    const float* __restrict__ inv_freq, int rotary_dim,
+                                    T* __restrict__ k_cache, T* __restrict__ v_cache,
+                                    const int* __restrict__ entry_of_token, const int* __restrict__ block_table,
+                                    int table_width, int block_size, int heads, int kv_heads, int hd) {
+  const int t = blockIdx.x;
+  const int pos = positions[t];
+  const int row_width = (heads + 2 * kv_heads) * hd;
+  T* row = qkv + (size_t)t * row_width;
+  const int half = rotary_dim / 2;
+  if (half > 0) {
+    const int pairs = (heads + kv_heads) * half;
+    for (int idx = threadIdx.x; idx < pairs; idx += blockDim.x) {
+      const int head = idx / half, i = idx - head * half;
+      T* h = row + (size_t)head * hd;  // q heads then k heads are contiguous
+      float sn, cs;
+      sincosf((float)pos * inv_freq[i], &sn, &cs);
+      const float lo = to_float<T>(h[i]), hi = to_float<T>(h[i + half]);
+      h[i] = from_float<T>(lo * cs - hi * sn);
+      h[i + half] = from_float<T>(lo * sn + hi * cs);
+    }
+    __syncthreads();
+  }
+  if (k_cache == nullptr) return;
+  const int page = block_table[(size_t)entry_of_token[t] * table_width + pos / block_size];
+  if (page < 0) return;
+  const int slot = pos % block_size;
+  const T* k_row = row + (size_t)heads * hd;
+  const T* v_row = k_row + (size_t)kv_heads * hd;
+  for (int idx = threadIdx.x; idx < kv_heads * hd; idx += blockDim.x) {
+    const int kvh = idx / hd, d = idx - kvh * hd;
+    const size_t at = (((size_t)page * kv_heads + kvh) * block_size + slot) * hd + d;
+    k_cache[at] = k_row[idx];
+    v_cache[at] = v_row[idx];
+  }
+}
+
+extern "C" int vk_rope_kvwrite(void* qkv, int dtype, const int* positions, const float* inv_freq, int rotary_dim,
+                               void* k_cache, void* v_cache, const int* entry_of_token, const int* block_table,
+                               int table_width, int block_size, int num_tokens, int heads, int kv_heads, int hd,
+                               void* stream) {
+  if (num_tokens <= 0) return 0;
+  if (hd <= 0 || heads <= 0 || kv_heads <= 0 || rotary_dim < 0 || rotary_dim > hd || (rotary_dim & 1))
+    return VK_BAD_ARGUMENT;
+  if (k_cache && (block_size <= 0 || table_width <= 0)) return VK_BAD_ARGUMENT;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == DT_F32)
+    rope_kvwrite_kernel<float><<<num_tokens, 256, 0, s>>>((float*)qkv, positions, inv_freq, rotary_dim,
+                                                           (float*)k_cache, (float*)v_cache, entry_of_token,
+                                                           block_table, table_width, block_size, heads, kv_heads, hd);
+  else if (dtype == DT_BF16)
+    rope_kvwrite_kernel<bf16_t><<<num_tokens, 256, 0, s>>>((bf16_t*)qkv, positions, inv_freq, rotary_dim,
+                                                            (bf16_t*)k_cache, (bf16_t*)v_cache, entry_of_token,
+                                                            block_table, table_width, block_size, heads, kv_heads, hd);
+  else
+    return VK_BAD_ARGUMENT;
+  VK_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------------
+// out[t, i] = up * silu(gate), gate = gate_up[t, i], up = gate_up[t, inter + i]; math in 32-bit.
+template <typename T>
+__global__ void swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out, int inter, long long total) {
+  for (long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (long long)gridDim.x * blockDim.x) {
+    const long long t = idx / inter;
+    const int i = (int)(idx - t * inter);
+    const T* row = gate_up + t * 2 * inter;
+    const float g = to_float<T>(row[i]), u = to_float<T>(row[inter + i]);
+    out[idx] = from_float<T>(u * (g / (1.0f + expf(-g))));
+  }
+}
+
+extern "C" int vk_swiglu(const void* gate_up, void* out, int dtype, int num_tokens, int inter, void* stream) {
+  if (num_tokens <= 0) return 0;
+  if (inter <= 0) return VK_BAD_ARGUMENT;
+  const long long total = (long long)num_tokens * inter;
+  long long blocks = (total + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == DT_F32)
+    swiglu_kernel<float><<<(int)blocks, 256, 0, s>>>((const float*)gate_up, (float*)out, inter, total);
+  else if (dtype == DT_BF16)
+    swiglu_kernel<bf16_t><<<(int)blocks, 256, 0, s>>>((const bf16_t*)gate_up, (bf16_t*)out, inter, total);
+  else
+    return VK_BAD_ARGUMENT;
+  VK_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Counter-based normal fill: element i of a stream is a function of (key, i) alone.
+//   z = mix(key + (i+1)*GOLDEN); u1 = (hi32(z)+0.5)/2^32; u2 = lo32(z)/2^32;
+//   n = sqrt(-2 ln u1) * cos(2 pi u2) in 64-bit; out = offset + std * n
+template <typename T>
+__global__ void fill_normal_kernel(T* __restrict__ out, long long count, unsigned long long key, float std_,
+                                   float offset) {
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < count;
+       i += (long long)gridDim.x * blockDim.x) {
+    unsigned long long z = key + (unsigned long long)(i + 1) * 0x9E3779B97F4A7C15ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    z = z ^ (z >> 31);
+    const double u1 = ((double)(z >> 32) + 0.5) / 4294967296.0;
+    const double u2 = (double)(z & 0xFFFFFFFFull) / 4294967296.0;
+    const double n = sqrt(-2.0 * log(u1)) * cos(6.283185307179586476925286766559 * u2);
+    const double scaled = n * (double)std_;
+    out[i] = from_float<T>((float)(offset != 0.f ? (double)offset + scaled : scaled));
+  }
+}
+
+extern "C" int vk_fill_normal(void* out, int dtype, long long count, unsigned long long key, float std_,
+                              float offset, void* stream) {
+  if (count <= 0) return 0;
+  long long blocks = (count + 255) / 256;
+  if (blocks > 16384) blocks = 16384;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == DT_F32)
+    fill_normal_kernel<float><<<(int)blocks, 256, 0, s>>>((float*)out, count, key, std_, offset);
+  else if (dtype == DT_BF16)
+    fill_normal_kernel<bf16_t><<<(int)blocks, 256, 0, s>>>((bf16_t*)out, count, key, std_, offset);
+  else
+    return VK_BAD_ARGUMENT;
+  VK_LAUNCH_CHECK();
+  return 0;
+}

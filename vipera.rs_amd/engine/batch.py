@@ -1,0 +1,129 @@
+"""The batch of one step as the parts see it: flat tokens with per-token and per-entry metadata.
+
+A step holds *entries*; an entry is a request with its next tokens (a portion of a prompt, or one
+decoded token).  All tokens of all entries form one flat batch.  The reference's interface has the
+same shape (``BatchEntry`` with ``new_tokens``, ``first_position`` and ``block_table``,
+crates/vipera-runtime/src/pipeline.rs:138-152) but its CPU backend runs mixed entries one after
+another (crates/vipera-backend-cpu/src/model.rs:796-827); here a mixed batch is the normal case.
+
+Everything is packed into one int32 host buffer and copied to the device once.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Sequence
+
+import numpy as np
+import torch
+
+from ..errors import InternalError, InvalidArgumentError
+
+
+@dataclass
+class StepEntry:
+    """One request's share of a step: ``tokens`` start at position ``start``; ``want`` lists the
+    indices (within ``tokens``) whose logits are asked for."""
+
+    request: int
+    start: int
+    tokens: Sequence[int]
+    want: Sequence[int] = ()
+
+
+@dataclass
+class StepBatch:
+    num_tokens: int
+    num_entries: int
+    num_logit_rows: int
+    tokens: torch.Tensor           # [T] int32
+    positions: torch.Tensor        # [T] int32
+    entry_of_token: torch.Tensor   # [T] int32
+    entry_start: torch.Tensor      # [E + 1] int32, offsets of the entries' tokens
+    entry_first_pos: torch.Tensor  # [E] int32
+    entry_kv_len: torch.Tensor     # [E] int32, tokens in the cache after this step
+    slots: torch.Tensor            # [E] int32, state slot of each entry's request
+    logit_rows: torch.Tensor       # [R] int32, flat token indices
+    block_tables: Dict[int, torch.Tensor]  # group -> [E, width] int32
+    # host copies, for launch decisions
+    host_counts: List[int] = field(default_factory=list)
+    host_first_pos: List[int] = field(default_factory=list)
+    host_slots: List[int] = field(default_factory=list)
+    max_count: int = 0
+    max_kv_len: int = 0
+    all_single: bool = False
+
+
+def build_batch(entries: Sequence[StepEntry], cache, vocab_size: int, device, min_table_width: int = 1) -> StepBatch:
+    """Pack ``entries`` for the device. The pages of every token must already be reserved in ``cache``."""
+    if not entries:
+        raise InvalidArgumentError("a step needs at least one entry")
+    counts = [len(e.tokens) for e in entries]
+    if min(counts) < 1:
+        raise InvalidArgumentError("every entry of a step needs at least one token")
+    seen = set()
+    for e in entries:
+        if e.request in seen:
+            raise InvalidArgumentError(f"request {e.request} appears twice in one step")
+        seen.add(e.request)
+    T, E = sum(counts), len(entries)
+    flat = np.fromiter((t for e in entries for t in e.tokens), dtype=np.int64, count=T)
+    if flat.min() < 0 or flat.max() >= vocab_size:
+        bad = int(flat[(flat < 0) | (flat >= vocab_size)][0])
+        raise InvalidArgumentError(f"token {bad} is outside the vocabulary of {vocab_size}")
+    starts = np.zeros(E + 1, dtype=np.int32)
+    starts[1:] = np.cumsum(counts)
+    first = np.array([e.start for e in entries], dtype=np.int32)
+    if first.min() < 0:
+        raise InvalidArgumentError("an entry starts at a negative position")
+    kv_len = first + np.array(counts, dtype=np.int32)
+    entry_of = np.repeat(np.arange(E, dtype=np.int32), counts)
+    positions = np.arange(T, dtype=np.int32) - starts[entry_of] + first[entry_of]
+    rows: List[int] = []
+    for k, e in enumerate(entries):
+        for w in e.want:
+            if not 0 <= w < counts[k]:
+                raise InvalidArgumentError(
+                    f"request {e.request}: wanted place {w} is outside its {counts[k]} tokens of this step")
+            rows.append(int(starts[k]) + int(w))
+    R = len(rows)
+    slots = np.array([cache.slot(e.request) for e in entries], dtype=np.int32)
+    if slots.min() < 0:
+        missing = entries[int(np.argmin(slots))].request
+        raise InternalError(f"request {missing} has no slot: nothing was reserved for it")
+
+    groups = cache.groups
+    tables = []
+    for g, spec in enumerate(groups):
+        width = max(min_table_width, int((int(kv_len.max()) + spec.block_size - 1) // spec.block_size))
+        table = np.full((E, width), -1, dtype=np.int32)
+        for k, e in enumerate(entries):
+            row = cache.table(e.request, g)
+            need_to = (int(kv_len[k]) + spec.block_size - 1) // spec.block_size
+            lo = max(0, e.start + 1 - spec.window) if spec.window > 0 else 0
+            need_from = lo // spec.block_size
+            if len(row) < need_to or any(p < 0 for p in row[need_from:need_to]):
+                raise InternalError(
+                    f"request {e.request}: positions {lo}..{int(kv_len[k]) - 1} are not all backed by pages "
+                    f"in cache group {g}; reserve before the step")
+            n = min(len(row), width)
+            table[k, :n] = row[:n]
+        tables.append(table)
+
+    parts = [flat.astype(np.int32), positions, entry_of, starts, first, kv_len.astype(np.int32), slots,
+             np.array(rows, dtype=np.int32)] + [t.reshape(-1) for t in tables]
+    sizes = [p.size for p in parts]
+    host = torch.from_numpy(np.concatenate(parts)) if sum(sizes) else torch.zeros(0, dtype=torch.int32)
+    dev = host.pin_memory().to(device, non_blocking=True) if device.type == "cuda" else host
+    views, at = [], 0
+    for size in sizes:
+        views.append(dev[at:at + size])
+        at += size
+    block_tables = {g: views[8 + g].view(E, tables[g].shape[1]) for g in range(len(groups))}
+    return StepBatch(
+        num_tokens=T, num_entries=E, num_logit_rows=R,
+        tokens=views[0], positions=views[1], entry_of_token=views[2], entry_start=views[3],
+        entry_first_pos=views[4], entry_kv_len=views[5], slots=views[6], logit_rows=views[7],
+        block_tables=block_tables, host_counts=counts, host_first_pos=[int(v) for v in first],
+        host_slots=[int(v) for v in slots], max_count=max(counts), max_kv_len=int(kv_len.max()),
+        all_single=max(counts) == 1,
+    )

@@ -1,0 +1,66 @@
+"""The step function: run a batch of (request, its next tokens) through the model from the cache.
+
+``ModelRunner`` owns the model, the cache manager and the cache's device memory.  ``step`` takes
+entries whose pages are already reserved, runs only the tokens it is given as one batch, and
+returns the logits at the wanted places.  It corresponds to the reference's ``ForwardPass`` seam
+(crates/vipera-runtime/src/pipeline.rs:192-230), with ``logits``, ``logits_range`` and
+``logits_batch`` folded into one call.
+"""
+from __future__ import annotations
+
+import os
+from typing import List, Optional, Sequence
+
+import torch
+
+from ..cache import CacheManager, CacheStorage, plan_groups
+from ..config.base import ModelConfig
+from ..config.registry import load_config
+from ..errors import InvalidArgumentError
+from ..models import build_model
+from ..runtime import Runtime
+from ..weights import Checkpoint, load_tensors
+from .batch import StepBatch, StepEntry, build_batch
+
+
+class ModelRunner:
+    def __init__(self, model, runtime: Runtime, block_size: int, num_blocks: int, num_slots: int):
+        if not model.loaded:
+            raise InvalidArgumentError("the model has no weights yet; load them before building a runner")
+        self.model = model
+        self.runtime = runtime
+        self.block_size = block_size
+        self.num_blocks = num_blocks
+        self.needs = model.cache_needs()
+        groups = plan_groups(self.needs, block_size, num_blocks)
+        self.cache = CacheManager(groups, num_slots)
+        self.storage = CacheStorage(self.needs, groups, num_slots, runtime)
+        self.vocab_size = model.vocab_size
+        self.steps = 0
+
+    # --- construction helpers -----------------------------------------------------------------
+    @classmethod
+    def from_folder(cls, folder: str, dtype="bfloat16", device="cuda:0", block_size: int = 16,
+                    num_blocks: int = 256, num_slots: int = 8, progress=None) -> "ModelRunner":
+        runtime = Runtime(device, dtype)
+        config = load_config(folder)
+        model = build_model(config, runtime)
+        checkpoint = Checkpoint(folder)
+        try:
+            tensors = load_tensors(checkpoint, model.tensor_specs(), runtime.dtype, runtime.device, progress)
+        finally:
+            checkpoint.close()
+        model.load(tensors)
+        return cls(model, runtime, block_size, num_blocks, num_slots)
+
+    # --- the step ---------------------------------------------------------------------------------
+    def prepare(self, entries: Sequence[StepEntry]) -> StepBatch:
+        return build_batch(entries, self.cache, self.vocab_size, self.runtime.device)
+
+    def run(self, batch: StepBatch) -> Optional[torch.Tensor]:
+        self.steps += 1
+        return self.model.forward(batch, self.storage)
+
+    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        """Logits ``[wanted, vocab]`` (32-bit, on the device) in the order of the entries and their ``want``."""
+        return self.run(self.prepare(entries))

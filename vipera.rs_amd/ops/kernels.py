@@ -1,0 +1,202 @@
+"""Python bindings of the HIP kernels: shape checks on the host, then one launch on the current stream.
+
+Every function takes device tensors, checks that their shapes and dtypes are what the kernel
+and its grid assume, and launches on ``torch.cuda.current_stream()``.  There is no fallback:
+when a library cannot be built or loaded the call raises.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from ..errors import InternalError, InvalidArgumentError, UnsupportedError
+from .build import load_module
+
+_DT = {torch.float32: 0, torch.bfloat16: 1}
+_p = ctypes.c_void_p
+_i = ctypes.c_int
+_ll = ctypes.c_longlong
+_f = ctypes.c_float
+
+
+def _dt(tensor: torch.Tensor, what: str) -> int:
+    if tensor.dtype not in _DT:
+        raise UnsupportedError(f"{what} has dtype {tensor.dtype}; float32 and bfloat16 are implemented")
+    return _DT[tensor.dtype]
+
+
+def _ptr(tensor: Optional[torch.Tensor]):
+    return _p(tensor.data_ptr()) if tensor is not None else _p(0)
+
+
+def _stream():
+    return _p(torch.cuda.current_stream().cuda_stream)
+
+
+def _need(cond: bool, text: str) -> None:
+    if not cond:
+        raise InvalidArgumentError(text)
+
+
+def _dev(*tensors: Optional[torch.Tensor]) -> None:
+    for tensor in tensors:
+        if tensor is not None and not tensor.is_cuda:
+            raise InvalidArgumentError("kernel operands must live on the GPU; got a CPU tensor")
+
+
+def _status(code: int, name: str) -> None:
+    if code == 0:
+        return
+    if code == -1:
+        raise InvalidArgumentError(f"{name}: the launcher refused its arguments")
+    if code == -2:
+        raise UnsupportedError(f"{name}: a size is outside what this kernel is built for")
+    raise InternalError(f"{name}: HIP error {code} at launch")
+
+
+_signatures_done = set()
+
+
+def _fn(module: str, name: str, argtypes):
+    library = load_module(module)
+    fn = getattr(library, name)
+    if name not in _signatures_done:
+        fn.argtypes = argtypes
+        fn.restype = ctypes.c_int
+        _signatures_done.add(name)
+    return fn
+
+
+# ----------------------------------------------------------------------------------------------
+def embed_gather(table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor) -> None:
+    """``out[t, :] = table[tokens[t], :]`` widened to 32-bit.  The caller has checked the ids."""
+    _dev(table, tokens, out)
+    num_tokens, width = out.shape
+    _need(table.dim() == 2 and table.shape[1] == width and table.is_contiguous(), "embed_gather: table shape")
+    _need(tokens.dtype == torch.int32 and tokens.numel() >= num_tokens and tokens.is_contiguous(), "embed_gather: tokens")
+    _need(out.dtype == torch.float32 and out.is_contiguous(), "embed_gather: out must be contiguous float32")
+    fn = _fn("elementwise", "vk_embed_gather", [_p, _i, _p, _p, _i, _i, _p])
+    _status(fn(_ptr(table), _dt(table, "table"), _ptr(tokens), _ptr(out), num_tokens, width, _stream()), "embed_gather")
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor,
+            rows: Optional[torch.Tensor] = None) -> None:
+    """``out[r] = x[rows[r]] * rsqrt(mean(x^2) + eps) * weight`` (``rows`` absent: every row in order)."""
+    _dev(x, weight, out, rows)
+    num_rows, width = out.shape
+    _need(x.dtype == torch.float32 and x.dim() == 2 and x.shape[1] == width and x.is_contiguous(), "rmsnorm: x")
+    _need(weight.dtype == torch.float32 and weight.numel() == width and weight.is_contiguous(), "rmsnorm: weight")
+    _need(out.is_contiguous(), "rmsnorm: out must be contiguous")
+    if rows is None:
+        _need(x.shape[0] >= num_rows, "rmsnorm: fewer input rows than output rows")
+    else:
+        _need(rows.dtype == torch.int32 and rows.numel() >= num_rows and rows.is_contiguous(), "rmsnorm: rows")
+    fn = _fn("elementwise", "vk_rmsnorm", [_p, _p, _p, _p, _i, _i, _i, _f, _p])
+    _status(fn(_ptr(x), _ptr(weight), _ptr(rows), _ptr(out), _dt(out, "out"), num_rows, width, float(eps), _stream()),
+            "rmsnorm")
+
+
+def rope_kvwrite(qkv: torch.Tensor, positions: torch.Tensor, inv_freq: Optional[torch.Tensor], rotary_dim: int,
+                 k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor], entry_of_token: torch.Tensor,
+                 block_table: Optional[torch.Tensor], heads: int, kv_heads: int, head_dim: int) -> None:
+    """Rotate the q and k heads of ``qkv`` in place, then store the tokens' K and V in their pages.
+
+    ``k_cache``/``v_cache``: ``[pages, kv_heads, block_size, head_dim]``; ``block_table``: ``[entries, width]``.
+    The caller guarantees that every token's page exists in its entry's row of the table.
+    """
+    _dev(qkv, positions, inv_freq, k_cache, v_cache, entry_of_token, block_table)
+    num_tokens = qkv.shape[0]
+    _need(qkv.dim() == 2 and qkv.shape[1] == (heads + 2 * kv_heads) * head_dim and qkv.is_contiguous(),
+          "rope_kvwrite: qkv must be [tokens, (heads + 2 kv_heads) * head_dim]")
+    _need(positions.dtype == torch.int32 and positions.numel() >= num_tokens, "rope_kvwrite: positions")
+    _need(0 <= rotary_dim <= head_dim and rotary_dim % 2 == 0, "rope_kvwrite: rotary_dim")
+    if rotary_dim:
+        _need(inv_freq is not None and inv_freq.dtype == torch.float32 and inv_freq.numel() == rotary_dim // 2,
+              "rope_kvwrite: inv_freq must hold rotary_dim / 2 floats")
+    table_width = block_size = 0
+    if k_cache is not None:
+        _need(v_cache is not None and block_table is not None, "rope_kvwrite: cache without table")
+        _need(k_cache.dim() == 4 and k_cache.shape[1] == kv_heads and k_cache.shape[3] == head_dim
+              and k_cache.shape == v_cache.shape and k_cache.dtype == qkv.dtype == v_cache.dtype
+              and k_cache.is_contiguous() and v_cache.is_contiguous(), "rope_kvwrite: cache shape or dtype")
+        _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(),
+              "rope_kvwrite: block table")
+        _need(entry_of_token.dtype == torch.int32 and entry_of_token.numel() >= num_tokens, "rope_kvwrite: entries")
+        table_width, block_size = block_table.shape[1], k_cache.shape[2]
+    fn = _fn("elementwise", "vk_rope_kvwrite", [_p, _i, _p, _p, _i, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p])
+    _status(fn(_ptr(qkv), _dt(qkv, "qkv"), _ptr(positions), _ptr(inv_freq), rotary_dim, _ptr(k_cache), _ptr(v_cache),
+               _ptr(entry_of_token), _ptr(block_table), table_width, block_size, num_tokens, heads, kv_heads,
+               head_dim, _stream()), "rope_kvwrite")
+
+
+def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:
+    """``out = up * silu(gate)`` with ``gate_up = [gate | up]`` along the last axis."""
+    _dev(gate_up, out)
+    num_tokens, inter = out.shape
+    _need(gate_up.shape == (num_tokens, 2 * inter) and gate_up.dtype == out.dtype and gate_up.is_contiguous()
+          and out.is_contiguous(), "swiglu: gate_up must be [tokens, 2 * intermediate] of out's dtype")
+    fn = _fn("elementwise", "vk_swiglu", [_p, _p, _i, _i, _i, _p])
+    _status(fn(_ptr(gate_up), _ptr(out), _dt(out, "out"), num_tokens, inter, _stream()), "swiglu")
+
+
+def fill_normal(out: torch.Tensor, key: int, std: float, offset: float = 0.0) -> None:
+    """Fill with ``offset + std * n_i``, ``n_i`` the counter-based normal stream of ``key``."""
+    _dev(out)
+    _need(out.is_contiguous(), "fill_normal: out must be contiguous")
+    fn = _fn("elementwise", "vk_fill_normal", [_p, _i, _ll, ctypes.c_ulonglong, _f, _f, _p])
+    _status(fn(_ptr(out), _dt(out, "out"), out.numel(), key & ((1 << 64) - 1), float(std), float(offset), _stream()),
+            "fill_normal")
+
+
+# ----------------------------------------------------------------------------------------------
+def gemm_generic(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
+                 accumulate: bool = False) -> None:
+    """``out (+)= a @ w.T + bias`` in 32-bit FMA; ``a`` and ``out`` may be row-strided views."""
+    _dev(a, w, bias, out)
+    _need(a.dim() == 2 and w.dim() == 2 and out.dim() == 2, "gemm: operands must be matrices")
+    m, k = a.shape
+    n = w.shape[0]
+    _need(w.shape[1] == k and out.shape == (m, n), f"gemm: shapes {tuple(a.shape)} x {tuple(w.shape)}^T -> {tuple(out.shape)}")
+    _need(a.stride(1) == 1 and out.stride(1) == 1 and w.is_contiguous(), "gemm: inner strides must be 1")
+    _need(a.stride(0) >= k or m == 1, "gemm: a's row stride")
+    _need(out.stride(0) >= n or m == 1, "gemm: out's row stride")
+    if bias is not None:
+        _need(bias.dtype == torch.float32 and bias.numel() == n and bias.is_contiguous(), "gemm: bias must be float32 [n]")
+    if accumulate:
+        _need(out.dtype == torch.float32, "gemm: accumulation needs a float32 output")
+    fn = _fn("gemm_generic", "vk_gemm_generic", [_p, _i, _p, _i, _p, _p, _i, _i, _i, _i, _ll, _ll, _i, _p])
+    lda = a.stride(0) if m > 1 else max(a.stride(0), k)
+    ldc = out.stride(0) if m > 1 else max(out.stride(0), n)
+    _status(fn(_ptr(a), _dt(a, "a"), _ptr(w), _dt(w, "w"), _ptr(bias), _ptr(out), _dt(out, "out"), m, n, k, lda, ldc,
+               1 if accumulate else 0, _stream()), "gemm_generic")
+
+
+# ----------------------------------------------------------------------------------------------
+def attn_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
+                 positions: torch.Tensor, entry_of_token: torch.Tensor, block_table: torch.Tensor,
+                 heads: int, kv_heads: int, head_dim: int, scale: float, window: int) -> None:
+    """Causal GQA over the paged cache for every token of the step, in 32-bit arithmetic.
+
+    ``q``: a view ``[tokens, >= heads * head_dim]`` whose row holds the query heads first (the fused
+    qkv buffer qualifies); ``out``: ``[tokens, heads * head_dim]``.
+    """
+    _dev(q, k_cache, v_cache, out, positions, entry_of_token, block_table)
+    num_tokens = out.shape[0]
+    _need(q.dim() == 2 and q.shape[0] == num_tokens and q.stride(1) == 1 and q.shape[1] >= heads * head_dim, "attention: q")
+    _need(out.shape == (num_tokens, heads * head_dim) and out.is_contiguous() and out.dtype == q.dtype, "attention: out")
+    _need(k_cache.dim() == 4 and k_cache.shape[1] == kv_heads and k_cache.shape[3] == head_dim
+          and k_cache.shape == v_cache.shape and k_cache.dtype == q.dtype == v_cache.dtype
+          and k_cache.is_contiguous() and v_cache.is_contiguous(), "attention: cache shape or dtype")
+    _need(positions.dtype == torch.int32 and positions.numel() >= num_tokens, "attention: positions")
+    _need(entry_of_token.dtype == torch.int32 and entry_of_token.numel() >= num_tokens, "attention: entries")
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(), "attention: table")
+    _need(heads % kv_heads == 0, "attention: heads must be a multiple of kv_heads")
+    if head_dim > 256:
+        raise UnsupportedError(f"attention: head_dim {head_dim} is above the kernel's limit of 256")
+    fn = _fn("attn_generic", "vk_attn_generic",
+             [_p, _ll, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _i, _p])
+    _status(fn(_ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(out), _dt(q, "q"), _ptr(positions),
+               _ptr(entry_of_token), _ptr(block_table), block_table.shape[1], k_cache.shape[2], num_tokens, heads,
+               kv_heads, head_dim, float(scale), int(window), _stream()), "attn_generic")

@@ -1,0 +1,103 @@
+"""Grouped-query attention over the paged cache.
+
+Order of work as in the reference's batched pass (crates/vipera-backend-cpu/src/model.rs:1005-1126):
+``q, k, v = h W^T + b``; rotate q and k; write K (rotated) and V of every token of the step into the
+cache; attend causally by count (a token at position p reads positions ``<= p`` of its own request,
+or the last ``window`` of them); ``x += attn Wo^T``.  The three projections run as one product over
+the concatenated weight ``[Wq; Wk; Wv]``, whose rows equal the separate products' rows.
+"""
+from __future__ import annotations
+
+import math
+from typing import Dict, List, Optional
+
+import torch
+
+from ..config.base import PartSpec
+from ..errors import InvalidArgumentError
+from ..ops import kernels
+from ..ops.attention import paged_attention
+from ..ops.linear import linear
+from ..weights.checkpoint import MATRIX, VECTOR, TensorSpec
+from .base import KVCacheSpec, Mixer, register_mixer
+
+
+def _cat(tensors: List[torch.Tensor]) -> torch.Tensor:
+    dtypes = {t.dtype for t in tensors}
+    if len(dtypes) > 1:  # a matrix kept in 32-bit pulls its companions up with it
+        tensors = [t.float() for t in tensors]
+    return torch.cat(tensors, dim=0).contiguous()
+
+
+class Attention(Mixer):
+    def __init__(self, spec: PartSpec, prefix: str, runtime):
+        super().__init__(spec, prefix, runtime)
+        p = spec.params
+        self.hidden = int(p["hidden"])
+        self.heads = int(p["heads"])
+        self.kv_heads = int(p["kv_heads"])
+        self.head_dim = int(p["head_dim"])
+        self.window = int(p.get("window") or 0)
+        self.qkv_bias = bool(p.get("qkv_bias", False))
+        self.out_bias = bool(p.get("out_bias", False))
+        scale = p.get("scale")
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.head_dim)
+        if self.heads % self.kv_heads:
+            raise InvalidArgumentError(f"heads {self.heads} is not a multiple of kv_heads {self.kv_heads}")
+        self.q_width = self.heads * self.head_dim
+        self.kv_width = self.kv_heads * self.head_dim
+        self.w_qkv = self.b_qkv = self.w_o = self.b_o = None
+
+    @classmethod
+    def declare(cls, spec: PartSpec, prefix: str) -> List[TensorSpec]:
+        p = spec.params
+        base = f"{prefix}{p['name']}."
+        hidden, hd = int(p["hidden"]), int(p["head_dim"])
+        q, kv = int(p["heads"]) * hd, int(p["kv_heads"]) * hd
+        specs: List[TensorSpec] = []
+        for name, rows in (("q", q), ("k", kv), ("v", kv)):
+            specs.append(TensorSpec(f"{base}{name}_proj.weight", (rows, hidden), MATRIX))
+            if p.get("qkv_bias"):
+                specs.append(TensorSpec(f"{base}{name}_proj.bias", (rows,), VECTOR))
+        specs.append(TensorSpec(base + "o_proj.weight", (hidden, q), MATRIX))
+        if p.get("out_bias"):
+            specs.append(TensorSpec(base + "o_proj.bias", (hidden,), VECTOR))
+        return specs
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        base = f"{self.prefix}{self.spec.params['name']}."
+        self.w_qkv = _cat([tensors[base + f"{n}_proj.weight"] for n in "qkv"])
+        if self.qkv_bias:
+            self.b_qkv = torch.cat([tensors[base + f"{n}_proj.bias"] for n in "qkv"]).contiguous()
+        self.w_o = tensors[base + "o_proj.weight"]
+        if self.out_bias:
+            self.b_o = tensors[base + "o_proj.bias"]
+
+    def cache_spec(self) -> Optional[KVCacheSpec]:
+        return KVCacheSpec(self.kv_heads, self.head_dim, self.window)
+
+    def forward(self, h, batch, cache, state, position, residual, reads_only: bool = False) -> None:
+        tokens = h.shape[0]
+        qkv = self.runtime.empty((tokens, self.q_width + 2 * self.kv_width))
+        linear(h, self.w_qkv, self.b_qkv, qkv)
+        table = batch.block_tables[cache.group]
+        fused = position.fused_rotary()
+        if fused is None:
+            position.apply(qkv, batch, self.heads, self.kv_heads, self.head_dim)
+            inv_freq, rotary_dim = None, 0
+        else:
+            inv_freq, rotary_dim = fused
+        if reads_only:
+            if rotary_dim:
+                kernels.rope_kvwrite(qkv, batch.positions, inv_freq, rotary_dim, None, None, batch.entry_of_token,
+                                     None, self.heads, self.kv_heads, self.head_dim)
+        else:
+            kernels.rope_kvwrite(qkv, batch.positions, inv_freq, rotary_dim, cache.k, cache.v, batch.entry_of_token,
+                                 table, self.heads, self.kv_heads, self.head_dim)
+        attn = self.runtime.empty((tokens, self.q_width))
+        paged_attention(qkv, cache.k, cache.v, attn, batch, table, self.heads, self.kv_heads, self.head_dim,
+                        self.scale, self.window)
+        linear(attn, self.w_o, self.b_o, residual, accumulate=True)
+
+
+register_mixer("attention", Attention)

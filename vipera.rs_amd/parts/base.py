@@ -1,0 +1,175 @@
+"""Interfaces of the parts a layer is put together from, and the registries that name them.
+
+A part is built from a :class:`~vipera_rs_amd.config.PartSpec` (its kind and parameters), a
+tensor-name prefix and a :class:`~vipera_rs_amd.runtime.Runtime`.  It knows nothing about the model
+it sits in.  Before any GPU work a part can *declare* the tensors it needs (names, shapes, how they
+are kept), which is what the loader checks a model folder against and what random weights are made
+from.
+
+Kinds of parts and what each must provide:
+
+``Norm``              ``forward(x, out=None, rows=None) -> h``: ``x`` is the 32-bit residual
+                      ``[tokens, width]``; ``h`` has the run's dtype; ``rows`` (int32 indices)
+                      selects rows.
+``PositionEncoding``  ``apply(qkv, batch, heads, kv_heads, head_dim)`` rotates (or otherwise marks)
+                      the q and k heads of the fused buffer in place; ``fused_rotary()`` may return
+                      ``(inv_freq, rotary_dim)`` to let a mixer fold the rotation into its cache write.
+``Mixer``             ``cache_spec()`` / ``state_spec()`` say what it keeps per request;
+                      ``forward(h, batch, cache, state, position, residual, reads_only)`` adds its
+                      output to ``residual`` (32-bit, in place).
+``FeedForward``       ``forward(h, batch, residual)`` adds its output to ``residual``.
+``Block``             ``forward(x, batch, cache, state, reads_only)`` runs its parts on the residual ``x``.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Callable, Dict, List, Optional, Tuple, Type
+
+import torch
+
+from ..config.base import LayerSpec, PartSpec
+from ..errors import UnsupportedError
+from ..weights.checkpoint import TensorSpec
+
+
+@dataclass(frozen=True)
+class KVCacheSpec:
+    """Keys and values in pages: per position ``kv_heads * head_dim`` of each; ``window`` 0 keeps all."""
+
+    kv_heads: int
+    head_dim: int
+    window: int = 0
+
+
+@dataclass(frozen=True)
+class StateSpec:
+    """Per-request state of fixed size: one tensor of ``shape`` and ``dtype`` per slot."""
+
+    shape: Tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+class Part:
+    kind = ""
+
+    def __init__(self, spec: PartSpec, prefix: str, runtime):
+        self.spec = spec
+        self.prefix = prefix
+        self.runtime = runtime
+
+    @classmethod
+    def declare(cls, spec: PartSpec, prefix: str) -> List[TensorSpec]:
+        """Tensors this part needs, by full name. No GPU is touched."""
+        return []
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        """Take the declared tensors (already on the device in their kept dtype)."""
+
+
+class Norm(Part):
+    def forward(self, x: torch.Tensor, out: Optional[torch.Tensor] = None,
+                rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    def fused_rotary(self):
+        return None
+
+    def apply(self, qkv: torch.Tensor, batch, heads: int, kv_heads: int, head_dim: int) -> None:
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    def cache_spec(self) -> Optional[KVCacheSpec]:
+        return None
+
+    def state_spec(self) -> Optional[StateSpec]:
+        return None
+
+    def forward(self, h, batch, cache, state, position, residual, reads_only: bool = False) -> None:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, h, batch, residual) -> None:
+        raise NotImplementedError
+
+
+class Block:
+    """An arrangement of a layer's parts. Built from a LayerSpec and the part registries."""
+
+    kind = ""
+
+    def __init__(self, spec: LayerSpec, runtime):
+        self.spec = spec
+        self.runtime = runtime
+
+    @classmethod
+    def declare(cls, spec: LayerSpec) -> List[TensorSpec]:
+        raise NotImplementedError
+
+    def load(self, tensors) -> None:
+        raise NotImplementedError
+
+    def forward(self, x, batch, cache, state, reads_only: bool = False) -> None:
+        raise NotImplementedError
+
+
+# --- registries ---------------------------------------------------------------------------------
+_REGISTRIES: Dict[str, Dict[str, type]] = {
+    "mixer": {}, "ffn": {}, "norm": {}, "position": {}, "block": {}, "embedding": {}, "head": {},
+}
+
+
+def _register(family: str, kind: str, cls: type) -> None:
+    cls.kind = kind
+    _REGISTRIES[family][kind] = cls
+
+
+def _lookup(family: str, kind: str) -> type:
+    registry = _REGISTRIES[family]
+    if kind not in registry:
+        known = ", ".join(registry) or "(none)"
+        raise UnsupportedError(f"{family} kind \"{kind}\" is not registered; registered: {known}")
+    return registry[kind]
+
+
+def register_mixer(kind: str, cls: Type[Mixer]) -> None:
+    _register("mixer", kind, cls)
+
+
+def register_ffn(kind: str, cls: Type[FeedForward]) -> None:
+    _register("ffn", kind, cls)
+
+
+def register_norm(kind: str, cls: Type[Norm]) -> None:
+    _register("norm", kind, cls)
+
+
+def register_position(kind: str, cls: Type[PositionEncoding]) -> None:
+    _register("position", kind, cls)
+
+
+def register_block(kind: str, cls: Type[Block]) -> None:
+    _register("block", kind, cls)
+
+
+def register_embedding(kind: str, cls: Type[Part]) -> None:
+    _register("embedding", kind, cls)
+
+
+def register_head(kind: str, cls: Type[Part]) -> None:
+    _register("head", kind, cls)
+
+
+def part_class(family: str, kind: str) -> type:
+    return _lookup(family, kind)
+
+
+def registered(family: str) -> List[str]:
+    return list(_REGISTRIES[family])
+
+
+def unregister(family: str, kind: str) -> None:
+    _REGISTRIES[family].pop(kind, None)

@@ -1,0 +1,67 @@
+"""Token embedding and the output projection.
+
+Reference: the embedding is a row read with no scaling (crates/vipera-backend-cpu/src/model.rs:607-616);
+the head is ``logits = Wout h`` on the normed rows that are wanted, and when the model has no output
+matrix the embedding table serves as one (model.rs:425, 1201-1237).
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional
+
+import torch
+
+from ..config.base import PartSpec
+from ..ops import kernels
+from ..ops.linear import linear
+from ..weights.checkpoint import MATRIX, TensorSpec
+from .base import Part, register_embedding, register_head
+
+
+class Embedding(Part):
+    def __init__(self, spec: PartSpec, prefix: str, runtime):
+        super().__init__(spec, prefix, runtime)
+        self.vocab = int(spec.params["vocab"])
+        self.width = int(spec.params["width"])
+        self.table: Optional[torch.Tensor] = None
+
+    @classmethod
+    def declare(cls, spec: PartSpec, prefix: str) -> List[TensorSpec]:
+        return [TensorSpec(f"{prefix}{spec.params['name']}.weight",
+                           (int(spec.params["vocab"]), int(spec.params["width"])), MATRIX)]
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        self.table = tensors[f"{self.prefix}{self.spec.params['name']}.weight"]
+
+    def forward(self, tokens: torch.Tensor, count: int) -> torch.Tensor:
+        out = self.runtime.empty((count, self.width), torch.float32)
+        kernels.embed_gather(self.table, tokens, out)
+        return out
+
+
+class LMHead(Part):
+    def __init__(self, spec: PartSpec, prefix: str, runtime):
+        super().__init__(spec, prefix, runtime)
+        self.vocab = int(spec.params["vocab"])
+        self.width = int(spec.params["width"])
+        self.tied_to = spec.params.get("tied_to")
+        self.weight: Optional[torch.Tensor] = None
+
+    @classmethod
+    def declare(cls, spec: PartSpec, prefix: str) -> List[TensorSpec]:
+        if spec.params.get("tied_to"):
+            return []
+        return [TensorSpec(f"{prefix}{spec.params['name']}.weight",
+                           (int(spec.params["vocab"]), int(spec.params["width"])), MATRIX)]
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        name = self.tied_to if self.tied_to else f"{self.prefix}{self.spec.params['name']}"
+        self.weight = tensors[f"{name}.weight"]  # tied: the same buffer, no copy
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        logits = self.runtime.empty((h.shape[0], self.vocab), torch.float32)
+        linear(h, self.weight, None, logits)
+        return logits
+
+
+register_embedding("embedding", Embedding)
+register_head("lm_head", LMHead)
