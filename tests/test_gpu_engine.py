@@ -1,0 +1,156 @@
+"""Generation through the entry point: greedy tokens against the plain implementation, sampling that
+does not depend on a request's company, preemption when pages run out, cancelling, long decoding."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import CONFIG_A, CONFIG_B, make_folder, random_tokens
+from plain import qwen2_plain
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    return {
+        "A": make_folder(tmp_path_factory.mktemp("engine_A"), CONFIG_A, 0, torch.float32),
+        "B": make_folder(tmp_path_factory.mktemp("engine_B"), CONFIG_B, 1, torch.float32),
+    }
+
+
+def _engine(folder, **kw):
+    from vipera_rs_amd import Engine
+    kw.setdefault("dtype", "float32")
+    return Engine(folder, **kw)
+
+
+def test_greedy_generation_equals_the_plain_implementation(folders):
+    # workload of the first tiny configuration: prompts of 5, 8 and 13 tokens, 8 new tokens each
+    cfg, weights = qwen2_plain.load_folder(folders["A"])
+    prompts = [random_tokens(CONFIG_A["vocab_size"], n, 40 + n) for n in (5, 8, 13)]
+    want = [qwen2_plain.greedy_generate(cfg, weights, p, 8) for p in prompts]
+    engine = _engine(folders["A"], block_size=16, num_blocks=12, max_num_seqs=4)
+    got = engine.generate(prompts, max_new_tokens=8)
+    assert [g.tokens for g in got] == want
+    assert all(g.finish == "length" and g.prompt_tokens == len(p) for g, p in zip(got, prompts))
+    assert engine.runner.cache.check() == "" and engine.runner.cache.live_requests() == 0
+    # the last sampled token is never fed back (engine.rs:1509-1514)
+    assert [g.processed_tokens for g in got] == [len(p) + 7 for p in prompts]
+
+
+def test_greedy_generation_with_an_untied_head_and_windowed_layers(folders):
+    # tied embeddings make a random model repeat its last token; the second configuration does not
+    cfg, weights = qwen2_plain.load_folder(folders["B"])
+    prompts = [random_tokens(CONFIG_B["vocab_size"], n, 60 + n) for n in (3, 30, 11)]
+    want = [qwen2_plain.greedy_generate(cfg, weights, p, 12) for p in prompts]
+    assert any(len(set(w)) > 3 for w in want), "the continuation should not be one repeated token"
+    engine = _engine(folders["B"], block_size=8, num_blocks=24, max_num_seqs=3, chunk_size=7)
+    assert [g.tokens for g in engine.generate(prompts, max_new_tokens=12)] == want
+
+
+def test_bfloat16_generation_runs_and_mostly_agrees(folders):
+    prompts = [random_tokens(CONFIG_A["vocab_size"], n, 40 + n) for n in (5, 8, 13)]
+    ref = _engine(folders["A"], num_blocks=12, max_num_seqs=4).generate(prompts, max_new_tokens=8)
+    got = _engine(folders["A"], dtype="bfloat16", num_blocks=12, max_num_seqs=4).generate(prompts, max_new_tokens=8)
+    assert all(len(g.tokens) == 8 for g in got)
+    assert sum(a.tokens[0] == b.tokens[0] for a, b in zip(ref, got)) >= 2
+
+
+def test_end_of_sequence_stops_and_is_kept_in_the_tokens(folders):
+    cfg, weights = qwen2_plain.load_folder(folders["A"])
+    prompt = random_tokens(CONFIG_A["vocab_size"], 9, 3)
+    free_run = qwen2_plain.greedy_generate(cfg, weights, prompt, 6)
+    eos = free_run[3]
+    stop_at = free_run.index(eos)
+    engine = _engine(folders["A"], num_blocks=8)
+    streamed = []
+    rid = engine.add_request(prompt, 6, eos_token_ids=[eos], on_token=streamed.append)
+    done = None
+    while done is None:
+        for g in engine.step().finished:
+            done = g
+    assert done.request == rid and done.finish == "stop"
+    assert done.tokens == free_run[:stop_at + 1]
+    assert streamed == free_run[:stop_at]  # the end token is not streamed (engine.rs:571-575)
+
+
+def test_seeded_sampling_is_independent_of_company_and_arrival(folders):
+    # workload of the second tiny configuration: prompts of 1, 7, 19 and 33 tokens in portions of 6
+    # mixed with decoding, temperature 0.8 with a seed, 10 new tokens each
+    from vipera_rs_amd import SamplingParams
+    prompts = [random_tokens(CONFIG_B["vocab_size"], n, 70 + n) for n in (1, 7, 19, 33)]
+    params = [SamplingParams(temperature=0.8, seed=11 + k) for k in range(4)]
+    alone = []
+    for p, s in zip(prompts, params):
+        engine = _engine(folders["B"], block_size=8, num_blocks=16, max_num_seqs=1, chunk_size=6)
+        alone.append(engine.generate([p], 10, s)[0].tokens)
+    engine = _engine(folders["B"], block_size=8, num_blocks=40, max_num_seqs=4, chunk_size=6,
+                     max_num_batched_tokens=16)
+    together = [g.tokens for g in engine.generate(prompts, 10, params)]
+    assert together == alone
+    engine = _engine(folders["B"], block_size=8, num_blocks=40, max_num_seqs=4, chunk_size=6,
+                     max_num_batched_tokens=16)
+    order = [3, 1, 0, 2]
+    shuffled = engine.generate([prompts[i] for i in order], 10, [params[i] for i in order])
+    assert [g.tokens for g in shuffled] == [alone[i] for i in order]
+    assert all(len(t) == 10 for t in alone)
+
+
+def test_preemption_when_pages_run_out_keeps_every_request_right(folders):
+    prompts = [random_tokens(CONFIG_A["vocab_size"], n, 90 + n) for n in (30, 28, 25, 31)]
+    solo = []
+    for p in prompts:
+        solo.append(_engine(folders["A"], num_blocks=8, max_num_seqs=1).generate([p], 40)[0].tokens)
+    # 4 requests growing to ~70 tokens need ~20 pages of 16; 10 pages force preemption
+    engine = _engine(folders["A"], block_size=16, num_blocks=10, max_num_seqs=4, chunk_size=16)
+    got = engine.generate(prompts, 40)
+    assert [g.tokens for g in got] == solo
+    assert engine.stats()["preemptions"] > 0 and sum(g.preemptions for g in got) == engine.stats()["preemptions"]
+    assert engine.runner.cache.check() == "" and engine.runner.cache.live_requests() == 0
+    assert engine.runner.cache.free_blocks(0) == 10
+
+
+def test_a_request_that_can_never_fit_is_refused_at_admission(folders):
+    from vipera_rs_amd.errors import InfeasibleError, InvalidArgumentError
+    engine = _engine(folders["A"], block_size=16, num_blocks=2, max_num_seqs=2)
+    with pytest.raises(InfeasibleError):
+        engine.add_request(random_tokens(256, 40, 1), 8)
+    with pytest.raises(InvalidArgumentError):
+        engine.add_request([], 8)
+    with pytest.raises(InvalidArgumentError):
+        engine.add_request([1, 2], 0)
+    with pytest.raises(InvalidArgumentError):
+        engine.add_request([1, 256], 4)
+    assert not engine.has_work()
+
+
+def test_cancel_frees_pages_at_a_step_boundary(folders):
+    engine = _engine(folders["A"], block_size=16, num_blocks=8, max_num_seqs=2)
+    a = engine.add_request(random_tokens(256, 20, 1), 30)
+    b = engine.add_request(random_tokens(256, 20, 2), 5)
+    engine.step()
+    assert engine.runner.cache.used_blocks(0) == 4
+    cancelled = engine.cancel(a)
+    assert cancelled.finish == "cancelled" and engine.runner.cache.used_blocks(0) == 2
+    done = []
+    while engine.has_work():
+        done += engine.step().finished
+    assert [g.request for g in done] == [b] and engine.runner.cache.used_blocks(0) == 0
+    assert engine.runner.cache.check() == ""
+
+
+def test_long_decoding_follows_the_plain_implementation(folders):
+    cfg, weights = qwen2_plain.load_folder(folders["B"])
+    prompt = random_tokens(CONFIG_B["vocab_size"], 6, 5)
+    engine = _engine(folders["B"], block_size=8, num_blocks=40, max_num_seqs=1)
+    tokens = engine.generate([prompt], 240)[0].tokens
+    assert len(tokens) == 240
+    logits = qwen2_plain.forward(cfg, weights, prompt + tokens[:-1])
+    checked = 0
+    for k, token in enumerate(tokens):
+        row = logits[len(prompt) - 1 + k]
+        order = np.argsort(row)
+        if row[order[-1]] - row[order[-2]] > 1e-4 * np.max(np.abs(row)):
+            assert token == int(order[-1]), f"token {k} differs from the plain implementation"
+            checked += 1
+    assert checked > 200

@@ -1,0 +1,378 @@
+// Sampling on the device: logit penalties, greedy argmax, and temperature sampling with the
+// top-k, top-p and min-p cuts. One workgroup of 1024 threads per row of logits.
+//
+// Meaning of the options as in the reference (crates/vipera-sampler/src/lib.rs):
+//   greedy        argmax over finite logits, ties to the lowest id (135-156)
+//   temperature   weights exp(l/T - peak), peak = best l/T; the denominator is the mass of every
+//                 finite logit (172-203)
+//   top_k         keep the k best by (logit descending, id ascending); 0 keeps all (176-186, 440-444)
+//   top_p         keep the shortest head whose mass reaches top_p * total mass (213-229, 421-430)
+//   min_p         drop weights below min_p times the best weight (231-232)
+//   draw          target = u * kept mass, first candidate whose running sum exceeds it (234-242)
+//   penalties     a token seen recently: positive logit / factor, negative * factor, minus
+//                 presence + frequency * count; plus a per-token bias (596-616)
+// What differs: no sort. The cuts are found by radix selection over an order-preserving integer
+// key of the logit, masses are summed as 2^-40 fixed-point integers (so every sum is exact and has
+// no order), and the draw walks the kept tokens in id order. The kept set is the reference's up to
+// rounding at a cut's edge; which kept token a given u selects differs, the distribution does not.
+#include "common.h"
+
+namespace {
+constexpr int THREADS = 1024;
+constexpr int WAVES = THREADS / WAVE;
+constexpr float FIXED_ONE = 1099511627776.0f;  // 2^40
+
+__device__ __forceinline__ bool finite_f(float v) { return (__float_as_uint(v) & 0x7f800000u) != 0x7f800000u; }
+
+// larger float <=> larger key; finite keys are above 0x007fffff
+__device__ __forceinline__ uint32_t key_of(float v) {
+  const uint32_t b = __float_as_uint(v);
+  return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+
+__device__ __forceinline__ unsigned long long wave_sum_u64(unsigned long long v) {
+#pragma unroll
+  for (int off = WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, WAVE);
+  return v;
+}
+
+__device__ __forceinline__ unsigned long long block_sum_u64(unsigned long long v, unsigned long long* scratch) {
+  const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+  v = wave_sum_u64(v);
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  unsigned long long total = 0;
+  for (int i = 0; i < WAVES; ++i) total += scratch[i];
+  return total;
+}
+
+__device__ __forceinline__ unsigned long long fixed_weight(float logit, float scale, float peak) {
+  return (unsigned long long)(expf(logit * scale - peak) * FIXED_ONE);
+}
+
+struct Cut {
+  uint32_t key;     // keys above it are kept
+  int ties;         // of the tokens with exactly this key, the first `ties` by id are kept
+};
+
+// One row. Returns the chosen token in *out (or -1 when no logit is finite).
+__global__ __launch_bounds__(THREADS) void sample_kernel(const float* __restrict__ logits, int vocab,
+                                                         const float* __restrict__ temperature,
+                                                         const int* __restrict__ top_k,
+                                                         const float* __restrict__ top_p,
+                                                         const float* __restrict__ min_p,
+                                                         const double* __restrict__ uniform, int* __restrict__ out) {
+  __shared__ float red_f[16];
+  __shared__ int red_i[WAVES];
+  __shared__ unsigned long long red_u[WAVES];
+  __shared__ unsigned long long hist[256];
+  __shared__ uint32_t sh_key;
+  __shared__ long long sh_remaining;
+  __shared__ unsigned long long sh_below;
+
+  const int row = blockIdx.x, tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
+  const float* x = logits + (size_t)row * vocab;
+
+  // --- best finite logit, ties to the lowest id ----------------------------------------------
+  float best = -INFINITY;
+  int best_id = 0x7fffffff;
+  for (int i = tid; i < vocab; i += THREADS) {
+    const float v = x[i];
+    if (finite_f(v) && (v > best || (v == best && i < best_id))) {
+      best = v;
+      best_id = i;
+    }
+  }
+#pragma unroll
+  for (int off = WAVE / 2; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(best, off, WAVE);
+    const int oi = __shfl_xor(best_id, off, WAVE);
+    if (ov > best || (ov == best && oi < best_id)) {
+      best = ov;
+      best_id = oi;
+    }
+  }
+  if (lane == 0) {
+    red_f[wave] = best;
+    red_i[wave] = best_id;
+  }
+  __syncthreads();
+  best = red_f[0];
+  best_id = red_i[0];
+  for (int w = 1; w < WAVES; ++w)
+    if (red_f[w] > best || (red_f[w] == best && red_i[w] < best_id)) {
+      best = red_f[w];
+      best_id = red_i[w];
+    }
+  __syncthreads();
+  if (best_id == 0x7fffffff) {
+    if (tid == 0) out[row] = -1;
+    return;
+  }
+  const float temp = temperature[row];
+  if (!(temp > 0.f)) {
+    if (tid == 0) out[row] = best_id;
+    return;
+  }
+  const float scale = 1.0f / temp;
+  const float peak = best * scale;
+
+  // --- top-k: the key of the k-th best token and how many of its ties are inside --------------
+  Cut cut = {0u, 0x7fffffff};  // everything finite
+  const int k = top_k[row];
+  int finite_count = 0;
+  for (int i = tid; i < vocab; i += THREADS) finite_count += finite_f(x[i]) ? 1 : 0;
+  finite_count = (int)block_sum_u64((unsigned long long)finite_count, red_u);
+  if (k > 0 && k < finite_count) {
+    uint32_t prefix = 0;
+    long long remaining = k;  // the k-th best lies among the keys that match the prefix
+    for (int shift = 24; shift >= 0; shift -= 8) {
+      for (int b = tid; b < 256; b += THREADS) hist[b] = 0;
+      __syncthreads();
+      const uint32_t mask = shift == 24 ? 0u : (0xffffffffu << (shift + 8));
+      for (int i = tid; i < vocab; i += THREADS) {
+        const float v = x[i];
+        if (!finite_f(v)) continue;
+        const uint32_t key = key_of(v);
+        if ((key & mask) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1ull);
+      }
+      __syncthreads();
+      if (tid == 0) {
+        long long left = remaining;
+        int b = 255;
+        for (; b > 0; --b) {
+          if ((long long)hist[b] >= left) break;
+          left -= (long long)hist[b];
+        }
+        sh_key = prefix | ((uint32_t)b << shift);
+        sh_remaining = left;
+      }
+      __syncthreads();
+      prefix = sh_key;
+      remaining = sh_remaining;
+      __syncthreads();
+    }
+    cut.key = prefix;
+    cut.ties = (int)remaining;
+  }
+
+  // --- top-p: the shortest head of the top-k set whose mass reaches top_p * total --------------
+  const float p = top_p[row];
+  if (p < 1.0f) {
+    unsigned long long total = 0;
+    for (int i = tid; i < vocab; i += THREADS) {
+      const float v = x[i];
+      if (finite_f(v)) total += fixed_weight(v, scale, peak);
+    }
+    total = block_sum_u64(total, red_u);
+    const unsigned long long target = (unsigned long long)((double)p * (double)total);
+    // how many tokens share the top-k cut's key, and their weight: only cut.ties of them count
+    int at_cut = 0;
+    for (int i = tid; i < vocab; i += THREADS) {
+      const float v = x[i];
+      at_cut += (finite_f(v) && key_of(v) == cut.key) ? 1 : 0;
+    }
+    at_cut = (int)block_sum_u64((unsigned long long)at_cut, red_u);
+    const int cut_excess = cut.ties < at_cut ? at_cut - cut.ties : 0;
+    unsigned long long cut_weight = 0;
+    if (cut_excess > 0) {
+      const uint32_t kb = cut.key;
+      const float cv = __uint_as_float((kb & 0x80000000u) ? (kb & 0x7fffffffu) : ~kb);
+      cut_weight = fixed_weight(cv, scale, peak);
+    }
+    uint32_t prefix = 0;
+    unsigned long long above = 0;  // mass of keys above everything that matches the prefix
+    bool reached = true;
+    for (int shift = 24; shift >= 0; shift -= 8) {
+      for (int b = tid; b < 256; b += THREADS) hist[b] = 0;
+      __syncthreads();
+      const uint32_t mask = shift == 24 ? 0u : (0xffffffffu << (shift + 8));
+      for (int i = tid; i < vocab; i += THREADS) {
+        const float v = x[i];
+        if (!finite_f(v)) continue;
+        const uint32_t key = key_of(v);
+        if (key < cut.key) continue;  // outside the top-k set
+        if ((key & mask) == prefix) atomicAdd(&hist[(key >> shift) & 255u], fixed_weight(v, scale, peak));
+      }
+      __syncthreads();
+      if (tid == 0) {
+        if (cut_excess > 0 && (cut.key & mask) == prefix)
+          hist[(cut.key >> shift) & 255u] -= (unsigned long long)cut_excess * cut_weight;
+        unsigned long long running = above;
+        int b = 255;
+        bool found = false;
+        for (; b >= 0; --b) {
+          if (running + hist[b] >= target) {
+            found = true;
+            break;
+          }
+          running += hist[b];
+        }
+        if (!found) b = 0;
+        sh_key = prefix | ((uint32_t)b << shift);
+        sh_below = running;
+        sh_remaining = found ? 1 : 0;
+      }
+      __syncthreads();
+      prefix = sh_key;
+      above = sh_below;
+      reached = sh_remaining != 0;
+      __syncthreads();
+      if (!reached) break;
+    }
+    if (reached && prefix >= cut.key) {
+      // tokens with key == prefix all weigh the same; take as many as the target still needs
+      const float cv = __uint_as_float((prefix & 0x80000000u) ? (prefix & 0x7fffffffu) : ~prefix);
+      const unsigned long long w = fixed_weight(cv, scale, peak);
+      long long need = 1;
+      if (w > 0 && target > above) need = (long long)((target - above + w - 1) / w);
+      if (need < 1) need = 1;
+      int limit = 0x7fffffff;
+      if (prefix == cut.key) limit = cut.ties;
+      cut.key = prefix;
+      cut.ties = need < (long long)limit ? (int)need : limit;
+    }
+  }
+  const float floor_weight = min_p[row];  // the best weight is exp(0) = 1
+
+  // --- draw among the kept tokens in id order ------------------------------------------------------
+  // every wave owns a contiguous range of ids and walks it in runs of 64
+  const int span = ((vocab + WAVES - 1) / WAVES + WAVE - 1) / WAVE * WAVE;
+  const int begin = wave * span, end = min(vocab, begin + span);
+
+  // ties at the cut: rank base of every wave
+  int ties_here = 0;
+  for (int base = begin; base < end; base += WAVE) {
+    const int i = base + lane;
+    const float v = i < end ? x[i] : NAN;
+    ties_here += (finite_f(v) && key_of(v) == cut.key) ? 1 : 0;
+  }
+  ties_here = (int)wave_sum_u64((unsigned long long)ties_here);
+  if (lane == 0) red_i[wave] = ties_here;
+  __syncthreads();
+  int tie_base = 0;
+  for (int w = 0; w < wave; ++w) tie_base += red_i[w];
+  __syncthreads();
+
+  // kept mass of every wave
+  unsigned long long mass_here = 0;
+  {
+    int tie_rank = tie_base;
+    for (int base = begin; base < end; base += WAVE) {
+      const int i = base + lane;
+      const float v = i < end ? x[i] : NAN;
+      const bool fin = finite_f(v);
+      const uint32_t key = fin ? key_of(v) : 0u;
+      const bool tie = fin && key == cut.key;
+      const unsigned long long ballot = __ballot(tie);
+      const int rank = tie_rank + __popcll(ballot & ((1ull << lane) - 1ull));
+      tie_rank += __popcll(ballot);
+      bool kept = fin && (key > cut.key || (tie && rank < cut.ties));
+      if (kept) kept = expf(v * scale - peak) >= floor_weight;
+      mass_here += kept ? fixed_weight(v, scale, peak) : 0ull;
+    }
+  }
+  mass_here = wave_sum_u64(mass_here);
+  if (lane == 0) red_u[wave] = mass_here;
+  __syncthreads();
+  unsigned long long mass = 0, before = 0;
+  for (int w = 0; w < WAVES; ++w) {
+    if (w < wave) before += red_u[w];
+    mass += red_u[w];
+  }
+  if (mass == 0) {  // every kept weight underflowed: the best token stands
+    if (tid == 0) out[row] = best_id;
+    return;
+  }
+  unsigned long long target = (unsigned long long)(uniform[row] * (double)mass);
+  if (target >= mass) target = mass - 1;
+  // the wave whose share holds the target walks its range once more
+  if (target >= before && target < before + red_u[wave]) {
+    unsigned long long running = before;
+    int tie_rank = tie_base;
+    for (int base = begin; base < end; base += WAVE) {
+      const int i = base + lane;
+      const float v = i < end ? x[i] : NAN;
+      const bool fin = finite_f(v);
+      const uint32_t key = fin ? key_of(v) : 0u;
+      const bool tie = fin && key == cut.key;
+      const unsigned long long ballot = __ballot(tie);
+      const int rank = tie_rank + __popcll(ballot & ((1ull << lane) - 1ull));
+      tie_rank += __popcll(ballot);
+      bool kept = fin && (key > cut.key || (tie && rank < cut.ties));
+      if (kept) kept = expf(v * scale - peak) >= floor_weight;
+      const unsigned long long w = kept ? fixed_weight(v, scale, peak) : 0ull;
+      // inclusive scan over the 64 lanes
+      unsigned long long incl = w;
+#pragma unroll
+      for (int off = 1; off < WAVE; off <<= 1) {
+        const unsigned long long other = __shfl_up(incl, off, WAVE);
+        if (lane >= off) incl += other;
+      }
+      const bool hit = kept && target < running + incl;
+      const unsigned long long hits = __ballot(hit);
+      if (hits) {
+        const int first = __ffsll((long long)hits) - 1;
+        if (lane == first) out[row] = i;
+        break;
+      }
+      running += __shfl(incl, WAVE - 1, WAVE);
+    }
+  }
+}
+
+// entries: (row, token, count) triples, unique per (row, token); applied in place
+__global__ void penalize_kernel(float* __restrict__ logits, int vocab, const int* __restrict__ rows,
+                                const int* __restrict__ tokens, const int* __restrict__ counts,
+                                const float* __restrict__ repetition, const float* __restrict__ presence,
+                                const float* __restrict__ frequency, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int row = rows[i], token = tokens[i];
+  if (token < 0 || token >= vocab) return;
+  float* at = logits + (size_t)row * vocab + token;
+  float v = *at;
+  const float factor = repetition[row];
+  if (factor != 1.0f) v = v > 0.f ? v / factor : v * factor;
+  v -= presence[row] + frequency[row] * (float)counts[i];
+  *at = v;
+}
+
+__global__ void bias_kernel(float* __restrict__ logits, int vocab, const int* __restrict__ rows,
+                            const int* __restrict__ tokens, const float* __restrict__ values, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int token = tokens[i];
+  if (token < 0 || token >= vocab) return;
+  logits[(size_t)rows[i] * vocab + token] += values[i];
+}
+}  // namespace
+
+extern "C" int vk_sample(const float* logits, int num_rows, int vocab, const float* temperature, const int* top_k,
+                         const float* top_p, const float* min_p, const double* uniform, int* out, void* stream) {
+  if (num_rows <= 0) return 0;
+  if (vocab <= 0) return VK_BAD_ARGUMENT;
+  sample_kernel<<<num_rows, THREADS, 0, (hipStream_t)stream>>>(logits, vocab, temperature, top_k, top_p, min_p,
+                                                                uniform, out);
+  VK_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" int vk_penalize(float* logits, int vocab, const int* rows, const int* tokens, const int* counts,
+                           const float* repetition, const float* presence, const float* frequency, int n,
+                           void* stream) {
+  if (n <= 0) return 0;
+  penalize_kernel<<<(n + 255) / 256, 256, 0, (hipStream_t)stream>>>(logits, vocab, rows, tokens, counts, repetition,
+                                                                    presence, frequency, n);
+  VK_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" int vk_logit_bias(float* logits, int vocab, const int* rows, const int* tokens, const float* values, int n,
+                             void* stream) {
+  if (n <= 0) return 0;
+  bias_kernel<<<(n + 255) / 256, 256, 0, (hipStream_t)stream>>>(logits, vocab, rows, tokens, values, n);
+  VK_LAUNCH_CHECK();
+  return 0;
+}

@@ -1,0 +1,261 @@
+"""The Python entry point: requests in, tokens out.
+
+``Engine`` puts the parts together: a model with its weights, the cache manager and its device
+memory, the step function, the scheduler above it and the sampler.  Its methods mirror the
+reference's ``Engine`` (crates/vipera-runtime/src/engine.rs:329-1232): ``add_request`` is ``admit`` +
+``enqueue``, ``step`` makes one scheduling decision and one forward pass and samples, ``generate``
+runs until the given requests are done.
+"""
+from __future__ import annotations
+
+import time
+from dataclasses import dataclass, field
+from typing import Callable, Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+from ..errors import InfeasibleError, InvalidArgumentError, ViperaError
+from ..runtime import Runtime
+from ..sampling import BatchSampler, Rng, RowRequest, SamplingParams
+from .batch import StepEntry
+from .runner import ModelRunner
+from .scheduler import FINISH_NAMES, NOT_FINISHED, Scheduler
+
+
+@dataclass
+class Generation:
+    """A finished request (engine.rs:308-327)."""
+
+    request: int
+    prompt_tokens: int
+    tokens: List[int]            # generated ids, the end-of-sequence token included when one ended it
+    finish: str                  # "stop" | "length" | "cancelled" | "error"
+    processed_tokens: int = 0    # tokens run through the model, recomputation after preemption included
+    preemptions: int = 0
+    error: Optional[str] = None
+
+
+@dataclass
+class StepToken:
+    request: int
+    token: int
+
+
+@dataclass
+class StepReport:
+    """What one step did (engine.rs:283-304), plus the requests it preempted."""
+
+    tokens: List[StepToken] = field(default_factory=list)
+    finished: List[Generation] = field(default_factory=list)
+    failed: List[Tuple[int, str]] = field(default_factory=list)
+    preempted: List[int] = field(default_factory=list)
+    num_batched_tokens: int = 0
+
+
+@dataclass
+class _Live:
+    prompt: List[int]
+    generated: List[int]
+    params: SamplingParams
+    rng: Rng
+    eos: frozenset
+    processed: int = 0
+    preemptions: int = 0
+    on_token: Optional[Callable[[int], None]] = None
+
+
+class Engine:
+    """Continuous-batching generation on one GPU.
+
+    ``model``: a folder with ``config.json`` and ``model.safetensors``.  ``dtype``: ``"bfloat16"``
+    or ``"float32"``.  The cache has ``num_blocks`` pages of ``block_size`` positions per group of
+    layers; when ``num_blocks`` is absent it is sized for ``max_num_seqs`` requests of
+    ``max_model_len`` tokens, bounded by free device memory.
+    """
+
+    def __init__(self, model: str, dtype: str = "bfloat16", device: str = "cuda:0", block_size: int = 16,
+                 num_blocks: Optional[int] = None, max_num_seqs: int = 8, max_num_batched_tokens: int = 2048,
+                 chunk_size: int = 512, max_model_len: Optional[int] = None,
+                 eos_token_ids: Optional[Sequence[int]] = None, runner: Optional[ModelRunner] = None):
+        if runner is None:
+            runtime = Runtime(device, dtype)
+            from ..config.registry import load_config
+            config = load_config(model)
+            limit = int(max_model_len or config.context_limit)
+            if limit > config.context_limit:
+                raise InvalidArgumentError(
+                    f"requested context {limit} exceeds the model's maximum of {config.context_limit}")
+            if num_blocks is None:
+                num_blocks = max_num_seqs * ((limit + block_size - 1) // block_size)
+            runner = self._load(model, config, runtime, block_size, num_blocks, max_num_seqs)
+        else:
+            config = runner.model.config
+            limit = int(max_model_len or config.context_limit)
+        self.runner = runner
+        self.config = config
+        self.max_model_len = limit
+        self.scheduler = Scheduler(runner.cache, max_num_seqs, max_num_batched_tokens, chunk_size, limit)
+        self.sampler = BatchSampler(runner.runtime.device)
+        default_eos = getattr(config, "eos_token_ids", ()) or ()
+        self.eos_token_ids = frozenset(eos_token_ids if eos_token_ids is not None else default_eos)
+        self._live: Dict[int, _Live] = {}
+        self._next_id = 0
+        self.generations = 0
+        self.failed = 0
+        self.step_count = 0
+        self.micros = {"schedule": 0, "compute": 0, "sample": 0}
+
+    @staticmethod
+    def _load(folder, config, runtime, block_size, num_blocks, num_slots) -> ModelRunner:
+        from ..models import build_model
+        from ..weights import Checkpoint, load_tensors
+
+        model = build_model(config, runtime)
+        checkpoint = Checkpoint(folder)
+        try:
+            tensors = load_tensors(checkpoint, model.tensor_specs(), runtime.dtype, runtime.device)
+        finally:
+            checkpoint.close()
+        model.load(tensors)
+        free, _ = torch.cuda.mem_get_info(runtime.device)
+        needs = model.cache_needs()
+        element = 4 if runtime.dtype == torch.float32 else 2
+        per_page = sum(2 * n.kv.kv_heads * n.kv.head_dim * block_size * element
+                       for i, n in enumerate(needs) if n.kv is not None and n.owner == i)
+        if per_page and num_blocks * per_page > 0.9 * free:
+            fit = int(0.9 * free // per_page)
+            if fit < 1:
+                raise InfeasibleError(
+                    f"no room for a single cache page of {per_page} bytes in {free} free bytes of device memory")
+            num_blocks = fit
+        return ModelRunner(model, runtime, block_size, num_blocks, max(num_slots, 1))
+
+    # --- requests ---------------------------------------------------------------------------------
+    def add_request(self, prompt: Sequence[int], max_new_tokens: int = 32,
+                    sampling: Optional[SamplingParams] = None, eos_token_ids: Optional[Sequence[int]] = None,
+                    on_token: Optional[Callable[[int], None]] = None) -> int:
+        """Queue a request and return its id. Refuses what can never run, before any work."""
+        params = sampling or SamplingParams()
+        params.validate()
+        prompt = [int(t) for t in prompt]
+        for token in prompt:
+            if not 0 <= token < self.runner.vocab_size:
+                raise InvalidArgumentError(f"token {token} is outside the vocabulary of {self.runner.vocab_size}")
+        request = self._next_id
+        self.scheduler.add(request, prompt, int(max_new_tokens))
+        self._next_id += 1
+        eos = frozenset(eos_token_ids) if eos_token_ids is not None else self.eos_token_ids
+        self._live[request] = _Live(prompt, [], params, Rng(params.seed), eos, on_token=on_token)
+        return request
+
+    def cancel(self, request: int) -> Optional[Generation]:
+        """Remove a request at a step boundary; its pages are free afterwards."""
+        live = self._live.pop(request, None)
+        if live is None:
+            return None
+        self.scheduler.cancel(request)
+        return Generation(request, len(live.prompt), live.generated, "cancelled", live.processed, live.preemptions)
+
+    def has_work(self) -> bool:
+        return self.scheduler.has_work()
+
+    # --- one step -----------------------------------------------------------------------------------
+    def step(self) -> StepReport:
+        report = StepReport()
+        started = time.perf_counter()
+        plan = self.scheduler.plan()
+        for request in plan.preempted:
+            if request in self._live:
+                self._live[request].preemptions += 1
+        report.preempted = list(plan.preempted)
+        scheduled = time.perf_counter()
+        self.micros["schedule"] += int((scheduled - started) * 1e6)
+        if not plan.entries:
+            return report
+        entries = [StepEntry(e.request, e.start, e.tokens, [len(e.tokens) - 1] if e.wants_logits else [])
+                   for e in plan.entries]
+        report.num_batched_tokens = plan.num_tokens
+        self.step_count += 1
+        try:
+            logits = self.runner.step(entries)
+        except ViperaError as err:  # every request of the batch fails and gives back what it holds
+            for e in plan.entries:
+                self._fail(e.request, str(err), report)
+            return report
+        for e in plan.entries:
+            self.scheduler.advance(e.request)
+            self._live[e.request].processed += len(e.tokens)
+        wanting = [e for e in plan.entries if e.wants_logits]
+        computed = time.perf_counter()
+        if wanting:
+            rows = []
+            for e in wanting:
+                live = self._live[e.request]
+                rows.append(RowRequest(live.params, live.rng, live.prompt + live.generated))
+            tokens = self.sampler.sample(logits, rows)
+            for e, token in zip(wanting, tokens):
+                if token < 0:
+                    self._fail(e.request, "the logits hold no finite value", report)
+                    continue
+                live = self._live[e.request]
+                live.generated.append(token)
+                is_eos = token in live.eos
+                reason = self.scheduler.append(e.request, token, is_eos)
+                report.tokens.append(StepToken(e.request, token))
+                if not is_eos and live.on_token is not None:
+                    live.on_token(token)
+                if reason != NOT_FINISHED:
+                    self._live.pop(e.request)
+                    self.generations += 1
+                    report.finished.append(Generation(e.request, len(live.prompt), live.generated,
+                                                      FINISH_NAMES[reason], live.processed, live.preemptions))
+        done = time.perf_counter()
+        self.micros["compute"] += int((computed - scheduled) * 1e6)
+        self.micros["sample"] += int((done - computed) * 1e6)
+        return report
+
+    def _fail(self, request: int, message: str, report: StepReport) -> None:
+        live = self._live.pop(request, None)
+        self.scheduler.cancel(request)
+        self.failed += 1
+        report.failed.append((request, message))
+        if live is not None:
+            report.finished.append(Generation(request, len(live.prompt), live.generated, "error", live.processed,
+                                              live.preemptions, message))
+
+    # --- whole generations --------------------------------------------------------------------------
+    def generate(self, prompts: Sequence[Sequence[int]], max_new_tokens: int = 32,
+                 sampling=None, eos_token_ids: Optional[Sequence[int]] = None) -> List[Generation]:
+        """Run ``prompts`` to the end; ``sampling`` is one :class:`SamplingParams` or one per prompt."""
+        if sampling is None or isinstance(sampling, SamplingParams):
+            sampling = [sampling] * len(prompts)
+        if len(sampling) != len(prompts):
+            raise InvalidArgumentError(f"{len(sampling)} sampling settings for {len(prompts)} prompts")
+        ids = [self.add_request(p, max_new_tokens, s, eos_token_ids) for p, s in zip(prompts, sampling)]
+        done: Dict[int, Generation] = {}
+        idle = 0
+        while len(done) < len(ids):
+            report = self.step()
+            for generation in report.finished:
+                done[generation.request] = generation
+            idle = idle + 1 if report.num_batched_tokens == 0 else 0
+            if idle > 2:
+                raise InfeasibleError("the scheduler can run none of the waiting requests")
+        return [done[i] for i in ids]
+
+    def stats(self) -> dict:
+        """Counters in the manner of the reference's ``RuntimeStats`` (engine.rs:95-110)."""
+        cache = self.runner.cache
+        return {
+            "requests": len(self._live),
+            "waiting": self.scheduler.num_waiting,
+            "running": self.scheduler.num_running,
+            "kv_used_blocks": [cache.used_blocks(g) for g in range(len(cache.groups))],
+            "kv_free_blocks": [cache.free_blocks(g) for g in range(len(cache.groups))],
+            "kv_bytes": self.runner.storage.bytes,
+            "generations": self.generations,
+            "failed": self.failed,
+            "preemptions": self.scheduler.preemptions,
+            "steps": self.step_count,
+            "micros": dict(self.micros),
+        }

@@ -200,3 +200,55 @@ def attn_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, 
     _status(fn(_ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(out), _dt(q, "q"), _ptr(positions),
                _ptr(entry_of_token), _ptr(block_table), block_table.shape[1], k_cache.shape[2], num_tokens, heads,
                kv_heads, head_dim, float(scale), int(window), _stream()), "attn_generic")
+
+
+# ----------------------------------------------------------------------------------------------
+def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
+           min_p: torch.Tensor, uniform: torch.Tensor, out: torch.Tensor) -> None:
+    """One token per row: greedy where ``temperature`` is 0, else a draw after the top-k/top-p/min-p cuts.
+
+    ``out[r]`` is -1 when row ``r`` has no finite logit.
+    """
+    _dev(logits, temperature, top_k, top_p, min_p, uniform, out)
+    rows, vocab = logits.shape
+    _need(logits.dtype == torch.float32 and logits.is_contiguous(), "sample: logits must be contiguous float32")
+    for name, tensor, dtype in (("temperature", temperature, torch.float32), ("top_k", top_k, torch.int32),
+                                ("top_p", top_p, torch.float32), ("min_p", min_p, torch.float32),
+                                ("uniform", uniform, torch.float64), ("out", out, torch.int32)):
+        _need(tensor.dtype == dtype and tensor.numel() == rows and tensor.is_contiguous(),
+              f"sample: {name} must hold one {dtype} per row")
+    fn = _fn("sampling", "vk_sample", [_p, _i, _i, _p, _p, _p, _p, _p, _p, _p])
+    _status(fn(_ptr(logits), rows, vocab, _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(min_p), _ptr(uniform),
+               _ptr(out), _stream()), "sample")
+
+
+def penalize(logits: torch.Tensor, rows: torch.Tensor, tokens: torch.Tensor, counts: torch.Tensor,
+             repetition: torch.Tensor, presence: torch.Tensor, frequency: torch.Tensor) -> None:
+    """Apply the repetition, presence and frequency penalties in place to the listed (row, token) pairs."""
+    _dev(logits, rows, tokens, counts, repetition, presence, frequency)
+    num_rows, vocab = logits.shape
+    n = rows.numel()
+    _need(logits.dtype == torch.float32 and logits.is_contiguous(), "penalize: logits must be contiguous float32")
+    _need(tokens.numel() == n and counts.numel() == n and all(t.dtype == torch.int32 for t in (rows, tokens, counts)),
+          "penalize: rows, tokens and counts must be int32 of one length")
+    _need(all(t.dtype == torch.float32 and t.numel() == num_rows for t in (repetition, presence, frequency)),
+          "penalize: one float32 factor per row")
+    if n:
+        _need(int(rows.max()) < num_rows and int(rows.min()) >= 0, "penalize: row index out of range")
+    fn = _fn("sampling", "vk_penalize", [_p, _i, _p, _p, _p, _p, _p, _p, _i, _p])
+    _status(fn(_ptr(logits), vocab, _ptr(rows), _ptr(tokens), _ptr(counts), _ptr(repetition), _ptr(presence),
+               _ptr(frequency), n, _stream()), "penalize")
+
+
+def logit_bias(logits: torch.Tensor, rows: torch.Tensor, tokens: torch.Tensor, values: torch.Tensor) -> None:
+    """``logits[rows[i], tokens[i]] += values[i]`` (pairs are unique)."""
+    _dev(logits, rows, tokens, values)
+    num_rows, vocab = logits.shape
+    n = rows.numel()
+    _need(logits.dtype == torch.float32 and logits.is_contiguous(), "logit_bias: logits must be contiguous float32")
+    _need(tokens.numel() == n and values.numel() == n and rows.dtype == torch.int32 and tokens.dtype == torch.int32
+          and values.dtype == torch.float32, "logit_bias: operand types")
+    if n:
+        _need(int(rows.max()) < num_rows and int(rows.min()) >= 0, "logit_bias: row index out of range")
+    fn = _fn("sampling", "vk_logit_bias", [_p, _i, _p, _p, _p, _i, _p])
+    _status(fn(_ptr(logits), vocab, _ptr(rows), _ptr(tokens), _ptr(values), n, _stream()), "logit_bias")

@@ -1,0 +1,140 @@
+"""Sampling options and the batched sampler that runs them on the device.
+
+Names, meanings, defaults and validation of the options follow the reference's ``SamplerConfig``
+(crates/vipera-sampler/src/lib.rs:36-115); a temperature of 0 selects greedy decoding and skips
+every other filter (lib.rs:273-280).  The engine's default temperature is 0, as the reference's
+engine and command line set it (crates/vipera-runtime/src/engine.rs:50-53, bins/vipera/src/main.rs:557-560).
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass, field
+from typing import List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+from ..errors import InvalidArgumentError
+from ..ops import kernels
+from .rng import Rng
+
+MAX_LOGIT_BIAS = 16
+RECENT_WINDOW = 128  # tokens the penalties look back over (bins/vipera/src/main.rs:685)
+
+
+@dataclass(frozen=True)
+class SamplingParams:
+    temperature: float = 0.0
+    top_k: int = 40
+    top_p: float = 0.95
+    min_p: float = 0.05
+    repetition_penalty: float = 1.0
+    presence_penalty: float = 0.0
+    frequency_penalty: float = 0.0
+    logit_bias: Tuple[Tuple[int, float], ...] = ()
+    seed: int = 0
+
+    def validate(self) -> None:
+        """Reject values that cannot describe a distribution (lib.rs:73-115)."""
+        def finite(v):
+            return isinstance(v, (int, float)) and math.isfinite(v)
+
+        if not finite(self.temperature) or self.temperature < 0.0:
+            raise InvalidArgumentError("temperature must be a finite number at or above 0")
+        if not isinstance(self.top_k, int) or self.top_k < 0:
+            raise InvalidArgumentError("top_k must be an integer at or above 0")
+        if not finite(self.top_p) or self.top_p <= 0.0 or self.top_p > 1.0:
+            raise InvalidArgumentError("top_p must be greater than 0 and at most 1")
+        if not finite(self.min_p) or self.min_p < 0.0 or self.min_p >= 1.0:
+            raise InvalidArgumentError("min_p must be at least 0 and below 1")
+        if not finite(self.repetition_penalty) or self.repetition_penalty <= 0.0:
+            raise InvalidArgumentError("repetition_penalty must be a finite number above 0")
+        for name in ("presence_penalty", "frequency_penalty"):
+            value = getattr(self, name)
+            if not finite(value) or not -2.0 <= value <= 2.0:
+                raise InvalidArgumentError(f"{name} must be a finite number from -2 to 2")
+        if len(self.logit_bias) > MAX_LOGIT_BIAS:
+            raise InvalidArgumentError(f"logit_bias holds at most {MAX_LOGIT_BIAS} entries")
+        for _, value in self.logit_bias:
+            if not finite(value) or not -100.0 <= value <= 100.0:
+                raise InvalidArgumentError("logit_bias values must be finite numbers from -100 to 100")
+
+    @property
+    def greedy(self) -> bool:
+        return self.temperature == 0.0
+
+    @property
+    def penalizes(self) -> bool:
+        return (self.repetition_penalty != 1.0 or self.presence_penalty != 0.0 or self.frequency_penalty != 0.0)
+
+
+@dataclass
+class RowRequest:
+    """What one row of logits is sampled with: options, the request's generator, its recent tokens."""
+
+    params: SamplingParams
+    rng: Rng
+    recent: Sequence[int] = ()
+
+
+class BatchSampler:
+    """Samples one token per row of ``[rows, vocab]`` logits on the device.
+
+    Per-row options go up in one small copy; the drawn ids come back in one.  Each random row
+    consumes exactly one uniform of its request's generator per token, so a request's stream does
+    not depend on its company in the batch or on the order of arrival (the invariant of
+    crates/vipera-runtime/src/engine.rs:665-670).
+    """
+
+    def __init__(self, device):
+        self.device = torch.device(device)
+
+    def sample(self, logits: torch.Tensor, rows: Sequence[RowRequest]) -> List[int]:
+        count, vocab = logits.shape
+        if count != len(rows):
+            raise InvalidArgumentError(f"{count} rows of logits for {len(rows)} requests")
+        if logits.dtype != torch.float32 or not logits.is_contiguous():
+            raise InvalidArgumentError("logits must be contiguous float32")
+        self._penalize(logits, rows, vocab)
+        temperature = np.array([r.params.temperature for r in rows], dtype=np.float32)
+        top_k = np.array([r.params.top_k for r in rows], dtype=np.int32)
+        top_p = np.array([r.params.top_p for r in rows], dtype=np.float32)
+        min_p = np.array([r.params.min_p for r in rows], dtype=np.float32)
+        uniform = np.array([0.0 if r.params.greedy else r.rng.next_f64() for r in rows], dtype=np.float64)
+        dev = lambda a: torch.from_numpy(a).to(self.device)  # noqa: E731
+        out = torch.empty(count, dtype=torch.int32, device=self.device)
+        kernels.sample(logits, dev(temperature), dev(top_k), dev(top_p), dev(min_p), dev(uniform), out)
+        return [int(t) for t in out.cpu().tolist()]
+
+    def _penalize(self, logits: torch.Tensor, rows: Sequence[RowRequest], vocab: int) -> None:
+        pen_rows: List[int] = []
+        pen_tokens: List[int] = []
+        pen_counts: List[int] = []
+        bias_rows: List[int] = []
+        bias_tokens: List[int] = []
+        bias_values: List[float] = []
+        for index, row in enumerate(rows):
+            if row.params.penalizes and row.recent:
+                counts = {}
+                for token in list(row.recent)[-RECENT_WINDOW:]:
+                    counts[token] = counts.get(token, 0) + 1
+                for token, n in counts.items():
+                    pen_rows.append(index)
+                    pen_tokens.append(token)
+                    pen_counts.append(n)
+            seen = set()
+            for token, value in sorted(row.params.logit_bias, key=lambda item: item[0]):
+                if token not in seen and 0 <= token < vocab:  # the first entry of a token id stands
+                    seen.add(token)
+                    bias_rows.append(index)
+                    bias_tokens.append(token)
+                    bias_values.append(value)
+        ints = lambda a: torch.tensor(a, dtype=torch.int32, device=self.device)  # noqa: E731
+        floats = lambda a: torch.tensor(a, dtype=torch.float32, device=self.device)  # noqa: E731
+        if pen_rows:
+            kernels.penalize(logits, ints(pen_rows), ints(pen_tokens), ints(pen_counts),
+                             floats([r.params.repetition_penalty for r in rows]),
+                             floats([r.params.presence_penalty for r in rows]),
+                             floats([r.params.frequency_penalty for r in rows]))
+        if bias_rows:
+            kernels.logit_bias(logits, ints(bias_rows), ints(bias_tokens), floats(bias_values))

@@ -15,6 +15,7 @@ import json
 import mmap
 import os
 import struct
+import warnings
 from dataclasses import dataclass
 from typing import Dict, Iterable, List, Tuple
 
@@ -103,7 +104,9 @@ class SafetensorsFile:
             count *= dim
         if count == 0:
             return torch.empty(info.shape, dtype=info.torch_dtype)
-        flat = torch.frombuffer(self._map, dtype=info.torch_dtype, count=count, offset=info.begin)
+        with warnings.catch_warnings():  # the map is read-only on purpose; nothing writes through the view
+            warnings.simplefilter("ignore", UserWarning)
+            flat = torch.frombuffer(self._map, dtype=info.torch_dtype, count=count, offset=info.begin)
         return flat.reshape(info.shape)
 
     def close(self) -> None:
