@@ -252,3 +252,34 @@ def logit_bias(logits: torch.Tensor, rows: torch.Tensor, tokens: torch.Tensor, v
         _need(int(rows.max()) < num_rows and int(rows.min()) >= 0, "logit_bias: row index out of range")
     fn = _fn("sampling", "vk_logit_bias", [_p, _i, _p, _p, _p, _i, _p])
     _status(fn(_ptr(logits), vocab, _ptr(rows), _ptr(tokens), _ptr(values), n, _stream()), "logit_bias")
+
+
+# ----------------------------------------------------------------------------------------------
+def gemm_bf16_supported(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> bool:
+    """Whether the matrix-core kernels take these operands (16-byte chunks along K)."""
+    k = a.shape[1]
+    return (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out.dtype in _DT and k % 8 == 0
+            and a.stride(1) == 1 and (a.stride(0) % 8 == 0 or a.shape[0] == 1) and a.data_ptr() % 16 == 0
+            and w.is_contiguous() and w.data_ptr() % 16 == 0 and out.stride(1) == 1)
+
+
+def gemm_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
+              accumulate: bool = False, skinny_limit: int = 64, skinny_shape: int = 0) -> None:
+    """``out (+)= a @ w.T + bias`` on the matrix cores: bfloat16 products, 32-bit sums."""
+    _dev(a, w, bias, out)
+    _need(a.dim() == 2 and w.dim() == 2 and out.dim() == 2, "gemm: operands must be matrices")
+    m, k = a.shape
+    n = w.shape[0]
+    _need(w.shape[1] == k and out.shape == (m, n), f"gemm: shapes {tuple(a.shape)} x {tuple(w.shape)}^T -> {tuple(out.shape)}")
+    _need(gemm_bf16_supported(a, w, out), "gemm_bf16: operands must be bfloat16, K a multiple of 8, rows 16-byte aligned")
+    if bias is not None:
+        _need(bias.dtype == torch.float32 and bias.numel() == n and bias.is_contiguous(), "gemm: bias must be float32 [n]")
+    if accumulate:
+        _need(out.dtype == torch.float32, "gemm: accumulation needs a float32 output")
+    lda = a.stride(0) if m > 1 else max(a.stride(0), k)
+    lda = lda if lda % 8 == 0 else k
+    ldc = out.stride(0) if m > 1 else max(out.stride(0), n)
+    _need(ldc >= n, "gemm: out's row stride")
+    fn = _fn("gemm_bf16", "vk_gemm_bf16", [_p, _p, _p, _p, _i, _i, _i, _i, _ll, _ll, _i, _i, _i, _p])
+    _status(fn(_ptr(a), _ptr(w), _ptr(bias), _ptr(out), _dt(out, "out"), m, n, k, lda, ldc, 1 if accumulate else 0,
+               int(skinny_limit), int(skinny_shape), _stream()), "gemm_bf16")
