@@ -89,3 +89,142 @@ def test_gemm_generic_does_not_depend_on_the_batch():
     single = torch.empty(1, 90, device=DEV)
     kernels.gemm_generic(a[37:38].contiguous(), w, None, single)
     assert torch.equal(single[0], whole[37])  # bit for bit: one thread sums each element in k order
+
+
+# --- attention -------------------------------------------------------------------------------------
+def _plain_attention(q, k, v, first_pos, window, scale):
+    """q: [T, heads, hd] at positions first_pos..; k, v: [P, kv_heads, hd] for positions 0..P-1. float64."""
+    T, heads, hd = q.shape
+    group = heads // k.shape[1]
+    out = torch.zeros(T, heads, hd, dtype=torch.float64)
+    for t in range(T):
+        pos = first_pos + t
+        lo = max(0, pos + 1 - window) if window > 0 else 0
+        for h in range(heads):
+            kk, vv = k[lo:pos + 1, h // group], v[lo:pos + 1, h // group]
+            w = torch.softmax((kk @ q[t, h]) * scale, dim=0)
+            out[t, h] = w @ vv
+    return out
+
+
+class _Paged:
+    """A paged cache filled by hand: shuffled pages, K [page, kvh, slot, hd], V [page, kvh, hd, slot]."""
+
+    def __init__(self, seqs, kv_heads, hd, block_size, dtype, seed):
+        g = torch.Generator().manual_seed(seed)
+        self.block_size = block_size
+        need = [(n + block_size - 1) // block_size for n in seqs]
+        pages = sum(need) + 3
+        order = torch.randperm(pages, generator=g).tolist()
+        self.k = (torch.randn(pages, kv_heads, block_size, hd, generator=g) * 7).to(dtype)   # stale values everywhere
+        self.v = (torch.randn(pages, kv_heads, hd, block_size, generator=g) * 7).to(dtype)
+        self.tables, self.keys, self.values = [], [], []
+        for n, blocks in zip(seqs, need):
+            table = [order.pop() for _ in range(blocks)]
+            keys = torch.randn(n, kv_heads, hd, generator=g).to(dtype)
+            values = torch.randn(n, kv_heads, hd, generator=g).to(dtype)
+            for p in range(n):
+                page, slot = table[p // block_size], p % block_size
+                self.k[page, :, slot, :] = keys[p]
+                self.v[page, :, :, slot] = values[p]
+            self.tables.append(table)
+            self.keys.append(keys)
+            self.values.append(values)
+        width = max(need)
+        self.table = torch.full((len(seqs), width), -1, dtype=torch.int32)
+        for i, t in enumerate(self.tables):
+            self.table[i, :len(t)] = torch.tensor(t, dtype=torch.int32)
+
+
+ATTN_CASES = [
+    # heads, kv_heads, hd, block_size, window, entries as (kv length after the step, tokens in the step)
+    (4, 2, 16, 16, 0, [(37, 37), (70, 1), (5, 2)]),
+    (3, 1, 32, 8, 21, [(90, 17), (64, 1), (33, 33), (130, 1)]),
+    (6, 3, 48, 16, 0, [(100, 64), (65, 65)]),
+    (28, 4, 128, 16, 0, [(300, 1), (257, 130), (31, 1)]),
+    (20, 1, 80, 32, 50, [(200, 1), (97, 96)]),
+    (2, 2, 256, 64, 0, [(129, 1), (70, 70)]),
+]
+
+
+@pytest.mark.parametrize("case", ATTN_CASES, ids=[f"h{c[0]}kv{c[1]}d{c[2]}b{c[3]}w{c[4]}" for c in ATTN_CASES])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_kernels_against_plain_softmax(case, dtype):
+    from vipera_rs_amd.ops import kernels
+    from vipera_rs_amd.ops.attention import decode_chunking
+    heads, kv_heads, hd, bs, window, entries = case
+    scale = 1.0 / math.sqrt(hd)
+    cache = _Paged([kv for kv, _ in entries], kv_heads, hd, bs, dtype, seed=heads * 100 + hd)
+    g = torch.Generator().manual_seed(hd)
+    counts = [n for _, n in entries]
+    T = sum(counts)
+    width = (heads + 2 * kv_heads) * hd
+    qkv = torch.randn(T, width, generator=g).to(dtype)
+    starts = [0]
+    for n in counts:
+        starts.append(starts[-1] + n)
+    first = [kv - n for kv, n in entries]
+    positions = torch.tensor([first[e] + i for e, n in enumerate(counts) for i in range(n)], dtype=torch.int32)
+    entry_of = torch.tensor([e for e, n in enumerate(counts) for _ in range(n)], dtype=torch.int32)
+    want = torch.zeros(T, heads, hd, dtype=torch.float64)
+    for e, (kv, n) in enumerate(entries):
+        q = qkv[starts[e]:starts[e + 1], :heads * hd].double().view(n, heads, hd)
+        want[starts[e]:starts[e + 1]] = _plain_attention(q, cache.keys[e].double(), cache.values[e].double(),
+                                                         first[e], window, scale)
+    want = want.view(T, heads * hd)
+    dev = lambda t: t.to(DEV)  # noqa: E731
+    qkv_d, k_d, v_d, table_d = dev(qkv), dev(cache.k), dev(cache.v), dev(cache.table)
+    tol = 2e-6 if dtype == torch.float32 else 1.2e-2
+
+    out = torch.zeros(T, heads * hd, dtype=dtype, device=DEV)
+    kernels.attn_generic(qkv_d, k_d, v_d, out, dev(positions), dev(entry_of), table_d, heads, kv_heads, hd, scale, window)
+    assert _rel(out.cpu(), want) < tol, "32-bit-arithmetic kernel"
+
+    if dtype == torch.bfloat16:
+        tiles = [x for e, n in enumerate(counts) if n > 1 for off in range(0, n, 64) for x in (e, off)]
+        singles = [e for e, n in enumerate(counts) if n == 1]
+        out2 = torch.zeros(T, heads * hd, dtype=dtype, device=DEV)
+        es, fp = dev(torch.tensor(starts, dtype=torch.int32)), dev(torch.tensor(first, dtype=torch.int32))
+        if tiles:
+            kernels.attn_bf16_prefill(qkv_d, k_d, v_d, out2, dev(torch.tensor(tiles, dtype=torch.int32)), es, fp,
+                                      table_d, heads, kv_heads, hd, scale, window)
+        if singles:
+            longest = max(entries[e][0] for e in singles)
+            for chunk, chunks in {decode_chunking(longest, len(singles), kv_heads, (heads // kv_heads + 15) // 16),
+                                  (32, (longest + 31) // 32), (512, (longest + 511) // 512)}:
+                partial = torch.empty(len(singles) * heads * chunks * (hd + 2), device=DEV)
+                kernels.attn_bf16_decode(qkv_d, k_d, v_d, out2, partial, dev(torch.tensor(singles, dtype=torch.int32)),
+                                         es, fp, table_d, heads, kv_heads, hd, scale, window, chunk, chunks)
+                assert _rel(out2.cpu(), want) < tol, f"matrix-core kernels, chunk {chunk}"
+        assert _rel(out2.cpu(), want) < tol, "matrix-core kernels"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_finds_one_far_key_among_hundreds(dtype):
+    """One early key is made to dominate: every later token must return (almost exactly) its value.
+    An off-by-one in the visible range, a missed page or a wrong tile would lose it."""
+    from vipera_rs_amd.ops import kernels
+    heads, kv_heads, hd, bs, n = 4, 2, 64, 16, 700
+    far = 17
+    cache = _Paged([n], kv_heads, hd, bs, dtype, seed=1)
+    direction = torch.randn(hd, generator=torch.Generator().manual_seed(3))
+    direction = (direction / direction.norm()).to(dtype)
+    page, slot = cache.tables[0][far // bs], far % bs
+    cache.k[page, :, slot, :] = direction * 40
+    q = torch.zeros(2, (heads + 2 * kv_heads) * hd, dtype=dtype)
+    q[:, :heads * hd] = (direction * 40).repeat(heads)
+    dev = lambda t: t.to(DEV)  # noqa: E731
+    out = torch.zeros(2, heads * hd, dtype=dtype, device=DEV)
+    positions = torch.tensor([n - 2, n - 1], dtype=torch.int32)
+    kernels.attn_generic(dev(q), dev(cache.k), dev(cache.v), out, dev(positions), dev(torch.zeros(2, dtype=torch.int32)),
+                         dev(cache.table), heads, kv_heads, hd, 1.0 / math.sqrt(hd), 0)
+    want = cache.values[0][far].double().repeat_interleave(heads // kv_heads, dim=0).reshape(-1)
+    for row in out.cpu().double():
+        assert float((row - want).abs().max()) < (1e-5 if dtype == torch.float32 else 2e-2)
+    if dtype == torch.bfloat16:
+        out2 = torch.zeros_like(out)
+        es, fp = dev(torch.tensor([0, 2], dtype=torch.int32)), dev(torch.tensor([n - 2], dtype=torch.int32))
+        kernels.attn_bf16_prefill(dev(q), dev(cache.k), dev(cache.v), out2, dev(torch.tensor([0, 0], dtype=torch.int32)),
+                                  es, fp, dev(cache.table), heads, kv_heads, hd, 1.0 / math.sqrt(hd), 0)
+        for row in out2.cpu().double():
+            assert float((row - want).abs().max()) < 2e-2

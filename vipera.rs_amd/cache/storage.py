@@ -1,7 +1,9 @@
 """Device memory of the caches: paged keys and values per cache-owning layer entry, and state slots.
 
-Layout of a paged tensor: ``[pages + 1, kv_heads, block_size, head_dim]``; the last page is a
-scratch page that is never handed out, which padding tokens of a captured step write to.  A state
+Layout of the paged tensors: keys ``[pages + 1, kv_heads, block_size, head_dim]``, values transposed
+``[pages + 1, kv_heads, head_dim, block_size]`` (the attention kernels read consecutive positions of
+one output dim); the last page is a scratch page that is never handed out, which padding tokens of
+a captured step write to.  A state
 tensor is ``[slots, *shape]``.
 """
 from __future__ import annotations
@@ -46,9 +48,8 @@ class CacheStorage:
                 if group is None:
                     raise InvalidArgumentError(f"no cache group keeps a window of {need.kv.window}")
                 spec = self.groups[group]
-                shape = (spec.num_blocks + 1, need.kv.kv_heads, spec.block_size, need.kv.head_dim)
-                k = runtime.zeros(shape)
-                v = runtime.zeros(shape)
+                k = runtime.zeros((spec.num_blocks + 1, need.kv.kv_heads, spec.block_size, need.kv.head_dim))
+                v = runtime.zeros((spec.num_blocks + 1, need.kv.kv_heads, need.kv.head_dim, spec.block_size))
                 self.kv[index] = PagedKV(k, v, group, spec.block_size)
                 self.bytes += 2 * k.numel() * k.element_size()
             if need.state is not None:

@@ -1,0 +1,320 @@
+// Causal grouped-query attention over the paged cache on the matrix cores (bfloat16 in, 32-bit
+// scores, softmax and sums). Compiled once per padded head width: -DHDP=32..256 in steps of 32.
+//
+// What is computed is the reference's attention (crates/vipera-backend-cpu/src/model.rs:1811-1857):
+// head h uses key head h / group; score = dot(q, k) * scale; a token at position p sees positions
+// [lo, p], lo = 0 or p + 1 - window (model.rs:2509); output = softmax-weighted sum of V. The decode
+// form splits the positions into chunks whose partial (max, sum, weighted sum) are merged afterwards,
+// as the reference's split kernels do (crates/vipera-backend-gpu/src/layer.cu:307-467).
+//
+// One wave works on a block of 16 columns and a range of positions. A column is a (token, query
+// head) pair: 16 consecutive tokens of one head (prompts), or up to 16 query heads of one key head at
+// one token (decoding; they share every K and V read). Nothing goes through LDS: the operand layout
+// of v_mfma_f32_16x16x32_bf16 (a lane holds 8 consecutive k of one row) is how K lies in the cache,
+// [page, kv_head, slot, head_dim], and V is cached transposed, [page, kv_head, head_dim, slot], so
+// that a lane reads consecutive positions of one output dim.
+//     S^T = K Q^T : lane (c = l % 16, g = l / 16), register j  <->  S[position 4g + j of a 16-tile][column c]
+//     O^T = V^T P : the 32 positions of a step feed the instruction in the order the scores arrive in
+//                   (slot 8g + i <-> position 4g + i for i < 4, 16 + 4g + i - 4 for i >= 4); V is read in
+//                   that same order, and a sum does not care how its terms are numbered.
+// The softmax is online over steps of 32 positions that start at multiples of 32, so a token's
+// arithmetic depends on its position and the cache only.
+#include "common.h"
+
+#ifndef HDP
+#define HDP 128
+#endif
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+namespace {
+constexpr int KS = HDP / 32;  // instruction steps over the head width
+constexpr int DT = HDP / 16;  // 16-wide tiles of the output width
+
+__device__ __forceinline__ bf16x8 zero8() {
+  bf16x8 z;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) z[i] = (__bf16)0.f;
+  return z;
+}
+
+struct CacheView {
+  const __bf16* k;
+  const __bf16* v;
+  const int* table;  // this request's row of the block table
+  int table_width, block_size, kv_heads, hd, kvh;
+};
+
+// Online-softmax attention of 16 columns over positions [begin, end). Per lane: col_lo / col_pos are
+// the visible range [lo, pos] of the lane's column (pos < 0: the column is empty).
+// State: o[DT] (O^T tiles), m (running max of the column), l (this lane's share of the running sum).
+__device__ __forceinline__ void attend_range(const bf16x8 (&qf)[KS], int col_lo, int col_pos, int begin, int end,
+                                             const CacheView& cv, float scale, f32x4 (&o)[DT], float& m, float& l) {
+  const int lane = threadIdx.x & 63, lr = lane & 15, lg = lane >> 4;
+  const int bs = cv.block_size, hd = cv.hd;
+  for (int kb = begin & ~31; kb < end; kb += 32) {
+    // ---- scores of two 16-position tiles
+    f32x4 s[2];
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub) {
+      const int p = kb + sub * 16 + lr;
+      const __bf16* row = nullptr;
+      if (p >= begin && p < end) {
+        const int page = cv.table[p / bs];
+        if (page >= 0) row = cv.k + (((size_t)page * cv.kv_heads + cv.kvh) * bs + (p % bs)) * hd + lg * 8;
+      }
+      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const bf16x8 kf = (row && ks * 32 + lg * 8 < hd) ? *(const bf16x8*)(row + ks * 32) : zero8();
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[ks], acc, 0, 0, 0);
+      }
+      s[sub] = acc;
+    }
+    // ---- V^T operands of the step: positions kb + 4g .. +3 and kb + 16 + 4g .. +3 of output dim 16 dt + lr
+    bf16x8 vf[DT];
+    {
+      const __bf16* vrow[2] = {nullptr, nullptr};
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        const int p = kb + half * 16 + lg * 4;
+        if (p + 3 >= begin && p < end) {  // a group of four positions lies in one page (4 divides the page size)
+          const int page = cv.table[p / bs];
+          if (page >= 0) vrow[half] = cv.v + (((size_t)page * cv.kv_heads + cv.kvh) * hd) * bs + (p % bs);
+        }
+      }
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        const int d = dt * 16 + lr;
+        bf16x8 f = zero8();
+        if (d < hd) {
+#pragma unroll
+          for (int half = 0; half < 2; ++half)
+            if (vrow[half]) {
+              const bf16x4 x = *(const bf16x4*)(vrow[half] + (size_t)d * bs);
+#pragma unroll
+              for (int i = 0; i < 4; ++i) f[half * 4 + i] = x[i];
+            }
+        }
+        vf[dt] = f;
+      }
+    }
+    // ---- mask, running max, weights
+    float sv[8];
+    float tile_max = -INFINITY;
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int p = kb + sub * 16 + lg * 4 + j;
+        const bool visible = p >= col_lo && p <= col_pos && p >= begin && p < end;
+        const float x = visible ? s[sub][j] * scale : -INFINITY;
+        sv[sub * 4 + j] = x;
+        tile_max = fmaxf(tile_max, x);
+      }
+    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, 64));
+    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
+    const float m_new = fmaxf(m, tile_max);
+    float alpha = 1.f;
+    bf16x8 pf = zero8();
+    if (m_new > -INFINITY) {
+      alpha = __expf(m - m_new);  // m = -inf gives 0
+      float sum = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float w = __expf(sv[i] - m_new);
+        sum += w;
+        pf[i] = (__bf16)w;
+      }
+      l = l * alpha + sum;
+      m = m_new;
+    }
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      o[dt] *= alpha;
+      o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pf, o[dt], 0, 0, 0);
+    }
+  }
+}
+
+__device__ __forceinline__ void load_q(const __bf16* qrow, int hd, bf16x8 (&qf)[KS]) {
+  const int lg = (threadIdx.x & 63) >> 4;
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks)
+    qf[ks] = (qrow && ks * 32 + lg * 8 < hd) ? *(const bf16x8*)(qrow + ks * 32 + lg * 8) : zero8();
+}
+
+// ---------------------------------------------------------------------------------------------
+// Prompts: grid (tiles, heads), four waves; tile = 64 consecutive tokens of one entry, 16 per wave.
+__global__ __launch_bounds__(256) void attn_prefill_kernel(
+    const __bf16* __restrict__ q, long long q_stride, const __bf16* __restrict__ k_cache,
+    const __bf16* __restrict__ v_cache, __bf16* __restrict__ out, const int* __restrict__ tiles,
+    const int* __restrict__ entry_start, const int* __restrict__ entry_first_pos,
+    const int* __restrict__ block_table, int table_width, int block_size, int heads, int kv_heads, int hd,
+    float scale, int window) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, lr = lane & 15, lg = lane >> 4;
+  const int entry = tiles[2 * blockIdx.x], q_off = tiles[2 * blockIdx.x + 1] + wave * 16;
+  const int h = blockIdx.y;
+  const int tok0 = entry_start[entry], count = entry_start[entry + 1] - tok0;
+  if (q_off >= count) return;
+  const int first_pos = entry_first_pos[entry];
+  const int cols = min(16, count - q_off);
+  const bool col_ok = lr < cols;
+  const int col_pos = col_ok ? first_pos + q_off + lr : -1;
+  const int col_lo = (window > 0 && col_pos + 1 > window) ? col_pos + 1 - window : 0;
+  const int token = tok0 + q_off + lr;
+  bf16x8 qf[KS];
+  load_q(col_ok ? q + (size_t)token * q_stride + (size_t)h * hd : nullptr, hd, qf);
+  CacheView cv{k_cache, v_cache, block_table + (size_t)entry * table_width, table_width, block_size,
+               kv_heads, hd, h / (heads / kv_heads)};
+  f32x4 o[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+  const int first_col_pos = first_pos + q_off;
+  const int begin = (window > 0 && first_col_pos + 1 > window) ? first_col_pos + 1 - window : 0;
+  const int end = first_pos + q_off + cols;  // one past the last column's position
+  attend_range(qf, col_lo, col_pos, begin, end, cv, scale, o, m, l);
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+  if (!col_ok) return;
+  const float inv = 1.f / l;
+  __bf16* dst = out + (size_t)token * heads * hd + (size_t)h * hd;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) {
+    const int d = dt * 16 + lg * 4;
+    if (d < hd) {
+      bf16x4 r;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) r[j] = (__bf16)(o[dt][j] * inv);
+      *(bf16x4*)(dst + d) = r;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Decoding: grid (entries, kv_heads * head_blocks, chunks), one wave. Columns are the query heads of
+// one key head. Chunk c covers positions [c * chunk, (c + 1) * chunk) of the visible range and leaves
+// (max, sum, weighted sum) in `partial`: [entry, head, chunk, hd + 2] floats.
+__global__ __launch_bounds__(64) void attn_decode_kernel(
+    const __bf16* __restrict__ q, long long q_stride, const __bf16* __restrict__ k_cache,
+    const __bf16* __restrict__ v_cache, float* __restrict__ partial, const int* __restrict__ entries,
+    const int* __restrict__ entry_start, const int* __restrict__ entry_first_pos,
+    const int* __restrict__ block_table, int table_width, int block_size, int heads, int kv_heads, int hd,
+    float scale, int window, int chunk, int head_blocks) {
+  const int lane = threadIdx.x & 63, lr = lane & 15, lg = lane >> 4;
+  const int slot = blockIdx.x, entry = entries[slot];
+  const int kvh = blockIdx.y / head_blocks, hb = blockIdx.y % head_blocks;
+  const int group = heads / kv_heads;
+  const int token = entry_start[entry];
+  const int pos = entry_first_pos[entry];
+  const int lo = (window > 0 && pos + 1 > window) ? pos + 1 - window : 0;
+  const int begin = max(lo, blockIdx.z * chunk), end = min(pos + 1, (blockIdx.z + 1) * chunk);
+  const int head_in_group = hb * 16 + lr;
+  const bool col_ok = head_in_group < group;
+  const int h = kvh * group + head_in_group;
+  float* dst = partial + (((size_t)slot * heads + (col_ok ? h : 0)) * gridDim.z + blockIdx.z) * (hd + 2);
+  if (begin >= end) {  // nothing of this chunk is visible
+    if (col_ok && lg == 0) {
+      dst[hd] = -INFINITY;
+      dst[hd + 1] = 0.f;
+    }
+    return;
+  }
+  bf16x8 qf[KS];
+  load_q(col_ok ? q + (size_t)token * q_stride + (size_t)h * hd : nullptr, hd, qf);
+  CacheView cv{k_cache, v_cache, block_table + (size_t)entry * table_width, table_width, block_size,
+               kv_heads, hd, kvh};
+  f32x4 o[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+  attend_range(qf, lo, col_ok ? pos : -1, begin, end, cv, scale, o, m, l);
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+  if (!col_ok) return;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) {
+    const int d = dt * 16 + lg * 4;
+    if (d < hd) *(f32x4*)(dst + d) = o[dt];
+  }
+  if (lg == 0) {
+    dst[hd] = m;
+    dst[hd + 1] = l;
+  }
+}
+
+// Merge the chunks of one (entry, head): M = max m_c; out = sum_c acc_c e^(m_c - M) / sum_c l_c e^(m_c - M),
+// chunks in ascending order (layer.cu:443-467).
+__global__ void attn_combine_kernel(const float* __restrict__ partial, __bf16* __restrict__ out,
+                                    const int* __restrict__ entries, const int* __restrict__ entry_start, int heads,
+                                    int hd, int chunks) {
+  const int slot = blockIdx.x, h = blockIdx.y;
+  const float* src = partial + ((size_t)slot * heads + h) * chunks * (hd + 2);
+  float best = -INFINITY;
+  for (int c = 0; c < chunks; ++c) best = fmaxf(best, src[(size_t)c * (hd + 2) + hd]);
+  float total = 0.f;
+  for (int c = 0; c < chunks; ++c) {
+    const float mc = src[(size_t)c * (hd + 2) + hd];
+    if (mc > -INFINITY) total += src[(size_t)c * (hd + 2) + hd + 1] * __expf(mc - best);
+  }
+  const int token = entry_start[entries[slot]];
+  for (int d = threadIdx.x; d < hd; d += blockDim.x) {
+    float acc = 0.f;
+    for (int c = 0; c < chunks; ++c) {
+      const float mc = src[(size_t)c * (hd + 2) + hd];
+      if (mc > -INFINITY) acc += src[(size_t)c * (hd + 2) + d] * __expf(mc - best);
+    }
+    out[(size_t)token * heads * hd + (size_t)h * hd + d] = (__bf16)(acc / total);
+  }
+}
+}  // namespace
+
+extern "C" int vk_attn_bf16_hdp() { return HDP; }
+
+// tiles: pairs (entry, first token of the tile within the entry), 64 tokens per tile.
+extern "C" int vk_attn_bf16_prefill(const void* q, long long q_stride, const void* k_cache, const void* v_cache,
+                                    void* out, const int* tiles, int num_tiles, const int* entry_start,
+                                    const int* entry_first_pos, const int* block_table, int table_width,
+                                    int block_size, int heads, int kv_heads, int hd, float scale, int window,
+                                    void* stream) {
+  if (num_tiles <= 0) return 0;
+  if (hd <= 0 || hd > HDP || (hd & 7) || block_size <= 0 || (block_size & 7) || heads <= 0 || kv_heads <= 0 ||
+      heads % kv_heads || heads > 65535 || (q_stride & 7) || window < 0)
+    return VK_UNSUPPORTED_SIZE;
+  dim3 grid(num_tiles, heads);
+  attn_prefill_kernel<<<grid, 256, 0, (hipStream_t)stream>>>(
+      (const __bf16*)q, q_stride, (const __bf16*)k_cache, (const __bf16*)v_cache, (__bf16*)out, tiles, entry_start,
+      entry_first_pos, block_table, table_width, block_size, heads, kv_heads, hd, scale, window);
+  VK_LAUNCH_CHECK();
+  return 0;
+}
+
+// entries: indices of the step's entries that hold exactly one token. partial: at least
+// num_entries * heads * chunks * (hd + 2) floats. `chunks` must cover the longest visible range:
+// chunks * chunk >= longest position + 1.
+extern "C" int vk_attn_bf16_decode(const void* q, long long q_stride, const void* k_cache, const void* v_cache,
+                                   void* out, float* partial, const int* entries, int num_entries,
+                                   const int* entry_start, const int* entry_first_pos, const int* block_table,
+                                   int table_width, int block_size, int heads, int kv_heads, int hd, float scale,
+                                   int window, int chunk, int chunks, void* stream) {
+  if (num_entries <= 0) return 0;
+  if (hd <= 0 || hd > HDP || (hd & 7) || block_size <= 0 || (block_size & 7) || heads <= 0 || kv_heads <= 0 ||
+      heads % kv_heads || (q_stride & 7) || window < 0 || chunk < 32 || (chunk & 31) || chunks <= 0 ||
+      chunks > 65535)
+    return VK_UNSUPPORTED_SIZE;
+  const int group = heads / kv_heads, head_blocks = (group + 15) / 16;
+  if (kv_heads * head_blocks > 65535 || heads > 65535) return VK_UNSUPPORTED_SIZE;
+  hipStream_t s = (hipStream_t)stream;
+  dim3 grid(num_entries, kv_heads * head_blocks, chunks);
+  attn_decode_kernel<<<grid, 64, 0, s>>>((const __bf16*)q, q_stride, (const __bf16*)k_cache, (const __bf16*)v_cache,
+                                         partial, entries, entry_start, entry_first_pos, block_table, table_width,
+                                         block_size, heads, kv_heads, hd, scale, window, chunk, head_blocks);
+  VK_LAUNCH_CHECK();
+  dim3 cgrid(num_entries, heads);
+  attn_combine_kernel<<<cgrid, 64, 0, s>>>(partial, (__bf16*)out, entries, entry_start, heads, hd, chunks);
+  VK_LAUNCH_CHECK();
+  return 0;
+}

@@ -10,7 +10,8 @@
 // online over tiles of 256 keys that start at lo, so the arithmetic of a token depends only on
 // its position and the cache contents, not on how the step was cut or batched.
 //
-// Cache layout: [page, kv_head, slot, head_dim]; page of position p = table[entry, p / block_size].
+// Cache layout: K [page, kv_head, slot, head_dim], V transposed [page, kv_head, head_dim, slot];
+// page of position p = table[entry, p / block_size].
 #include "common.h"
 
 namespace {
@@ -71,8 +72,8 @@ __global__ __launch_bounds__(THREADS) void attn_generic_kernel(
       const int count = min(THREADS, hi - base);
       for (int j = vpart; j < count; j += parts) {
         const int pj = base + j;
-        const T* v_row = v_cache + (((size_t)page_s[j] * kv_heads + kvh) * block_size + (pj % block_size)) * hd;
-        acc = fmaf(p_s[j], to_float<T>(v_row[vd]), acc);
+        const T* v_at = v_cache + (((size_t)page_s[j] * kv_heads + kvh) * hd + vd) * block_size + (pj % block_size);
+        acc = fmaf(p_s[j], to_float<T>(*v_at), acc);
       }
     }
     __syncthreads();

@@ -71,8 +71,10 @@ extern "C" int vk_rmsnorm(const float* x, const float* weight, const int* rows, 
 // ---------------------------------------------------------------------------------------------
 // One block per token. `qkv` row layout: [heads*hd | kv_heads*hd | kv_heads*hd].
 // The first `rotary_dim` dims of every q and k head are rotated in place (angles in 32-bit:
-// float(pos) * inv_freq[i]); then the token's K and V rows go to the paged cache, whose layout is
-// [page, kv_head, slot, hd]. A token whose page id is negative writes nothing to the cache.
+// float(pos) * inv_freq[i]); then the token's K and V rows go to the paged cache. K pages are
+// [page, kv_head, slot, hd]; V pages are transposed, [page, kv_head, hd, slot], so that the
+// attention kernels read consecutive positions of one output dim. A token whose page id is
+// negative writes nothing to the cache.
 template <typename T>
 __global__ void rope_kvwrite_kernel(T* __restrict__ qkv, const int* __restrict__ positions,
                                     const float* __restrict__ inv_freq, int rotary_dim,
@@ -105,9 +107,9 @@ __global__ void rope_kvwrite_kernel(T* __restrict__ qkv, const int* __restrict__
   const T* v_row = k_row + (size_t)kv_heads * hd;
   for (int idx = threadIdx.x; idx < kv_heads * hd; idx += blockDim.x) {
     const int kvh = idx / hd, d = idx - kvh * hd;
-    const size_t at = (((size_t)page * kv_heads + kvh) * block_size + slot) * hd + d;
-    k_cache[at] = k_row[idx];
-    v_cache[at] = v_row[idx];
+    const size_t head = (size_t)page * kv_heads + kvh;
+    k_cache[(head * block_size + slot) * hd + d] = k_row[idx];
+    v_cache[(head * hd + d) * block_size + slot] = v_row[idx];
   }
 }
 

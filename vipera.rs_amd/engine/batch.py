@@ -18,6 +18,8 @@ import torch
 
 from ..errors import InternalError, InvalidArgumentError
 
+TILE_TOKENS = 64  # tokens of one prompt tile of the matrix-core attention kernel
+
 
 @dataclass
 class StepEntry:
@@ -44,6 +46,8 @@ class StepBatch:
     slots: torch.Tensor            # [E] int32, state slot of each entry's request
     logit_rows: torch.Tensor       # [R] int32, flat token indices
     block_tables: Dict[int, torch.Tensor]  # group -> [E, width] int32
+    prefill_tiles: torch.Tensor    # [tiles, 2] int32: (entry, first token within it) per 64 tokens of multi-token entries
+    decode_entries: torch.Tensor   # [n] int32: entries that hold exactly one token
     # host copies, for launch decisions
     host_counts: List[int] = field(default_factory=list)
     host_first_pos: List[int] = field(default_factory=list)
@@ -51,6 +55,9 @@ class StepBatch:
     max_count: int = 0
     max_kv_len: int = 0
     all_single: bool = False
+    num_prefill_tiles: int = 0
+    num_decode_entries: int = 0
+    max_decode_kv_len: int = 0
 
 
 def build_batch(entries: Sequence[StepEntry], cache, vocab_size: int, device, min_table_width: int = 1) -> StepBatch:
@@ -109,8 +116,20 @@ def build_batch(entries: Sequence[StepEntry], cache, vocab_size: int, device, mi
             table[k, :n] = row[:n]
         tables.append(table)
 
+    tiles: List[int] = []
+    singles: List[int] = []
+    for k, n in enumerate(counts):
+        if n == 1:
+            singles.append(k)
+        else:
+            for off in range(0, n, TILE_TOKENS):
+                tiles += [k, off]
+    max_decode_kv = max((int(kv_len[k]) for k in singles), default=0)
+
     parts = [flat.astype(np.int32), positions, entry_of, starts, first, kv_len.astype(np.int32), slots,
-             np.array(rows, dtype=np.int32)] + [t.reshape(-1) for t in tables]
+             np.array(rows, dtype=np.int32), np.array(tiles, dtype=np.int32), np.array(singles, dtype=np.int32)]
+    fixed = len(parts)
+    parts += [t.reshape(-1) for t in tables]
     sizes = [p.size for p in parts]
     host = torch.from_numpy(np.concatenate(parts)) if sum(sizes) else torch.zeros(0, dtype=torch.int32)
     dev = host.pin_memory().to(device, non_blocking=True) if device.type == "cuda" else host
@@ -118,12 +137,14 @@ def build_batch(entries: Sequence[StepEntry], cache, vocab_size: int, device, mi
     for size in sizes:
         views.append(dev[at:at + size])
         at += size
-    block_tables = {g: views[8 + g].view(E, tables[g].shape[1]) for g in range(len(groups))}
+    block_tables = {g: views[fixed + g].view(E, tables[g].shape[1]) for g in range(len(groups))}
     return StepBatch(
         num_tokens=T, num_entries=E, num_logit_rows=R,
         tokens=views[0], positions=views[1], entry_of_token=views[2], entry_start=views[3],
         entry_first_pos=views[4], entry_kv_len=views[5], slots=views[6], logit_rows=views[7],
-        block_tables=block_tables, host_counts=counts, host_first_pos=[int(v) for v in first],
+        block_tables=block_tables, prefill_tiles=views[8].view(-1, 2), decode_entries=views[9],
+        num_prefill_tiles=len(tiles) // 2, num_decode_entries=len(singles), max_decode_kv_len=max_decode_kv,
+        host_counts=counts, host_first_pos=[int(v) for v in first],
         host_slots=[int(v) for v in slots], max_count=max(counts), max_kv_len=int(kv_len.max()),
         all_single=max(counts) == 1,
     )

@@ -1,22 +1,49 @@
-"""Attention dispatch: which kernel attends over the paged cache for a step's tokens."""
+"""Attention dispatch: which kernel attends over the paged cache for a step's tokens.
+
+A bfloat16 run whose head width and page size allow 16-byte reads uses the matrix-core kernels: one
+launch for the tiles of multi-token entries (prompt portions), one (plus the merge) for the entries
+that hold a single token, whose positions are split into chunks.  Everything else (the 32-bit run,
+odd sizes) uses the 32-bit kernel, which serves both kinds alike.
+"""
 from __future__ import annotations
 
 import torch
 
 from . import kernels
 
-_bf16_attention = None
+DECODE_WAVES_WANTED = 2048   # enough waves to keep the memory system busy
+DECODE_CHUNKS_MAX = 128
 
 
-def set_bf16_attention(fn) -> None:
-    """Install the matrix-core implementation; ``fn(...) -> bool`` (False: not taken, fall through)."""
-    global _bf16_attention
-    _bf16_attention = fn
+def decode_chunking(max_kv_len: int, num_entries: int, kv_heads: int, head_blocks: int):
+    """``(chunk, chunks)``: positions per chunk (a multiple of 32) and chunks that cover ``max_kv_len``."""
+    chunk = 512
+    while chunk > 32:
+        chunks = (max_kv_len + chunk - 1) // chunk
+        if num_entries * kv_heads * head_blocks * chunks >= DECODE_WAVES_WANTED:
+            break
+        chunk //= 2
+    chunks = max(1, (max_kv_len + chunk - 1) // chunk)
+    while chunks > DECODE_CHUNKS_MAX:
+        chunk *= 2
+        chunks = (max_kv_len + chunk - 1) // chunk
+    return chunk, chunks
 
 
 def paged_attention(qkv, k_cache, v_cache, out, batch, table, heads, kv_heads, head_dim, scale, window) -> None:
-    if _bf16_attention is not None and qkv.dtype == torch.bfloat16:
-        if _bf16_attention(qkv, k_cache, v_cache, out, batch, table, heads, kv_heads, head_dim, scale, window):
-            return
+    if kernels.attn_bf16_supported(qkv, k_cache, head_dim):
+        if batch.num_prefill_tiles:
+            kernels.attn_bf16_prefill(qkv, k_cache, v_cache, out, batch.prefill_tiles, batch.entry_start,
+                                      batch.entry_first_pos, table, heads, kv_heads, head_dim, scale, window)
+        if batch.num_decode_entries:
+            group = heads // kv_heads
+            visible = batch.max_decode_kv_len
+            chunk, chunks = decode_chunking(visible, batch.num_decode_entries, kv_heads, (group + 15) // 16)
+            partial = torch.empty(batch.num_decode_entries * heads * chunks * (head_dim + 2), dtype=torch.float32,
+                                  device=qkv.device)
+            kernels.attn_bf16_decode(qkv, k_cache, v_cache, out, partial, batch.decode_entries, batch.entry_start,
+                                     batch.entry_first_pos, table, heads, kv_heads, head_dim, scale, window, chunk,
+                                     chunks)
+        return
     kernels.attn_generic(qkv, k_cache, v_cache, out, batch.positions, batch.entry_of_token, table, heads, kv_heads,
                          head_dim, scale, window)

@@ -28,7 +28,7 @@ HIP_FLAGS = [
 ]
 HOST_FLAGS = ["-O2", "-std=c++17", "-shared", "-fPIC", "-Wall"]
 
-# module name -> (compiler kind, sources relative to csrc, extra dependencies that enter the hash)
+# module name -> (compiler kind, sources relative to csrc, extra dependencies that enter the hash[, extra flags])
 MODULES: Dict[str, tuple] = {
     "elementwise": ("hip", ["kernels/elementwise.hip"], ["kernels/common.h"]),
     "gemm_generic": ("hip", ["kernels/gemm_generic.hip"], ["kernels/common.h"]),
@@ -38,6 +38,10 @@ MODULES: Dict[str, tuple] = {
     "host": ("host", ["host/cache_manager.cpp", "host/scheduler.cpp", "host/c_api.cpp"],
              ["host/cache_manager.h", "host/scheduler.h"]),
 }
+
+# matrix-core attention: one module per padded head width, compiled when a model of that width runs
+for _width in range(32, 257, 32):
+    MODULES[f"attn_bf16_hd{_width}"] = ("hip", ["kernels/attn_bf16.hip"], ["kernels/common.h"], [f"-DHDP={_width}"])
 
 _loaded: Dict[str, ctypes.CDLL] = {}
 _lock = threading.Lock()
@@ -55,14 +59,19 @@ def _hipcc() -> str:
 
 
 def _module_hash(name: str) -> str:
-    kind, sources, deps = MODULES[name]
+    kind, sources, deps = MODULES[name][:3]
     digest = hashlib.sha256()
-    digest.update(" ".join(HIP_FLAGS if kind == "hip" else HOST_FLAGS).encode())
+    digest.update(" ".join((HIP_FLAGS if kind == "hip" else HOST_FLAGS) + _extra_flags(name)).encode())
     for rel in list(sources) + list(deps):
         with open(os.path.join(_CSRC, rel), "rb") as handle:
             digest.update(rel.encode())
             digest.update(handle.read())
     return digest.hexdigest()[:12]
+
+
+def _extra_flags(name: str) -> List[str]:
+    entry = MODULES[name]
+    return list(entry[3]) if len(entry) > 3 else []
 
 
 def _build_dirs() -> List[str]:
@@ -94,14 +103,14 @@ def library_path(name: str, for_writing: bool = False) -> Optional[str]:
 
 def compile_module(name: str, verbose: bool = True) -> str:
     """Compile ``name`` now (even if a library exists) and return the library's path."""
-    kind, sources, _ = MODULES[name]
+    kind, sources = MODULES[name][:2]
     target = library_path(name, for_writing=True)
     tmp = f"{target}.{os.getpid()}.tmp"
     if kind == "hip":
         command = [_hipcc()] + HIP_FLAGS
     else:
         command = [os.environ.get("CXX") or shutil.which("g++") or "g++"] + HOST_FLAGS
-    command += ["-o", tmp] + [os.path.join(_CSRC, rel) for rel in sources]
+    command += _extra_flags(name) + ["-o", tmp] + [os.path.join(_CSRC, rel) for rel in sources]
     started = time.time()
     if verbose:
         print(f"[vipera build] compiling {name} ({', '.join(sources)})", file=sys.stderr, flush=True)

@@ -56,16 +56,26 @@ def _status(code: int, name: str) -> None:
     raise InternalError(f"{name}: HIP error {code} at launch")
 
 
+def _cache_ok(k_cache, v_cache, kv_heads: int, head_dim: int, dtype) -> bool:
+    """K pages ``[pages, kv_heads, block_size, head_dim]``, V pages ``[pages, kv_heads, head_dim, block_size]``."""
+    return (k_cache.dim() == 4 and v_cache.dim() == 4 and k_cache.shape[1] == kv_heads
+            and k_cache.shape[3] == head_dim and v_cache.shape[1] == kv_heads and v_cache.shape[2] == head_dim
+            and v_cache.shape[0] == k_cache.shape[0] and v_cache.shape[3] == k_cache.shape[2]
+            and k_cache.dtype == dtype and v_cache.dtype == dtype and k_cache.is_contiguous()
+            and v_cache.is_contiguous())
+
+
 _signatures_done = set()
 
 
-def _fn(module: str, name: str, argtypes):
+def _fn(module: str, name: str, argtypes, key: str = None):
     library = load_module(module)
     fn = getattr(library, name)
-    if name not in _signatures_done:
+    key = key or name
+    if key not in _signatures_done:
         fn.argtypes = argtypes
         fn.restype = ctypes.c_int
-        _signatures_done.add(name)
+        _signatures_done.add(key)
     return fn
 
 
@@ -103,7 +113,8 @@ def rope_kvwrite(qkv: torch.Tensor, positions: torch.Tensor, inv_freq: Optional[
                  block_table: Optional[torch.Tensor], heads: int, kv_heads: int, head_dim: int) -> None:
     """Rotate the q and k heads of ``qkv`` in place, then store the tokens' K and V in their pages.
 
-    ``k_cache``/``v_cache``: ``[pages, kv_heads, block_size, head_dim]``; ``block_table``: ``[entries, width]``.
+    ``k_cache``: ``[pages, kv_heads, block_size, head_dim]``; ``v_cache`` is transposed,
+    ``[pages, kv_heads, head_dim, block_size]``; ``block_table``: ``[entries, width]``.
     The caller guarantees that every token's page exists in its entry's row of the table.
     """
     _dev(qkv, positions, inv_freq, k_cache, v_cache, entry_of_token, block_table)
@@ -118,9 +129,7 @@ def rope_kvwrite(qkv: torch.Tensor, positions: torch.Tensor, inv_freq: Optional[
     table_width = block_size = 0
     if k_cache is not None:
         _need(v_cache is not None and block_table is not None, "rope_kvwrite: cache without table")
-        _need(k_cache.dim() == 4 and k_cache.shape[1] == kv_heads and k_cache.shape[3] == head_dim
-              and k_cache.shape == v_cache.shape and k_cache.dtype == qkv.dtype == v_cache.dtype
-              and k_cache.is_contiguous() and v_cache.is_contiguous(), "rope_kvwrite: cache shape or dtype")
+        _need(_cache_ok(k_cache, v_cache, kv_heads, head_dim, qkv.dtype), "rope_kvwrite: cache shape or dtype")
         _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(),
               "rope_kvwrite: block table")
         _need(entry_of_token.dtype == torch.int32 and entry_of_token.numel() >= num_tokens, "rope_kvwrite: entries")
@@ -186,9 +195,7 @@ def attn_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, 
     num_tokens = out.shape[0]
     _need(q.dim() == 2 and q.shape[0] == num_tokens and q.stride(1) == 1 and q.shape[1] >= heads * head_dim, "attention: q")
     _need(out.shape == (num_tokens, heads * head_dim) and out.is_contiguous() and out.dtype == q.dtype, "attention: out")
-    _need(k_cache.dim() == 4 and k_cache.shape[1] == kv_heads and k_cache.shape[3] == head_dim
-          and k_cache.shape == v_cache.shape and k_cache.dtype == q.dtype == v_cache.dtype
-          and k_cache.is_contiguous() and v_cache.is_contiguous(), "attention: cache shape or dtype")
+    _need(_cache_ok(k_cache, v_cache, kv_heads, head_dim, q.dtype), "attention: cache shape or dtype")
     _need(positions.dtype == torch.int32 and positions.numel() >= num_tokens, "attention: positions")
     _need(entry_of_token.dtype == torch.int32 and entry_of_token.numel() >= num_tokens, "attention: entries")
     _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(), "attention: table")
@@ -283,3 +290,62 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], ou
     fn = _fn("gemm_bf16", "vk_gemm_bf16", [_p, _p, _p, _p, _i, _i, _i, _i, _ll, _ll, _i, _i, _i, _p])
     _status(fn(_ptr(a), _ptr(w), _ptr(bias), _ptr(out), _dt(out, "out"), m, n, k, lda, ldc, 1 if accumulate else 0,
                int(skinny_limit), int(skinny_shape), _stream()), "gemm_bf16")
+
+
+# ----------------------------------------------------------------------------------------------
+def attn_bf16_padded_width(head_dim: int) -> int:
+    """The padded head width a matrix-core attention module is compiled for (a multiple of 32)."""
+    return (head_dim + 31) // 32 * 32
+
+
+def attn_bf16_supported(q: torch.Tensor, k_cache: torch.Tensor, head_dim: int) -> bool:
+    return (q.dtype == torch.bfloat16 and head_dim % 8 == 0 and head_dim <= 256 and k_cache.shape[2] % 8 == 0
+            and q.stride(0) % 8 == 0 and q.data_ptr() % 16 == 0)
+
+
+def attn_bf16_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
+                      tiles: torch.Tensor, entry_start: torch.Tensor, entry_first_pos: torch.Tensor,
+                      block_table: torch.Tensor, heads: int, kv_heads: int, head_dim: int, scale: float,
+                      window: int) -> None:
+    """Attention of the entries' 64-token tiles listed in ``tiles`` (pairs: entry, first token within it)."""
+    _dev(q, k_cache, v_cache, out, tiles, entry_start, entry_first_pos, block_table)
+    _need(attn_bf16_supported(q, k_cache, head_dim), "attn_bf16: operands must be bfloat16 with 16-byte rows")
+    _need(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= heads * head_dim, "attention: q")
+    _need(out.shape == (q.shape[0], heads * head_dim) and out.is_contiguous() and out.dtype == q.dtype, "attention: out")
+    _need(_cache_ok(k_cache, v_cache, kv_heads, head_dim, q.dtype), "attention: cache shape or dtype")
+    _need(tiles.dtype == torch.int32 and tiles.numel() % 2 == 0 and tiles.is_contiguous(), "attention: tiles")
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(), "attention: table")
+    _need(entry_start.dtype == torch.int32 and entry_first_pos.dtype == torch.int32
+          and entry_start.numel() == block_table.shape[0] + 1 and entry_first_pos.numel() == block_table.shape[0],
+          "attention: entry arrays")
+    module = f"attn_bf16_hd{attn_bf16_padded_width(head_dim)}"
+    fn = _fn(module, "vk_attn_bf16_prefill", [_p, _ll, _p, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _f, _i, _p],
+             key=module + ".prefill")
+    _status(fn(_ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(tiles), tiles.numel() // 2,
+               _ptr(entry_start), _ptr(entry_first_pos), _ptr(block_table), block_table.shape[1], k_cache.shape[2],
+               heads, kv_heads, head_dim, float(scale), int(window), _stream()), "attn_bf16_prefill")
+
+
+def attn_bf16_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
+                     partial: torch.Tensor, entries: torch.Tensor, entry_start: torch.Tensor,
+                     entry_first_pos: torch.Tensor, block_table: torch.Tensor, heads: int, kv_heads: int,
+                     head_dim: int, scale: float, window: int, chunk: int, chunks: int) -> None:
+    """Attention of the single-token entries listed in ``entries``, positions split into ``chunks`` of ``chunk``."""
+    _dev(q, k_cache, v_cache, out, partial, entries, entry_start, entry_first_pos, block_table)
+    _need(attn_bf16_supported(q, k_cache, head_dim), "attn_bf16: operands must be bfloat16 with 16-byte rows")
+    _need(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= heads * head_dim, "attention: q")
+    _need(out.shape == (q.shape[0], heads * head_dim) and out.is_contiguous() and out.dtype == q.dtype, "attention: out")
+    _need(_cache_ok(k_cache, v_cache, kv_heads, head_dim, q.dtype), "attention: cache shape or dtype")
+    count = entries.numel()
+    _need(entries.dtype == torch.int32 and entries.is_contiguous(), "attention: entries")
+    _need(partial.dtype == torch.float32 and partial.is_contiguous()
+          and partial.numel() >= count * heads * chunks * (head_dim + 2), "attention: workspace too small")
+    _need(chunk >= 32 and chunk % 32 == 0 and chunks >= 1, "attention: chunk must be a multiple of 32")
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(), "attention: table")
+    module = f"attn_bf16_hd{attn_bf16_padded_width(head_dim)}"
+    fn = _fn(module, "vk_attn_bf16_decode",
+             [_p, _ll, _p, _p, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _f, _i, _i, _i, _p], key=module + ".decode")
+    _status(fn(_ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(partial), _ptr(entries), count,
+               _ptr(entry_start), _ptr(entry_first_pos), _ptr(block_table), block_table.shape[1], k_cache.shape[2],
+               heads, kv_heads, head_dim, float(scale), int(window), int(chunk), int(chunks), _stream()),
+            "attn_bf16_decode")
