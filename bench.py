@@ -1,0 +1,199 @@
+#!/usr/bin/env python3
+"""Throughput of the engine on one MI355X: decode tokens per second at batch 8 (the headline value),
+at batch 1 and 64, and prefill tokens per second at 2,048 tokens, each with its roofline fraction.
+
+    python bench.py --gpus 1 --steps K --warmup W
+
+The model has the layer sizes of Qwen2.5-7B (28 layers, hidden 3584, 28 heads over 4 KV heads of
+width 128, feed-forward 18944, vocabulary 152064, rotary base 1e6, untied output matrix) with seeded
+random weights N(0, 0.02) in bfloat16; token ids are seeded uniform-random.  Every request is
+prefilled for real and then decoded up to a context of 4,096 tokens; the timed steps are the last K
+decode steps of that run, through the engine's scheduler, captured step and greedy sampler.  A step
+is one decode step of the whole batch.
+
+Bytes a decode step has to read: every weight it uses once (all layer matrices, norms and the output
+matrix; of the embedding table only the batch's rows) and the keys and values of the live requests.
+Peaks are MI355X's published ones: HBM 8 TB/s; dense bfloat16 matrix cores 2.5 PFLOP/s.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK = 8.0e12
+MFMA_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+QWEN25_7B = {
+    "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2",
+    "num_hidden_layers": 28, "hidden_size": 3584, "num_attention_heads": 28, "num_key_value_heads": 4,
+    "intermediate_size": 18944, "vocab_size": 152064, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6,
+    "tie_word_embeddings": False, "max_position_embeddings": 32768, "hidden_act": "silu",
+    "use_sliding_window": False, "sliding_window": 131072, "max_window_layers": 28, "torch_dtype": "bfloat16",
+}
+
+
+def log(text):
+    print(f"[bench] {text}", file=sys.stderr, flush=True)
+
+
+def main() -> int:
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=64)
+    parser.add_argument("--warmup", type=int, default=8)
+    parser.add_argument("--batch", type=int, default=8, help="batch of the headline decode measurement")
+    parser.add_argument("--ctx", type=int, default=4096, help="context length the decode steps end at")
+    parser.add_argument("--layers", type=int, default=28, help="fewer layers than 28 only where memory or time needs it")
+    parser.add_argument("--points", default="1,64", help="further decode batch sizes to report")
+    parser.add_argument("--prefill-tokens", type=int, default=2048)
+    parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    parser.add_argument("--block-size", type=int, default=16)
+    args = parser.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU: this engine runs on a single MI355X, so --gpus {args.gpus} is not run")
+        return 2
+
+    import torch
+
+    import vipera_rs_amd  # noqa: F401
+    from vipera_rs_amd import Engine
+    from vipera_rs_amd.config import config_from_dict
+    from vipera_rs_amd.engine.batch import StepEntry
+    from vipera_rs_amd.engine.runner import ModelRunner
+    from vipera_rs_amd.models import build_model
+    from vipera_rs_amd.runtime import Runtime
+    from vipera_rs_amd.weights import random_device_tensors
+
+    dtype_key = "bf16" if args.dtype == "bfloat16" else "fp32"
+    element = 2 if dtype_key == "bf16" else 4
+    data = dict(QWEN25_7B, num_hidden_layers=args.layers)
+    config = config_from_dict(data)
+    runtime = Runtime("cuda:0", args.dtype)
+    model = build_model(config, runtime)
+    started = time.perf_counter()
+    model.load(random_device_tensors(model.tensor_specs(), 0, runtime.dtype, runtime.device))
+    torch.cuda.synchronize()
+    log(f"random weights for {args.layers} layers on the device in {time.perf_counter() - started:.1f} s")
+
+    batches = [args.batch] + [int(b) for b in args.points.split(",") if b.strip()]
+    largest = max(batches)
+    ctx = args.ctx
+    pages_per_request = (ctx + args.block_size - 1) // args.block_size
+    num_blocks = largest * pages_per_request + (args.prefill_tokens + args.block_size - 1) // args.block_size + 8
+    runner = ModelRunner(model, runtime, args.block_size, num_blocks, largest + 1, use_graphs=True, max_context=ctx)
+
+    H, L, V = config.hidden_size, args.layers, config.vocab_size
+    Q, KV, I = config.num_attention_heads * config.head_dim, config.num_key_value_heads * config.head_dim, \
+        config.intermediate_size
+    layer_matrix = H * (Q + 2 * KV) + Q * H + 2 * I * H + I * H
+    layer_vectors = (Q + 2 * KV) + 2 * H
+    kv_per_token = 2 * KV * element * L
+    weight_bytes = L * (layer_matrix * element + layer_vectors * 4) + V * H * element + H * 4
+
+    gen = torch.Generator().manual_seed(0)
+
+    def tokens(n):
+        return torch.randint(0, V, (n,), generator=gen).tolist()
+
+    # --- prefill of 2,048 tokens -----------------------------------------------------------------------
+    T = args.prefill_tokens
+    prompt = tokens(T)
+
+    def prefill_once(request):
+        runner.cache.reserve(request, 0, T)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        runner.step([StepEntry(request, 0, prompt, [T - 1])])
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        runner.cache.release(request)
+        return dt
+
+    prefill_once(10_000)
+    prefill_s = min(prefill_once(10_001 + k) for k in range(3))
+    prefill_flops = 2.0 * T * L * layer_matrix + 2.0 * V * H + L * 4.0 * config.num_attention_heads * config.head_dim \
+        * (T * (T + 1) / 2)
+    prefill = {"value": round(T / prefill_s, 1), "tokens": T, "ms": round(prefill_s * 1e3, 3),
+               "frac": round(prefill_flops / prefill_s / MFMA_PEAK[dtype_key], 4)}
+    log(f"prefill {T} tokens: {prefill['ms']} ms, {prefill['value']} tok/s, {prefill['frac']:.3f} of peak")
+
+    # --- decode ---------------------------------------------------------------------------------------------
+    def decode(batch, steps, warmup):
+        engine = Engine(None, runner=runner, max_num_seqs=batch, max_num_batched_tokens=8192, chunk_size=2048,
+                        max_model_len=ctx + 8)
+        prompt_len = ctx - steps - warmup - 1
+        for _ in range(batch):
+            engine.add_request(tokens(prompt_len), max_new_tokens=steps + warmup + 4)
+        last = time.perf_counter()
+        while True:  # prefill, until every request has its first token and the next step is all decode
+            report = engine.step()
+            if time.perf_counter() - last > 20:
+                log(f"  prefilling batch {batch}: {engine.scheduler.num_waiting} requests still waiting")
+                last = time.perf_counter()
+            if engine.scheduler.num_waiting == 0 and report.num_batched_tokens == batch:
+                break
+        for _ in range(warmup - 1):
+            engine.step()
+        torch.cuda.synchronize()
+        engine.micros = {key: 0 for key in engine.micros}
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            report = engine.step()
+            assert report.num_batched_tokens == batch and len(report.tokens) == batch
+        torch.cuda.synchronize()
+        seconds = time.perf_counter() - t0
+        log(f"  host microseconds per step: " + ", ".join(f"{k} {v // steps}" for k, v in engine.micros.items()))
+        mean_ctx = ctx - steps / 2.0
+        for request in list(engine._live):
+            engine.cancel(request)
+        assert runner.cache.check() == "" and runner.cache.live_requests() == 0
+        step_bytes = weight_bytes + batch * H * element + batch * mean_ctx * kv_per_token
+        return seconds, step_bytes
+
+    results = {}
+    for batch in batches:
+        steps = args.steps if batch == args.batch else max(16, args.steps // 2)
+        seconds, step_bytes = decode(batch, steps, args.warmup)
+        ms = seconds / steps * 1e3
+        results[batch] = {"tok_s": batch * steps / seconds, "ms": ms, "bytes": step_bytes,
+                          "gbs": step_bytes / (seconds / steps) / 1e9}
+        log(f"decode batch {batch}: {ms:.3f} ms/step, {results[batch]['tok_s']:.1f} tok/s, "
+            f"{results[batch]['gbs']:.0f} GB/s of {HBM_PEAK / 1e9:.0f}")
+
+    head = results[args.batch]
+    line = {
+        "metric": f"decode tokens per second at batch {args.batch}, context {ctx}",
+        "value": round(head["tok_s"], 1),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(head["ms"], 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": dtype_key,
+        "data": "synthetic: seeded random weights N(0, 0.02) and uniform-random token ids",
+        "config": {
+            "model": "Qwen2.5-7B shape", "layers": args.layers, "layers_full": 28, "hidden": H,
+            "heads": config.num_attention_heads, "kv_heads": config.num_key_value_heads,
+            "head_dim": config.head_dim, "intermediate": I, "vocab": V, "global_batch": args.batch,
+            "seq_len": ctx, "prefill_tokens": T, "block_size": args.block_size, "parallelism": "single GPU",
+            "sampling": "greedy", "weights_gb": round(weight_bytes / 1e9, 2),
+        },
+        "prefill": prefill,
+        "roofline": {"bound": "hbm", "achieved": round(head["gbs"], 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                     "frac": round(head["gbs"] * 1e9 / HBM_PEAK, 4)},
+        "points": {f"decode_b{b}": round(r["tok_s"], 1) for b, r in results.items() if b != args.batch},
+        "points_ms": {f"decode_b{b}": round(r["ms"], 4) for b, r in results.items() if b != args.batch},
+    }
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -154,3 +154,45 @@ def test_long_decoding_follows_the_plain_implementation(folders):
             assert token == int(order[-1]), f"token {k} differs from the plain implementation"
             checked += 1
     assert checked > 200
+
+
+def test_captured_decode_steps_equal_eager_steps_on_every_replay(folders):
+    """A graph is replayed many times, with eager prompt steps and synchronizations in between; each
+    replay must give the logits of the same step run eagerly."""
+    from vipera_rs_amd.engine.batch import StepEntry
+    from vipera_rs_amd.engine.runner import ModelRunner
+    vocab = CONFIG_B["vocab_size"]
+    runners = [ModelRunner.from_folder(folders["B"], dtype="bfloat16", block_size=8, num_blocks=64, num_slots=8)
+               for _ in range(2)]
+    from vipera_rs_amd.engine.graphs import DecodeGraphs
+    runners[1].graphs = DecodeGraphs(runners[1], 512)
+    prompts = {r: random_tokens(vocab, n, 300 + r) for r, n in enumerate((9, 30, 17))}
+    lengths = {r: 0 for r in prompts}
+    feed = {r: random_tokens(vocab, 40, 400 + r) for r in prompts}
+    for runner in runners:
+        for r, tokens in prompts.items():
+            runner.cache.reserve(r, 0, len(tokens))
+        runner.step([StepEntry(r, 0, tokens, [len(tokens) - 1]) for r, tokens in prompts.items()])
+    for r, tokens in prompts.items():
+        lengths[r] = len(tokens)
+    for step in range(24):
+        live = [r for r in prompts if not (step % 7 == 3 and r == 1)]  # one request sits out now and then
+        outs = []
+        for runner in runners:
+            entries = []
+            for r in live:
+                runner.cache.reserve(r, lengths[r], lengths[r] + 1)
+                entries.append(StepEntry(r, lengths[r], [feed[r][step]], [0]))
+            outs.append(runner.step(entries).float().cpu())
+            torch.cuda.synchronize()
+        assert torch.equal(outs[0], outs[1]), f"replay {step} differs from the eager step"
+        for r in live:
+            lengths[r] += 1
+        if step == 10:  # a new request arrives: an eager prompt step between replays, then a wider graph
+            prompts[3] = random_tokens(vocab, 21, 303)
+            feed[3] = random_tokens(vocab, 40, 403)
+            for runner in runners:
+                runner.cache.reserve(3, 0, 21)
+                runner.step([StepEntry(3, 0, prompts[3], [20])])
+            lengths[3] = 21
+    assert runners[1].graphs.replays == 24 and len(runners[1].graphs.graphs) >= 2

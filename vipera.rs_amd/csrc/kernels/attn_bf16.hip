@@ -247,27 +247,49 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
 }
 
 // Merge the chunks of one (entry, head): M = max m_c; out = sum_c acc_c e^(m_c - M) / sum_c l_c e^(m_c - M),
-// chunks in ascending order (layer.cu:443-467).
-__global__ void attn_combine_kernel(const float* __restrict__ partial, __bf16* __restrict__ out,
-                                    const int* __restrict__ entries, const int* __restrict__ entry_start, int heads,
-                                    int hd, int chunks) {
-  const int slot = blockIdx.x, h = blockIdx.y;
+// chunks in ascending order (layer.cu:443-467). One wave per (entry, head): the chunk weights are worked
+// out in parallel over the chunks (their sum by a fixed tree), then every lane owns output dims.
+constexpr int MAX_CHUNKS = 128;
+__global__ __launch_bounds__(64) void attn_combine_kernel(const float* __restrict__ partial, __bf16* __restrict__ out,
+                                                          const int* __restrict__ entries,
+                                                          const int* __restrict__ entry_start, int heads, int hd,
+                                                          int chunks) {
+  __shared__ float weight[MAX_CHUNKS];
+  const int slot = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const float* src = partial + ((size_t)slot * heads + h) * chunks * (hd + 2);
+  float mc[MAX_CHUNKS / 64], lc[MAX_CHUNKS / 64];
   float best = -INFINITY;
-  for (int c = 0; c < chunks; ++c) best = fmaxf(best, src[(size_t)c * (hd + 2) + hd]);
-  float total = 0.f;
-  for (int c = 0; c < chunks; ++c) {
-    const float mc = src[(size_t)c * (hd + 2) + hd];
-    if (mc > -INFINITY) total += src[(size_t)c * (hd + 2) + hd + 1] * __expf(mc - best);
+#pragma unroll
+  for (int i = 0; i < MAX_CHUNKS / 64; ++i) {
+    const int c = lane + 64 * i;
+    mc[i] = c < chunks ? src[(size_t)c * (hd + 2) + hd] : -INFINITY;
+    lc[i] = c < chunks ? src[(size_t)c * (hd + 2) + hd + 1] : 0.f;
+    best = fmaxf(best, mc[i]);
   }
+  best = wave_max(best);
+  float total = 0.f;
+#pragma unroll
+  for (int i = 0; i < MAX_CHUNKS / 64; ++i) {
+    const float w = mc[i] > -INFINITY ? __expf(mc[i] - best) : 0.f;
+    const int c = lane + 64 * i;
+    if (c < chunks) weight[c] = w;
+    total += w * lc[i];
+  }
+  total = wave_sum(total);
+  __syncthreads();
+  const float inv = 1.f / total;
   const int token = entry_start[entries[slot]];
-  for (int d = threadIdx.x; d < hd; d += blockDim.x) {
-    float acc = 0.f;
+  __bf16* dst = out + (size_t)token * heads * hd + (size_t)h * hd;
+  for (int d = lane * 4; d < hd; d += 256) {
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
     for (int c = 0; c < chunks; ++c) {
-      const float mc = src[(size_t)c * (hd + 2) + hd];
-      if (mc > -INFINITY) acc += src[(size_t)c * (hd + 2) + d] * __expf(mc - best);
+      const float w = weight[c];
+      if (w != 0.f) acc += *(const f32x4*)(src + (size_t)c * (hd + 2) + d) * w;
     }
-    out[(size_t)token * heads * hd + (size_t)h * hd + d] = (__bf16)(acc / total);
+    bf16x4 r;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) r[j] = (__bf16)(acc[j] * inv);
+    *(bf16x4*)(dst + d) = r;
   }
 }
 }  // namespace
@@ -303,7 +325,7 @@ extern "C" int vk_attn_bf16_decode(const void* q, long long q_stride, const void
   if (num_entries <= 0) return 0;
   if (hd <= 0 || hd > HDP || (hd & 7) || block_size <= 0 || (block_size & 7) || heads <= 0 || kv_heads <= 0 ||
       heads % kv_heads || (q_stride & 7) || window < 0 || chunk < 32 || (chunk & 31) || chunks <= 0 ||
-      chunks > 65535)
+      chunks > MAX_CHUNKS)
     return VK_UNSUPPORTED_SIZE;
   const int group = heads / kv_heads, head_blocks = (group + 15) / 16;
   if (kv_heads * head_blocks > 65535 || heads > 65535) return VK_UNSUPPORTED_SIZE;

@@ -36,12 +36,43 @@ extern "C" int vk_embed_gather(const void* table, int table_dtype, const int* to
 
 // ---------------------------------------------------------------------------------------------
 // One block per output row. `rows` (may be null) picks the input row of each output row.
+// The row is read once into registers (four floats at a time when the width allows) and the sum of
+// squares is reduced in a fixed order.
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
 template <typename TO>
-__global__ void rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ weight,
-                               const int* __restrict__ rows, TO* __restrict__ out, int width, float eps) {
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ weight,
+                                                      const int* __restrict__ rows, TO* __restrict__ out, int width,
+                                                      float eps) {
   __shared__ float scratch[16];
   const int r = blockIdx.x;
   const float* src = x + (size_t)(rows ? rows[r] : r) * width;
+  TO* dst = out + (size_t)r * width;
+  constexpr int MAXV = 8;  // up to 8 * 4 * 256 = 8192 columns stay in registers
+  if ((width & 3) == 0 && width <= MAXV * 4 * 256) {
+    f32x4_t v[MAXV];
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < MAXV; ++i) {
+      const int c = (threadIdx.x + 256 * i) * 4;
+      if (c < width) {
+        v[i] = *(const f32x4_t*)(src + c);
+        sum += v[i][0] * v[i][0] + v[i][1] * v[i][1] + v[i][2] * v[i][2] + v[i][3] * v[i][3];
+      }
+    }
+    sum = block_sum(sum, scratch);
+    const float inv = 1.0f / sqrtf(sum / (float)width + eps);
+#pragma unroll
+    for (int i = 0; i < MAXV; ++i) {
+      const int c = (threadIdx.x + 256 * i) * 4;
+      if (c < width) {
+        const f32x4_t w = *(const f32x4_t*)(weight + c);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) dst[c + j] = from_float<TO>(v[i][j] * inv * w[j]);
+      }
+    }
+    return;
+  }
   float sum = 0.f;
   for (int i = threadIdx.x; i < width; i += blockDim.x) {
     const float v = src[i];
@@ -49,7 +80,6 @@ __global__ void rmsnorm_kernel(const float* __restrict__ x, const float* __restr
   }
   sum = block_sum(sum, scratch);
   const float inv = 1.0f / sqrtf(sum / (float)width + eps);
-  TO* dst = out + (size_t)r * width;
   for (int i = threadIdx.x; i < width; i += blockDim.x) dst[i] = from_float<TO>(src[i] * inv * weight[i]);
 }
 

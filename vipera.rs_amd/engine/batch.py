@@ -6,12 +6,14 @@ same shape (``BatchEntry`` with ``new_tokens``, ``first_position`` and ``block_t
 crates/vipera-runtime/src/pipeline.rs:138-152) but its CPU backend runs mixed entries one after
 another (crates/vipera-backend-cpu/src/model.rs:796-827); here a mixed batch is the normal case.
 
-Everything is packed into one int32 host buffer and copied to the device once.
+Everything is packed into one int32 host buffer and copied to the device once.  The packing has a
+fixed order of sections, so a step of single tokens can also be copied into the standing buffer of
+a captured graph.
 """
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Dict, List, Sequence
+from typing import Dict, List, Optional, Sequence
 
 import numpy as np
 import torch
@@ -45,9 +47,9 @@ class StepBatch:
     entry_kv_len: torch.Tensor     # [E] int32, tokens in the cache after this step
     slots: torch.Tensor            # [E] int32, state slot of each entry's request
     logit_rows: torch.Tensor       # [R] int32, flat token indices
-    block_tables: Dict[int, torch.Tensor]  # group -> [E, width] int32
     prefill_tiles: torch.Tensor    # [tiles, 2] int32: (entry, first token within it) per 64 tokens of multi-token entries
     decode_entries: torch.Tensor   # [n] int32: entries that hold exactly one token
+    block_tables: Dict[int, torch.Tensor]  # group -> [E, width] int32
     # host copies, for launch decisions
     host_counts: List[int] = field(default_factory=list)
     host_first_pos: List[int] = field(default_factory=list)
@@ -60,8 +62,33 @@ class StepBatch:
     max_decode_kv_len: int = 0
 
 
-def build_batch(entries: Sequence[StepEntry], cache, vocab_size: int, device, min_table_width: int = 1) -> StepBatch:
-    """Pack ``entries`` for the device. The pages of every token must already be reserved in ``cache``."""
+@dataclass
+class PackedStep:
+    """Host side of a step: the sections in their fixed order, and what the launch decisions need."""
+
+    sections: List[np.ndarray]     # tokens, positions, entry_of, starts, first, kv_len, slots, rows, tiles, singles, tables...
+    table_widths: List[int]
+    num_tokens: int
+    num_entries: int
+    num_logit_rows: int
+    counts: List[int]
+    first: List[int]
+    slots: List[int]
+    max_kv_len: int
+    max_decode_kv_len: int
+
+    def flat(self) -> np.ndarray:
+        return np.concatenate([s.reshape(-1) for s in self.sections]) if self.sections else np.zeros(0, np.int32)
+
+
+def pack_entries(entries: Sequence[StepEntry], cache, vocab_size: int, min_table_width: int = 1,
+                 pad_entries: int = 0, pad_page: int = -1) -> PackedStep:
+    """Check ``entries`` and lay them out for the device.
+
+    The pages of every token must already be reserved in ``cache``.  ``pad_entries`` appends
+    single-token dummy entries (token 0 at position 0, every table entry ``pad_page``), which a
+    captured graph of a fixed batch size needs; their logits are computed and ignored.
+    """
     if not entries:
         raise InvalidArgumentError("a step needs at least one entry")
     counts = [len(e.tokens) for e in entries]
@@ -72,19 +99,32 @@ def build_batch(entries: Sequence[StepEntry], cache, vocab_size: int, device, mi
         if e.request in seen:
             raise InvalidArgumentError(f"request {e.request} appears twice in one step")
         seen.add(e.request)
-    T, E = sum(counts), len(entries)
-    flat = np.fromiter((t for e in entries for t in e.tokens), dtype=np.int64, count=T)
+    real = len(entries)
+    T_real = sum(counts)
+    flat = np.fromiter((t for e in entries for t in e.tokens), dtype=np.int64, count=T_real)
     if flat.min() < 0 or flat.max() >= vocab_size:
         bad = int(flat[(flat < 0) | (flat >= vocab_size)][0])
         raise InvalidArgumentError(f"token {bad} is outside the vocabulary of {vocab_size}")
-    starts = np.zeros(E + 1, dtype=np.int32)
-    starts[1:] = np.cumsum(counts)
-    first = np.array([e.start for e in entries], dtype=np.int32)
-    if first.min() < 0:
+    first_real = [int(e.start) for e in entries]
+    if min(first_real) < 0:
         raise InvalidArgumentError("an entry starts at a negative position")
-    kv_len = first + np.array(counts, dtype=np.int32)
-    entry_of = np.repeat(np.arange(E, dtype=np.int32), counts)
+    slots_real = [cache.slot(e.request) for e in entries]
+    if min(slots_real) < 0:
+        missing = entries[int(np.argmin(slots_real))].request
+        raise InternalError(f"request {missing} has no slot: nothing was reserved for it")
+
+    counts_all = counts + [1] * pad_entries
+    E = real + pad_entries
+    T = T_real + pad_entries
+    tokens = np.zeros(T, dtype=np.int32)
+    tokens[:T_real] = flat
+    starts = np.zeros(E + 1, dtype=np.int32)
+    starts[1:] = np.cumsum(counts_all)
+    first = np.array(first_real + [0] * pad_entries, dtype=np.int32)
+    kv_len = first + np.array(counts_all, dtype=np.int32)
+    entry_of = np.repeat(np.arange(E, dtype=np.int32), counts_all)
     positions = np.arange(T, dtype=np.int32) - starts[entry_of] + first[entry_of]
+    slots = np.array(slots_real + [0] * pad_entries, dtype=np.int32)
     rows: List[int] = []
     for k, e in enumerate(entries):
         for w in e.want:
@@ -92,15 +132,18 @@ def build_batch(entries: Sequence[StepEntry], cache, vocab_size: int, device, mi
                 raise InvalidArgumentError(
                     f"request {e.request}: wanted place {w} is outside its {counts[k]} tokens of this step")
             rows.append(int(starts[k]) + int(w))
-    R = len(rows)
-    slots = np.array([cache.slot(e.request) for e in entries], dtype=np.int32)
-    if slots.min() < 0:
-        missing = entries[int(np.argmin(slots))].request
-        raise InternalError(f"request {missing} has no slot: nothing was reserved for it")
+    tiles: List[int] = []
+    singles: List[int] = []
+    for k, n in enumerate(counts_all):
+        if n == 1:
+            singles.append(k)
+        else:
+            for off in range(0, n, TILE_TOKENS):
+                tiles += [k, off]
+    max_decode_kv = max((int(kv_len[k]) for k in singles), default=0)
 
-    groups = cache.groups
-    tables = []
-    for g, spec in enumerate(groups):
+    tables, widths = [], []
+    for g, spec in enumerate(cache.groups):
         width = max(min_table_width, int((int(kv_len.max()) + spec.block_size - 1) // spec.block_size))
         table = np.full((E, width), -1, dtype=np.int32)
         for k, e in enumerate(entries):
@@ -114,37 +157,41 @@ def build_batch(entries: Sequence[StepEntry], cache, vocab_size: int, device, mi
                     f"in cache group {g}; reserve before the step")
             n = min(len(row), width)
             table[k, :n] = row[:n]
+        if pad_entries:
+            table[real:, :] = pad_page
         tables.append(table)
+        widths.append(width)
+    sections = [tokens, positions, entry_of, starts, first, kv_len.astype(np.int32), slots,
+                np.array(rows, dtype=np.int32), np.array(tiles, dtype=np.int32), np.array(singles, dtype=np.int32)]
+    sections += tables
+    return PackedStep(sections, widths, T, E, len(rows), counts_all, [int(v) for v in first], [int(v) for v in slots],
+                      int(kv_len.max()), max_decode_kv)
 
-    tiles: List[int] = []
-    singles: List[int] = []
-    for k, n in enumerate(counts):
-        if n == 1:
-            singles.append(k)
-        else:
-            for off in range(0, n, TILE_TOKENS):
-                tiles += [k, off]
-    max_decode_kv = max((int(kv_len[k]) for k in singles), default=0)
 
-    parts = [flat.astype(np.int32), positions, entry_of, starts, first, kv_len.astype(np.int32), slots,
-             np.array(rows, dtype=np.int32), np.array(tiles, dtype=np.int32), np.array(singles, dtype=np.int32)]
-    fixed = len(parts)
-    parts += [t.reshape(-1) for t in tables]
-    sizes = [p.size for p in parts]
-    host = torch.from_numpy(np.concatenate(parts)) if sum(sizes) else torch.zeros(0, dtype=torch.int32)
-    dev = host.pin_memory().to(device, non_blocking=True) if device.type == "cuda" else host
+def batch_from_buffer(packed: PackedStep, dev: torch.Tensor) -> StepBatch:
+    """A StepBatch whose tensors are views of ``dev``, which holds ``packed.flat()``."""
     views, at = [], 0
-    for size in sizes:
-        views.append(dev[at:at + size])
-        at += size
-    block_tables = {g: views[fixed + g].view(E, tables[g].shape[1]) for g in range(len(groups))}
+    for section in packed.sections:
+        views.append(dev[at:at + section.size])
+        at += section.size
+    E = packed.num_entries
+    fixed = 10
+    block_tables = {g: views[fixed + g].view(E, packed.table_widths[g]) for g in range(len(packed.table_widths))}
     return StepBatch(
-        num_tokens=T, num_entries=E, num_logit_rows=R,
+        num_tokens=packed.num_tokens, num_entries=E, num_logit_rows=packed.num_logit_rows,
         tokens=views[0], positions=views[1], entry_of_token=views[2], entry_start=views[3],
         entry_first_pos=views[4], entry_kv_len=views[5], slots=views[6], logit_rows=views[7],
-        block_tables=block_tables, prefill_tiles=views[8].view(-1, 2), decode_entries=views[9],
-        num_prefill_tiles=len(tiles) // 2, num_decode_entries=len(singles), max_decode_kv_len=max_decode_kv,
-        host_counts=counts, host_first_pos=[int(v) for v in first],
-        host_slots=[int(v) for v in slots], max_count=max(counts), max_kv_len=int(kv_len.max()),
-        all_single=max(counts) == 1,
+        prefill_tiles=views[8].view(-1, 2), decode_entries=views[9], block_tables=block_tables,
+        host_counts=packed.counts, host_first_pos=packed.first, host_slots=packed.slots,
+        max_count=max(packed.counts), max_kv_len=packed.max_kv_len, all_single=max(packed.counts) == 1,
+        num_prefill_tiles=packed.sections[8].size // 2, num_decode_entries=packed.sections[9].size,
+        max_decode_kv_len=packed.max_decode_kv_len,
     )
+
+
+def build_batch(entries: Sequence[StepEntry], cache, vocab_size: int, device, min_table_width: int = 1) -> StepBatch:
+    """Pack ``entries`` and copy them to the device."""
+    packed = pack_entries(entries, cache, vocab_size, min_table_width)
+    host = torch.from_numpy(packed.flat())
+    dev = host.pin_memory().to(device, non_blocking=True) if device.type == "cuda" else host
+    return batch_from_buffer(packed, dev)

@@ -70,13 +70,15 @@ class Engine:
     ``model``: a folder with ``config.json`` and ``model.safetensors``.  ``dtype``: ``"bfloat16"``
     or ``"float32"``.  The cache has ``num_blocks`` pages of ``block_size`` positions per group of
     layers; when ``num_blocks`` is absent it is sized for ``max_num_seqs`` requests of
-    ``max_model_len`` tokens, bounded by free device memory.
+    ``max_model_len`` tokens, bounded by free device memory.  ``use_graphs`` (default on) replays
+    steps of single tokens as captured HIP graphs.
     """
 
     def __init__(self, model: str, dtype: str = "bfloat16", device: str = "cuda:0", block_size: int = 16,
                  num_blocks: Optional[int] = None, max_num_seqs: int = 8, max_num_batched_tokens: int = 2048,
                  chunk_size: int = 512, max_model_len: Optional[int] = None,
-                 eos_token_ids: Optional[Sequence[int]] = None, runner: Optional[ModelRunner] = None):
+                 eos_token_ids: Optional[Sequence[int]] = None, runner: Optional[ModelRunner] = None,
+                 use_graphs: Optional[bool] = None):
         if runner is None:
             runtime = Runtime(device, dtype)
             from ..config.registry import load_config
@@ -87,8 +89,10 @@ class Engine:
                     f"requested context {limit} exceeds the model's maximum of {config.context_limit}")
             if num_blocks is None:
                 num_blocks = max_num_seqs * ((limit + block_size - 1) // block_size)
-            runner = self._load(model, config, runtime, block_size, num_blocks, max_num_seqs)
-        else:
+            if use_graphs is None:
+                use_graphs = True
+            runner = self._load(model, config, runtime, block_size, num_blocks, max_num_seqs, use_graphs, limit)
+        else:  # a runner that is already set up (its model, cache and graphs are used as they are)
             config = runner.model.config
             limit = int(max_model_len or config.context_limit)
         self.runner = runner
@@ -106,7 +110,7 @@ class Engine:
         self.micros = {"schedule": 0, "compute": 0, "sample": 0}
 
     @staticmethod
-    def _load(folder, config, runtime, block_size, num_blocks, num_slots) -> ModelRunner:
+    def _load(folder, config, runtime, block_size, num_blocks, num_slots, use_graphs, max_context) -> ModelRunner:
         from ..models import build_model
         from ..weights import Checkpoint, load_tensors
 
@@ -128,7 +132,7 @@ class Engine:
                 raise InfeasibleError(
                     f"no room for a single cache page of {per_page} bytes in {free} free bytes of device memory")
             num_blocks = fit
-        return ModelRunner(model, runtime, block_size, num_blocks, max(num_slots, 1))
+        return ModelRunner(model, runtime, block_size, num_blocks, max(num_slots, 1), use_graphs, max_context)
 
     # --- requests ---------------------------------------------------------------------------------
     def add_request(self, prompt: Sequence[int], max_new_tokens: int = 32,

@@ -24,7 +24,8 @@ from .batch import StepBatch, StepEntry, build_batch
 
 
 class ModelRunner:
-    def __init__(self, model, runtime: Runtime, block_size: int, num_blocks: int, num_slots: int):
+    def __init__(self, model, runtime: Runtime, block_size: int, num_blocks: int, num_slots: int,
+                 use_graphs: bool = False, max_context: int = 0):
         if not model.loaded:
             raise InvalidArgumentError("the model has no weights yet; load them before building a runner")
         self.model = model
@@ -37,6 +38,10 @@ class ModelRunner:
         self.storage = CacheStorage(self.needs, groups, num_slots, runtime)
         self.vocab_size = model.vocab_size
         self.steps = 0
+        self.graphs = None
+        if use_graphs:
+            from .graphs import DecodeGraphs
+            self.graphs = DecodeGraphs(self, max_context or block_size * num_blocks)
 
     # --- construction helpers -----------------------------------------------------------------
     @classmethod
@@ -63,4 +68,7 @@ class ModelRunner:
 
     def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
         """Logits ``[wanted, vocab]`` (32-bit, on the device) in the order of the entries and their ``want``."""
+        if self.graphs is not None and self.graphs.wants(entries):
+            self.steps += 1
+            return self.graphs.step(entries)
         return self.run(self.prepare(entries))

@@ -87,3 +87,27 @@ def write_random_model(folder: str, config: ModelConfig, specs: Sequence[TensorS
         metadata={"format": "pt", "seed": seed},
     )
     return folder
+
+
+def random_device_tensors(specs: Sequence[TensorSpec], seed: int, run_dtype: torch.dtype, device):
+    """Seeded random weights made on the device, for models too large to write to a folder first.
+
+    The same counter-based streams as :func:`random_tensor`, evaluated by the ``fill_normal`` kernel;
+    values agree with the host's up to the last bit of the device's ``log`` and ``cos``.
+    """
+    from ..ops import kernels
+    from .checkpoint import kept_dtype
+
+    out: Dict[str, torch.Tensor] = {}
+    for spec in specs:
+        dtype = kept_dtype(spec, run_dtype, run_dtype)
+        tensor = torch.empty(spec.shape, dtype=dtype, device=device)
+        if spec.role == INT_TABLE or spec.init == "zeros":
+            tensor.zero_()
+        elif spec.init == "ones":
+            tensor.fill_(1.0)
+        else:
+            kernels.fill_normal(tensor, tensor_key(seed, spec.name), spec.std,
+                                1.0 if spec.init == "one_plus_normal" else 0.0)
+        out[spec.name] = tensor
+    return out
