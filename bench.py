@@ -123,13 +123,16 @@ def main() -> int:
 
     # --- decode ---------------------------------------------------------------------------------------------
     def decode(batch, steps, warmup):
-        engine = Engine(None, runner=runner, max_num_seqs=batch, max_num_batched_tokens=8192, chunk_size=2048,
+        # every prompt gets a portion in every prefill step, so that all requests start decoding together
+        engine = Engine(None, runner=runner, max_num_seqs=batch, max_num_batched_tokens=batch * 2048, chunk_size=2048,
                         max_model_len=ctx + 8)
         prompt_len = ctx - steps - warmup - 1
         for _ in range(batch):
             engine.add_request(tokens(prompt_len), max_new_tokens=steps + warmup + 4)
         last = time.perf_counter()
-        while True:  # prefill, until every request has its first token and the next step is all decode
+        for guard in range(10_000):  # prefill, until every request has its first token and the next step is all decode
+            if guard == 9_999 or not engine.has_work():
+                raise RuntimeError("the requests ended before a step of decode tokens only was reached")
             report = engine.step()
             if time.perf_counter() - last > 20:
                 log(f"  prefilling batch {batch}: {engine.scheduler.num_waiting} requests still waiting")
