@@ -47,59 +47,81 @@ struct CacheView {
   int table_width, block_size, kv_heads, hd, kvh;
 };
 
+// The K and V^T operands of one step of 32 positions.
+struct StepOperands {
+  bf16x8 kf[2][KS];  // two 16-position tiles of K
+  bf16x8 vf[DT];     // V^T: positions kb + 4g .. +3 and kb + 16 + 4g .. +3 of output dim 16 dt + lr
+};
+
+// Issue the loads of the step that starts at kb. Positions outside [begin, end), pages that are not
+// held and dims past the head width read as zero.
+__device__ __forceinline__ void load_step(int kb, int begin, int end, const CacheView& cv, StepOperands& r) {
+  const int lane = threadIdx.x & 63, lr = lane & 15, lg = lane >> 4;
+  const int bs = cv.block_size, hd = cv.hd;
+#pragma unroll
+  for (int sub = 0; sub < 2; ++sub) {
+    const int p = kb + sub * 16 + lr;
+    const __bf16* row = nullptr;
+    if (p >= begin && p < end) {
+      const int page = cv.table[p / bs];
+      if (page >= 0) row = cv.k + (((size_t)page * cv.kv_heads + cv.kvh) * bs + (p % bs)) * hd + lg * 8;
+    }
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+      r.kf[sub][ks] = (row && ks * 32 + lg * 8 < hd) ? *(const bf16x8*)(row + ks * 32) : zero8();
+  }
+  const __bf16* vrow[2] = {nullptr, nullptr};
+#pragma unroll
+  for (int half = 0; half < 2; ++half) {
+    const int p = kb + half * 16 + lg * 4;
+    if (p + 3 >= begin && p < end) {  // a group of four positions lies in one page (4 divides the page size)
+      const int page = cv.table[p / bs];
+      if (page >= 0) vrow[half] = cv.v + (((size_t)page * cv.kv_heads + cv.kvh) * hd) * bs + (p % bs);
+    }
+  }
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) {
+    const int d = dt * 16 + lr;
+    bf16x8 f = zero8();
+    if (d < hd) {
+#pragma unroll
+      for (int half = 0; half < 2; ++half)
+        if (vrow[half]) {
+          const bf16x4 x = *(const bf16x4*)(vrow[half] + (size_t)d * bs);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) f[half * 4 + i] = x[i];
+        }
+    }
+    r.vf[dt] = f;
+  }
+}
+
 // Online-softmax attention of 16 columns over positions [begin, end). Per lane: col_lo / col_pos are
 // the visible range [lo, pos] of the lane's column (pos < 0: the column is empty).
 // State: o[DT] (O^T tiles), m (running max of the column), l (this lane's share of the running sum).
+// With AHEAD the loads of a step are issued one step ahead of its arithmetic (twice the operand
+// registers, fewer waves per SIMD: right for decoding, where a wave has few steps and memory is the bound).
+template <bool AHEAD>
 __device__ __forceinline__ void attend_range(const bf16x8 (&qf)[KS], int col_lo, int col_pos, int begin, int end,
                                              const CacheView& cv, float scale, f32x4 (&o)[DT], float& m, float& l) {
-  const int lane = threadIdx.x & 63, lr = lane & 15, lg = lane >> 4;
-  const int bs = cv.block_size, hd = cv.hd;
-  for (int kb = begin & ~31; kb < end; kb += 32) {
+  const int lane = threadIdx.x & 63, lg = lane >> 4;
+  StepOperands cur, next;
+  const int first = begin & ~31;
+  if (first >= end) return;
+  if (AHEAD) load_step(first, begin, end, cv, cur);
+  for (int kb = first; kb < end; kb += 32) {
+    if (!AHEAD)
+      load_step(kb, begin, end, cv, cur);
+    else if (kb + 32 < end)
+      load_step(kb + 32, begin, end, cv, next);
     // ---- scores of two 16-position tiles
     f32x4 s[2];
 #pragma unroll
     for (int sub = 0; sub < 2; ++sub) {
-      const int p = kb + sub * 16 + lr;
-      const __bf16* row = nullptr;
-      if (p >= begin && p < end) {
-        const int page = cv.table[p / bs];
-        if (page >= 0) row = cv.k + (((size_t)page * cv.kv_heads + cv.kvh) * bs + (p % bs)) * hd + lg * 8;
-      }
       f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const bf16x8 kf = (row && ks * 32 + lg * 8 < hd) ? *(const bf16x8*)(row + ks * 32) : zero8();
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[ks], acc, 0, 0, 0);
-      }
+      for (int ks = 0; ks < KS; ++ks) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.kf[sub][ks], qf[ks], acc, 0, 0, 0);
       s[sub] = acc;
-    }
-    // ---- V^T operands of the step: positions kb + 4g .. +3 and kb + 16 + 4g .. +3 of output dim 16 dt + lr
-    bf16x8 vf[DT];
-    {
-      const __bf16* vrow[2] = {nullptr, nullptr};
-#pragma unroll
-      for (int half = 0; half < 2; ++half) {
-        const int p = kb + half * 16 + lg * 4;
-        if (p + 3 >= begin && p < end) {  // a group of four positions lies in one page (4 divides the page size)
-          const int page = cv.table[p / bs];
-          if (page >= 0) vrow[half] = cv.v + (((size_t)page * cv.kv_heads + cv.kvh) * hd) * bs + (p % bs);
-        }
-      }
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
-        const int d = dt * 16 + lr;
-        bf16x8 f = zero8();
-        if (d < hd) {
-#pragma unroll
-          for (int half = 0; half < 2; ++half)
-            if (vrow[half]) {
-              const bf16x4 x = *(const bf16x4*)(vrow[half] + (size_t)d * bs);
-#pragma unroll
-              for (int i = 0; i < 4; ++i) f[half * 4 + i] = x[i];
-            }
-        }
-        vf[dt] = f;
-      }
     }
     // ---- mask, running max, weights
     float sv[8];
@@ -134,8 +156,9 @@ __device__ __forceinline__ void attend_range(const bf16x8 (&qf)[KS], int col_lo,
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
       o[dt] *= alpha;
-      o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pf, o[dt], 0, 0, 0);
+      o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.vf[dt], pf, o[dt], 0, 0, 0);
     }
+    if (AHEAD && kb + 32 < end) cur = next;
   }
 }
 
@@ -176,7 +199,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
   const int first_col_pos = first_pos + q_off;
   const int begin = (window > 0 && first_col_pos + 1 > window) ? first_col_pos + 1 - window : 0;
   const int end = first_pos + q_off + cols;  // one past the last column's position
-  attend_range(qf, col_lo, col_pos, begin, end, cv, scale, o, m, l);
+  attend_range<false>(qf, col_lo, col_pos, begin, end, cv, scale, o, m, l);
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
   if (!col_ok) return;
@@ -198,7 +221,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
 // Decoding: grid (entries, kv_heads * head_blocks, chunks), one wave. Columns are the query heads of
 // one key head. Chunk c covers positions [c * chunk, (c + 1) * chunk) of the visible range and leaves
 // (max, sum, weighted sum) in `partial`: [entry, head, chunk, hd + 2] floats.
-__global__ __launch_bounds__(64) void attn_decode_kernel(
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void attn_decode_kernel(
     const __bf16* __restrict__ q, long long q_stride, const __bf16* __restrict__ k_cache,
     const __bf16* __restrict__ v_cache, float* __restrict__ partial, const int* __restrict__ entries,
     const int* __restrict__ entry_start, const int* __restrict__ entry_first_pos,
@@ -231,7 +254,7 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
-  attend_range(qf, lo, col_ok ? pos : -1, begin, end, cv, scale, o, m, l);
+  attend_range<true>(qf, lo, col_ok ? pos : -1, begin, end, cv, scale, o, m, l);
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
   if (!col_ok) return;
@@ -255,15 +278,17 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(const float* __restric
                                                           const int* __restrict__ entry_start, int heads, int hd,
                                                           int chunks) {
   __shared__ float weight[MAX_CHUNKS];
+  __shared__ f32x4 part_sum[64];
   const int slot = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-  const float* src = partial + ((size_t)slot * heads + h) * chunks * (hd + 2);
+  const size_t stride = hd + 2;
+  const float* src = partial + ((size_t)slot * heads + h) * chunks * stride;
   float mc[MAX_CHUNKS / 64], lc[MAX_CHUNKS / 64];
   float best = -INFINITY;
 #pragma unroll
   for (int i = 0; i < MAX_CHUNKS / 64; ++i) {
     const int c = lane + 64 * i;
-    mc[i] = c < chunks ? src[(size_t)c * (hd + 2) + hd] : -INFINITY;
-    lc[i] = c < chunks ? src[(size_t)c * (hd + 2) + hd + 1] : 0.f;
+    mc[i] = c < chunks ? src[(size_t)c * stride + hd] : -INFINITY;
+    lc[i] = c < chunks ? src[(size_t)c * stride + hd + 1] : 0.f;
     best = fmaxf(best, mc[i]);
   }
   best = wave_max(best);
@@ -278,18 +303,39 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(const float* __restric
   total = wave_sum(total);
   __syncthreads();
   const float inv = 1.f / total;
+  // lane -> (part, four output dims); part p sums the chunks c = p, p + parts, ... ; parts are added in order
+  const int quads = hd / 4;                         // hd is a multiple of 8
+  const int parts = quads >= 64 ? 1 : 64 / quads;
   const int token = entry_start[entries[slot]];
   __bf16* dst = out + (size_t)token * heads * hd + (size_t)h * hd;
-  for (int d = lane * 4; d < hd; d += 256) {
+  for (int q0 = 0; q0 < quads; q0 += 64) {
+    const int quad = q0 + (parts > 1 ? lane % quads : lane);
+    const int part = parts > 1 ? lane / quads : 0;
+    const bool active = quad < quads && part < parts;
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-    for (int c = 0; c < chunks; ++c) {
-      const float w = weight[c];
-      if (w != 0.f) acc += *(const f32x4*)(src + (size_t)c * (hd + 2) + d) * w;
-    }
-    bf16x4 r;
+    if (active) {
+      for (int c = part; c < chunks; c += parts) {
+        const float w = weight[c];
+        const f32x4 v = *(const f32x4*)(src + (size_t)c * stride + quad * 4);  // an empty chunk holds stale numbers
 #pragma unroll
-    for (int j = 0; j < 4; ++j) r[j] = (__bf16)(acc[j] * inv);
-    *(bf16x4*)(dst + d) = r;
+        for (int j = 0; j < 4; ++j) acc[j] += w != 0.f ? v[j] * w : 0.f;
+      }
+    }
+    if (parts > 1) {
+      __syncthreads();
+      part_sum[lane] = acc;
+      __syncthreads();
+      if (part == 0 && active) {
+        acc = part_sum[quad];
+        for (int p = 1; p < parts; ++p) acc += part_sum[p * quads + quad];
+      }
+    }
+    if (part == 0 && active) {
+      bf16x4 r;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) r[j] = (__bf16)(acc[j] * inv);
+      *(bf16x4*)(dst + quad * 4) = r;
+    }
   }
 }
 }  // namespace

@@ -196,36 +196,37 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const __bf16* _
     for (int cb = 0; cb < CB; ++cb) acc[rt][cb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   const int spans = (K + SPAN - 1) / SPAN;
-  bf16x8 w_cur[RT][4], w_next[RT][4];
-  auto load_w = [&](int span, bf16x8 (*dst)[4]) {
-    const int kb = span * SPAN;
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int k = kb + i * 32 + lg * 8;
-        dst[rt][i] = (span < spans && k < K) ? *(const bf16x8*)(wp[rt] + kb + i * 32) : zero8();
-      }
-  };
-  load_w(wave, w_cur);
-  for (int span = wave; span < spans; span += WAVES) {
-    load_w(span + WAVES, w_next);
+  // two spans are in flight: while one is multiplied, the loads of the next (weights and activations)
+  // are already issued, and nothing of the current span waits for them
+  bf16x8 w_cur[RT][4], w_next[RT][4], a_cur[CB][4], a_next[CB][4];
+  auto load_span = [&](int span, bf16x8 (*w_dst)[4], bf16x8 (*a_dst)[4]) {
     const int kb = span * SPAN;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int k = kb + i * 32 + lg * 8;
+      const bool ok = span < spans && kb + i * 32 + lg * 8 < K;
 #pragma unroll
-      for (int cb = 0; cb < CB; ++cb) {
-        const bf16x8 a = (a_ok[cb] && k < K) ? *(const bf16x8*)(ap[cb] + kb + i * 32) : zero8();
+      for (int rt = 0; rt < RT; ++rt) w_dst[rt][i] = ok ? *(const bf16x8*)(wp[rt] + kb + i * 32) : zero8();
+#pragma unroll
+      for (int cb = 0; cb < CB; ++cb) a_dst[cb][i] = (ok && a_ok[cb]) ? *(const bf16x8*)(ap[cb] + kb + i * 32) : zero8();
+    }
+  };
+  load_span(wave, w_cur, a_cur);
+  for (int span = wave; span < spans; span += WAVES) {
+    load_span(span + WAVES, w_next, a_next);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt)
-          acc[rt][cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_cur[rt][i], a, acc[rt][cb], 0, 0, 0);
-      }
+          acc[rt][cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_cur[rt][i], a_cur[cb][i], acc[rt][cb], 0, 0, 0);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) w_cur[rt][i] = w_next[rt][i];
+#pragma unroll
+      for (int cb = 0; cb < CB; ++cb) a_cur[cb][i] = a_next[cb][i];
     }
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) w_cur[rt][i] = w_next[rt][i];
   }
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt)
@@ -257,7 +258,8 @@ template <int CB, typename TC, bool ACC>
 int launch_skinny_cb(const __bf16* A, const __bf16* W, const float* bias, TC* C, int M, int N, int K, long long lda,
                      long long ldc, int vector_ok, int shape, hipStream_t s) {
   const int tiles = (N + 15) / 16;
-  if (shape == 0) shape = tiles >= 1024 ? ((CB >= 2 || M > 4) ? 2 : 1) : 3;  // measured on the 7B shapes
+  // measured on the 7B shapes; sixteen waves with more than one token block would not fit the registers
+  if (shape == 0) shape = tiles >= 1024 ? ((CB >= 2 || M > 4) ? 2 : 1) : (CB == 1 ? 3 : 1);
   switch (shape) {
     case 1: return launch_skinny_as<CB, 1, 4, TC, ACC>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, s);
     case 2: return launch_skinny_as<CB, 2, 4, TC, ACC>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, s);
