@@ -1,0 +1,425 @@
+"""The small kernels alone, each part of a layer alone, a run order that repeats a layer and shares a
+cache, and a toy mixer with state of its own that is registered, built and stepped from this file
+without any change to the package."""
+import math
+from dataclasses import dataclass
+from typing import List
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import CONFIG_A, CONFIG_B, make_folder, random_tokens, rel_err
+from plain import qwen2_plain as P
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _runtime(dtype):
+    from vipera_rs_amd.runtime import Runtime
+    return Runtime(DEV, dtype)
+
+
+# --- kernels alone ------------------------------------------------------------------------------------
+@pytest.mark.parametrize("table_dtype", [torch.float32, torch.bfloat16])
+def test_embed_gather(table_dtype):
+    from vipera_rs_amd.ops import kernels
+    table = torch.randn(331, 100).to(table_dtype).to(DEV)
+    tokens = torch.tensor([330, 0, 17, 17, 200], dtype=torch.int32, device=DEV)
+    out = torch.empty(5, 100, device=DEV)
+    kernels.embed_gather(table, tokens, out)
+    assert torch.equal(out, table.float()[tokens.long()])
+
+
+@pytest.mark.parametrize("width", [100, 3584, 8200, 97])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+def test_rmsnorm_kernel(width, out_dtype):
+    from vipera_rs_amd.ops import kernels
+    g = torch.Generator().manual_seed(width)
+    x = (torch.randn(6, width, generator=g) * 3).to(DEV)
+    w = (1 + 0.1 * torch.randn(width, generator=g)).to(DEV)
+    want = torch.tensor(P.rms_norm(x.cpu().double().numpy(), w.cpu().double().numpy(), 1e-5))
+    out = torch.empty(6, width, dtype=out_dtype, device=DEV)
+    kernels.rmsnorm(x, w, 1e-5, out)
+    tol = 2e-6 if out_dtype == torch.float32 else 5e-3
+    assert rel_err(out.float().cpu().numpy(), want.numpy()) < tol
+    rows = torch.tensor([4, 1], dtype=torch.int32, device=DEV)       # rows picked by index
+    picked = torch.empty(2, width, dtype=out_dtype, device=DEV)
+    kernels.rmsnorm(x, w, 1e-5, picked, rows)
+    assert torch.equal(picked, out[[4, 1]])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("hd,rotary_dim", [(16, 16), (48, 48), (128, 128), (64, 32), (32, 0)])
+def test_rope_and_cache_write(dtype, hd, rotary_dim):
+    from vipera_rs_amd.ops import kernels
+    from vipera_rs_amd.parts.rotary import neox_inverse_frequencies
+    heads, kv_heads, bs, base = 3, 2, 8, 50000.0
+    positions = [0, 1, 7, 8, 300, 41]
+    entry_of = [0, 0, 0, 0, 1, 1]
+    table = torch.tensor([[5, 2, -1, -1, -1, -1], [9, 9, 9, 9, 9, 0] + [-1] * 0], dtype=torch.int32)
+    table = torch.full((2, 40), -1, dtype=torch.int32)
+    table[0, 0], table[0, 1] = 5, 2
+    table[1, 300 // bs], table[1, 41 // bs] = 7, 3
+    g = torch.Generator().manual_seed(hd)
+    qkv = torch.randn(6, (heads + 2 * kv_heads) * hd, generator=g).to(dtype)
+    k_cache = torch.zeros(10, kv_heads, bs, hd, dtype=dtype)
+    v_cache = torch.zeros(10, kv_heads, hd, bs, dtype=dtype)
+    inv = torch.from_numpy(neox_inverse_frequencies(rotary_dim, base)) if rotary_dim else None
+    dev = lambda t: t.to(DEV) if t is not None else None  # noqa: E731
+    qkv_d, k_d, v_d = dev(qkv.clone()), dev(k_cache), dev(v_cache)
+    kernels.rope_kvwrite(qkv_d, dev(torch.tensor(positions, dtype=torch.int32)), dev(inv), rotary_dim, k_d, v_d,
+                         dev(torch.tensor(entry_of, dtype=torch.int32)), dev(table), heads, kv_heads, hd)
+    got = qkv_d.float().cpu().numpy()
+    tol = 2e-6 if dtype == torch.float32 else 8e-3
+    for t, pos in enumerate(positions):
+        # 32-bit rows make the plain rotation round the angle to 32-bit as the reference does (model.rs:4199-4201);
+        # with a 64-bit angle the two differ by the angle's rounding, about position * 6e-8
+        row = qkv[t].float().numpy()
+        for head in range(heads + kv_heads):
+            x = row[head * hd:(head + 1) * hd].reshape(1, hd)
+            want = x.copy()
+            if rotary_dim:
+                want[:, :rotary_dim] = P.rope_neox(x[:, :rotary_dim].copy(), pos, base)
+            assert np.max(np.abs(got[t, head * hd:(head + 1) * hd] - want[0])) < tol * max(1.0, np.max(np.abs(want)))
+        # v is untouched, and the cache holds the rotated k and the v at the token's page and slot
+        v_in = qkv[t, (heads + kv_heads) * hd:].float().numpy()
+        assert np.array_equal(got[t, (heads + kv_heads) * hd:], v_in)
+        page, slot = int(table[entry_of[t], pos // bs]), pos % bs
+        k_now = qkv_d[t, heads * hd:(heads + kv_heads) * hd].view(kv_heads, hd)
+        assert torch.equal(k_d[page, :, slot, :], k_now)
+        assert torch.equal(v_d[page, :, :, slot].float().cpu(), torch.tensor(v_in).view(kv_heads, hd))
+    written = {(int(table[e, p // bs]), p % bs) for e, p in zip(entry_of, positions)}
+    for page in range(10):
+        for slot in range(bs):
+            if (page, slot) not in written:
+                assert float(k_d[page, :, slot, :].abs().max()) == 0.0 and float(v_d[page, :, :, slot].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_swiglu_kernel(dtype):
+    from vipera_rs_amd.ops import kernels
+    gate_up = (torch.randn(7, 2 * 200) * 4).to(dtype).to(DEV)
+    out = torch.empty(7, 200, dtype=dtype, device=DEV)
+    kernels.swiglu(gate_up, out)
+    g, u = gate_up[:, :200].double().cpu().numpy(), gate_up[:, 200:].double().cpu().numpy()
+    assert rel_err(out.float().cpu().numpy(), u * P.silu(g)) < (2e-6 if dtype == torch.float32 else 5e-3)
+
+
+def test_device_random_weights_follow_the_host_stream():
+    from vipera_rs_amd.ops import kernels
+    from vipera_rs_amd.weights import standard_normal, tensor_key
+    key = tensor_key(5, "model.layers.3.mlp.down_proj.weight")
+    out = torch.empty(10_001, device=DEV)
+    kernels.fill_normal(out, key, 0.02, 1.0)
+    want = 1.0 + 0.02 * standard_normal(key, 10_001)
+    np.testing.assert_allclose(out.cpu().numpy(), want.astype(np.float32), rtol=2e-6, atol=1e-7)
+
+
+# --- parts alone -------------------------------------------------------------------------------------------
+def _random_part_tensors(cls, spec, prefix, seed, runtime):
+    from vipera_rs_amd.weights import kept_dtype, random_tensor
+    host, device = {}, {}
+    for t in cls.declare(spec, prefix):
+        value = random_tensor(t, seed, torch.float32)
+        kept = kept_dtype(t, torch.float32 if runtime.dtype == torch.float32 else torch.bfloat16, runtime.dtype)
+        device[t.name] = value.to(kept).to(runtime.device)
+        host[t.name] = device[t.name].double().cpu().numpy()
+    return host, device
+
+
+class _OneLayerCache:
+    """A cache manager and storage for a single attention part, and batches over them."""
+
+    def __init__(self, runtime, kv_spec, block_size=8, pages=40):
+        from vipera_rs_amd.cache import CacheGroupSpec, CacheManager, CacheStorage
+        from vipera_rs_amd.models.decoder import CacheNeed
+        groups = [CacheGroupSpec(block_size, pages, kv_spec.window)]
+        self.cache = CacheManager(groups, 4)
+        self.storage = CacheStorage([CacheNeed(0, kv_spec, None)], groups, 4, runtime)
+        self.runtime = runtime
+
+    def batch(self, entries):
+        from vipera_rs_amd.engine.batch import build_batch
+        for e in entries:
+            self.cache.reserve(e.request, e.start, e.start + len(e.tokens))
+        return build_batch(entries, self.cache, 1000, self.runtime.device)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_norm_mlp_embedding_and_head_parts(dtype):
+    from vipera_rs_amd.config import PartSpec
+    from vipera_rs_amd.parts import part_class
+    rt = _runtime(dtype)
+    tol = 1e-5 if dtype == "float32" else 1.5e-2
+    x = torch.randn(9, 72).to(DEV)
+    # norm
+    spec = PartSpec("rmsnorm", {"width": 72, "eps": 1e-5, "name": "ln"})
+    cls = part_class("norm", "rmsnorm")
+    host, dev = _random_part_tensors(cls, spec, "p.", 1, rt)
+    norm = cls(spec, "p.", rt)
+    norm.load(dev)
+    h = norm.forward(x)
+    assert h.dtype == rt.dtype
+    assert rel_err(h.float().cpu().numpy(), P.rms_norm(x.double().cpu().numpy(), host["p.ln.weight"], 1e-5)) < tol
+    # feed-forward adds into the 32-bit residual
+    spec = PartSpec("gated_mlp", {"hidden": 72, "intermediate": 200, "activation": "silu", "name": "mlp"})
+    cls = part_class("ffn", "gated_mlp")
+    host, dev = _random_part_tensors(cls, spec, "p.", 2, rt)
+    mlp = cls(spec, "p.", rt)
+    mlp.load(dev)
+    residual = torch.randn(9, 72).to(DEV)
+    before = residual.double().cpu().numpy()
+    mlp.forward(h, None, residual)
+    hh = h.double().cpu().numpy()
+    want = before + P.swiglu_mlp(hh, host["p.mlp.gate_proj.weight"], host["p.mlp.up_proj.weight"], host["p.mlp.down_proj.weight"])
+    assert rel_err(residual.cpu().numpy(), want) < tol
+    # embedding and output projection, untied and tied
+    espec = PartSpec("embedding", {"vocab": 331, "width": 72, "name": "emb"})
+    ecls = part_class("embedding", "embedding")
+    ehost, edev = _random_part_tensors(ecls, espec, "", 3, rt)
+    emb = ecls(espec, "", rt)
+    emb.load(edev)
+    tokens = torch.tensor([0, 330, 5], dtype=torch.int32, device=DEV)
+    got = emb.forward(tokens, 3)
+    assert got.dtype == torch.float32 and np.array_equal(got.cpu().numpy(), ehost["emb.weight"][[0, 330, 5]].astype(np.float32))
+    hcls = part_class("head", "lm_head")
+    for tied in (None, "emb"):
+        hspec = PartSpec("lm_head", {"vocab": 331, "width": 72, "name": "out", "tied_to": tied})
+        hhost, hdev = _random_part_tensors(hcls, hspec, "", 4, rt)
+        assert (len(hhost) == 0) == (tied is not None)
+        head = hcls(hspec, "", rt)
+        head.load({**edev, **hdev})
+        logits = head.forward(h)
+        weight = ehost["emb.weight"] if tied else hhost["out.weight"]
+        assert logits.dtype == torch.float32 and rel_err(logits.cpu().numpy(), hh @ weight.T) < tol
+        if tied:
+            assert head.weight.data_ptr() == emb.table.data_ptr()      # the same buffer, no copy
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("heads,kv_heads,hd,window,bias", [(4, 2, 16, 0, True), (3, 1, 32, 11, True), (6, 6, 48, 0, False)])
+def test_attention_part_in_portions(dtype, heads, kv_heads, hd, window, bias):
+    from vipera_rs_amd.config import PartSpec
+    from vipera_rs_amd.engine.batch import StepEntry
+    from vipera_rs_amd.parts import part_class
+    rt = _runtime(dtype)
+    hidden = 56
+    spec = PartSpec("attention", {"hidden": hidden, "heads": heads, "kv_heads": kv_heads, "head_dim": hd, "qkv_bias": bias,
+                                  "out_bias": False, "window": window, "scale": None, "name": "attn"})
+    cls = part_class("mixer", "attention")
+    host, dev = _random_part_tensors(cls, spec, "l.", 5, rt)
+    for name in host:                       # larger weights, so that the scores are not all alike
+        if name.endswith("proj.weight"):
+            dev[name] = (dev[name].float() * 8).to(dev[name].dtype)
+            host[name] = dev[name].double().cpu().numpy()
+    mixer = cls(spec, "l.", rt)
+    mixer.load(dev)
+    pos_spec = PartSpec("rotary_neox", {"head_dim": hd, "rotary_dim": hd, "base": 10000.0})
+    position = part_class("position", "rotary_neox")(pos_spec, "l.", rt)
+    T = 37
+    h = torch.randn(T, hidden).to(rt.dtype).to(DEV)
+    cfg = {"num_attention_heads": heads, "num_key_value_heads": kv_heads, "head_dim": hd, "rope_theta": 10000.0}
+    w = {k.replace("l.attn.", ""): v for k, v in host.items()}
+    want = P.attention_block(h.double().cpu().numpy(), w, "", cfg, window)
+    env = _OneLayerCache(rt, mixer.cache_spec())
+    residual = torch.zeros(T, hidden, device=DEV)
+    at = 0
+    for size in (5, 1, 16, 2, 13):          # portions of changing size; every one adds its rows
+        batch = env.batch([StepEntry(0, at, [1] * size)])
+        mixer.forward(h[at:at + size].contiguous(), batch, env.storage.kv[0], None, position, residual[at:at + size])
+        env.cache.advance(0, at + size)
+        at += size
+    assert rel_err(residual.cpu().numpy(), want) < (2e-5 if dtype == "float32" else 2e-2)
+
+
+# --- a run order that names a layer twice and lets an entry read another entry's cache ---------------------------
+def _plain_scheduled(cfg, w, tokens, schedule):
+    """Plain forward with an explicit run order: (layer, cache_of) pairs; a reading entry uses the keys
+    and values that the owning entry computed (from the owner's input), and its own queries."""
+    cfg = P.normalize_config(cfg)
+    T = len(tokens)
+    heads, kv_heads, hd = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    x = w["model.embed_tokens.weight"][np.asarray(tokens)]
+    kept = {}
+    for index, (layer, cache_of) in enumerate(schedule):
+        p = f"model.layers.{layer}."
+        h = P.rms_norm(x, w[p + "input_layernorm.weight"], cfg["rms_norm_eps"])
+        a = p + "self_attn."
+        q = P.linear(h, w[a + "q_proj.weight"], w[a + "q_proj.bias"]).reshape(T, heads, hd)
+        for t in range(T):
+            q[t] = P.rope_neox(q[t], t, cfg["rope_theta"])
+        if cache_of is None:
+            k = P.linear(h, w[a + "k_proj.weight"], w[a + "k_proj.bias"]).reshape(T, kv_heads, hd)
+            v = P.linear(h, w[a + "v_proj.weight"], w[a + "v_proj.bias"]).reshape(T, kv_heads, hd)
+            for t in range(T):
+                k[t] = P.rope_neox(k[t], t, cfg["rope_theta"])
+            kept[index] = (k, v)
+        else:
+            k, v = kept[cache_of]
+        x = x + P.linear(P.attention(q, k, v).reshape(T, heads * hd), w[a + "o_proj.weight"])
+        h = P.rms_norm(x, w[p + "post_attention_layernorm.weight"], cfg["rms_norm_eps"])
+        x = x + P.swiglu_mlp(h, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+    h = P.rms_norm(x, w["model.norm.weight"], cfg["rms_norm_eps"])
+    return P.linear(h, w["model.embed_tokens.weight"])
+
+
+def test_the_run_order_is_data(tmp_path):
+    from vipera_rs_amd.config import Qwen2Config, ScheduleEntry, register_architecture, unregister_architecture
+    from vipera_rs_amd.engine.batch import StepEntry
+    from vipera_rs_amd.engine.runner import ModelRunner
+    from vipera_rs_amd.models.decoder import DecoderModel
+
+    order = [(0, None), (1, None), (0, None), (1, 1)]     # layer 0 twice (two caches); the last entry reads entry 1's cache
+
+    class Looped(Qwen2Config):
+        architecture = "LoopedForCausalLM"
+
+        def schedule(self):
+            return [ScheduleEntry(layer, cache_of) for layer, cache_of in order]
+
+    register_architecture("LoopedForCausalLM", Looped, lambda config, runtime: DecoderModel(config, runtime))
+    try:
+        folder = make_folder(tmp_path / "looped", dict(CONFIG_A, architectures=["LoopedForCausalLM"]), 4)
+        cfg, w = P.load_folder(folder)
+        tokens = random_tokens(256, 29, 9)
+        want = _plain_scheduled(cfg, w, tokens, order)
+        runner = ModelRunner.from_folder(folder, dtype="float32", block_size=8, num_blocks=16, num_slots=2)
+        assert sum(kv is not None for kv in runner.storage.kv) == 4
+        assert runner.storage.kv[3] is runner.storage.kv[1] and runner.storage.kv[2] is not runner.storage.kv[0]
+        rows, at = [], 0
+        for size in (11, 1, 2, 15):
+            runner.cache.reserve(0, at, at + size)
+            rows.append(runner.step([StepEntry(0, at, tokens[at:at + size], list(range(size)))]).cpu().numpy())
+            at += size
+        assert rel_err(np.concatenate(rows), want) < 1e-4
+    finally:
+        unregister_architecture("LoopedForCausalLM")
+
+
+# --- a toy mixer with state of its own, defined here ----------------------------------------------------------------
+def test_a_stateful_toy_mixer_is_registered_built_and_stepped(tmp_path):
+    """``s_t = decay * s_{t-1} + W_in h_t``, ``y_t = W_out s_t``: one vector of state per request, no pages.
+    Layer 0 uses it, layer 1 is ordinary attention: different mixers in different layers of one model."""
+    from vipera_rs_amd.config import (LayerSpec, PartSpec, Qwen2Config, register_architecture, unregister_architecture)
+    from vipera_rs_amd.engine.batch import StepEntry
+    from vipera_rs_amd.engine.runner import ModelRunner
+    from vipera_rs_amd.models.decoder import DecoderModel
+    from vipera_rs_amd.parts import Mixer, StateSpec, register_mixer, unregister
+    from vipera_rs_amd.weights import MATRIX, TensorSpec
+
+    DECAY, WIDTH = 0.9, 24
+
+    class RunningState(Mixer):
+        def __init__(self, spec, prefix, runtime):
+            super().__init__(spec, prefix, runtime)
+            self.hidden = spec.params["hidden"]
+            self.w_in = self.w_out = None
+
+        @classmethod
+        def declare(cls, spec, prefix):
+            base = f"{prefix}{spec.params['name']}."
+            return [TensorSpec(base + "in.weight", (WIDTH, spec.params["hidden"]), MATRIX, std=0.3),
+                    TensorSpec(base + "out.weight", (spec.params["hidden"], WIDTH), MATRIX, std=0.3)]
+
+        def load(self, tensors):
+            base = f"{self.prefix}{self.spec.params['name']}."
+            self.w_in, self.w_out = tensors[base + "in.weight"].float(), tensors[base + "out.weight"].float()
+
+        def state_spec(self):
+            return StateSpec((WIDTH,), torch.float32)
+
+        def forward(self, h, batch, cache, state, position, residual, reads_only=False):
+            u = h.float() @ self.w_in.T
+            at = 0
+            for count, first, slot in zip(batch.host_counts, batch.host_first_pos, batch.host_slots):
+                s = torch.zeros(WIDTH, device=h.device) if first == 0 else state[slot].clone()   # zero on first use
+                for t in range(at, at + count):
+                    s = DECAY * s + u[t]
+                    residual[t] += s @ self.w_out.T
+                state[slot] = s
+                at += count
+
+    class ToyConfig(Qwen2Config):
+        architecture = "ToyStateForCausalLM"
+
+        def layer_specs(self) -> List[LayerSpec]:
+            specs = super().layer_specs()
+            first = specs[0]
+            specs[0] = LayerSpec(first.block, PartSpec("running_state", {"hidden": self.hidden_size, "name": "state"}),
+                                 first.ffn, first.mixer_norm, first.ffn_norm, PartSpec("none", {}), first.prefix)
+            return specs
+
+    def plain(cfg, w, tokens):
+        cfg = P.normalize_config(cfg)
+        x = w["model.embed_tokens.weight"][np.asarray(tokens)]
+        h = P.rms_norm(x, w["model.layers.0.input_layernorm.weight"], cfg["rms_norm_eps"])
+        s, ys = np.zeros(WIDTH), []
+        for t in range(len(tokens)):
+            s = DECAY * s + w["model.layers.0.state.in.weight"] @ h[t]
+            ys.append(w["model.layers.0.state.out.weight"] @ s)
+        x = x + np.stack(ys)
+        h = P.rms_norm(x, w["model.layers.0.post_attention_layernorm.weight"], cfg["rms_norm_eps"])
+        x = x + P.swiglu_mlp(h, *(w[f"model.layers.0.mlp.{n}_proj.weight"] for n in ("gate", "up", "down")))
+        h = P.rms_norm(x, w["model.layers.1.input_layernorm.weight"], cfg["rms_norm_eps"])
+        x = x + P.attention_block(h, w, "model.layers.1.self_attn.", cfg, 0)
+        h = P.rms_norm(x, w["model.layers.1.post_attention_layernorm.weight"], cfg["rms_norm_eps"])
+        x = x + P.swiglu_mlp(h, *(w[f"model.layers.1.mlp.{n}_proj.weight"] for n in ("gate", "up", "down")))
+        return P.linear(P.rms_norm(x, w["model.norm.weight"], cfg["rms_norm_eps"]), w["model.embed_tokens.weight"])
+
+    register_mixer("running_state", RunningState)
+    register_architecture("ToyStateForCausalLM", ToyConfig, lambda config, runtime: DecoderModel(config, runtime))
+    try:
+        folder = make_folder(tmp_path / "toy", dict(CONFIG_A, architectures=["ToyStateForCausalLM"]), 6)
+        cfg, w = P.load_folder(folder)
+        assert "model.layers.0.state.in.weight" in w and "model.layers.0.self_attn.q_proj.weight" not in w
+        runner = ModelRunner.from_folder(folder, dtype="float32", block_size=8, num_blocks=24, num_slots=3)
+        assert runner.storage.state[0].shape == (3, WIDTH) and runner.storage.kv[0] is None
+        assert runner.storage.kv[1] is not None and runner.storage.state[1] is None
+        requests = {0: random_tokens(256, 23, 1), 1: random_tokens(256, 17, 2), 2: random_tokens(256, 9, 3)}
+        want = {r: plain(cfg, w, toks) for r, toks in requests.items()}
+        # mixed steps: portions of some requests beside single tokens of others; request 2 starts late in the
+        # slot and pages that request 1 gave back, so state left in a slot must not leak into a new request
+        at = {r: 0 for r in requests}
+        plan = [[(0, 7), (1, 2)], [(0, 1), (1, 9)], [(1, 6)], [(0, 13), (2, 4)], [(0, 2), (2, 1)], [(2, 4)]]
+        for step in plan:
+            entries = []
+            for r, size in step:
+                runner.cache.reserve(r, at[r], at[r] + size)
+                entries.append(StepEntry(r, at[r], requests[r][at[r]:at[r] + size], list(range(size))))
+            logits = runner.step(entries).cpu().numpy()
+            row = 0
+            for r, size in step:
+                assert rel_err(logits[row:row + size], want[r][at[r]:at[r] + size]) < 1e-4, (r, at[r])
+                row += size
+                at[r] += size
+                if at[r] == len(requests[r]):
+                    runner.cache.release(r)
+        assert at == {r: len(t) for r, t in requests.items()} and runner.cache.check() == ""
+    finally:
+        unregister_architecture("ToyStateForCausalLM")
+        unregister("mixer", "running_state")
+
+
+# --- the first tokens of a sequence --------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_first_tokens_of_a_sequence(tmp_path, dtype):
+    from vipera_rs_amd.engine.batch import StepEntry
+    from vipera_rs_amd.engine.runner import ModelRunner
+    folder = make_folder(tmp_path / "m", CONFIG_B, 1, torch.float32 if dtype == "float32" else torch.bfloat16)
+    cfg, w = P.load_folder(folder)
+    runner = ModelRunner.from_folder(folder, dtype=dtype, block_size=8, num_blocks=8, num_slots=4)
+    tol = 1e-4 if dtype == "float32" else 3e-2
+    for rid, tokens in enumerate(([7], [7, 7], [299, 0, 150])):
+        want = P.forward(cfg, w, tokens)
+        runner.cache.reserve(rid, 0, len(tokens))
+        whole = runner.step([StepEntry(rid, 0, tokens, list(range(len(tokens))))]).cpu().numpy()
+        assert rel_err(whole, want) < tol
+        runner.cache.release(rid)
+        rows = []
+        for pos, token in enumerate(tokens):     # and one by one from position 0
+            runner.cache.reserve(10 + rid, pos, pos + 1)
+            rows.append(runner.step([StepEntry(10 + rid, pos, [token], [0])]).cpu().numpy()[0])
+        runner.cache.release(10 + rid)
+        assert rel_err(np.stack(rows), want) < tol
