@@ -282,6 +282,281 @@ int launch_skinny(const __bf16* A, const __bf16* W, const float* bias, TC* C, in
   return VK_UNSUPPORTED_SIZE;
 }
 
+// ---------------------------------------------------------------------------------------------
+// M <= 16, activations stationary. A workgroup owns a range of weight rows and one slice of K
+// (SLICE_SPANS * 128 wide). Each wave loads the slice of the activations once into registers and then
+// streams the 16-row weight tiles of the range through them: no LDS, no barrier in the loop, the next
+// tile's loads in flight while the current one is multiplied. The slices' partial sums go to a
+// workspace, [slice, M, N] floats; the workgroup that finishes a row range last (an atomic counter per
+// range says who) adds the slices in ascending order, applies the epilogue and resets the counter. The
+// sum has one fixed order whoever is last. Workgroups of one row range run on different XCDs, whose L2
+// caches do not see each other's lines: the partial sums are therefore written and read with device-scope
+// accesses (they go through to memory), the writers wait for their stores to complete before the counter
+// is bumped, and no cache-wide fence is needed (one per workgroup would flush the L2 a thousand times).
+constexpr int SLICE_SPANS = 4;
+constexpr int SLICE_K = SLICE_SPANS * SPAN;
+
+template <typename TC, bool ACCUMULATE>
+__global__ __launch_bounds__(256) void gemm_stationary_kernel(const __bf16* __restrict__ A,
+                                                              const __bf16* __restrict__ W,
+                                                              const float* __restrict__ bias, TC* __restrict__ C,
+                                                              float* __restrict__ partial,
+                                                              int* __restrict__ counters, int M, int N, int K,
+                                                              long long lda, long long ldc, int rows_per_group,
+                                                              int vector_ok) {
+  __shared__ int is_last;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int lr = lane & 15, lg = lane >> 4;
+  const int group = blockIdx.x, slice = blockIdx.y, slices = gridDim.y;
+  const int row0 = group * rows_per_group, row_end = min(N, row0 + rows_per_group);
+  const int k0 = slice * SLICE_K;
+
+  // the slice of the activations: lane (m = lr, g = lg), step i holds A[m][k0 + 32 i + 8 g .. + 8]
+  bf16x8 act[SLICE_SPANS * 4];
+  {
+    const bool a_ok = lr < M;
+    const __bf16* ap = A + (size_t)(a_ok ? lr : 0) * lda + k0 + lg * 8;
+#pragma unroll
+    for (int i = 0; i < SLICE_SPANS * 4; ++i)
+      act[i] = (a_ok && k0 + i * 32 + lg * 8 < K) ? *(const bf16x8*)(ap + i * 32) : zero8();
+  }
+  const int tiles = (row_end - row0 + 15) / 16;
+  bf16x8 w_cur[SLICE_SPANS * 4], w_next[SLICE_SPANS * 4];
+  auto load_tile = [&](int tile, bf16x8* dst) {
+    const int wrow = min(row0 + tile * 16 + lr, N - 1);
+    const __bf16* wp = W + (size_t)wrow * K + k0 + lg * 8;
+#pragma unroll
+    for (int i = 0; i < SLICE_SPANS * 4; ++i)
+      dst[i] = (tile < tiles && k0 + i * 32 + lg * 8 < K) ? *(const bf16x8*)(wp + i * 32) : zero8();
+  };
+  load_tile(wave, w_cur);
+  for (int tile = wave; tile < tiles; tile += 4) {
+    load_tile(tile + 4, w_next);
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < SLICE_SPANS * 4; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_cur[i], act[i], acc, 0, 0, 0);
+    const int n = row0 + tile * 16 + lg * 4;
+    if (lr < M && n < N) {
+      float* dst = partial + ((size_t)slice * M + lr) * N + n;
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (n + j < N) __hip_atomic_store(dst + j, acc[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+#pragma unroll
+    for (int i = 0; i < SLICE_SPANS * 4; ++i) w_cur[i] = w_next[i];
+  }
+  // who is last for this row range? every store above has completed before the counter moves
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __syncthreads();
+  if (tid == 0) {
+    const int before = __hip_atomic_fetch_add(&counters[group], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    is_last = before == slices - 1;
+  }
+  __syncthreads();
+  if (!is_last) return;
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  const int width = row_end - row0;
+  for (int idx = tid * 4; idx < M * ((width + 3) & ~3); idx += 256 * 4) {
+    const int per_row = (width + 3) & ~3;
+    const int m = idx / per_row, n = row0 + (idx - m * per_row);
+    if (n >= N) continue;
+    f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+    for (int sl = 0; sl < slices; ++sl) {
+      const float* src = partial + ((size_t)sl * M + m) * N + n;
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (n + j < N) sum[j] += __hip_atomic_load(src + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    store4<TC, ACCUMULATE>(C, ldc, m, n, M, N, sum, bias, vector_ok != 0);
+  }
+  if (tid == 0) __hip_atomic_store(&counters[group], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next product
+}
+
+template <typename TC, bool ACC>
+int launch_stationary(const __bf16* A, const __bf16* W, const float* bias, TC* C, float* partial, int* counters,
+                      int max_groups, long long partial_floats, int M, int N, int K, long long lda, long long ldc,
+                      int vector_ok, hipStream_t s) {
+  const int slices = (K + SLICE_K - 1) / SLICE_K;
+  // about a thousand workgroups, at least one tile per wave
+  long long rows = ((long long)N * slices / 1024 + 63) / 64 * 64;
+  if (rows < 64) rows = 64;
+  if (rows > 512) rows = 512;
+  const int groups = (int)((N + rows - 1) / rows);
+  if (groups > max_groups || (long long)slices * M * N > partial_floats || slices > 65535) return VK_UNSUPPORTED_SIZE;
+  dim3 grid(groups, slices);
+  gemm_stationary_kernel<TC, ACC><<<grid, 256, 0, s>>>(A, W, bias, C, partial, counters, M, N, K, lda, ldc, (int)rows,
+                                                         vector_ok);
+  VK_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------------
+// M <= 64, activations shared through LDS. A workgroup owns 64 * RT weight rows (16 * RT per wave)
+// and a range of K; all four waves walk that range together in chunks of 256. A chunk's activations
+// (16 * CB tokens x 256) are fetched once per workgroup into LDS, double-buffered, one barrier per
+// chunk; the weights go from HBM straight into the instruction's operand layout, the next chunk's
+// loads in flight while the current one is multiplied. With several K ranges (gridDim.y > 1) every
+// range writes its partial sums, [range, M, N] floats, and gemm_reduce_kernel adds the ranges in
+// ascending order afterwards (a second launch: kernel boundaries are what keeps the XCDs' caches coherent).
+constexpr int MID_CHUNK = 256;
+constexpr int MID_ROW = MID_CHUNK + 8;  // elements per LDS row: 528 bytes, so 16 rows hit 16 different 16-byte slots
+
+template <int CB, int RT, typename TC, bool ACCUMULATE>
+__global__ __launch_bounds__(256) void gemm_mid_kernel(const __bf16* __restrict__ A, const __bf16* __restrict__ W,
+                                                       const float* __restrict__ bias, TC* __restrict__ C, int M,
+                                                       int N, int K, long long lda, long long ldc, int k_per_range,
+                                                       long long range_stride, int vector_ok) {
+  extern __shared__ __attribute__((aligned(16))) __bf16 lds[];  // [2][CB * 16][MID_ROW]
+  constexpr int BUF = CB * 16 * MID_ROW;
+  constexpr int A_LOADS = CB * 2;  // 16-byte pieces of a chunk per thread
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int lr = lane & 15, lg = lane >> 4;
+  const int n0 = blockIdx.x * 64 * RT + wave * 16 * RT;
+  const int k_begin = blockIdx.y * k_per_range, k_end = min(K, k_begin + k_per_range);
+  C += (size_t)blockIdx.y * range_stride;
+
+  const __bf16* wp[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) wp[rt] = W + (size_t)min(n0 + rt * 16 + lr, N - 1) * K + lg * 8;
+  f32x4 acc[RT][CB];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb) acc[rt][cb] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  bf16x8 a_stage[A_LOADS], w_cur[RT][8], w_next[RT][8];
+  auto load_acts = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) {
+      const int id = tid + 256 * i, row = id >> 5, k = k0 + (id & 31) * 8;
+      a_stage[i] = (row < M && k < k_end) ? *(const bf16x8*)(A + (size_t)row * lda + k) : zero8();
+    }
+  };
+  auto store_acts = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) {
+      const int id = tid + 256 * i, row = id >> 5, c = id & 31;
+      *(bf16x8*)(lds + buf * BUF + row * MID_ROW + c * 8) = a_stage[i];
+    }
+  };
+  auto load_weights = [&](int k0, bf16x8 (*dst)[8]) {
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        dst[rt][i] = (k0 + i * 32 + lg * 8 < k_end) ? *(const bf16x8*)(wp[rt] + k0 + i * 32) : zero8();
+  };
+
+  load_acts(k_begin);
+  load_weights(k_begin, w_cur);
+  store_acts(0);
+  __syncthreads();
+  int buf = 0;
+  for (int k0 = k_begin; k0 < k_end; k0 += MID_CHUNK) {
+    const bool more = k0 + MID_CHUNK < k_end;
+    if (more) {
+      load_acts(k0 + MID_CHUNK);
+      load_weights(k0 + MID_CHUNK, w_next);
+    }
+    const __bf16* tile = lds + buf * BUF + lr * MID_ROW + lg * 8;
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int cb = 0; cb < CB; ++cb) {
+        const bf16x8 a = *(const bf16x8*)(tile + cb * 16 * MID_ROW + i * 32);
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+          acc[rt][cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_cur[rt][i], a, acc[rt][cb], 0, 0, 0);
+      }
+    if (more) store_acts(buf ^ 1);
+    __syncthreads();
+    buf ^= 1;
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) w_cur[rt][i] = w_next[rt][i];
+  }
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb)
+      store4<TC, ACCUMULATE>(C, ldc, cb * 16 + lr, n0 + rt * 16 + lg * 4, M, N, acc[rt][cb], bias, vector_ok != 0);
+}
+
+// C (+)= sum over ranges of partial[range] (+ bias): ranges in ascending order, four columns per thread.
+template <typename TC, bool ACCUMULATE>
+__global__ void gemm_reduce_kernel(const float* __restrict__ partial, const float* __restrict__ bias,
+                                   TC* __restrict__ C, int M, int N, long long ldc, int ranges, int vector_ok) {
+  const int quads = (N + 3) / 4;
+  const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (long long)M * quads) return;
+  const int m = (int)(idx / quads), n = (int)(idx % quads) * 4;
+  f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+  const bool whole = n + 3 < N && (N & 3) == 0;
+  for (int r = 0; r < ranges; ++r) {
+    const float* src = partial + ((size_t)r * M + m) * N + n;
+    if (whole) {
+      sum += *(const f32x4*)src;
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (n + j < N) sum[j] += src[j];
+    }
+  }
+  store4<TC, ACCUMULATE>(C, ldc, m, n, M, N, sum, bias, vector_ok != 0);
+}
+
+template <int CB, int RT, typename TC, bool ACC>
+int launch_mid_as(const __bf16* A, const __bf16* W, const float* bias, TC* C, float* partial, long long partial_floats,
+                  int ranges, int M, int N, int K, long long lda, long long ldc, int vector_ok, hipStream_t s) {
+  constexpr int lds_bytes = 2 * CB * 16 * MID_ROW * (int)sizeof(__bf16);
+  const int blocks = (N + 64 * RT - 1) / (64 * RT);
+  if (ranges <= 1) {
+    auto kernel = gemm_mid_kernel<CB, RT, TC, ACC>;
+    static bool configured = false;
+    if (!configured) {
+      hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+      if (e != hipSuccess) return (int)e;
+      configured = true;
+    }
+    kernel<<<dim3(blocks, 1), 256, lds_bytes, s>>>(A, W, bias, C, M, N, K, lda, ldc, K, 0, vector_ok);
+    VK_LAUNCH_CHECK();
+    return 0;
+  }
+  if (!partial || (long long)ranges * M * N > partial_floats) return VK_UNSUPPORTED_SIZE;
+  auto kernel = gemm_mid_kernel<CB, RT, float, false>;
+  static bool configured_partial = false;
+  if (!configured_partial) {
+    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    if (e != hipSuccess) return (int)e;
+    configured_partial = true;
+  }
+  const int k_per_range = ((K + ranges - 1) / ranges + MID_CHUNK - 1) / MID_CHUNK * MID_CHUNK;
+  const int used = (K + k_per_range - 1) / k_per_range;
+  kernel<<<dim3(blocks, used), 256, lds_bytes, s>>>(A, W, nullptr, partial, M, N, K, lda, N, k_per_range,
+                                                    (long long)M * N, (N & 3) == 0 ? 1 : 0);
+  VK_LAUNCH_CHECK();
+  const long long threads = (long long)M * ((N + 3) / 4);
+  gemm_reduce_kernel<TC, ACC><<<(int)((threads + 255) / 256), 256, 0, s>>>(partial, bias, C, M, N, ldc, used, vector_ok);
+  VK_LAUNCH_CHECK();
+  return 0;
+}
+
+template <typename TC, bool ACC>
+int launch_mid(const __bf16* A, const __bf16* W, const float* bias, TC* C, float* partial, long long partial_floats,
+               int ranges, int rows_per_wave, int M, int N, int K, long long lda, long long ldc, int vector_ok,
+               hipStream_t s) {
+  const int cb = (M + 15) / 16;
+#define VK_MID(CBV, RTV) return launch_mid_as<CBV, RTV, TC, ACC>(A, W, bias, C, partial, partial_floats, ranges, M, N, K, lda, ldc, vector_ok, s)
+  if (rows_per_wave == 2) {
+    switch (cb) { case 1: VK_MID(1, 2); case 2: VK_MID(2, 2); case 3: VK_MID(3, 2); case 4: VK_MID(4, 2); }
+  } else {
+    switch (cb) { case 1: VK_MID(1, 1); case 2: VK_MID(2, 1); case 3: VK_MID(3, 1); case 4: VK_MID(4, 1); }
+  }
+#undef VK_MID
+  return VK_UNSUPPORTED_SIZE;
+}
+
 template <typename TC, bool ACC>
 int launch_tile(const __bf16* A, const __bf16* W, const float* bias, TC* C, int M, int N, int K, long long lda,
                 long long ldc, int vector_ok, hipStream_t s) {
@@ -330,5 +605,60 @@ extern "C" int vk_gemm_bf16(const void* A, const void* W, const float* bias, voi
   if (c_dtype == DT_BF16)
     return skinny ? launch_skinny<__bf16, false>(a, w, bias, (__bf16*)C, M, N, K, lda, ldc, vector_ok, skinny_shape, s)
                   : launch_tile<__bf16, false>(a, w, bias, (__bf16*)C, M, N, K, lda, ldc, vector_ok, s);
+  return VK_BAD_ARGUMENT;
+}
+
+// The same product for M <= 16 with the activations held in registers and K split over workgroups.
+// partial: workspace of `partial_floats` floats, at least ceil(K / 512) * M * N. counters: `max_groups`
+// ints that are zero before the first call; every call leaves them zero. Calls that share a workspace
+// must not overlap (one stream).
+extern "C" int vk_gemm_bf16_stationary(const void* A, const void* W, const float* bias, void* C, int c_dtype, int M,
+                                       int N, int K, long long lda, long long ldc, int accumulate, float* partial,
+                                       long long partial_floats, int* counters, int max_groups, void* stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (M > 16) return VK_UNSUPPORTED_SIZE;
+  if (K <= 0 || (K & 7) || (lda & 7) || lda < K || ldc < N) return VK_BAD_ARGUMENT;
+  if (((uintptr_t)A & 15) || ((uintptr_t)W & 15) || ((uintptr_t)partial & 15) || !partial || !counters) return VK_BAD_ARGUMENT;
+  if (accumulate && c_dtype != DT_F32) return VK_BAD_ARGUMENT;
+  const int elem = c_dtype == DT_F32 ? 4 : 2;
+  const int vector_ok = ((ldc & 3) == 0 && ((uintptr_t)C & (4 * elem - 1)) == 0 &&
+                         (bias == nullptr || ((uintptr_t)bias & 15) == 0)) ? 1 : 0;
+  hipStream_t s = (hipStream_t)stream;
+  const __bf16* a = (const __bf16*)A;
+  const __bf16* w = (const __bf16*)W;
+  if (c_dtype == DT_F32) {
+    if (accumulate)
+      return launch_stationary<float, true>(a, w, bias, (float*)C, partial, counters, max_groups, partial_floats, M, N, K, lda, ldc, vector_ok, s);
+    return launch_stationary<float, false>(a, w, bias, (float*)C, partial, counters, max_groups, partial_floats, M, N, K, lda, ldc, vector_ok, s);
+  }
+  if (c_dtype == DT_BF16)
+    return launch_stationary<__bf16, false>(a, w, bias, (__bf16*)C, partial, counters, max_groups, partial_floats, M, N, K, lda, ldc, vector_ok, s);
+  return VK_BAD_ARGUMENT;
+}
+
+// The same product for M <= 64 with the activations shared through LDS. `ranges` > 1 splits K over
+// workgroups: partial sums go to `partial` (at least ranges * M * N floats) and a second kernel adds them.
+// rows_per_wave: 1 or 2 tiles of 16 weight rows per wave.
+extern "C" int vk_gemm_bf16_mid(const void* A, const void* W, const float* bias, void* C, int c_dtype, int M, int N,
+                                int K, long long lda, long long ldc, int accumulate, int ranges, int rows_per_wave,
+                                float* partial, long long partial_floats, void* stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (M > 64) return VK_UNSUPPORTED_SIZE;
+  if (K <= 0 || (K & 7) || (lda & 7) || lda < K || ldc < N || ranges < 1) return VK_BAD_ARGUMENT;
+  if (((uintptr_t)A & 15) || ((uintptr_t)W & 15) || ((uintptr_t)partial & 15)) return VK_BAD_ARGUMENT;
+  if (accumulate && c_dtype != DT_F32) return VK_BAD_ARGUMENT;
+  const int elem = c_dtype == DT_F32 ? 4 : 2;
+  const int vector_ok = ((ldc & 3) == 0 && ((uintptr_t)C & (4 * elem - 1)) == 0 &&
+                         (bias == nullptr || ((uintptr_t)bias & 15) == 0)) ? 1 : 0;
+  hipStream_t s = (hipStream_t)stream;
+  const __bf16* a = (const __bf16*)A;
+  const __bf16* w = (const __bf16*)W;
+  if (c_dtype == DT_F32) {
+    if (accumulate)
+      return launch_mid<float, true>(a, w, bias, (float*)C, partial, partial_floats, ranges, rows_per_wave, M, N, K, lda, ldc, vector_ok, s);
+    return launch_mid<float, false>(a, w, bias, (float*)C, partial, partial_floats, ranges, rows_per_wave, M, N, K, lda, ldc, vector_ok, s);
+  }
+  if (c_dtype == DT_BF16)
+    return launch_mid<__bf16, false>(a, w, bias, (__bf16*)C, partial, partial_floats, ranges, rows_per_wave, M, N, K, lda, ldc, vector_ok, s);
   return VK_BAD_ARGUMENT;
 }

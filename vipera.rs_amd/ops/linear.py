@@ -2,20 +2,47 @@
 
 All-bfloat16 operands whose rows are 16-byte aligned go to the matrix-core kernels; every other
 combination (the 32-bit run, or a matrix kept in 32-bit inside a bfloat16 run) goes to the
-32-bit FMA kernel.
+32-bit FMA kernel.  Among the matrix-core kernels the number of rows of ``a`` (tokens) decides:
+
+* more than 64: the 128x128 tiled kernel (prompts);
+* up to 64 (decoding): the product is a stream of the weights.  Few tokens, or few weight rows at up
+  to 16 tokens, use the kernel whose waves split K inside a workgroup; otherwise the kernel that
+  shares the activations through LDS, with K split over workgroups where the weight has too few rows
+  to fill the GPU otherwise.  The thresholds were measured on the 7B shapes on an MI355X.
 """
 from __future__ import annotations
 
-from typing import Optional
+from typing import Optional, Tuple
 
 import torch
 
 from . import kernels
 
+STATIONARY = False   # the register-stationary split-K product is measured slower than the others; kept for tests
+
+
+def mid_plan(m: int, n: int, k: int) -> Tuple[int, int]:
+    """``(ranges of K, 16-row tiles per wave)`` for the LDS-shared kernel."""
+    if n >= 100_000:
+        return (1, 2) if m > 16 else (1, 1)
+    if n >= 16_384:
+        return (2, 1) if m > 16 else (1, 1)
+    return min(16, max(1, k // 448)), 1
+
+
 def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
            accumulate: bool = False) -> torch.Tensor:
     if a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and kernels.gemm_bf16_supported(a, w, out):
-        kernels.gemm_bf16(a, w, bias, out, accumulate)
+        m, k = a.shape
+        n = w.shape[0]
+        if m > 64 or m <= 4 or (m <= 16 and n < 16_384):
+            if m <= 16 and STATIONARY:
+                kernels.gemm_bf16_stationary(a, w, bias, out, accumulate)
+            else:
+                kernels.gemm_bf16(a, w, bias, out, accumulate)
+        else:
+            ranges, rows_per_wave = mid_plan(m, n, k)
+            kernels.gemm_bf16_mid(a, w, bias, out, accumulate, ranges, rows_per_wave)
     else:
         kernels.gemm_generic(a, w, bias, out, accumulate)
     return out
