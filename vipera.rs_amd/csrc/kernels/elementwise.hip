@@ -99,47 +99,51 @@ extern "C" int vk_rmsnorm(const float* x, const float* weight, const int* rows, 
 }
 
 // ---------------------------------------------------------------------------------------------
-// One block per token. `qkv` row layout: [heads*hd | kv_heads*hd | kv_heads*hd].
+// One workgroup of 64 threads per (token, head): grid (tokens, heads + 2 * kv_heads); the last
+// kv_heads of a row are the value heads. `qkv` row layout: [heads*hd | kv_heads*hd | kv_heads*hd].
 // The first `rotary_dim` dims of every q and k head are rotated in place (angles in 32-bit:
 // float(pos) * inv_freq[i]); then the token's K and V rows go to the paged cache. K pages are
 // [page, kv_head, slot, hd]; V pages are transposed, [page, kv_head, hd, slot], so that the
 // attention kernels read consecutive positions of one output dim. A token whose page id is
 // negative writes nothing to the cache.
 template <typename T>
-__global__ void rope_kvwrite_kernel(T* __restrict__ qkv, const int* __restrict__ positions,
-                                    const float* __restrict__ inv_freq, int rotary_dim,
-                                    T* __restrict__ k_cache, T* __restrict__ v_cache,
-                                    const int* __restrict__ entry_of_token, const int* __restrict__ block_table,
-                                    int table_width, int block_size, int heads, int kv_heads, int hd) {
-  const int t = blockIdx.x;
+__global__ __launch_bounds__(64) void rope_kvwrite_kernel(T* __restrict__ qkv, const int* __restrict__ positions,
+                                                          const float* __restrict__ inv_freq, int rotary_dim,
+                                                          T* __restrict__ k_cache, T* __restrict__ v_cache,
+                                                          const int* __restrict__ entry_of_token,
+                                                          const int* __restrict__ block_table, int table_width,
+                                                          int block_size, int heads, int kv_heads, int hd) {
+  const int t = blockIdx.x, head = blockIdx.y;
   const int pos = positions[t];
-  const int row_width = (heads + 2 * kv_heads) * hd;
-  T* row = qkv + (size_t)t * row_width;
+  T* h = qkv + (size_t)t * (heads + 2 * kv_heads) * hd + (size_t)head * hd;
+  const bool is_q = head < heads, is_k = !is_q && head < heads + kv_heads;
   const int half = rotary_dim / 2;
-  if (half > 0) {
-    const int pairs = (heads + kv_heads) * half;
-    for (int idx = threadIdx.x; idx < pairs; idx += blockDim.x) {
-      const int head = idx / half, i = idx - head * half;
-      T* h = row + (size_t)head * hd;  // q heads then k heads are contiguous
-      float sn, cs;
-      sincosf((float)pos * inv_freq[i], &sn, &cs);
-      const float lo = to_float<T>(h[i]), hi = to_float<T>(h[i + half]);
-      h[i] = from_float<T>(lo * cs - hi * sn);
-      h[i + half] = from_float<T>(lo * sn + hi * cs);
-    }
-    __syncthreads();
-  }
-  if (k_cache == nullptr) return;
-  const int page = block_table[(size_t)entry_of_token[t] * table_width + pos / block_size];
-  if (page < 0) return;
+  int page = -1;
+  if (!is_q && k_cache != nullptr) page = block_table[(size_t)entry_of_token[t] * table_width + pos / block_size];
   const int slot = pos % block_size;
-  const T* k_row = row + (size_t)heads * hd;
-  const T* v_row = k_row + (size_t)kv_heads * hd;
-  for (int idx = threadIdx.x; idx < kv_heads * hd; idx += blockDim.x) {
-    const int kvh = idx / hd, d = idx - kvh * hd;
-    const size_t head = (size_t)page * kv_heads + kvh;
-    k_cache[(head * block_size + slot) * hd + d] = k_row[idx];
-    v_cache[(head * hd + d) * block_size + slot] = v_row[idx];
+  if (is_q || is_k) {
+    const int kvh = head - heads;
+    const size_t k_at = is_k && page >= 0 ? (((size_t)page * kv_heads + kvh) * block_size + slot) * hd : 0;
+    for (int i = threadIdx.x; i < hd; i += 64) {
+      if (i < half) {
+        float sn, cs;
+        sincosf((float)pos * inv_freq[i], &sn, &cs);
+        const float lo = to_float<T>(h[i]), hi = to_float<T>(h[i + half]);
+        const T a = from_float<T>(lo * cs - hi * sn), b = from_float<T>(lo * sn + hi * cs);
+        h[i] = a;
+        h[i + half] = b;
+        if (is_k && page >= 0) {
+          k_cache[k_at + i] = a;
+          k_cache[k_at + i + half] = b;
+        }
+      } else if (i >= rotary_dim && is_k && page >= 0) {
+        k_cache[k_at + i] = h[i];
+      }
+    }
+  } else if (page >= 0) {
+    const int kvh = head - heads - kv_heads;
+    const size_t v_at = (((size_t)page * kv_heads + kvh) * hd) * block_size + slot;
+    for (int i = threadIdx.x; i < hd; i += 64) v_cache[v_at + (size_t)i * block_size] = h[i];
   }
 }
 
@@ -151,13 +155,15 @@ extern "C" int vk_rope_kvwrite(void* qkv, int dtype, const int* positions, const
   if (hd <= 0 || heads <= 0 || kv_heads <= 0 || rotary_dim < 0 || rotary_dim > hd || (rotary_dim & 1))
     return VK_BAD_ARGUMENT;
   if (k_cache && (block_size <= 0 || table_width <= 0)) return VK_BAD_ARGUMENT;
+  if (heads + 2 * kv_heads > 65535) return VK_UNSUPPORTED_SIZE;
   hipStream_t s = (hipStream_t)stream;
+  const dim3 grid(num_tokens, heads + (k_cache ? 2 : 1) * kv_heads);  // without a cache the value heads have nothing to do
   if (dtype == DT_F32)
-    rope_kvwrite_kernel<float><<<num_tokens, 256, 0, s>>>((float*)qkv, positions, inv_freq, rotary_dim,
+    rope_kvwrite_kernel<float><<<grid, 64, 0, s>>>((float*)qkv, positions, inv_freq, rotary_dim,
                                                            (float*)k_cache, (float*)v_cache, entry_of_token,
                                                            block_table, table_width, block_size, heads, kv_heads, hd);
   else if (dtype == DT_BF16)
-    rope_kvwrite_kernel<bf16_t><<<num_tokens, 256, 0, s>>>((bf16_t*)qkv, positions, inv_freq, rotary_dim,
+    rope_kvwrite_kernel<bf16_t><<<grid, 64, 0, s>>>((bf16_t*)qkv, positions, inv_freq, rotary_dim,
                                                             (bf16_t*)k_cache, (bf16_t*)v_cache, entry_of_token,
                                                             block_table, table_width, block_size, heads, kv_heads, hd);
   else

@@ -77,12 +77,27 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(const float* __restrict
   // --- best finite logit, ties to the lowest id ----------------------------------------------
   float best = -INFINITY;
   int best_id = 0x7fffffff;
-  for (int i = tid; i < vocab; i += THREADS) {
-    const float v = x[i];
-    if (finite_f(v) && (v > best || (v == best && i < best_id))) {
-      best = v;
-      best_id = i;
+  {
+    // four independent candidates per thread keep four loads in flight; they are merged in index order
+    float b4[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+    int i4[4] = {0x7fffffff, 0x7fffffff, 0x7fffffff, 0x7fffffff};
+    for (int base = tid; base < vocab; base += 4 * THREADS) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int i = base + u * THREADS;
+        const float v = i < vocab ? x[i] : NAN;
+        if (finite_f(v) && v > b4[u]) {  // within one candidate the indices ascend, so ties keep the lower one
+          b4[u] = v;
+          i4[u] = i;
+        }
+      }
     }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (b4[u] > best || (b4[u] == best && i4[u] < best_id)) {
+        best = b4[u];
+        best_id = i4[u];
+      }
   }
 #pragma unroll
   for (int off = WAVE / 2; off > 0; off >>= 1) {

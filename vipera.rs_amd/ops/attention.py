@@ -11,7 +11,7 @@ import torch
 
 from . import kernels
 
-DECODE_WAVES_WANTED = 2048   # enough waves to keep the memory system busy
+DECODE_WAVES_WANTED = 1024   # enough waves to keep the memory system busy
 DECODE_CHUNKS_MAX = 128
 
 
