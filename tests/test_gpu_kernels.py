@@ -281,3 +281,28 @@ def test_gemm_mid_against_float64(m, n, k, ranges, rows_per_wave):
     acc = base.clone()
     kernels.gemm_bf16_mid(a, w, None, acc, accumulate=True, ranges=ranges, rows_per_wave=rows_per_wave)
     assert _rel(acc, base.double() + a.double() @ w.double().T) < 1e-5
+
+
+@pytest.mark.parametrize("m,inter,k", [(1, 32, 64), (5, 48, 96), (8, 18944, 512), (16, 176, 200), (33, 128, 264), (64, 1024, 256),
+                                       (65, 64, 72), (300, 208, 136), (2048, 512, 128)])
+def test_gated_product_and_interleaved_swiglu(m, inter, k):
+    from vipera_rs_amd.ops import kernels
+    from vipera_rs_amd.ops.linear import interleave_gate_up, linear_gated
+    g = torch.Generator().manual_seed(m + inter + k)
+    a = torch.randn(m, k, generator=g).to(torch.bfloat16).to(DEV)
+    gate = torch.randn(inter, k, generator=g).to(torch.bfloat16).to(DEV)
+    up = torch.randn(inter, k, generator=g).to(torch.bfloat16).to(DEV)
+    gd, ud = a.double() @ gate.double().T, a.double() @ up.double().T
+    want = ud * (gd / (1 + torch.exp(-gd)))
+    fused = interleave_gate_up(gate, up)
+    assert torch.equal(fused[:16], gate[:16]) and torch.equal(fused[16:32], up[:16])
+    for rows_per_wave in (1, 2):
+        out = torch.full((m, inter), 7.0, dtype=torch.bfloat16, device=DEV)
+        kernels.gemm_bf16_gated(a, fused, out, rows_per_wave)
+        assert _rel(out, want) < 8e-3, f"fused epilogue, {rows_per_wave} tiles per wave"
+    out = torch.empty(m, inter, dtype=torch.bfloat16, device=DEV)
+    linear_gated(a, fused, out, True)                       # whichever path the dispatch takes
+    assert _rel(out, want) < 1.2e-2
+    plain = torch.empty(m, inter, dtype=torch.bfloat16, device=DEV)
+    linear_gated(a, torch.cat([gate, up]).contiguous(), plain, False)
+    assert _rel(plain, want) < 1.2e-2

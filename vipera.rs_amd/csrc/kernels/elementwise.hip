@@ -173,30 +173,36 @@ extern "C" int vk_rope_kvwrite(void* qkv, int dtype, const int* positions, const
 }
 
 // ---------------------------------------------------------------------------------------------
-// out[t, i] = up * silu(gate), gate = gate_up[t, i], up = gate_up[t, inter + i]; math in 32-bit.
+// out[t, i] = up * silu(gate); math in 32-bit. Two layouts of a gate_up row: [gate | up] halves, or
+// `interleaved` in groups of 16 (gate of outputs 16 p .. 16 p + 15 at columns 32 p .., their up values
+// at columns 32 p + 16 ..), which is what the fused matrix-core product of the feed-forward wants.
 template <typename T>
-__global__ void swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out, int inter, long long total) {
+__global__ void swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out, int inter, long long total,
+                              int interleaved) {
   for (long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
        idx += (long long)gridDim.x * blockDim.x) {
     const long long t = idx / inter;
     const int i = (int)(idx - t * inter);
     const T* row = gate_up + t * 2 * inter;
-    const float g = to_float<T>(row[i]), u = to_float<T>(row[inter + i]);
+    const int gi = interleaved ? (i / 16) * 32 + (i % 16) : i;
+    const int ui = interleaved ? gi + 16 : inter + i;
+    const float g = to_float<T>(row[gi]), u = to_float<T>(row[ui]);
     out[idx] = from_float<T>(u * (g / (1.0f + expf(-g))));
   }
 }
 
-extern "C" int vk_swiglu(const void* gate_up, void* out, int dtype, int num_tokens, int inter, void* stream) {
+extern "C" int vk_swiglu(const void* gate_up, void* out, int dtype, int num_tokens, int inter, int interleaved,
+                         void* stream) {
   if (num_tokens <= 0) return 0;
-  if (inter <= 0) return VK_BAD_ARGUMENT;
+  if (inter <= 0 || (interleaved && (inter & 15))) return VK_BAD_ARGUMENT;
   const long long total = (long long)num_tokens * inter;
   long long blocks = (total + 255) / 256;
   if (blocks > 65536) blocks = 65536;
   hipStream_t s = (hipStream_t)stream;
   if (dtype == DT_F32)
-    swiglu_kernel<float><<<(int)blocks, 256, 0, s>>>((const float*)gate_up, (float*)out, inter, total);
+    swiglu_kernel<float><<<(int)blocks, 256, 0, s>>>((const float*)gate_up, (float*)out, inter, total, interleaved);
   else if (dtype == DT_BF16)
-    swiglu_kernel<bf16_t><<<(int)blocks, 256, 0, s>>>((const bf16_t*)gate_up, (bf16_t*)out, inter, total);
+    swiglu_kernel<bf16_t><<<(int)blocks, 256, 0, s>>>((const bf16_t*)gate_up, (bf16_t*)out, inter, total, interleaved);
   else
     return VK_BAD_ARGUMENT;
   VK_LAUNCH_CHECK();

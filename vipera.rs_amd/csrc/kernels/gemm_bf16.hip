@@ -68,13 +68,33 @@ __device__ __forceinline__ void store4(TC* __restrict__ C, long long ldc, int m,
   }
 }
 
+// The gated epilogue. The fused gate/up weight interleaves its rows in groups of 16: fused rows
+// [32 p, 32 p + 16) are gate rows [16 p, 16 p + 16) and fused rows [32 p + 16, 32 p + 32) are the up rows of
+// the same outputs. A pair of accumulators (gate, up) of one token block gives
+// out[m][16 p + 4 g + j] = up * gate / (1 + exp(-gate)) (crates/vipera-backend-cpu/src/model.rs:4368-4374).
+__device__ __forceinline__ void store_gated(__bf16* __restrict__ C, long long ldc, int m, int n, int M, int inter,
+                                            f32x4 gate, f32x4 up) {
+  if (m >= M || n >= inter) return;
+  __bf16* dst = C + (size_t)m * ldc + n;
+  bf16x4 o;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) o[j] = (__bf16)(up[j] * (gate[j] / (1.0f + __expf(-gate[j]))));
+  if (n + 3 < inter && (ldc & 3) == 0 && ((uintptr_t)C & 7) == 0) {
+    *(bf16x4*)dst = o;
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (n + j < inter) dst[j] = o[j];
+  }
+}
+
 // ---------------------------------------------------------------------------------------------
 constexpr int BM = 128, BN = 128, BK = 64;
 constexpr int ROW = BK + 8;  // elements per LDS row: 144 bytes
 constexpr int TILE_ELEMS = BM * ROW;
 constexpr int XCDS = 8;
 
-template <typename TC, bool ACCUMULATE>
+template <typename TC, bool ACCUMULATE, bool GATED>
 __global__ __launch_bounds__(256) void gemm_tile_kernel(const __bf16* __restrict__ A, const __bf16* __restrict__ W,
                                                         const float* __restrict__ bias, TC* __restrict__ C, int M,
                                                         int N, int K, long long lda, long long ldc, int tiles_m,
@@ -152,12 +172,22 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(const __bf16* __restrict
     __syncthreads();
   }
 
+  if constexpr (GATED) {
+    // N counts fused rows; the output has N / 2 columns
 #pragma unroll
-  for (int tn = 0; tn < 4; ++tn)
+    for (int pair = 0; pair < 2; ++pair)
 #pragma unroll
-    for (int tm = 0; tm < 4; ++tm)
-      store4<TC, ACCUMULATE>(C, ldc, m0 + wm * 64 + tm * 16 + lr, n0 + wn * 64 + tn * 16 + lg * 4, M, N, acc[tn][tm],
-                             bias, vector_ok != 0);
+      for (int tm = 0; tm < 4; ++tm)
+        store_gated((__bf16*)C, ldc, m0 + wm * 64 + tm * 16 + lr, (n0 + wn * 64 + pair * 32) / 2 + lg * 4, M, N / 2,
+                    acc[2 * pair][tm], acc[2 * pair + 1][tm]);
+  } else {
+#pragma unroll
+    for (int tn = 0; tn < 4; ++tn)
+#pragma unroll
+      for (int tm = 0; tm < 4; ++tm)
+        store4<TC, ACCUMULATE>(C, ldc, m0 + wm * 64 + tm * 16 + lr, n0 + wn * 64 + tn * 16 + lg * 4, M, N, acc[tn][tm],
+                               bias, vector_ok != 0);
+  }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -401,7 +431,7 @@ int launch_stationary(const __bf16* A, const __bf16* W, const float* bias, TC* C
 constexpr int MID_CHUNK = 256;
 constexpr int MID_ROW = MID_CHUNK + 8;  // elements per LDS row: 528 bytes, so 16 rows hit 16 different 16-byte slots
 
-template <int CB, int RT, typename TC, bool ACCUMULATE>
+template <int CB, int RT, typename TC, bool ACCUMULATE, bool GATED = false>
 __global__ __launch_bounds__(256) void gemm_mid_kernel(const __bf16* __restrict__ A, const __bf16* __restrict__ W,
                                                        const float* __restrict__ bias, TC* __restrict__ C, int M,
                                                        int N, int K, long long lda, long long ldc, int k_per_range,
@@ -476,11 +506,32 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const __bf16* __restrict_
 #pragma unroll
       for (int i = 0; i < 8; ++i) w_cur[rt][i] = w_next[rt][i];
   }
+  if constexpr (GATED) {
+    if constexpr (RT == 2) {  // a wave's two tiles are the gate and up rows of the same outputs
 #pragma unroll
-  for (int rt = 0; rt < RT; ++rt)
+      for (int cb = 0; cb < CB; ++cb)
+        store_gated((__bf16*)C, ldc, cb * 16 + lr, n0 / 2 + lg * 4, M, N / 2, acc[0][cb], acc[1][cb]);
+    } else {  // waves 0 and 2 hold gate rows, waves 1 and 3 the up rows of the same outputs: hand them over in LDS
+      f32x4* swap = (f32x4*)lds;  // the loop's last barrier has passed: the activation buffers are free
+      if (wave & 1) {
 #pragma unroll
-    for (int cb = 0; cb < CB; ++cb)
-      store4<TC, ACCUMULATE>(C, ldc, cb * 16 + lr, n0 + rt * 16 + lg * 4, M, N, acc[rt][cb], bias, vector_ok != 0);
+        for (int cb = 0; cb < CB; ++cb) swap[((wave >> 1) * CB + cb) * 64 + lane] = acc[0][cb];
+      }
+      __syncthreads();
+      if (!(wave & 1)) {
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb)
+          store_gated((__bf16*)C, ldc, cb * 16 + lr, n0 / 2 + lg * 4, M, N / 2, acc[0][cb],
+                      swap[((wave >> 1) * CB + cb) * 64 + lane]);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int cb = 0; cb < CB; ++cb)
+        store4<TC, ACCUMULATE>(C, ldc, cb * 16 + lr, n0 + rt * 16 + lg * 4, M, N, acc[rt][cb], bias, vector_ok != 0);
+  }
 }
 
 // C (+)= sum over ranges of partial[range] (+ bias): ranges in ascending order, four columns per thread.
@@ -557,12 +608,12 @@ int launch_mid(const __bf16* A, const __bf16* W, const float* bias, TC* C, float
   return VK_UNSUPPORTED_SIZE;
 }
 
-template <typename TC, bool ACC>
+template <typename TC, bool ACC, bool GATED = false>
 int launch_tile(const __bf16* A, const __bf16* W, const float* bias, TC* C, int M, int N, int K, long long lda,
                 long long ldc, int vector_ok, hipStream_t s) {
   static bool configured = false;
   constexpr int lds_bytes = 4 * TILE_ELEMS * (int)sizeof(__bf16);
-  auto kernel = gemm_tile_kernel<TC, ACC>;
+  auto kernel = gemm_tile_kernel<TC, ACC, GATED>;
   if (!configured) {
     hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
     if (e != hipSuccess) return (int)e;
@@ -661,4 +712,41 @@ extern "C" int vk_gemm_bf16_mid(const void* A, const void* W, const float* bias,
   if (c_dtype == DT_BF16)
     return launch_mid<__bf16, false>(a, w, bias, (__bf16*)C, partial, partial_floats, ranges, rows_per_wave, M, N, K, lda, ldc, vector_ok, s);
   return VK_BAD_ARGUMENT;
+}
+
+// out[M, N / 2] = up * silu(gate) of the product with a fused gate/up weight W[N, K] whose rows are
+// interleaved in groups of 16 (see store_gated). bfloat16 in and out; N a multiple of 32.
+// More than 64 tokens: the tiled kernel; up to 64: the LDS-shared kernel with one K range.
+extern "C" int vk_gemm_bf16_gated(const void* A, const void* W, void* C, int M, int N, int K, long long lda,
+                                  long long ldc, int rows_per_wave, void* stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (K <= 0 || (K & 7) || (lda & 7) || lda < K || (N & 31) || ldc < N / 2) return VK_BAD_ARGUMENT;
+  if (((uintptr_t)A & 15) || ((uintptr_t)W & 15)) return VK_BAD_ARGUMENT;
+  hipStream_t s = (hipStream_t)stream;
+  const __bf16* a = (const __bf16*)A;
+  const __bf16* w = (const __bf16*)W;
+  __bf16* c = (__bf16*)C;
+  if (M > 64) return launch_tile<__bf16, false, true>(a, w, nullptr, c, M, N, K, lda, ldc, 0, s);
+  const int cb = (M + 15) / 16;
+#define VK_GATED(CBV, RTV)                                                                                         \
+  {                                                                                                                \
+    constexpr int lds_bytes = 2 * CBV * 16 * MID_ROW * (int)sizeof(__bf16);                                       \
+    auto kernel = gemm_mid_kernel<CBV, RTV, __bf16, false, true>;                                                  \
+    static bool configured = false;                                                                                \
+    if (!configured) {                                                                                             \
+      hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes); \
+      if (e != hipSuccess) return (int)e;                                                                          \
+      configured = true;                                                                                           \
+    }                                                                                                              \
+    kernel<<<dim3((N + 64 * RTV - 1) / (64 * RTV), 1), 256, lds_bytes, s>>>(a, w, nullptr, c, M, N, K, lda, ldc, K, 0, 0); \
+    VK_LAUNCH_CHECK();                                                                                             \
+    return 0;                                                                                                      \
+  }
+  if (rows_per_wave == 2) {
+    switch (cb) { case 1: VK_GATED(1, 2) case 2: VK_GATED(2, 2) case 3: VK_GATED(3, 2) case 4: VK_GATED(4, 2) }
+  } else {
+    switch (cb) { case 1: VK_GATED(1, 1) case 2: VK_GATED(2, 1) case 3: VK_GATED(3, 1) case 4: VK_GATED(4, 1) }
+  }
+#undef VK_GATED
+  return VK_UNSUPPORTED_SIZE;
 }

@@ -140,14 +140,16 @@ def rope_kvwrite(qkv: torch.Tensor, positions: torch.Tensor, inv_freq: Optional[
                head_dim, _stream()), "rope_kvwrite")
 
 
-def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:
-    """``out = up * silu(gate)`` with ``gate_up = [gate | up]`` along the last axis."""
+def swiglu(gate_up: torch.Tensor, out: torch.Tensor, interleaved: bool = False) -> None:
+    """``out = up * silu(gate)``; a row of ``gate_up`` is ``[gate | up]``, or with ``interleaved`` groups of
+    16 gate columns followed by the 16 up columns of the same outputs."""
     _dev(gate_up, out)
     num_tokens, inter = out.shape
     _need(gate_up.shape == (num_tokens, 2 * inter) and gate_up.dtype == out.dtype and gate_up.is_contiguous()
           and out.is_contiguous(), "swiglu: gate_up must be [tokens, 2 * intermediate] of out's dtype")
-    fn = _fn("elementwise", "vk_swiglu", [_p, _p, _i, _i, _i, _p])
-    _status(fn(_ptr(gate_up), _ptr(out), _dt(out, "out"), num_tokens, inter, _stream()), "swiglu")
+    _need(not interleaved or inter % 16 == 0, "swiglu: the interleaved layout needs a multiple of 16 outputs")
+    fn = _fn("elementwise", "vk_swiglu", [_p, _p, _i, _i, _i, _i, _p])
+    _status(fn(_ptr(gate_up), _ptr(out), _dt(out, "out"), num_tokens, inter, 1 if interleaved else 0, _stream()), "swiglu")
 
 
 def fill_normal(out: torch.Tensor, key: int, std: float, offset: float = 0.0) -> None:
@@ -423,3 +425,18 @@ def gemm_bf16_mid(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor]
     _status(fn(_ptr(a), _ptr(w), _ptr(bias), _ptr(out), _dt(out, "out"), m, n, k, lda, ldc, 1 if accumulate else 0,
                int(ranges), int(rows_per_wave), _ptr(partial), partial.numel() if partial is not None else 0, _stream()),
             "gemm_bf16_mid")
+
+
+def gemm_bf16_gated(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, rows_per_wave: int = 1) -> None:
+    """``out = up * silu(gate)`` where ``[gate, up] = a @ w.T`` and ``w`` interleaves gate and up rows in
+    groups of 16.  ``out``: ``[tokens, w.shape[0] / 2]`` bfloat16."""
+    _dev(a, w, out)
+    m, k = a.shape
+    n = w.shape[0]
+    _need(w.shape[1] == k and out.shape == (m, n // 2) and n % 32 == 0, "gemm_gated: shapes")
+    _need(gemm_bf16_supported(a, w, out) and out.dtype == torch.bfloat16, "gemm_gated: operands must be bfloat16")
+    lda = a.stride(0) if m > 1 else max(a.stride(0), k)
+    lda = lda if lda % 8 == 0 else k
+    ldc = out.stride(0) if m > 1 else max(out.stride(0), n // 2)
+    fn = _fn("gemm_bf16", "vk_gemm_bf16_gated", [_p, _p, _p, _i, _i, _i, _ll, _ll, _i, _p])
+    _status(fn(_ptr(a), _ptr(w), _ptr(out), m, n, k, lda, ldc, int(rows_per_wave), _stream()), "gemm_bf16_gated")

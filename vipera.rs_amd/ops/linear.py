@@ -46,3 +46,27 @@ def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: 
     else:
         kernels.gemm_generic(a, w, bias, out, accumulate)
     return out
+
+
+def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """The fused weight of a gated feed-forward with rows interleaved in groups of 16: rows ``[32 p, 32 p + 16)``
+    are gate rows ``[16 p, 16 p + 16)``, rows ``[32 p + 16, 32 p + 32)`` the up rows of the same outputs."""
+    inter, width = gate.shape
+    fused = torch.stack([gate.view(inter // 16, 16, width), up.view(inter // 16, 16, width)], dim=1)
+    return fused.reshape(2 * inter, width).contiguous()
+
+
+def linear_gated(a: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor, interleaved: bool) -> torch.Tensor:
+    """``out = up(a) * silu(gate(a))`` with the fused weight ``w_gate_up`` (``interleaved`` or ``[gate; up]``)."""
+    m, k = a.shape
+    n = w_gate_up.shape[0]
+    fusable = (interleaved and a.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16
+               and out.dtype == torch.bfloat16 and kernels.gemm_bf16_supported(a, w_gate_up, out))
+    if fusable and (m > 64 or (4 < m <= 16 and n >= 16_384)):
+        # the epilogue of the tiled kernel, or of the LDS-shared kernel with one K range, applies the gate
+        kernels.gemm_bf16_gated(a, w_gate_up, out, rows_per_wave=1)
+        return out
+    gate_up = torch.empty((m, n), dtype=out.dtype, device=out.device)
+    linear(a, w_gate_up, None, gate_up)
+    kernels.swiglu(gate_up, out, interleaved)
+    return out

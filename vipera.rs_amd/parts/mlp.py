@@ -1,7 +1,8 @@
 """Gated feed-forward (SwiGLU): ``x += (up(h) * silu(gate(h))) Wd^T``.
 
 Reference: crates/vipera-backend-cpu/src/model.rs:672-680, 1159-1198; ``silu(z) = z / (1 + exp(-z))``
-(model.rs:4368-4370).  Gate and up run as one product over ``[Wg; Wu]``.
+(model.rs:4368-4370).  Gate and up run as one product over a fused weight; with bfloat16 weights its
+rows are interleaved in groups of 16 so that the product's epilogue can apply the gate.
 """
 from __future__ import annotations
 
@@ -12,7 +13,7 @@ import torch
 from ..config.base import PartSpec
 from ..errors import UnsupportedError
 from ..ops import kernels
-from ..ops.linear import linear
+from ..ops.linear import interleave_gate_up, linear, linear_gated
 from ..weights.checkpoint import MATRIX, TensorSpec
 from .attention import _cat
 from .base import FeedForward, register_ffn
@@ -26,6 +27,7 @@ class GatedMLP(FeedForward):
         if spec.params.get("activation", "silu") != "silu":
             raise UnsupportedError(f"activation {spec.params.get('activation')!r} is not implemented; only \"silu\"")
         self.w_gate_up = self.w_down = None
+        self.interleaved = False
 
     @classmethod
     def declare(cls, spec: PartSpec, prefix: str) -> List[TensorSpec]:
@@ -39,15 +41,17 @@ class GatedMLP(FeedForward):
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         base = f"{self.prefix}{self.spec.params['name']}."
-        self.w_gate_up = _cat([tensors[base + "gate_proj.weight"], tensors[base + "up_proj.weight"]])
+        gate, up = tensors[base + "gate_proj.weight"], tensors[base + "up_proj.weight"]
+        # all-bfloat16 weights of a width the kernels can pair are interleaved, so that the product's
+        # epilogue can apply the gate; anything else stays [gate; up]
+        self.interleaved = (gate.dtype == torch.bfloat16 and up.dtype == torch.bfloat16 and self.inter % 16 == 0)
+        self.w_gate_up = interleave_gate_up(gate, up) if self.interleaved else _cat([gate, up])
         self.w_down = tensors[base + "down_proj.weight"]
 
     def forward(self, h, batch, residual) -> None:
         tokens = h.shape[0]
-        gate_up = self.runtime.empty((tokens, 2 * self.inter))
-        linear(h, self.w_gate_up, None, gate_up)
         act = self.runtime.empty((tokens, self.inter))
-        kernels.swiglu(gate_up, act)
+        linear_gated(h, self.w_gate_up, act, self.interleaved)
         linear(act, self.w_down, None, residual, accumulate=True)
 
 
