@@ -181,7 +181,8 @@ def test_attention_kernels_against_plain_softmax(case, dtype):
     assert _rel(out.cpu(), want) < tol, "32-bit-arithmetic kernel"
 
     if dtype == torch.bfloat16:
-        tiles = [x for e, n in enumerate(counts) if n > 1 for off in range(0, n, 64) for x in (e, off)]
+        from vipera_rs_amd.engine.batch import TILE_TOKENS
+        tiles = [x for e, n in enumerate(counts) if n > 1 for off in range(0, n, TILE_TOKENS) for x in (e, off)]
         singles = [e for e, n in enumerate(counts) if n == 1]
         out2 = torch.zeros(T, heads * hd, dtype=dtype, device=DEV)
         es, fp = dev(torch.tensor(starts, dtype=torch.int32)), dev(torch.tensor(first, dtype=torch.int32))

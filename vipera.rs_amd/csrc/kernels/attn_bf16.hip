@@ -7,9 +7,10 @@
 // form splits the positions into chunks whose partial (max, sum, weighted sum) are merged afterwards,
 // as the reference's split kernels do (crates/vipera-backend-gpu/src/layer.cu:307-467).
 //
-// One wave works on a block of 16 columns and a range of positions. A column is a (token, query
-// head) pair: 16 consecutive tokens of one head (prompts), or up to 16 query heads of one key head at
-// one token (decoding; they share every K and V read). Nothing goes through LDS: the operand layout
+// A wave works on blocks of 16 columns and a range of positions. A column is a (token, query head)
+// pair: 16 consecutive tokens of one head (prompts), or up to 16 query heads of one key head at one
+// token (decoding; they share every K and V read). The decode kernel reads the cache straight into
+// the instruction's operands; the prompt kernel shares K/V tiles among its waves through LDS. The operand layout
 // of v_mfma_f32_16x16x32_bf16 (a lane holds 8 consecutive k of one row) is how K lies in the cache,
 // [page, kv_head, slot, head_dim], and V is cached transposed, [page, kv_head, head_dim, slot], so
 // that a lane reads consecutive positions of one output dim.
@@ -170,41 +171,188 @@ __device__ __forceinline__ void load_q(const __bf16* qrow, int hd, bf16x8 (&qf)[
 }
 
 // ---------------------------------------------------------------------------------------------
-// Prompts: grid (tiles, heads), four waves; tile = 64 consecutive tokens of one entry, 16 per wave.
-__global__ __launch_bounds__(256) void attn_prefill_kernel(
+// Prompts: grid (tiles, heads), eight waves. A tile is 128 consecutive tokens of one entry; a wave owns
+// 16 of them (one block of columns). The positions are walked in tiles of 64 whose K rows and V^T rows
+// are fetched once per workgroup into LDS and read from there by all eight waves: while a tile is being
+// multiplied the next one's loads are in flight in registers, and the page ids of the tile after that
+// are already being looked up. Two workgroups fit a CU, so one's barriers and loads hide behind the
+// other's arithmetic. LDS rows are padded by 16 bytes so that the 16 rows of an operand read fall into
+// different banks. Tiles are taken last-first: the long ones (late tokens see many positions) start first.
+constexpr int PT_WAVES = 8;
+constexpr int PT_THREADS = PT_WAVES * 64;
+constexpr int PT_TOKENS = PT_WAVES * 16;   // tokens of a tile
+constexpr int PT_KV = 64;                  // positions of a K/V tile
+constexpr int PT_KROW = HDP + 8;           // elements of a K row in LDS
+constexpr int PT_VROW = PT_KV + 8;         // elements of a V^T row in LDS
+constexpr int PT_PIECES = PT_KV * HDP / 8; // 16-byte pieces of a K tile, and of a V^T tile
+constexpr int PT_PER_THREAD = (PT_PIECES + PT_THREADS - 1) / PT_THREADS;
+
+__global__ __launch_bounds__(PT_THREADS) void attn_prefill_kernel(
     const __bf16* __restrict__ q, long long q_stride, const __bf16* __restrict__ k_cache,
     const __bf16* __restrict__ v_cache, __bf16* __restrict__ out, const int* __restrict__ tiles,
     const int* __restrict__ entry_start, const int* __restrict__ entry_first_pos,
     const int* __restrict__ block_table, int table_width, int block_size, int heads, int kv_heads, int hd,
     float scale, int window) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, lr = lane & 15, lg = lane >> 4;
-  const int entry = tiles[2 * blockIdx.x], q_off = tiles[2 * blockIdx.x + 1] + wave * 16;
-  const int h = blockIdx.y;
+  extern __shared__ __attribute__((aligned(16))) __bf16 lds[];
+  __bf16* sK = lds;                     // [PT_KV][PT_KROW]
+  __bf16* sV = lds + PT_KV * PT_KROW;   // [HDP][PT_VROW]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, lr = lane & 15, lg = lane >> 4;
+  const int tile = gridDim.x - 1 - blockIdx.x;
+  const int entry = tiles[2 * tile], tile_off = tiles[2 * tile + 1];
+  const int h = blockIdx.y, kvh = h / (heads / kv_heads);
   const int tok0 = entry_start[entry], count = entry_start[entry + 1] - tok0;
-  if (q_off >= count) return;
   const int first_pos = entry_first_pos[entry];
-  const int cols = min(16, count - q_off);
-  const bool col_ok = lr < cols;
-  const int col_pos = col_ok ? first_pos + q_off + lr : -1;
+  const int* table = block_table + (size_t)entry * table_width;
+  const int bs = block_size;
+
+  // the workgroup's range of positions
+  const int tile_cols = min(PT_TOKENS, count - tile_off);
+  const int tile_first_pos = first_pos + tile_off;
+  const int begin = (window > 0 && tile_first_pos + 1 > window) ? tile_first_pos + 1 - window : 0;
+  const int end = tile_first_pos + tile_cols;  // one past the last column's position
+
+  // this wave's columns
+  const int q_off = tile_off + wave * 16;
+  const int c = q_off + lr;
+  const bool col_ok = c < count;
+  const int col_pos = col_ok ? first_pos + c : -1;
   const int col_lo = (window > 0 && col_pos + 1 > window) ? col_pos + 1 - window : 0;
-  const int token = tok0 + q_off + lr;
   bf16x8 qf[KS];
-  load_q(col_ok ? q + (size_t)token * q_stride + (size_t)h * hd : nullptr, hd, qf);
-  CacheView cv{k_cache, v_cache, block_table + (size_t)entry * table_width, table_width, block_size,
-               kv_heads, hd, h / (heads / kv_heads)};
+  load_q(col_ok ? q + (size_t)(tok0 + c) * q_stride + (size_t)h * hd : nullptr, hd, qf);
+  const int wave_cols = max(0, min(16, count - q_off));
+  const int wave_end = wave_cols > 0 ? first_pos + q_off + wave_cols : 0;  // nothing at or past it is visible
+  const int wave_first = first_pos + q_off;
+  const int wave_begin = (window > 0 && wave_first + 1 > window) ? wave_first + 1 - window : 0;
+
   f32x4 o[DT];
+  float m = -INFINITY, l = 0.f;
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
-  float m = -INFINITY, l = 0.f;
-  const int first_col_pos = first_pos + q_off;
-  const int begin = (window > 0 && first_col_pos + 1 > window) ? first_col_pos + 1 - window : 0;
-  const int end = first_pos + q_off + cols;  // one past the last column's position
-  attend_range<false>(qf, col_lo, col_pos, begin, end, cv, scale, o, m, l);
+
+  // per thread: PT_PER_THREAD pieces of the K tile (row r, 8 dims) and of the V^T tile (dim d, 8 positions)
+  bf16x8 k_stage[PT_PER_THREAD], v_stage[PT_PER_THREAD];
+  int k_page[PT_PER_THREAD], v_page[PT_PER_THREAD];
+  auto lookup = [&](int p0) {  // page ids of the tile at p0 (-1: nothing to read)
+#pragma unroll
+    for (int i = 0; i < PT_PER_THREAD; ++i) {
+      const int id = tid + PT_THREADS * i;
+      const int pk = p0 + id / (HDP / 8);
+      k_page[i] = (id < PT_PIECES && pk >= begin && pk < end) ? table[pk / bs] : -1;
+      const int pv = p0 + (id % (PT_KV / 8)) * 8;  // eight positions of one page (8 divides the page size)
+      v_page[i] = (id < PT_PIECES && pv + 7 >= begin && pv < end) ? table[pv / bs] : -1;
+    }
+  };
+  auto fetch = [&](int p0) {
+#pragma unroll
+    for (int i = 0; i < PT_PER_THREAD; ++i) {
+      const int id = tid + PT_THREADS * i;
+      const int r = id / (HDP / 8), ck = id % (HDP / 8);
+      const int pk = p0 + r;
+      k_stage[i] = (k_page[i] >= 0 && ck * 8 < hd)
+                       ? *(const bf16x8*)(k_cache + (((size_t)k_page[i] * kv_heads + kvh) * bs + (pk % bs)) * hd + ck * 8)
+                       : zero8();
+      const int d = id / (PT_KV / 8), cv = id % (PT_KV / 8);
+      const int pv = p0 + cv * 8;
+      v_stage[i] = (v_page[i] >= 0 && d < hd)
+                       ? *(const bf16x8*)(v_cache + (((size_t)v_page[i] * kv_heads + kvh) * hd + d) * bs + (pv % bs))
+                       : zero8();
+    }
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int i = 0; i < PT_PER_THREAD; ++i) {
+      const int id = tid + PT_THREADS * i;
+      if (id < PT_PIECES) {
+        *(bf16x8*)(sK + (id / (HDP / 8)) * PT_KROW + (id % (HDP / 8)) * 8) = k_stage[i];
+        *(bf16x8*)(sV + (id / (PT_KV / 8)) * PT_VROW + (id % (PT_KV / 8)) * 8) = v_stage[i];
+      }
+    }
+  };
+
+  const int first_tile = begin & ~(PT_KV - 1);
+  lookup(first_tile);
+  fetch(first_tile);
+  lookup(first_tile + PT_KV);
+  stash();
+  __syncthreads();
+  for (int p0 = first_tile; p0 < end; p0 += PT_KV) {
+    const bool more = p0 + PT_KV < end;
+    if (more) {
+      fetch(p0 + PT_KV);        // with the page ids looked up one tile ago
+      lookup(p0 + 2 * PT_KV);
+    }
+    if (p0 < wave_end && p0 + PT_KV > wave_begin) {  // some of this tile is visible to this wave
+      // ---- scores of four 16-position tiles
+      f32x4 s[4];
+#pragma unroll
+      for (int sub = 0; sub < 4; ++sub) {
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          const bf16x8 kf = *(const bf16x8*)(sK + (sub * 16 + lr) * PT_KROW + ks * 32 + lg * 8);
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[ks], acc, 0, 0, 0);
+        }
+        s[sub] = acc;
+      }
+      // ---- mask, running max, weights
+      float sv[16];
+      float tile_max = -INFINITY;
+#pragma unroll
+      for (int sub = 0; sub < 4; ++sub)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int p = p0 + sub * 16 + lg * 4 + j;
+          const bool visible = p >= col_lo && p <= col_pos;
+          const float x = visible ? s[sub][j] * scale : -INFINITY;
+          sv[sub * 4 + j] = x;
+          tile_max = fmaxf(tile_max, x);
+        }
+      tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, 64));
+      tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
+      const float m_new = fmaxf(m, tile_max);
+      float alpha = 1.f;
+      bf16x8 pf[2] = {zero8(), zero8()};
+      if (m_new > -INFINITY) {
+        alpha = __expf(m - m_new);
+        float sum = 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const float w = __expf(sv[i] - m_new);
+          sum += w;
+          pf[i >> 3][i & 7] = (__bf16)w;   // step 0: tiles 0 and 1; step 1: tiles 2 and 3
+        }
+        l = l * alpha + sum;
+        m = m_new;
+      }
+      // ---- output: V^T operands from LDS
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        o[dt] *= alpha;
+#pragma unroll
+        for (int step = 0; step < 2; ++step) {
+          const __bf16* vrow = sV + (dt * 16 + lr) * PT_VROW + step * 32 + lg * 4;
+          const bf16x4 v0 = *(const bf16x4*)vrow, v1 = *(const bf16x4*)(vrow + 16);
+          bf16x8 vf;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            vf[i] = v0[i];
+            vf[4 + i] = v1[i];
+          }
+          o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[step], o[dt], 0, 0, 0);
+        }
+      }
+    }
+    __syncthreads();  // everyone is done with this tile
+    if (more) {
+      stash();
+      __syncthreads();
+    }
+  }
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
   if (!col_ok) return;
   const float inv = 1.f / l;
-  __bf16* dst = out + (size_t)token * heads * hd + (size_t)h * hd;
+  __bf16* dst = out + (size_t)(tok0 + c) * heads * hd + (size_t)h * hd;
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) {
     const int d = dt * 16 + lg * 4;
@@ -342,7 +490,7 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(const float* __restric
 
 extern "C" int vk_attn_bf16_hdp() { return HDP; }
 
-// tiles: pairs (entry, first token of the tile within the entry), 64 tokens per tile.
+// tiles: pairs (entry, first token of the tile within the entry), 128 tokens per tile.
 extern "C" int vk_attn_bf16_prefill(const void* q, long long q_stride, const void* k_cache, const void* v_cache,
                                     void* out, const int* tiles, int num_tiles, const int* entry_start,
                                     const int* entry_first_pos, const int* block_table, int table_width,
@@ -352,8 +500,16 @@ extern "C" int vk_attn_bf16_prefill(const void* q, long long q_stride, const voi
   if (hd <= 0 || hd > HDP || (hd & 7) || block_size <= 0 || (block_size & 7) || heads <= 0 || kv_heads <= 0 ||
       heads % kv_heads || heads > 65535 || (q_stride & 7) || window < 0)
     return VK_UNSUPPORTED_SIZE;
+  constexpr int lds_bytes = (PT_KV * PT_KROW + HDP * PT_VROW) * (int)sizeof(__bf16);
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute((const void*)attn_prefill_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       lds_bytes);
+    if (e != hipSuccess) return (int)e;
+    configured = true;
+  }
   dim3 grid(num_tiles, heads);
-  attn_prefill_kernel<<<grid, 256, 0, (hipStream_t)stream>>>(
+  attn_prefill_kernel<<<grid, PT_THREADS, lds_bytes, (hipStream_t)stream>>>(
       (const __bf16*)q, q_stride, (const __bf16*)k_cache, (const __bf16*)v_cache, (__bf16*)out, tiles, entry_start,
       entry_first_pos, block_table, table_width, block_size, heads, kv_heads, hd, scale, window);
   VK_LAUNCH_CHECK();

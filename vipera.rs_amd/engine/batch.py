@@ -20,7 +20,7 @@ import torch
 
 from ..errors import InternalError, InvalidArgumentError
 
-TILE_TOKENS = 64  # tokens of one prompt tile of the matrix-core attention kernel
+TILE_TOKENS = 128  # tokens of one prompt tile of the matrix-core attention kernel
 
 
 @dataclass
@@ -47,7 +47,7 @@ class StepBatch:
     entry_kv_len: torch.Tensor     # [E] int32, tokens in the cache after this step
     slots: torch.Tensor            # [E] int32, state slot of each entry's request
     logit_rows: torch.Tensor       # [R] int32, flat token indices
-    prefill_tiles: torch.Tensor    # [tiles, 2] int32: (entry, first token within it) per 64 tokens of multi-token entries
+    prefill_tiles: torch.Tensor    # [tiles, 2] int32: (entry, first token within it) per 128 tokens of multi-token entries
     decode_entries: torch.Tensor   # [n] int32: entries that hold exactly one token
     block_tables: Dict[int, torch.Tensor]  # group -> [E, width] int32
     # host copies, for launch decisions

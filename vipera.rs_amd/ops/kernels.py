@@ -309,7 +309,7 @@ def attn_bf16_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
                       tiles: torch.Tensor, entry_start: torch.Tensor, entry_first_pos: torch.Tensor,
                       block_table: torch.Tensor, heads: int, kv_heads: int, head_dim: int, scale: float,
                       window: int) -> None:
-    """Attention of the entries' 64-token tiles listed in ``tiles`` (pairs: entry, first token within it)."""
+    """Attention of the entries' 128-token tiles listed in ``tiles`` (pairs: entry, first token within it)."""
     _dev(q, k_cache, v_cache, out, tiles, entry_start, entry_first_pos, block_table)
     _need(attn_bf16_supported(q, k_cache, head_dim), "attn_bf16: operands must be bfloat16 with 16-byte rows")
     _need(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= heads * head_dim, "attention: q")
