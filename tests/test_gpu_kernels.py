@@ -16,7 +16,8 @@ def _rel(got, want):
 
 # --- matrix products -----------------------------------------------------------------------------
 GEMM_SHAPES = [(1, 48, 64), (7, 300, 96), (8, 3584, 512), (16, 200, 128), (17, 331, 80), (33, 1000, 264),
-               (64, 520, 1024), (65, 130, 72), (128, 128, 64), (200, 257, 136), (515, 384, 200)]
+               (64, 520, 1024), (65, 130, 72), (128, 128, 64), (100, 9000, 72), (200, 257, 136), (515, 384, 200),
+               (2050, 4100, 136)]   # the last ones take each tiling of the tiled kernel
 
 
 @pytest.mark.parametrize("m,n,k", GEMM_SHAPES)
@@ -285,7 +286,7 @@ def test_gemm_mid_against_float64(m, n, k, ranges, rows_per_wave):
 
 
 @pytest.mark.parametrize("m,inter,k", [(1, 32, 64), (5, 48, 96), (8, 18944, 512), (16, 176, 200), (33, 128, 264), (64, 1024, 256),
-                                       (65, 64, 72), (300, 208, 136), (2048, 512, 128)])
+                                       (65, 64, 72), (300, 208, 136), (2048, 512, 128), (2048, 8208, 72), (100, 4608, 64)])
 def test_gated_product_and_interleaved_swiglu(m, inter, k):
     from vipera_rs_amd.ops import kernels
     from vipera_rs_amd.ops.linear import interleave_gate_up, linear_gated

@@ -89,19 +89,25 @@ __device__ __forceinline__ void store_gated(__bf16* __restrict__ C, long long ld
 }
 
 // ---------------------------------------------------------------------------------------------
-constexpr int BM = 128, BN = 128, BK = 64;
+constexpr int BK = 64;
 constexpr int ROW = BK + 8;  // elements per LDS row: 144 bytes
-constexpr int TILE_ELEMS = BM * ROW;
 constexpr int XCDS = 8;
 
-template <typename TC, bool ACCUMULATE, bool GATED>
-__global__ __launch_bounds__(256) void gemm_tile_kernel(const __bf16* __restrict__ A, const __bf16* __restrict__ W,
-                                                        const float* __restrict__ bias, TC* __restrict__ C, int M,
-                                                        int N, int K, long long lda, long long ldc, int tiles_m,
-                                                        int tiles_n, int vector_ok) {
+// BM x BN: output tile of a workgroup (tokens x weight rows); WM x WN: its grid of waves. A wave owns
+// (BM / WM) x (BN / WN) outputs as TM x TN instruction tiles.
+template <int BM, int BN, int WM, int WN, typename TC, bool ACCUMULATE, bool GATED>
+__global__ __launch_bounds__(WM * WN * 64) void gemm_tile_kernel(const __bf16* __restrict__ A,
+                                                                   const __bf16* __restrict__ W,
+                                                                   const float* __restrict__ bias, TC* __restrict__ C,
+                                                                   int M, int N, int K, long long lda, long long ldc,
+                                                                   int tiles_m, int tiles_n, int vector_ok) {
+  constexpr int THREADS = WM * WN * 64;
+  constexpr int TM = BM / WM / 16, TN = BN / WN / 16;
+  constexpr int A_PIECES = BM * 8 / THREADS, W_PIECES = BN * 8 / THREADS;  // 16-byte pieces per thread and step
+  static_assert(BM * 8 % THREADS == 0 && BN * 8 % THREADS == 0, "tile rows must divide among the threads");
   extern __shared__ __attribute__((aligned(16))) __bf16 lds[];
-  __bf16* sA = lds;                   // [2][BM][ROW]
-  __bf16* sW = lds + 2 * TILE_ELEMS;  // [2][BN][ROW]
+  __bf16* sA = lds;                  // [2][BM][ROW]
+  __bf16* sW = lds + 2 * BM * ROW;   // [2][BN][ROW]
 
   // workgroups are dealt to the XCDs round-robin; give each XCD a contiguous run of tiles
   const int total = tiles_m * tiles_n;
@@ -113,35 +119,38 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(const __bf16* __restrict
   const int m0 = tile_m * BM, n0 = tile_n * BN;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / WN, wn = wave % WN;
   const int lr = lane & 15, lg = lane >> 4;
 
-  f32x4 acc[4][4];  // [n tile][m tile]
+  f32x4 acc[TN][TM];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < TN; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < TM; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  // staging: 1024 chunks of 16 bytes per operand tile, four per thread
-  bf16x8 ra[4], rw[4];
+  bf16x8 ra[A_PIECES], rw[W_PIECES];
   auto load_global = [&](int k0) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int id = tid + 256 * i;
-      const int row = id >> 3, c = id & 7;
-      const int k = k0 + c * 8;
-      const int am = m0 + row, wn_ = n0 + row;
-      ra[i] = (am < M && k < K) ? *(const bf16x8*)(A + (size_t)am * lda + k) : zero8();
-      rw[i] = (wn_ < N && k < K) ? *(const bf16x8*)(W + (size_t)wn_ * K + k) : zero8();
+    for (int i = 0; i < A_PIECES; ++i) {
+      const int id = tid + THREADS * i, row = id >> 3, k = k0 + (id & 7) * 8;
+      ra[i] = (m0 + row < M && k < K) ? *(const bf16x8*)(A + (size_t)(m0 + row) * lda + k) : zero8();
+    }
+#pragma unroll
+    for (int i = 0; i < W_PIECES; ++i) {
+      const int id = tid + THREADS * i, row = id >> 3, k = k0 + (id & 7) * 8;
+      rw[i] = (n0 + row < N && k < K) ? *(const bf16x8*)(W + (size_t)(n0 + row) * K + k) : zero8();
     }
   };
   auto store_lds = [&](int buf) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int id = tid + 256 * i;
-      const int row = id >> 3, c = id & 7;
-      *(bf16x8*)(sA + buf * TILE_ELEMS + row * ROW + c * 8) = ra[i];
-      *(bf16x8*)(sW + buf * TILE_ELEMS + row * ROW + c * 8) = rw[i];
+    for (int i = 0; i < A_PIECES; ++i) {
+      const int id = tid + THREADS * i;
+      *(bf16x8*)(sA + buf * BM * ROW + (id >> 3) * ROW + (id & 7) * 8) = ra[i];
+    }
+#pragma unroll
+    for (int i = 0; i < W_PIECES; ++i) {
+      const int id = tid + THREADS * i;
+      *(bf16x8*)(sW + buf * BN * ROW + (id >> 3) * ROW + (id & 7) * 8) = rw[i];
     }
   };
 
@@ -152,41 +161,42 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(const __bf16* __restrict
   for (int s = 0; s < steps; ++s) {
     const int buf = s & 1;
     if (s + 1 < steps) load_global((s + 1) * BK);
-    const __bf16* tA = sA + buf * TILE_ELEMS + (wm * 64 + lr) * ROW + lg * 8;
-    const __bf16* tW = sW + buf * TILE_ELEMS + (wn * 64 + lr) * ROW + lg * 8;
+    const __bf16* tA = sA + buf * BM * ROW + (wm * TM * 16 + lr) * ROW + lg * 8;
+    const __bf16* tW = sW + buf * BN * ROW + (wn * TN * 16 + lr) * ROW + lg * 8;
 #pragma unroll
     for (int ks = 0; ks < BK / 32; ++ks) {
-      bf16x8 fa[4], fw[4];
+      bf16x8 fa[TM], fw[TN];
 #pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        fa[t] = *(const bf16x8*)(tA + t * 16 * ROW + ks * 32);
-        fw[t] = *(const bf16x8*)(tW + t * 16 * ROW + ks * 32);
-      }
+      for (int t = 0; t < TM; ++t) fa[t] = *(const bf16x8*)(tA + t * 16 * ROW + ks * 32);
 #pragma unroll
-      for (int tn = 0; tn < 4; ++tn)
+      for (int t = 0; t < TN; ++t) fw[t] = *(const bf16x8*)(tW + t * 16 * ROW + ks * 32);
 #pragma unroll
-        for (int tm = 0; tm < 4; ++tm)
+      for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm)
           acc[tn][tm] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[tn], fa[tm], acc[tn][tm], 0, 0, 0);
     }
     if (s + 1 < steps) store_lds(buf ^ 1);
     __syncthreads();
   }
 
+  const int wave_m = m0 + wm * TM * 16, wave_n = n0 + wn * TN * 16;
   if constexpr (GATED) {
-    // N counts fused rows; the output has N / 2 columns
+    // N counts fused rows (pairs of 16-row tiles: gate, up); the output has N / 2 columns
+    static_assert(!GATED || TN % 2 == 0, "a wave must own whole gate/up pairs");
 #pragma unroll
-    for (int pair = 0; pair < 2; ++pair)
+    for (int pair = 0; pair < TN / 2; ++pair)
 #pragma unroll
-      for (int tm = 0; tm < 4; ++tm)
-        store_gated((__bf16*)C, ldc, m0 + wm * 64 + tm * 16 + lr, (n0 + wn * 64 + pair * 32) / 2 + lg * 4, M, N / 2,
+      for (int tm = 0; tm < TM; ++tm)
+        store_gated((__bf16*)C, ldc, wave_m + tm * 16 + lr, (wave_n + pair * 32) / 2 + lg * 4, M, N / 2,
                     acc[2 * pair][tm], acc[2 * pair + 1][tm]);
   } else {
 #pragma unroll
-    for (int tn = 0; tn < 4; ++tn)
+    for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
-      for (int tm = 0; tm < 4; ++tm)
-        store4<TC, ACCUMULATE>(C, ldc, m0 + wm * 64 + tm * 16 + lr, n0 + wn * 64 + tn * 16 + lg * 4, M, N, acc[tn][tm],
-                               bias, vector_ok != 0);
+      for (int tm = 0; tm < TM; ++tm)
+        store4<TC, ACCUMULATE>(C, ldc, wave_m + tm * 16 + lr, wave_n + tn * 16 + lg * 4, M, N, acc[tn][tm], bias,
+                               vector_ok != 0);
   }
 }
 
@@ -608,12 +618,12 @@ int launch_mid(const __bf16* A, const __bf16* W, const float* bias, TC* C, float
   return VK_UNSUPPORTED_SIZE;
 }
 
-template <typename TC, bool ACC, bool GATED = false>
-int launch_tile(const __bf16* A, const __bf16* W, const float* bias, TC* C, int M, int N, int K, long long lda,
-                long long ldc, int vector_ok, hipStream_t s) {
+template <int BM, int BN, int WM, int WN, typename TC, bool ACC, bool GATED>
+int launch_tile_as(const __bf16* A, const __bf16* W, const float* bias, TC* C, int M, int N, int K, long long lda,
+                   long long ldc, int vector_ok, hipStream_t s) {
   static bool configured = false;
-  constexpr int lds_bytes = 4 * TILE_ELEMS * (int)sizeof(__bf16);
-  auto kernel = gemm_tile_kernel<TC, ACC, GATED>;
+  constexpr int lds_bytes = 2 * (BM + BN) * ROW * (int)sizeof(__bf16);
+  auto kernel = gemm_tile_kernel<BM, BN, WM, WN, TC, ACC, GATED>;
   if (!configured) {
     hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
     if (e != hipSuccess) return (int)e;
@@ -623,9 +633,33 @@ int launch_tile(const __bf16* A, const __bf16* W, const float* bias, TC* C, int 
   const long long total = (long long)tiles_m * tiles_n;
   const long long grid = (total + XCDS - 1) / XCDS * XCDS;
   if (grid > 0x7fffffffLL) return VK_UNSUPPORTED_SIZE;
-  kernel<<<(int)grid, 256, lds_bytes, s>>>(A, W, bias, C, M, N, K, lda, ldc, tiles_m, tiles_n, vector_ok);
+  kernel<<<(int)grid, WM * WN * 64, lds_bytes, s>>>(A, W, bias, C, M, N, K, lda, ldc, tiles_m, tiles_n, vector_ok);
   VK_LAUNCH_CHECK();
   return 0;
+}
+
+int g_tile_config = -1;  // -1: chosen by shape; 0..5 force a tiling (vk_gemm_bf16_tile_config, for measurements)
+
+// Measured on the 7B shapes at 2,048 tokens: 256x256 tiles with sixteen waves are fastest when there are
+// enough of them to fill the GPU (about 1 PFLOP/s), 256x128 with eight waves otherwise; few tokens keep
+// the token side of the tile at 128.
+int choose_tile_config(int M, int N) {
+  if (M <= 128) return N >= 8192 ? 3 : 0;
+  const long long big = (long long)((M + 255) / 256) * ((N + 255) / 256);
+  return big >= 128 ? 4 : 2;
+}
+
+template <typename TC, bool ACC, bool GATED = false>
+int launch_tile(const __bf16* A, const __bf16* W, const float* bias, TC* C, int M, int N, int K, long long lda,
+                long long ldc, int vector_ok, hipStream_t s) {
+  switch (g_tile_config >= 0 ? g_tile_config : choose_tile_config(M, N)) {
+    case 1: return launch_tile_as<128, 128, 2, 4, TC, ACC, GATED>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, s);
+    case 2: return launch_tile_as<256, 128, 4, 2, TC, ACC, GATED>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, s);
+    case 3: return launch_tile_as<128, 256, 2, 4, TC, ACC, GATED>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, s);
+    case 4: return launch_tile_as<256, 256, 4, 4, TC, ACC, GATED>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, s);
+    case 5: return launch_tile_as<256, 256, 2, 4, TC, ACC, GATED>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, s);
+    default: return launch_tile_as<128, 128, 2, 2, TC, ACC, GATED>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, s);
+  }
 }
 }  // namespace
 
@@ -749,4 +783,9 @@ extern "C" int vk_gemm_bf16_gated(const void* A, const void* W, void* C, int M, 
   }
 #undef VK_GATED
   return VK_UNSUPPORTED_SIZE;
+}
+
+extern "C" int vk_gemm_bf16_tile_config(int config) {
+  g_tile_config = config;
+  return 0;
 }
