@@ -1,0 +1,82 @@
+"""The layer sizes of Qwen2.5-7B (hidden 3584, 28 heads over 4 key heads of width 128, feed-forward
+18944, rotary base 1e6, q/k/v bias) with one layer and a small vocabulary, so that the plain
+implementation stays affordable: whole prompts, portions and single tokens against it in 32-bit and
+bfloat16, and a vocabulary of 152064 for the output projection and the samplers alone."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import make_folder, random_tokens, rel_err
+from plain import qwen2_plain as P
+
+pytestmark = pytest.mark.gpu
+
+CONFIG_7B_LAYER = {
+    "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2",
+    "num_hidden_layers": 1, "hidden_size": 3584, "num_attention_heads": 28, "num_key_value_heads": 4,
+    "intermediate_size": 18944, "vocab_size": 1000, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6,
+    "tie_word_embeddings": False, "max_position_embeddings": 32768, "hidden_act": "silu",
+    "use_sliding_window": False, "sliding_window": 131072, "max_window_layers": 28,
+}
+
+
+@pytest.fixture(scope="module")
+def real(tmp_path_factory):
+    out = {}
+    tokens = random_tokens(1000, 150, 21)
+    for dtype, tdtype in (("float32", torch.float32), ("bfloat16", torch.bfloat16)):
+        folder = make_folder(tmp_path_factory.mktemp(f"real_{dtype}"), CONFIG_7B_LAYER, 3, tdtype)
+        cfg, w = P.load_folder(folder)
+        out[dtype] = (folder, P.forward(cfg, w, tokens))
+    out["tokens"] = tokens
+    return out
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 1e-4), ("bfloat16", 3e-2)])
+def test_real_layer_sizes_under_every_cut(real, dtype, tol):
+    from vipera_rs_amd.engine.batch import StepEntry
+    from vipera_rs_amd.engine.runner import ModelRunner
+    folder, want = real[dtype]
+    tokens = real["tokens"]
+    runner = ModelRunner.from_folder(folder, dtype=dtype, block_size=16, num_blocks=40, num_slots=4)
+    # whole
+    runner.cache.reserve(0, 0, len(tokens))
+    whole = runner.step([StepEntry(0, 0, tokens, list(range(len(tokens))))]).cpu().numpy()
+    assert rel_err(whole, want) < tol
+    runner.cache.release(0)
+    # portions of changing size, then the last 20 tokens one by one, beside another request's portions
+    other = random_tokens(1000, 90, 22)
+    rows, at, oat = [], 0, 0
+    sizes = [70, 3, 2, 40, 15]
+    for size in sizes + [1] * (len(tokens) - sum(sizes)):
+        entries = []
+        runner.cache.reserve(1, at, at + size)
+        entries.append(StepEntry(1, at, tokens[at:at + size], list(range(size))))
+        if oat < len(other):
+            osize = min(17, len(other) - oat)
+            runner.cache.reserve(2, oat, oat + osize)
+            entries.append(StepEntry(2, oat, other[oat:oat + osize], []))
+            oat += osize
+        rows.append(runner.step(entries).cpu().numpy())
+        at += size
+    assert rel_err(np.concatenate(rows), want) < tol
+    assert runner.cache.check() == ""
+
+
+def test_the_full_vocabulary_head_and_greedy_choice():
+    """152064 columns are no power of two: the output projection and the argmax at that width."""
+    from vipera_rs_amd.ops import kernels
+    from vipera_rs_amd.ops.linear import linear
+    g = torch.Generator().manual_seed(4)
+    h = torch.randn(5, 3584, generator=g).to(torch.bfloat16).to("cuda:0")
+    w = (torch.randn(152064, 3584, generator=g) * 0.02).to(torch.bfloat16).to("cuda:0")
+    logits = torch.empty(5, 152064, dtype=torch.float32, device="cuda:0")
+    linear(h, w, None, logits)
+    want = h.double() @ w.double().T
+    assert float((logits.double() - want).abs().max() / want.abs().max()) < 1e-5
+    rows = logits.shape[0]
+    out = torch.empty(rows, dtype=torch.int32, device="cuda:0")
+    zeros = lambda d: torch.zeros(rows, dtype=d, device="cuda:0")  # noqa: E731
+    kernels.sample(logits, zeros(torch.float32), zeros(torch.int32), torch.ones(rows, device="cuda:0"),
+                   zeros(torch.float32), zeros(torch.float64), out)
+    assert out.cpu().tolist() == want.argmax(dim=1).cpu().tolist()
