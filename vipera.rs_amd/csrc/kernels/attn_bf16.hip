@@ -46,7 +46,18 @@ struct CacheView {
   const __bf16* v;
   const int* table;  // this request's row of the block table
   int table_width, block_size, kv_heads, hd, kvh;
+  int page0, pages;  // REGS: lane i of `pages` holds the id of page page0 + i of the request
 };
+
+// Page id of position p. With REGS the ids of the wave's range were read once, one per lane, and come
+// back through a lane shuffle (every lane calls it), so no step waits for a table read before its
+// K and V reads can be issued.
+template <bool REGS>
+__device__ __forceinline__ int page_of(const CacheView& cv, int p) {
+  const int index = p / cv.block_size;
+  if (REGS) return __shfl(cv.pages, (index - cv.page0) & 63, 64);
+  return (index >= 0 && index < cv.table_width) ? cv.table[index] : -1;
+}
 
 // The K and V^T operands of one step of 32 positions.
 struct StepOperands {
@@ -56,17 +67,17 @@ struct StepOperands {
 
 // Issue the loads of the step that starts at kb. Positions outside [begin, end), pages that are not
 // held and dims past the head width read as zero.
+template <bool REGS>
 __device__ __forceinline__ void load_step(int kb, int begin, int end, const CacheView& cv, StepOperands& r) {
   const int lane = threadIdx.x & 63, lr = lane & 15, lg = lane >> 4;
   const int bs = cv.block_size, hd = cv.hd;
 #pragma unroll
   for (int sub = 0; sub < 2; ++sub) {
     const int p = kb + sub * 16 + lr;
+    const int page = page_of<REGS>(cv, p);
     const __bf16* row = nullptr;
-    if (p >= begin && p < end) {
-      const int page = cv.table[p / bs];
-      if (page >= 0) row = cv.k + (((size_t)page * cv.kv_heads + cv.kvh) * bs + (p % bs)) * hd + lg * 8;
-    }
+    if (p >= begin && p < end && page >= 0)
+      row = cv.k + (((size_t)page * cv.kv_heads + cv.kvh) * bs + (p % bs)) * hd + lg * 8;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks)
       r.kf[sub][ks] = (row && ks * 32 + lg * 8 < hd) ? *(const bf16x8*)(row + ks * 32) : zero8();
@@ -75,10 +86,10 @@ __device__ __forceinline__ void load_step(int kb, int begin, int end, const Cach
 #pragma unroll
   for (int half = 0; half < 2; ++half) {
     const int p = kb + half * 16 + lg * 4;
-    if (p + 3 >= begin && p < end) {  // a group of four positions lies in one page (4 divides the page size)
-      const int page = cv.table[p / bs];
-      if (page >= 0) vrow[half] = cv.v + (((size_t)page * cv.kv_heads + cv.kvh) * hd) * bs + (p % bs);
-    }
+    const int page = page_of<REGS>(cv, p);
+    // a group of four positions lies in one page (4 divides the page size)
+    if (p + 3 >= begin && p < end && page >= 0)
+      vrow[half] = cv.v + (((size_t)page * cv.kv_heads + cv.kvh) * hd) * bs + (p % bs);
   }
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) {
@@ -100,21 +111,18 @@ __device__ __forceinline__ void load_step(int kb, int begin, int end, const Cach
 // Online-softmax attention of 16 columns over positions [begin, end). Per lane: col_lo / col_pos are
 // the visible range [lo, pos] of the lane's column (pos < 0: the column is empty).
 // State: o[DT] (O^T tiles), m (running max of the column), l (this lane's share of the running sum).
-// With AHEAD the loads of a step are issued one step ahead of its arithmetic (twice the operand
-// registers, fewer waves per SIMD: right for decoding, where a wave has few steps and memory is the bound).
-template <bool AHEAD>
+// The loads of a step are issued one step ahead of its arithmetic: a wave has few steps and memory is
+// the bound.
+template <bool REGS>
 __device__ __forceinline__ void attend_range(const bf16x8 (&qf)[KS], int col_lo, int col_pos, int begin, int end,
                                              const CacheView& cv, float scale, f32x4 (&o)[DT], float& m, float& l) {
   const int lane = threadIdx.x & 63, lg = lane >> 4;
   StepOperands cur, next;
   const int first = begin & ~31;
   if (first >= end) return;
-  if (AHEAD) load_step(first, begin, end, cv, cur);
+  load_step<REGS>(first, begin, end, cv, cur);
   for (int kb = first; kb < end; kb += 32) {
-    if (!AHEAD)
-      load_step(kb, begin, end, cv, cur);
-    else if (kb + 32 < end)
-      load_step(kb + 32, begin, end, cv, next);
+    if (kb + 32 < end) load_step<REGS>(kb + 32, begin, end, cv, next);
     // ---- scores of two 16-position tiles
     f32x4 s[2];
 #pragma unroll
@@ -159,7 +167,7 @@ __device__ __forceinline__ void attend_range(const bf16x8 (&qf)[KS], int col_lo,
       o[dt] *= alpha;
       o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.vf[dt], pf, o[dt], 0, 0, 0);
     }
-    if (AHEAD && kb + 32 < end) cur = next;
+    if (kb + 32 < end) cur = next;
   }
 }
 
@@ -368,7 +376,9 @@ __global__ __launch_bounds__(PT_THREADS) void attn_prefill_kernel(
 // ---------------------------------------------------------------------------------------------
 // Decoding: grid (entries, kv_heads * head_blocks, chunks), one wave. Columns are the query heads of
 // one key head. Chunk c covers positions [c * chunk, (c + 1) * chunk) of the visible range and leaves
-// (max, sum, weighted sum) in `partial`: [entry, head, chunk, hd + 2] floats.
+// (max, sum, weighted sum) in `partial`: [entry, head, chunk, hd + 2] floats. REGS: a chunk spans at most
+// 64 pages, whose ids the wave reads once.
+template <bool REGS>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void attn_decode_kernel(
     const __bf16* __restrict__ q, long long q_stride, const __bf16* __restrict__ k_cache,
     const __bf16* __restrict__ v_cache, float* __restrict__ partial, const int* __restrict__ entries,
@@ -397,12 +407,16 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void at
   bf16x8 qf[KS];
   load_q(col_ok ? q + (size_t)token * q_stride + (size_t)h * hd : nullptr, hd, qf);
   CacheView cv{k_cache, v_cache, block_table + (size_t)entry * table_width, table_width, block_size,
-               kv_heads, hd, kvh};
+               kv_heads, hd, kvh, begin / block_size, -1};
+  if (REGS) {
+    const int index = cv.page0 + lane;
+    if (index <= (end - 1) / block_size && index < table_width) cv.pages = cv.table[index];
+  }
   f32x4 o[DT];
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
-  attend_range<true>(qf, lo, col_ok ? pos : -1, begin, end, cv, scale, o, m, l);
+  attend_range<REGS>(qf, lo, col_ok ? pos : -1, begin, end, cv, scale, o, m, l);
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
   if (!col_ok) return;
@@ -533,9 +547,11 @@ extern "C" int vk_attn_bf16_decode(const void* q, long long q_stride, const void
   if (kv_heads * head_blocks > 65535 || heads > 65535) return VK_UNSUPPORTED_SIZE;
   hipStream_t s = (hipStream_t)stream;
   dim3 grid(num_entries, kv_heads * head_blocks, chunks);
-  attn_decode_kernel<<<grid, 64, 0, s>>>((const __bf16*)q, q_stride, (const __bf16*)k_cache, (const __bf16*)v_cache,
-                                         partial, entries, entry_start, entry_first_pos, block_table, table_width,
-                                         block_size, heads, kv_heads, hd, scale, window, chunk, head_blocks);
+  // a chunk that does not start on a page's edge touches one page more than chunk / block_size
+  auto kernel = chunk / block_size + 2 <= 64 ? attn_decode_kernel<true> : attn_decode_kernel<false>;
+  kernel<<<grid, 64, 0, s>>>((const __bf16*)q, q_stride, (const __bf16*)k_cache, (const __bf16*)v_cache, partial,
+                             entries, entry_start, entry_first_pos, block_table, table_width, block_size, heads,
+                             kv_heads, hd, scale, window, chunk, head_blocks);
   VK_LAUNCH_CHECK();
   dim3 cgrid(num_entries, heads);
   attn_combine_kernel<<<cgrid, 64, 0, s>>>(partial, (__bf16*)out, entries, entry_start, heads, hd, chunks);
