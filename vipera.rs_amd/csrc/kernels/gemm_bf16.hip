@@ -23,6 +23,17 @@
 // reference's batched matvec (crates/vipera-backend-gpu/src/q4k_matvec_q8_batch.cu:40-116).
 #include "common.h"
 
+#include <type_traits>
+
+// Depth of the load pipelines of the weight-streaming kernels: register sets of operands, one being
+// multiplied while the others are in flight (measured on an MI355X).
+#ifndef VK_SKINNY_SETS
+#define VK_SKINNY_SETS 3
+#endif
+#ifndef VK_MID_SETS
+#define VK_MID_SETS 3
+#endif
+
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -34,6 +45,68 @@ __device__ __forceinline__ bf16x8 zero8() {
 #pragma unroll
   for (int i = 0; i < 8; ++i) z[i] = (__bf16)0.f;
   return z;
+}
+
+// A range of memory behind a buffer descriptor (wave-uniform): a 16-byte read at a byte offset at or
+// past `bytes` returns zero without touching memory. Offsets and sizes are 32-bit.
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+struct BufferView {
+  __amdgpu_buffer_rsrc_t rsrc;
+  __device__ __forceinline__ bf16x8 load(unsigned byte_offset) const {
+    return __builtin_bit_cast(bf16x8, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)byte_offset, 0, 0));
+  }
+};
+__device__ __forceinline__ BufferView buffer_view(const void* base, unsigned long long bytes) {
+  const unsigned range = bytes > 0xffffffffull ? 0xffffffffu : (unsigned)bytes;
+  // third word: raw buffer, 32-bit data format (what the compiler's own buffer accesses use on gfx9)
+  return BufferView{__builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)range, 0x00020000)};
+}
+
+template <int N, int I = 0, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<N, I + 1>(f);
+  }
+}
+
+// A software pipeline over `count` items with SETS rotating register sets. step(set, rem, i) works on
+// item i with register set `set` (std::integral_constant) and is told, as a compile-time constant `rem`
+// capped at NEED, how many items follow it: so what a step still requests (items i + 1 .. i + NEED) is
+// decided when it is compiled, no load of the loop sits behind a branch, the compiler can count exactly
+// which loads a use waits for, and the later ones stay in flight. The loop runs rounds of SETS steps
+// while every step of a round has NEED followers; the last items run as one straight-line sequence
+// chosen by how many are left. NEED >= SETS - 1.
+template <int SETS, int NEED, int R, int J = 0, typename Step>
+__device__ __forceinline__ void pipeline_last(Step& step, int i) {
+  if constexpr (J < R) {
+    step(std::integral_constant<int, J % SETS>{}, std::integral_constant<int, (R - J - 1 < NEED ? R - J - 1 : NEED)>{},
+         i + J);
+    pipeline_last<SETS, NEED, R, J + 1>(step, i);
+  }
+}
+template <int SETS, int NEED, int R = 1, typename Step>
+__device__ __forceinline__ void pipeline_last_of(Step& step, int i, int left) {
+  if constexpr (R < SETS + NEED) {
+    if (left == R)
+      pipeline_last<SETS, NEED, R>(step, i);
+    else
+      pipeline_last_of<SETS, NEED, R + 1>(step, i, left);
+  }
+}
+template <int SETS, int NEED, int S = 0, typename Step>
+__device__ __forceinline__ void pipeline_round(Step& step, int i) {
+  if constexpr (S < SETS) {
+    step(std::integral_constant<int, S>{}, std::integral_constant<int, NEED>{}, i + S);
+    pipeline_round<SETS, NEED, S + 1>(step, i);
+  }
+}
+template <int SETS, int NEED, typename Step>
+__device__ __forceinline__ void run_pipeline(Step& step, int count) {
+  static_assert(NEED >= SETS - 1 && NEED >= 1, "a step must know about every item it may request");
+  int i = 0;
+  for (; i + SETS + NEED <= count; i += SETS) pipeline_round<SETS, NEED>(step, i);
+  pipeline_last_of<SETS, NEED>(step, i, count - i);
 }
 
 template <typename TC, bool ACCUMULATE>
@@ -205,68 +278,83 @@ constexpr int SPAN = 128;  // k per wave per step: four instructions of 32
 
 // CB: blocks of 16 tokens (M <= 16 * CB). RT: tiles of 16 weight rows per wave. WAVES: waves of a
 // workgroup, which split K in interleaved spans. A workgroup owns 16 * RT weight rows.
-template <int CB, int RT, int WAVES, typename TC, bool ACCUMULATE>
+template <int CB, int RT, int WAVES, typename TC, bool ACCUMULATE, int SETS = (CB == 1 ? VK_SKINNY_SETS : 2)>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const __bf16* __restrict__ A,
                                                                   const __bf16* __restrict__ W,
                                                                   const float* __restrict__ bias,
                                                                   TC* __restrict__ C, int M, int N, int K,
                                                                   long long lda, long long ldc, int vector_ok) {
   __shared__ f32x4 partial[WAVES][RT * CB][64];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lr = lane & 15, lg = lane >> 4;
   const int n0 = blockIdx.x * 16 * RT;
-  const __bf16* wp[RT];
+  // reads past the last weight row or the last token return zero and fetch nothing (see BufferView)
+  const BufferView w_view = buffer_view(W + (size_t)n0 * K, (unsigned long long)(N - n0) * K * 2);
+  const BufferView a_view = buffer_view(A, ((unsigned long long)(M - 1) * lda + K) * 2);
+  unsigned w_off[RT], a_off[CB];
 #pragma unroll
-  for (int rt = 0; rt < RT; ++rt) {
-    const int wrow = min(n0 + rt * 16 + lr, N - 1);  // rows past N are read from the last row and never stored
-    wp[rt] = W + (size_t)wrow * K + lg * 8;
-  }
-  const __bf16* ap[CB];
-  bool a_ok[CB];
+  for (int rt = 0; rt < RT; ++rt) w_off[rt] = (unsigned)(((rt * 16 + lr) * K + lg * 8) * 2);
 #pragma unroll
-  for (int cb = 0; cb < CB; ++cb) {
-    const int m = cb * 16 + lr;
-    a_ok[cb] = m < M;
-    ap[cb] = A + (size_t)(a_ok[cb] ? m : 0) * lda + lg * 8;
-  }
+  for (int cb = 0; cb < CB; ++cb) a_off[cb] = (unsigned)(((cb * 16 + lr) * lda + lg * 8) * 2);
   f32x4 acc[RT][CB];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
     for (int cb = 0; cb < CB; ++cb) acc[rt][cb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  const int spans = (K + SPAN - 1) / SPAN;
-  // two spans are in flight: while one is multiplied, the loads of the next (weights and activations)
-  // are already issued, and nothing of the current span waits for them
-  bf16x8 w_cur[RT][4], w_next[RT][4], a_cur[CB][4], a_next[CB][4];
-  auto load_span = [&](int span, bf16x8 (*w_dst)[4], bf16x8 (*a_dst)[4]) {
-    const int kb = span * SPAN;
+  // SETS register sets of operands rotate through run_pipeline: the loads of SETS - 1 spans are in flight
+  // while one span is multiplied (three sets with one block of tokens, two with more).
+  bf16x8 wf[SETS][RT][4], af[SETS][CB][4];
+  auto load_span = [&](int span, bf16x8 (&w_dst)[RT][4], bf16x8 (&a_dst)[CB][4]) {
+    const unsigned kb = (unsigned)span * SPAN * 2;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const bool ok = span < spans && kb + i * 32 + lg * 8 < K;
 #pragma unroll
-      for (int rt = 0; rt < RT; ++rt) w_dst[rt][i] = ok ? *(const bf16x8*)(wp[rt] + kb + i * 32) : zero8();
+      for (int rt = 0; rt < RT; ++rt) w_dst[rt][i] = w_view.load(w_off[rt] + kb + i * 64);
 #pragma unroll
-      for (int cb = 0; cb < CB; ++cb) a_dst[cb][i] = (ok && a_ok[cb]) ? *(const bf16x8*)(ap[cb] + kb + i * 32) : zero8();
+      for (int cb = 0; cb < CB; ++cb) a_dst[cb][i] = a_view.load(a_off[cb] + kb + i * 64);
     }
   };
-  load_span(wave, w_cur, a_cur);
-  for (int span = wave; span < spans; span += WAVES) {
-    load_span(span + WAVES, w_next, a_next);
+  auto multiply = [&](const bf16x8 (&w_src)[RT][4], const bf16x8 (&a_src)[CB][4]) {
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
       for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt)
-          acc[rt][cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_cur[rt][i], a_cur[cb][i], acc[rt][cb], 0, 0, 0);
+          acc[rt][cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_src[rt][i], a_src[cb][i], acc[rt][cb], 0, 0, 0);
+  };
+  const int whole = K / SPAN;                                               // spans that lie inside K
+  const int count = wave < whole ? (whole - wave + WAVES - 1) / WAVES : 0;  // this wave's: wave + i * WAVES
+  auto step = [&](auto set_, auto rem_, int i) {
+    constexpr int SET = decltype(set_)::value;
+    if constexpr (decltype(rem_)::value >= SETS - 1)
+      load_span(wave + (i + SETS - 1) * WAVES, wf[(SET + SETS - 1) % SETS], af[(SET + SETS - 1) % SETS]);
+    multiply(wf[SET], af[SET]);
+  };
+  if (count >= SETS - 1) {
+    static_for<SETS - 1>([&](auto j) { load_span(wave + j.value * WAVES, wf[j.value], af[j.value]); });
+    run_pipeline<SETS, SETS - 1>(step, count);
+  } else {  // fewer spans than the pipeline is deep: request them all, then multiply
+    static_for<SETS - 1>([&](auto j) {
+      if (j.value < count) load_span(wave + j.value * WAVES, wf[j.value], af[j.value]);
+    });
+    static_for<SETS - 1>([&](auto j) {
+      if (j.value < count) multiply(wf[j.value], af[j.value]);
+    });
+  }
+  if (whole * SPAN < K && wave == whole % WAVES) {  // the rest of K, less than a span: operands past K are zeroed
+    load_span(whole, wf[0], af[0]);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < 4; ++i)
+      if (whole * SPAN + i * 32 + lg * 8 >= K) {
 #pragma unroll
-      for (int rt = 0; rt < RT; ++rt) w_cur[rt][i] = w_next[rt][i];
+        for (int rt = 0; rt < RT; ++rt) wf[0][rt][i] = zero8();
 #pragma unroll
-      for (int cb = 0; cb < CB; ++cb) a_cur[cb][i] = a_next[cb][i];
-    }
+        for (int cb = 0; cb < CB; ++cb) af[0][cb][i] = zero8();
+      }
+    multiply(wf[0], af[0]);
   }
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt)
@@ -292,14 +380,14 @@ int launch_skinny_as(const __bf16* A, const __bf16* W, const float* bias, TC* C,
   return 0;
 }
 
-// Shape of the launch: few weight rows (N / 16 tiles below `many`) want many waves per workgroup so
-// that enough loads are in flight; many rows want more rows per wave so that activations are re-read less.
+// Shape of the launch (rows per wave, waves that split K). Measured on the 7B shapes: with one block of
+// tokens four waves on 16 rows are fastest at every weight size; with more blocks, many rows want two
+// row tiles per wave so that activations are re-read less.
 template <int CB, typename TC, bool ACC>
 int launch_skinny_cb(const __bf16* A, const __bf16* W, const float* bias, TC* C, int M, int N, int K, long long lda,
                      long long ldc, int vector_ok, int shape, hipStream_t s) {
   const int tiles = (N + 15) / 16;
-  // measured on the 7B shapes; sixteen waves with more than one token block would not fit the registers
-  if (shape == 0) shape = tiles >= 1024 ? ((CB >= 2 || M > 4) ? 2 : 1) : (CB == 1 ? 3 : 1);
+  if (shape == 0) shape = (CB >= 2 && tiles >= 1024) ? 2 : 1;
   switch (shape) {
     case 1: return launch_skinny_as<CB, 1, 4, TC, ACC>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, s);
     case 2: return launch_skinny_as<CB, 2, 4, TC, ACC>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, s);
@@ -441,7 +529,8 @@ int launch_stationary(const __bf16* A, const __bf16* W, const float* bias, TC* C
 constexpr int MID_CHUNK = 256;
 constexpr int MID_ROW = MID_CHUNK + 8;  // elements per LDS row: 528 bytes, so 16 rows hit 16 different 16-byte slots
 
-template <int CB, int RT, typename TC, bool ACCUMULATE, bool GATED = false>
+template <int CB, int RT, typename TC, bool ACCUMULATE, bool GATED = false,
+          int SETS = (RT == 1 && CB <= 2 ? VK_MID_SETS : 2)>
 __global__ __launch_bounds__(256) void gemm_mid_kernel(const __bf16* __restrict__ A, const __bf16* __restrict__ W,
                                                        const float* __restrict__ bias, TC* __restrict__ C, int M,
                                                        int N, int K, long long lda, long long ldc, int k_per_range,
@@ -449,55 +538,51 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const __bf16* __restrict_
   extern __shared__ __attribute__((aligned(16))) __bf16 lds[];  // [2][CB * 16][MID_ROW]
   constexpr int BUF = CB * 16 * MID_ROW;
   constexpr int A_LOADS = CB * 2;  // 16-byte pieces of a chunk per thread
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lr = lane & 15, lg = lane >> 4;
   const int n0 = blockIdx.x * 64 * RT + wave * 16 * RT;
   const int k_begin = blockIdx.y * k_per_range, k_end = min(K, k_begin + k_per_range);
   C += (size_t)blockIdx.y * range_stride;
 
-  const __bf16* wp[RT];
+  // Reads go through buffer descriptors: one past the end (a weight row past N, a token past M) returns
+  // zero and fetches nothing, so no load of the pipeline below sits behind a branch, the compiler can
+  // count exactly which loads a use waits for, and the later ones stay in flight.
+  const BufferView w_view = buffer_view(W + (size_t)min(n0, N - 1) * K, n0 < N ? (unsigned long long)(N - n0) * K * 2 : 0);
+  const BufferView a_view = buffer_view(A, ((unsigned long long)(M - 1) * lda + K) * 2);
+  unsigned w_off[RT], a_off[A_LOADS];
 #pragma unroll
-  for (int rt = 0; rt < RT; ++rt) wp[rt] = W + (size_t)min(n0 + rt * 16 + lr, N - 1) * K + lg * 8;
+  for (int rt = 0; rt < RT; ++rt) w_off[rt] = (unsigned)(((rt * 16 + lr) * K + lg * 8) * 2);
+#pragma unroll
+  for (int i = 0; i < A_LOADS; ++i) {
+    const int id = tid + 256 * i;
+    a_off[i] = (unsigned)(((id >> 5) * lda + (id & 31) * 8) * 2);
+  }
   f32x4 acc[RT][CB];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
     for (int cb = 0; cb < CB; ++cb) acc[rt][cb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  bf16x8 a_stage[A_LOADS], w_cur[RT][8], w_next[RT][8];
+  bf16x8 a_stage[A_LOADS], w[SETS][RT][8];
   auto load_acts = [&](int k0) {
 #pragma unroll
-    for (int i = 0; i < A_LOADS; ++i) {
-      const int id = tid + 256 * i, row = id >> 5, k = k0 + (id & 31) * 8;
-      a_stage[i] = (row < M && k < k_end) ? *(const bf16x8*)(A + (size_t)row * lda + k) : zero8();
-    }
+    for (int i = 0; i < A_LOADS; ++i) a_stage[i] = a_view.load(a_off[i] + (unsigned)k0 * 2);
   };
   auto store_acts = [&](int buf) {
 #pragma unroll
     for (int i = 0; i < A_LOADS; ++i) {
-      const int id = tid + 256 * i, row = id >> 5, c = id & 31;
-      *(bf16x8*)(lds + buf * BUF + row * MID_ROW + c * 8) = a_stage[i];
+      const int id = tid + 256 * i;
+      *(bf16x8*)(lds + buf * BUF + (id >> 5) * MID_ROW + (id & 31) * 8) = a_stage[i];
     }
   };
-  auto load_weights = [&](int k0, bf16x8 (*dst)[8]) {
+  auto load_weights = [&](int k0, bf16x8 (&dst)[RT][8]) {
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-      for (int i = 0; i < 8; ++i)
-        dst[rt][i] = (k0 + i * 32 + lg * 8 < k_end) ? *(const bf16x8*)(wp[rt] + k0 + i * 32) : zero8();
+      for (int i = 0; i < 8; ++i) dst[rt][i] = w_view.load(w_off[rt] + (unsigned)(k0 + i * 32) * 2);
   };
-
-  load_acts(k_begin);
-  load_weights(k_begin, w_cur);
-  store_acts(0);
-  __syncthreads();
-  int buf = 0;
-  for (int k0 = k_begin; k0 < k_end; k0 += MID_CHUNK) {
-    const bool more = k0 + MID_CHUNK < k_end;
-    if (more) {
-      load_acts(k0 + MID_CHUNK);
-      load_weights(k0 + MID_CHUNK, w_next);
-    }
+  auto multiply = [&](const bf16x8 (&wf)[RT][8], int buf) {
     const __bf16* tile = lds + buf * BUF + lr * MID_ROW + lg * 8;
 #pragma unroll
     for (int i = 0; i < 8; ++i)
@@ -506,15 +591,53 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const __bf16* __restrict_
         const bf16x8 a = *(const bf16x8*)(tile + cb * 16 * MID_ROW + i * 32);
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt)
-          acc[rt][cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_cur[rt][i], a, acc[rt][cb], 0, 0, 0);
+          acc[rt][cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[rt][i], a, acc[rt][cb], 0, 0, 0);
       }
-    if (more) store_acts(buf ^ 1);
+  };
+
+  // Whole chunks run through run_pipeline: the weights of chunk c + SETS - 1 are requested before chunk c
+  // is multiplied (SETS register sets: three while registers allow three waves a SIMD, else two), the activations
+  // of chunk c + 1 wait in registers until the barrier frees their LDS buffer, those of chunk c + 2 are
+  // requested right after it.
+  const int whole = (k_end - k_begin) / MID_CHUNK;
+  int buf = 0;
+  constexpr int NEED = SETS - 1 > 2 ? SETS - 1 : 2;
+  auto chunk = [&](auto set_, auto rem_, int c) {
+    constexpr int SET = decltype(set_)::value, REM = decltype(rem_)::value;  // REM chunks follow (capped)
+    const int k0 = k_begin + c * MID_CHUNK;
+    if constexpr (REM >= SETS - 1) load_weights(k0 + (SETS - 1) * MID_CHUNK, w[(SET + SETS - 1) % SETS]);
+    multiply(w[SET], buf);
+    if constexpr (REM >= 1) store_acts(buf ^ 1);
     __syncthreads();
+    if constexpr (REM >= 2) load_acts(k0 + 2 * MID_CHUNK);
     buf ^= 1;
+  };
+  if (whole > 0) {
+    // requests past the range (fewer chunks than the pipeline is deep) read weights that are not used
+    load_acts(k_begin);
+    static_for<SETS - 1>([&](auto j) { load_weights(k_begin + j.value * MID_CHUNK, w[j.value]); });
+    store_acts(0);
+    load_acts(k_begin + MID_CHUNK);
+    __syncthreads();
+    run_pipeline<SETS, NEED>(chunk, whole);
+  }
+  // the rest of the range (less than a chunk): operands past k_end are zeroed
+  const int k_rest = k_begin + whole * MID_CHUNK;
+  if (k_rest < k_end) {
+    load_acts(k_rest);
+    load_weights(k_rest, w[0]);
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i)
+      if (k_rest + ((tid + 256 * i) & 31) * 8 >= k_end) a_stage[i] = zero8();
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-      for (int i = 0; i < 8; ++i) w_cur[rt][i] = w_next[rt][i];
+      for (int i = 0; i < 8; ++i)
+        if (k_rest + i * 32 + lg * 8 >= k_end) w[0][rt][i] = zero8();
+    store_acts(0);
+    __syncthreads();
+    multiply(w[0], 0);
+    __syncthreads();  // the epilogue may reuse the buffers
   }
   if constexpr (GATED) {
     if constexpr (RT == 2) {  // a wave's two tiles are the gate and up rows of the same outputs

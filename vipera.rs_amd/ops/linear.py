@@ -4,9 +4,9 @@ All-bfloat16 operands whose rows are 16-byte aligned go to the matrix-core kerne
 combination (the 32-bit run, or a matrix kept in 32-bit inside a bfloat16 run) goes to the
 32-bit FMA kernel.  Among the matrix-core kernels the number of rows of ``a`` (tokens) decides:
 
-* more than 64: the 128x128 tiled kernel (prompts);
-* up to 64 (decoding): the product is a stream of the weights.  Few tokens, or few weight rows at up
-  to 16 tokens, use the kernel whose waves split K inside a workgroup; otherwise the kernel that
+* more than 64: the LDS-tiled kernel (prompts);
+* up to 64 (decoding): the product is a stream of the weights.  Up to four tokens, or a small weight
+  at up to 16 tokens, use the kernel whose waves split K inside a workgroup; otherwise the kernel that
   shares the activations through LDS, with K split over workgroups where the weight has too few rows
   to fill the GPU otherwise.  The thresholds were measured on the 7B shapes on an MI355X.
 """
@@ -27,7 +27,10 @@ def mid_plan(m: int, n: int, k: int) -> Tuple[int, int]:
         return (1, 2) if m > 16 else (1, 1)
     if n >= 16_384:
         return (2, 1) if m > 16 else (1, 1)
-    return min(16, max(1, k // 448)), 1
+    # few weight rows: split K while the workgroups still fit the 256 CUs at once (one more range was
+    # measured a third slower), each range at least two chunks long
+    row_blocks = (n + 63) // 64
+    return max(1, min(k // 512, 256 // row_blocks)), 1
 
 
 def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
@@ -35,7 +38,7 @@ def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: 
     if a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and kernels.gemm_bf16_supported(a, w, out):
         m, k = a.shape
         n = w.shape[0]
-        if m > 64 or m <= 4 or (m <= 16 and n < 16_384):
+        if m > 64 or m <= 4 or (m <= 16 and n < 16_384 and k < 8_192):
             if m <= 16 and STATIONARY:
                 kernels.gemm_bf16_stationary(a, w, bias, out, accumulate)
             else:
@@ -62,7 +65,7 @@ def linear_gated(a: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor, in
     n = w_gate_up.shape[0]
     fusable = (interleaved and a.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16
                and out.dtype == torch.bfloat16 and kernels.gemm_bf16_supported(a, w_gate_up, out))
-    if fusable and (m > 64 or (4 < m <= 16 and n >= 16_384)):
+    if fusable and m > 4:
         # the epilogue of the tiled kernel, or of the LDS-shared kernel with one K range, applies the gate
         kernels.gemm_bf16_gated(a, w_gate_up, out, rows_per_wave=1)
         return out
