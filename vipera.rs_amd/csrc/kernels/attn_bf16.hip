@@ -21,6 +21,7 @@
 // The softmax is online over steps of 32 positions that start at multiples of 32, so a token's
 // arithmetic depends on its position and the cache only.
 #include "common.h"
+#include "pipeline.h"
 
 #ifndef HDP
 #define HDP 128
@@ -56,7 +57,7 @@ template <bool REGS>
 __device__ __forceinline__ int page_of(const CacheView& cv, int p) {
   const int index = p / cv.block_size;
   if (REGS) return __shfl(cv.pages, (index - cv.page0) & 63, 64);
-  return (index >= 0 && index < cv.table_width) ? cv.table[index] : -1;
+  return cv.table[min(max(index, 0), cv.table_width - 1)];
 }
 
 // The K and V^T operands of one step of 32 positions.
@@ -65,44 +66,46 @@ struct StepOperands {
   bf16x8 vf[DT];     // V^T: positions kb + 4g .. +3 and kb + 16 + 4g .. +3 of output dim 16 dt + lr
 };
 
-// Issue the loads of the step that starts at kb. Positions outside [begin, end), pages that are not
-// held and dims past the head width read as zero.
+// Issue the loads of the step that starts at kb. No load sits behind a branch (the compiler can then
+// count which loads a use waits for, and the next step's stay in flight): a position outside
+// [begin, end) reads a position inside it instead, a dim past the head width reads dim 0, a page id
+// that is not held reads page 0. None of these can reach a result: such a position's score is masked
+// before the softmax and its weight is zero, the query is zero in the padded dims and padded output
+// dims are not stored; what is read in their place is cache content of the same request, which is finite
+// (the pool starts zeroed). The block table is checked on the host before a step runs.
 template <bool REGS>
 __device__ __forceinline__ void load_step(int kb, int begin, int end, const CacheView& cv, StepOperands& r) {
   const int lane = threadIdx.x & 63, lr = lane & 15, lg = lane >> 4;
   const int bs = cv.block_size, hd = cv.hd;
 #pragma unroll
   for (int sub = 0; sub < 2; ++sub) {
-    const int p = kb + sub * 16 + lr;
-    const int page = page_of<REGS>(cv, p);
-    const __bf16* row = nullptr;
-    if (p >= begin && p < end && page >= 0)
-      row = cv.k + (((size_t)page * cv.kv_heads + cv.kvh) * bs + (p % bs)) * hd + lg * 8;
+    const int p = min(max(kb + sub * 16 + lr, begin), end - 1);
+    const int page = max(page_of<REGS>(cv, p), 0);
+    const __bf16* row = cv.k + (((size_t)page * cv.kv_heads + cv.kvh) * bs + (p % bs)) * hd;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks)
-      r.kf[sub][ks] = (row && ks * 32 + lg * 8 < hd) ? *(const bf16x8*)(row + ks * 32) : zero8();
+    for (int ks = 0; ks < KS; ++ks) {
+      const int dim = ks * 32 + lg * 8;
+      r.kf[sub][ks] = *(const bf16x8*)(row + (dim < hd ? dim : 0));
+    }
   }
-  const __bf16* vrow[2] = {nullptr, nullptr};
+  const __bf16* vrow[2];
 #pragma unroll
   for (int half = 0; half < 2; ++half) {
-    const int p = kb + half * 16 + lg * 4;
-    const int page = page_of<REGS>(cv, p);
-    // a group of four positions lies in one page (4 divides the page size)
-    if (p + 3 >= begin && p < end && page >= 0)
-      vrow[half] = cv.v + (((size_t)page * cv.kv_heads + cv.kvh) * hd) * bs + (p % bs);
+    // groups of four positions start at multiples of 4 and lie in one page (4 divides the page size)
+    const int p = min(max(kb + half * 16 + lg * 4, begin & ~3), (end - 1) & ~3);
+    const int page = max(page_of<REGS>(cv, p), 0);
+    vrow[half] = cv.v + (((size_t)page * cv.kv_heads + cv.kvh) * hd) * bs + (p % bs);
   }
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) {
     const int d = dt * 16 + lr;
-    bf16x8 f = zero8();
-    if (d < hd) {
+    const size_t offset = (size_t)(d < hd ? d : 0) * bs;
+    const bf16x4 x0 = *(const bf16x4*)(vrow[0] + offset), x1 = *(const bf16x4*)(vrow[1] + offset);
+    bf16x8 f;
 #pragma unroll
-      for (int half = 0; half < 2; ++half)
-        if (vrow[half]) {
-          const bf16x4 x = *(const bf16x4*)(vrow[half] + (size_t)d * bs);
-#pragma unroll
-          for (int i = 0; i < 4; ++i) f[half * 4 + i] = x[i];
-        }
+    for (int i = 0; i < 4; ++i) {
+      f[i] = x0[i];
+      f[4 + i] = x1[i];
     }
     r.vf[dt] = f;
   }
@@ -111,18 +114,20 @@ __device__ __forceinline__ void load_step(int kb, int begin, int end, const Cach
 // Online-softmax attention of 16 columns over positions [begin, end). Per lane: col_lo / col_pos are
 // the visible range [lo, pos] of the lane's column (pos < 0: the column is empty).
 // State: o[DT] (O^T tiles), m (running max of the column), l (this lane's share of the running sum).
-// The loads of a step are issued one step ahead of its arithmetic: a wave has few steps and memory is
-// the bound.
+// The loads of a step are issued one step ahead of its arithmetic (two operand sets that alternate by
+// unrolling): a wave has few steps and memory is the bound.
 template <bool REGS>
 __device__ __forceinline__ void attend_range(const bf16x8 (&qf)[KS], int col_lo, int col_pos, int begin, int end,
                                              const CacheView& cv, float scale, f32x4 (&o)[DT], float& m, float& l) {
   const int lane = threadIdx.x & 63, lg = lane >> 4;
-  StepOperands cur, next;
   const int first = begin & ~31;
   if (first >= end) return;
-  load_step<REGS>(first, begin, end, cv, cur);
-  for (int kb = first; kb < end; kb += 32) {
-    if (kb + 32 < end) load_step<REGS>(kb + 32, begin, end, cv, next);
+  StepOperands ops[2];
+  auto step = [&](auto set_, auto rem_, int i) {
+    constexpr int SET = decltype(set_)::value;
+    const int kb = first + i * 32;
+    if constexpr (decltype(rem_)::value >= 1) load_step<REGS>(kb + 32, begin, end, cv, ops[SET ^ 1]);
+    const StepOperands& cur = ops[SET];
     // ---- scores of two 16-position tiles
     f32x4 s[2];
 #pragma unroll
@@ -154,10 +159,10 @@ __device__ __forceinline__ void attend_range(const bf16x8 (&qf)[KS], int col_lo,
       alpha = __expf(m - m_new);  // m = -inf gives 0
       float sum = 0.f;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const float w = __expf(sv[i] - m_new);
+      for (int i8 = 0; i8 < 8; ++i8) {
+        const float w = __expf(sv[i8] - m_new);
         sum += w;
-        pf[i] = (__bf16)w;
+        pf[i8] = (__bf16)w;
       }
       l = l * alpha + sum;
       m = m_new;
@@ -167,8 +172,9 @@ __device__ __forceinline__ void attend_range(const bf16x8 (&qf)[KS], int col_lo,
       o[dt] *= alpha;
       o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.vf[dt], pf, o[dt], 0, 0, 0);
     }
-    if (kb + 32 < end) cur = next;
-  }
+  };
+  load_step<REGS>(first, begin, end, cv, ops[0]);
+  run_pipeline<2, 1>(step, (end - first + 31) / 32);
 }
 
 __device__ __forceinline__ void load_q(const __bf16* qrow, int hd, bf16x8 (&qf)[KS]) {

@@ -11,14 +11,14 @@ import torch
 
 from . import kernels
 
-DECODE_WAVES_WANTED = 2048   # enough waves to keep the memory system busy
+DECODE_WAVES_WANTED = 512    # enough waves to keep the memory system busy (each keeps a step of loads in flight)
 DECODE_CHUNK_MIN = 128       # below this the merge of the chunks costs more than the waves gain
 DECODE_CHUNKS_MAX = 128
 
 
 def decode_chunking(max_kv_len: int, num_entries: int, kv_heads: int, head_blocks: int):
     """``(chunk, chunks)``: positions per chunk (a multiple of 32) and chunks that cover ``max_kv_len``."""
-    chunk = 512
+    chunk = 1024
     while chunk > DECODE_CHUNK_MIN:
         chunks = (max_kv_len + chunk - 1) // chunk
         if num_entries * kv_heads * head_blocks * chunks >= DECODE_WAVES_WANTED:

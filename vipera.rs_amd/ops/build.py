@@ -33,7 +33,7 @@ MODULES: Dict[str, tuple] = {
     "elementwise": ("hip", ["kernels/elementwise.hip"], ["kernels/common.h"]),
     "gemm_generic": ("hip", ["kernels/gemm_generic.hip"], ["kernels/common.h"]),
     "attn_generic": ("hip", ["kernels/attn_generic.hip"], ["kernels/common.h"]),
-    "gemm_bf16": ("hip", ["kernels/gemm_bf16.hip"], ["kernels/common.h"]),
+    "gemm_bf16": ("hip", ["kernels/gemm_bf16.hip"], ["kernels/common.h", "kernels/pipeline.h"]),
     "sampling": ("hip", ["kernels/sampling.hip"], ["kernels/common.h"]),
     "host": ("host", ["host/cache_manager.cpp", "host/scheduler.cpp", "host/c_api.cpp"],
              ["host/cache_manager.h", "host/scheduler.h"]),
@@ -41,7 +41,8 @@ MODULES: Dict[str, tuple] = {
 
 # matrix-core attention: one module per padded head width, compiled when a model of that width runs
 for _width in range(32, 257, 32):
-    MODULES[f"attn_bf16_hd{_width}"] = ("hip", ["kernels/attn_bf16.hip"], ["kernels/common.h"], [f"-DHDP={_width}"])
+    MODULES[f"attn_bf16_hd{_width}"] = ("hip", ["kernels/attn_bf16.hip"], ["kernels/common.h", "kernels/pipeline.h"],
+                                         [f"-DHDP={_width}"])
 
 _loaded: Dict[str, ctypes.CDLL] = {}
 _lock = threading.Lock()
