@@ -747,6 +747,7 @@ extern "C" int vk_gemm_bf16(const void* A, const void* W, const float* bias, voi
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0 || (K & 7) || (lda & 7) || lda < K || ldc < N) return VK_BAD_ARGUMENT;
   if (((uintptr_t)A & 15) || ((uintptr_t)W & 15)) return VK_BAD_ARGUMENT;
+  if (K >= (1 << 24) || lda >= (1 << 24)) return VK_UNSUPPORTED_SIZE;  // byte offsets inside a tile of rows are 32-bit
   if (accumulate && c_dtype != DT_F32) return VK_BAD_ARGUMENT;
   const int elem = c_dtype == DT_F32 ? 4 : 2;
   const int vector_ok = ((ldc & 3) == 0 && ((uintptr_t)C & (4 * elem - 1)) == 0 &&
@@ -831,6 +832,7 @@ extern "C" int vk_gemm_bf16_gated(const void* A, const void* W, void* C, int M, 
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0 || (K & 7) || (lda & 7) || lda < K || (N & 31) || ldc < N / 2) return VK_BAD_ARGUMENT;
   if (((uintptr_t)A & 15) || ((uintptr_t)W & 15)) return VK_BAD_ARGUMENT;
+  if (K >= (1 << 24) || lda >= (1 << 24)) return VK_UNSUPPORTED_SIZE;  // byte offsets inside a tile of rows are 32-bit
   hipStream_t s = (hipStream_t)stream;
   const __bf16* a = (const __bf16*)A;
   const __bf16* w = (const __bf16*)W;
