@@ -807,6 +807,7 @@ extern "C" int vk_gemm_bf16_mid(const void* A, const void* W, const float* bias,
   if (M > 64) return VK_UNSUPPORTED_SIZE;
   if (K <= 0 || (K & 7) || (lda & 7) || lda < K || ldc < N || ranges < 1) return VK_BAD_ARGUMENT;
   if (((uintptr_t)A & 15) || ((uintptr_t)W & 15) || ((uintptr_t)partial & 15)) return VK_BAD_ARGUMENT;
+  if (K >= (1 << 24) || lda >= (1 << 24)) return VK_UNSUPPORTED_SIZE;  // byte offsets inside a tile of rows are 32-bit
   if (accumulate && c_dtype != DT_F32) return VK_BAD_ARGUMENT;
   const int elem = c_dtype == DT_F32 ? 4 : 2;
   const int vector_ok = ((ldc & 3) == 0 && ((uintptr_t)C & (4 * elem - 1)) == 0 &&
