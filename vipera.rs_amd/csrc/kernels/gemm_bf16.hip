@@ -153,17 +153,33 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_tile_kernel(const __bf16* _
 #pragma unroll
     for (int j = 0; j < TM; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+  // rows past M or N read zero through the buffer descriptors, so no load sits behind a branch
+  const BufferView a_view = buffer_view(A + (size_t)m0 * lda, ((unsigned long long)(M - m0 - 1) * lda + K) * 2);
+  const BufferView w_view = buffer_view(W + (size_t)n0 * K, (unsigned long long)(N - n0) * K * 2);
+  unsigned a_off[A_PIECES], w_off[W_PIECES];
+#pragma unroll
+  for (int i = 0; i < A_PIECES; ++i) {
+    const int id = tid + THREADS * i;
+    a_off[i] = (unsigned)(((id >> 3) * lda + (id & 7) * 8) * 2);
+  }
+#pragma unroll
+  for (int i = 0; i < W_PIECES; ++i) {
+    const int id = tid + THREADS * i;
+    w_off[i] = (unsigned)(((size_t)(id >> 3) * K + (id & 7) * 8) * 2);
+  }
   bf16x8 ra[A_PIECES], rw[W_PIECES];
   auto load_global = [&](int k0) {
 #pragma unroll
-    for (int i = 0; i < A_PIECES; ++i) {
-      const int id = tid + THREADS * i, row = id >> 3, k = k0 + (id & 7) * 8;
-      ra[i] = (m0 + row < M && k < K) ? *(const bf16x8*)(A + (size_t)(m0 + row) * lda + k) : zero8();
-    }
+    for (int i = 0; i < A_PIECES; ++i) ra[i] = a_view.load(a_off[i] + (unsigned)k0 * 2);
 #pragma unroll
-    for (int i = 0; i < W_PIECES; ++i) {
-      const int id = tid + THREADS * i, row = id >> 3, k = k0 + (id & 7) * 8;
-      rw[i] = (n0 + row < N && k < K) ? *(const bf16x8*)(W + (size_t)(n0 + row) * K + k) : zero8();
+    for (int i = 0; i < W_PIECES; ++i) rw[i] = w_view.load(w_off[i] + (unsigned)k0 * 2);
+    if (k0 + BK > K) {  // the last step of a K that is no multiple of 64: pieces past K are zero
+#pragma unroll
+      for (int i = 0; i < A_PIECES; ++i)
+        if (k0 + ((tid + THREADS * i) & 7) * 8 >= K) ra[i] = zero8();
+#pragma unroll
+      for (int i = 0; i < W_PIECES; ++i)
+        if (k0 + ((tid + THREADS * i) & 7) * 8 >= K) rw[i] = zero8();
     }
   };
   auto store_lds = [&](int buf) {
