@@ -185,13 +185,13 @@ __device__ __forceinline__ void load_q(const __bf16* qrow, int hd, bf16x8 (&qf)[
 }
 
 // ---------------------------------------------------------------------------------------------
-// Prompts: grid (tiles, heads), eight waves. A tile is 128 consecutive tokens of one entry; a wave owns
+// Prompts: one workgroup of eight waves per (tile, head). A tile is 128 consecutive tokens of one entry; a wave owns
 // 16 of them (one block of columns). The positions are walked in tiles of 64 whose K rows and V^T rows
 // are fetched once per workgroup into LDS and read from there by all eight waves: while a tile is being
 // multiplied the next one's loads are in flight in registers, and the page ids of the tile after that
 // are already being looked up. Two workgroups fit a CU, so one's barriers and loads hide behind the
 // other's arithmetic. LDS rows are padded by 16 bytes so that the 16 rows of an operand read fall into
-// different banks. Tiles are taken last-first: the long ones (late tokens see many positions) start first.
+// different banks.
 constexpr int PT_WAVES = 8;
 constexpr int PT_THREADS = PT_WAVES * 64;
 constexpr int PT_TOKENS = PT_WAVES * 16;   // tokens of a tile
@@ -206,14 +206,20 @@ __global__ __launch_bounds__(PT_THREADS) void attn_prefill_kernel(
     const __bf16* __restrict__ v_cache, __bf16* __restrict__ out, const int* __restrict__ tiles,
     const int* __restrict__ entry_start, const int* __restrict__ entry_first_pos,
     const int* __restrict__ block_table, int table_width, int block_size, int heads, int kv_heads, int hd,
-    float scale, int window) {
+    float scale, int window, int cus) {
   extern __shared__ __attribute__((aligned(16))) __bf16 lds[];
   __bf16* sK = lds;                     // [PT_KV][PT_KROW]
   __bf16* sV = lds + PT_KV * PT_KROW;   // [HDP][PT_VROW]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, lr = lane & 15, lg = lane >> 4;
-  const int tile = gridDim.x - 1 - blockIdx.x;
+  // Work items (tile, head) are numbered by rising length (the host sorts the tiles). Workgroups are
+  // handed out in rounds of one per CU and two share a CU: even rounds take the longest items left,
+  // odd rounds the shortest, so that a long tile's neighbour on its CU is a short one.
+  const int total = (int)gridDim.x, round = blockIdx.x / cus;
+  const int taken = (round >> 1) * cus + blockIdx.x % cus;
+  const int item = (round & 1) ? taken : total - 1 - taken;
+  const int tile = item / heads;
   const int entry = tiles[2 * tile], tile_off = tiles[2 * tile + 1];
-  const int h = blockIdx.y, kvh = h / (heads / kv_heads);
+  const int h = item % heads, kvh = h / (heads / kv_heads);
   const int tok0 = entry_start[entry], count = entry_start[entry + 1] - tok0;
   const int first_pos = entry_first_pos[entry];
   const int* table = block_table + (size_t)entry * table_width;
@@ -510,7 +516,8 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(const float* __restric
 
 extern "C" int vk_attn_bf16_hdp() { return HDP; }
 
-// tiles: pairs (entry, first token of the tile within the entry), 128 tokens per tile.
+// tiles: pairs (entry, first token of the tile within the entry), 128 tokens per tile; best sorted by the
+// number of positions a tile sees, rising (any order gives the same result).
 extern "C" int vk_attn_bf16_prefill(const void* q, long long q_stride, const void* k_cache, const void* v_cache,
                                     void* out, const int* tiles, int num_tiles, const int* entry_start,
                                     const int* entry_first_pos, const int* block_table, int table_width,
@@ -518,7 +525,7 @@ extern "C" int vk_attn_bf16_prefill(const void* q, long long q_stride, const voi
                                     void* stream) {
   if (num_tiles <= 0) return 0;
   if (hd <= 0 || hd > HDP || (hd & 7) || block_size <= 0 || (block_size & 7) || heads <= 0 || kv_heads <= 0 ||
-      heads % kv_heads || heads > 65535 || (q_stride & 7) || window < 0)
+      heads % kv_heads || (q_stride & 7) || window < 0)
     return VK_UNSUPPORTED_SIZE;
   constexpr int lds_bytes = (PT_KV * PT_KROW + HDP * PT_VROW) * (int)sizeof(__bf16);
   static bool configured = false;
@@ -528,10 +535,18 @@ extern "C" int vk_attn_bf16_prefill(const void* q, long long q_stride, const voi
     if (e != hipSuccess) return (int)e;
     configured = true;
   }
-  dim3 grid(num_tiles, heads);
-  attn_prefill_kernel<<<grid, PT_THREADS, lds_bytes, (hipStream_t)stream>>>(
+  static int cus = 0;  // compute units of the device, for the pairing of long and short tiles
+  if (cus == 0) {
+    int device = 0, count = 0;
+    hipError_t e = hipGetDevice(&device);
+    if (e == hipSuccess) e = hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, device);
+    if (e != hipSuccess) return (int)e;
+    cus = count > 0 ? count : 1;
+  }
+  if ((long long)num_tiles * heads > 0x7fffffffLL) return VK_UNSUPPORTED_SIZE;
+  attn_prefill_kernel<<<num_tiles * heads, PT_THREADS, lds_bytes, (hipStream_t)stream>>>(
       (const __bf16*)q, q_stride, (const __bf16*)k_cache, (const __bf16*)v_cache, (__bf16*)out, tiles, entry_start,
-      entry_first_pos, block_table, table_width, block_size, heads, kv_heads, hd, scale, window);
+      entry_first_pos, block_table, table_width, block_size, heads, kv_heads, hd, scale, window, cus);
   VK_LAUNCH_CHECK();
   return 0;
 }

@@ -132,14 +132,17 @@ def pack_entries(entries: Sequence[StepEntry], cache, vocab_size: int, min_table
                 raise InvalidArgumentError(
                     f"request {e.request}: wanted place {w} is outside its {counts[k]} tokens of this step")
             rows.append(int(starts[k]) + int(w))
-    tiles: List[int] = []
+    tile_list: List[tuple] = []
     singles: List[int] = []
     for k, n in enumerate(counts_all):
         if n == 1:
             singles.append(k)
         else:
             for off in range(0, n, TILE_TOKENS):
-                tiles += [k, off]
+                tile_list.append((int(first[k]) + off, k, off))
+    # by rising number of visible positions: the attention kernel pairs long tiles with short ones
+    tile_list.sort()
+    tiles: List[int] = [x for _, k, off in tile_list for x in (k, off)]
     max_decode_kv = max((int(kv_len[k]) for k in singles), default=0)
 
     tables, widths = [], []
