@@ -36,6 +36,17 @@ QWEN25_7B = {
 }
 
 
+# the other two Qwen2.5 shapes, for measurements beside the headline one (--shape)
+SHAPES = {
+    "7b": ("Qwen2.5-7B shape", QWEN25_7B),
+    "1.5b": ("Qwen2.5-1.5B shape", dict(QWEN25_7B, num_hidden_layers=28, hidden_size=1536, num_attention_heads=12,
+                                        num_key_value_heads=2, intermediate_size=8960, vocab_size=151936,
+                                        tie_word_embeddings=True, max_window_layers=21)),
+    "32b": ("Qwen2.5-32B shape", dict(QWEN25_7B, num_hidden_layers=64, hidden_size=5120, num_attention_heads=40,
+                                      num_key_value_heads=8, intermediate_size=27648, max_window_layers=64)),
+}
+
+
 def log(text):
     print(f"[bench] {text}", file=sys.stderr, flush=True)
 
@@ -47,7 +58,9 @@ def main() -> int:
     parser.add_argument("--warmup", type=int, default=8)
     parser.add_argument("--batch", type=int, default=8, help="batch of the headline decode measurement")
     parser.add_argument("--ctx", type=int, default=4096, help="context length the decode steps end at")
-    parser.add_argument("--layers", type=int, default=28, help="fewer layers than 28 only where memory or time needs it")
+    parser.add_argument("--shape", default="7b", choices=sorted(SHAPES), help="layer sizes; the headline run is 7b")
+    parser.add_argument("--layers", type=int, default=0,
+                        help="fewer layers than the shape has, only where memory or time needs it (0: all)")
     parser.add_argument("--points", default="1,64", help="further decode batch sizes to report")
     parser.add_argument("--prefill-tokens", type=int, default=2048)
     parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
@@ -70,7 +83,10 @@ def main() -> int:
 
     dtype_key = "bf16" if args.dtype == "bfloat16" else "fp32"
     element = 2 if dtype_key == "bf16" else 4
-    data = dict(QWEN25_7B, num_hidden_layers=args.layers)
+    shape_name, shape = SHAPES[args.shape]
+    layers_full = shape["num_hidden_layers"]
+    args.layers = args.layers or layers_full
+    data = dict(shape, num_hidden_layers=args.layers)
     config = config_from_dict(data)
     runtime = Runtime("cuda:0", args.dtype)
     model = build_model(config, runtime)
@@ -92,7 +108,7 @@ def main() -> int:
     layer_matrix = H * (Q + 2 * KV) + Q * H + 2 * I * H + I * H
     layer_vectors = (Q + 2 * KV) + 2 * H
     kv_per_token = 2 * KV * element * L
-    weight_bytes = L * (layer_matrix * element + layer_vectors * 4) + V * H * element + H * 4
+    weight_bytes = L * (layer_matrix * element + layer_vectors * 4) + V * H * element + H * 4  # output matrix (tied or not)
 
     gen = torch.Generator().manual_seed(0)
 
@@ -182,7 +198,7 @@ def main() -> int:
         "dtype": dtype_key,
         "data": "synthetic: seeded random weights N(0, 0.02) and uniform-random token ids",
         "config": {
-            "model": "Qwen2.5-7B shape", "layers": args.layers, "layers_full": 28, "hidden": H,
+            "model": shape_name, "layers": args.layers, "layers_full": layers_full, "hidden": H,
             "heads": config.num_attention_heads, "kv_heads": config.num_key_value_heads,
             "head_dim": config.head_dim, "intermediate": I, "vocab": V, "global_batch": args.batch,
             "seq_len": ctx, "prefill_tokens": T, "block_size": args.block_size, "parallelism": "single GPU",

@@ -39,6 +39,7 @@ def _host():
         "vk_cache_advance": ([p, u64, i], None),
         "vk_cache_release": ([p, u64], i),
         "vk_cache_table": ([p, u64, i, ip, i], i),
+        "vk_cache_fill_tables": ([p, c.POINTER(u64), i, i, ip, i, ip, ip], i),
         "vk_cache_slot": ([p, u64], i),
         "vk_cache_knows": ([p, u64], i),
         "vk_cache_free_blocks": ([p, i], i),
@@ -139,6 +140,18 @@ class CacheManager:
     def table_into(self, request: int, group: int, buffer, capacity: int) -> int:
         """Write the table into a ctypes int array; returns its length."""
         return self._lib.vk_cache_table(self._handle, request, group, buffer, capacity)
+
+    def fill_tables(self, requests, group: int, out, need_from, need_to) -> int:
+        """Write the block tables of ``requests`` into the rows of ``out`` (a C-contiguous int32 array
+        ``[len(requests), width]``, -1 where no page is held) and check that logical blocks
+        ``[need_from[k], need_to[k])`` of every request are backed by pages.  Returns -1, or the index
+        of the first request that fails the check."""
+        count = len(requests)
+        ids = (ctypes.c_ulonglong * count)(*requests)
+        lo = (ctypes.c_int * count)(*need_from)
+        hi = (ctypes.c_int * count)(*need_to)
+        return self._lib.vk_cache_fill_tables(self._handle, ids, count, group,
+                                              out.ctypes.data_as(ctypes.POINTER(ctypes.c_int)), out.shape[1], lo, hi)
 
     def slot(self, request: int) -> int:
         return self._lib.vk_cache_slot(self._handle, request)

@@ -53,6 +53,26 @@ int vk_cache_table(void* handle, unsigned long long id, int group, int* out, int
   return n;
 }
 
+// The block tables of `count` requests at once: row k of out[count][width] gets the table of ids[k]
+// (-1 where it holds no page, and past its end). Logical blocks [from[k], to[k]) of request k must all
+// be backed by a page and fit the row. Returns -1 when that holds for every request, else the index of
+// the first one for which it does not (rows up to that one are written).
+int vk_cache_fill_tables(void* handle, const unsigned long long* ids, int count, int group, int* out, int width,
+                         const int* from, const int* to) {
+  const CacheManager* cache = static_cast<CacheManager*>(handle);
+  for (int k = 0; k < count; ++k) {
+    const auto& table = cache->table(ids[k], group);
+    const int n = (int)table.size() < width ? (int)table.size() : width;
+    int* row = out + (size_t)k * width;
+    if (n > 0) std::memcpy(row, table.data(), sizeof(int) * (size_t)n);
+    for (int b = n; b < width; ++b) row[b] = -1;
+    if (to[k] > n) return k;
+    for (int b = from[k] < 0 ? 0 : from[k]; b < to[k]; ++b)
+      if (row[b] < 0) return k;
+  }
+  return -1;
+}
+
 int vk_cache_slot(void* handle, unsigned long long id) { return static_cast<CacheManager*>(handle)->slot(id); }
 int vk_cache_knows(void* handle, unsigned long long id) { return static_cast<CacheManager*>(handle)->knows(id) ? 1 : 0; }
 int vk_cache_free_blocks(void* handle, int group) { return static_cast<CacheManager*>(handle)->free_blocks(group); }

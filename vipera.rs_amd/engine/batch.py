@@ -146,20 +146,22 @@ def pack_entries(entries: Sequence[StepEntry], cache, vocab_size: int, min_table
     max_decode_kv = max((int(kv_len[k]) for k in singles), default=0)
 
     tables, widths = [], []
+    requests = [e.request for e in entries]
     for g, spec in enumerate(cache.groups):
         width = max(min_table_width, int((int(kv_len.max()) + spec.block_size - 1) // spec.block_size))
-        table = np.full((E, width), -1, dtype=np.int32)
-        for k, e in enumerate(entries):
-            row = cache.table(e.request, g)
-            need_to = (int(kv_len[k]) + spec.block_size - 1) // spec.block_size
+        table = np.empty((E, width), dtype=np.int32)
+        need_to = [(int(kv_len[k]) + spec.block_size - 1) // spec.block_size for k in range(real)]
+        if spec.window > 0:
+            need_from = [max(0, e.start + 1 - spec.window) // spec.block_size for e in entries]
+        else:
+            need_from = [0] * real
+        failed = cache.fill_tables(requests, g, table, need_from, need_to)
+        if failed >= 0:
+            e = entries[failed]
             lo = max(0, e.start + 1 - spec.window) if spec.window > 0 else 0
-            need_from = lo // spec.block_size
-            if len(row) < need_to or any(p < 0 for p in row[need_from:need_to]):
-                raise InternalError(
-                    f"request {e.request}: positions {lo}..{int(kv_len[k]) - 1} are not all backed by pages "
-                    f"in cache group {g}; reserve before the step")
-            n = min(len(row), width)
-            table[k, :n] = row[:n]
+            raise InternalError(
+                f"request {e.request}: positions {lo}..{int(kv_len[failed]) - 1} are not all backed by pages "
+                f"in cache group {g}; reserve before the step")
         if pad_entries:
             table[real:, :] = pad_page
         tables.append(table)
