@@ -88,6 +88,8 @@ class BatchSampler:
 
     def __init__(self, device):
         self.device = torch.device(device)
+        self._staging = None        # pinned host words of the per-row options, reused by every call
+        self._device_words = None   # their place on the device
 
     def sample(self, logits: torch.Tensor, rows: Sequence[RowRequest]) -> List[int]:
         count, vocab = logits.shape
@@ -96,14 +98,23 @@ class BatchSampler:
         if logits.dtype != torch.float32 or not logits.is_contiguous():
             raise InvalidArgumentError("logits must be contiguous float32")
         self._penalize(logits, rows, vocab)
-        temperature = np.array([r.params.temperature for r in rows], dtype=np.float32)
-        top_k = np.array([r.params.top_k for r in rows], dtype=np.int32)
-        top_p = np.array([r.params.top_p for r in rows], dtype=np.float32)
-        min_p = np.array([r.params.min_p for r in rows], dtype=np.float32)
-        uniform = np.array([0.0 if r.params.greedy else r.rng.next_f64() for r in rows], dtype=np.float64)
-        dev = lambda a: torch.from_numpy(a).to(self.device)  # noqa: E731
+        # one pinned staging buffer, one copy: 4-byte columns first, then the 8-byte uniforms
+        words = 6 * count
+        if self._staging is None or self._staging.numel() < words:
+            self._staging = torch.empty(max(words, 6 * 64), dtype=torch.int32).pin_memory()
+            self._device_words = torch.empty(self._staging.numel(), dtype=torch.int32, device=self.device)
+        host = self._staging.numpy()
+        host[0:count].view(np.float32)[:] = [r.params.temperature for r in rows]
+        host[count:2 * count] = [r.params.top_k for r in rows]
+        host[2 * count:3 * count].view(np.float32)[:] = [r.params.top_p for r in rows]
+        host[3 * count:4 * count].view(np.float32)[:] = [r.params.min_p for r in rows]
+        host[4 * count:6 * count].view(np.float64)[:] = [0.0 if r.params.greedy else r.rng.next_f64() for r in rows]
+        dev = self._device_words
+        dev[:words].copy_(self._staging[:words], non_blocking=True)
         out = torch.empty(count, dtype=torch.int32, device=self.device)
-        kernels.sample(logits, dev(temperature), dev(top_k), dev(top_p), dev(min_p), dev(uniform), out)
+        kernels.sample(logits, dev[0:count].view(torch.float32), dev[count:2 * count],
+                       dev[2 * count:3 * count].view(torch.float32), dev[3 * count:4 * count].view(torch.float32),
+                       dev[4 * count:6 * count].view(torch.float64), out)
         return [int(t) for t in out.cpu().tolist()]
 
     def _penalize(self, logits: torch.Tensor, rows: Sequence[RowRequest], vocab: int) -> None:
