@@ -193,12 +193,46 @@ def test_attention_kernels_against_plain_softmax(case, dtype):
         if singles:
             longest = max(entries[e][0] for e in singles)
             for chunk, chunks in {decode_chunking(longest, len(singles), kv_heads, (heads // kv_heads + 15) // 16),
-                                  (32, (longest + 31) // 32), (512, (longest + 511) // 512)}:
+                                  (32, (longest + 31) // 32), (512, (longest + 511) // 512),
+                                  (2048, (longest + 2047) // 2048)}:
                 partial = torch.empty(len(singles) * heads * chunks * (hd + 2), device=DEV)
                 kernels.attn_bf16_decode(qkv_d, k_d, v_d, out2, partial, dev(torch.tensor(singles, dtype=torch.int32)),
                                          es, fp, table_d, heads, kv_heads, hd, scale, window, chunk, chunks)
                 assert _rel(out2.cpu(), want) < tol, f"matrix-core kernels, chunk {chunk}"
         assert _rel(out2.cpu(), want) < tol, "matrix-core kernels"
+
+
+@pytest.mark.parametrize("window", [0, 1500])
+def test_decode_attention_over_thousands_of_positions(window):
+    """Single-token entries with long histories: many chunks, chunks that span more pages than a wave
+    keeps ids of in a register (the table is then read step by step), chunks cut by a window's edge."""
+    from vipera_rs_amd.ops import kernels
+    heads, kv_heads, hd, bs = 8, 2, 64, 16
+    lengths = [5000, 3333, 1, 4097]
+    scale = 1.0 / math.sqrt(hd)
+    dtype = torch.bfloat16
+    cache = _Paged(lengths, kv_heads, hd, bs, dtype, seed=11)
+    g = torch.Generator().manual_seed(5)
+    qkv = torch.randn(len(lengths), (heads + 2 * kv_heads) * hd, generator=g).to(dtype)
+    first = [n - 1 for n in lengths]
+    want = torch.zeros(len(lengths), heads, hd, dtype=torch.float64)
+    for e, n in enumerate(lengths):
+        q = qkv[e:e + 1, :heads * hd].double().view(1, heads, hd)
+        want[e] = _plain_attention(q, cache.keys[e].double(), cache.values[e].double(), first[e], window, scale)[0]
+    want = want.view(len(lengths), heads * hd)
+    dev = lambda t: t.to(DEV)  # noqa: E731
+    qkv_d, k_d, v_d, table_d = dev(qkv), dev(cache.k), dev(cache.v), dev(cache.table)
+    es = dev(torch.arange(len(lengths) + 1, dtype=torch.int32))
+    fp = dev(torch.tensor(first, dtype=torch.int32))
+    singles = dev(torch.arange(len(lengths), dtype=torch.int32))
+    longest = max(lengths)
+    for chunk in (128, 256, 1024, 4096):
+        chunks = (longest + chunk - 1) // chunk
+        out = torch.zeros(len(lengths), heads * hd, dtype=dtype, device=DEV)
+        partial = torch.empty(len(lengths) * heads * chunks * (hd + 2), device=DEV)
+        kernels.attn_bf16_decode(qkv_d, k_d, v_d, out, partial, singles, es, fp, table_d, heads, kv_heads, hd, scale,
+                                 window, chunk, chunks)
+        assert _rel(out.cpu(), want) < 1.2e-2, f"chunk {chunk}"
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
