@@ -568,8 +568,9 @@ extern "C" int vk_attn_bf16_decode(const void* q, long long q_stride, const void
   if (kv_heads * head_blocks > 65535 || heads > 65535) return VK_UNSUPPORTED_SIZE;
   hipStream_t s = (hipStream_t)stream;
   dim3 grid(num_entries, kv_heads * head_blocks, chunks);
-  // a chunk that does not start on a page's edge touches one page more than chunk / block_size
-  auto kernel = chunk / block_size + 2 <= 64 ? attn_decode_kernel<true> : attn_decode_kernel<false>;
+  // pages a chunk can touch: chunks start at multiples of `chunk`, which need not be page edges
+  const int chunk_pages = chunk % block_size == 0 ? chunk / block_size : chunk / block_size + 2;
+  auto kernel = chunk_pages <= 64 ? attn_decode_kernel<true> : attn_decode_kernel<false>;
   kernel<<<grid, 64, 0, s>>>((const __bf16*)q, q_stride, (const __bf16*)k_cache, (const __bf16*)v_cache, partial,
                              entries, entry_start, entry_first_pos, block_table, table_width, block_size, heads,
                              kv_heads, hd, scale, window, chunk, head_blocks);
