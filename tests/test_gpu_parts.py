@@ -402,6 +402,120 @@ def test_a_stateful_toy_mixer_is_registered_built_and_stepped(tmp_path):
         unregister("mixer", "running_state")
 
 
+# --- a feed-forward with routing and another position encoding, defined here --------------------------------------
+def test_a_routed_feed_forward_and_another_position_encoding(tmp_path):
+    """Layer 0 gets a top-1-of-three-experts feed-forward (router in 32-bit) and a position encoding that
+    is no rotation (a sinusoid of the position added to q and k); layer 1 stays as it is.  Both parts
+    live in this file and are only registered with the framework."""
+    from vipera_rs_amd.config import (LayerSpec, PartSpec, Qwen2Config, register_architecture, unregister_architecture)
+    from vipera_rs_amd.engine.batch import StepEntry
+    from vipera_rs_amd.engine.runner import ModelRunner
+    from vipera_rs_amd.models.decoder import DecoderModel
+    from vipera_rs_amd.parts import (FeedForward, PositionEncoding, register_ffn, register_position, unregister)
+    from vipera_rs_amd.weights import MATRIX, TensorSpec
+
+    EXPERTS, INNER = 3, 40
+
+    class TopOne(FeedForward):
+        @classmethod
+        def declare(cls, spec, prefix):
+            hidden = spec.params["hidden"]
+            base = f"{prefix}moe."
+            out = [TensorSpec(base + "router.weight", (EXPERTS, hidden), MATRIX, std=0.5)]
+            for e in range(EXPERTS):
+                out.append(TensorSpec(f"{base}experts.{e}.up.weight", (INNER, hidden), MATRIX, std=0.2))
+                out.append(TensorSpec(f"{base}experts.{e}.down.weight", (hidden, INNER), MATRIX, std=0.2))
+            return out
+
+        def load(self, tensors):
+            base = f"{self.prefix}moe."
+            self.router = tensors[base + "router.weight"].float()
+            self.up = [tensors[f"{base}experts.{e}.up.weight"].float() for e in range(EXPERTS)]
+            self.down = [tensors[f"{base}experts.{e}.down.weight"].float() for e in range(EXPERTS)]
+
+        def forward(self, h, batch, residual):
+            x = h.float()
+            probs = torch.softmax(x @ self.router.T, dim=-1)          # 32-bit router
+            weight, choice = probs.max(dim=-1)
+            for e in range(EXPERTS):
+                rows = (choice == e).nonzero().flatten()
+                if rows.numel():
+                    y = torch.relu(x[rows] @ self.up[e].T) @ self.down[e].T
+                    residual[rows] += weight[rows, None] * y
+
+    class Tilt(PositionEncoding):
+        @classmethod
+        def declare(cls, spec, prefix):
+            return []
+
+        def load(self, tensors):
+            pass
+
+        def apply(self, qkv, batch, heads, kv_heads, head_dim):
+            width = (heads + kv_heads) * head_dim                       # q and k, not v
+            dims = torch.arange(head_dim, device=qkv.device, dtype=torch.float32).repeat(heads + kv_heads)
+            signal = 0.5 * torch.sin(batch.positions.float()[:, None] * 0.1 * (dims[None, :] + 1.0))
+            qkv[:, :width] = (qkv[:, :width].float() + signal).to(qkv.dtype)
+
+    class MixedConfig(Qwen2Config):
+        architecture = "ToyRoutedForCausalLM"
+
+        def layer_specs(self) -> List[LayerSpec]:
+            specs = super().layer_specs()
+            first = specs[0]
+            specs[0] = LayerSpec(first.block, first.mixer, PartSpec("top_one", {"hidden": self.hidden_size}),
+                                 first.mixer_norm, first.ffn_norm, PartSpec("tilt", {}), first.prefix)
+            return specs
+
+    def plain(cfg, w, tokens):
+        cfg = P.normalize_config(cfg)
+        T = len(tokens)
+        heads, kv_heads, hd = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+        x = w["model.embed_tokens.weight"][np.asarray(tokens)]
+        h = P.rms_norm(x, w["model.layers.0.input_layernorm.weight"], cfg["rms_norm_eps"])
+        a = "model.layers.0.self_attn."
+        q = P.linear(h, w[a + "q_proj.weight"], w.get(a + "q_proj.bias")).reshape(T, heads, hd)
+        k = P.linear(h, w[a + "k_proj.weight"], w.get(a + "k_proj.bias")).reshape(T, kv_heads, hd)
+        v = P.linear(h, w[a + "v_proj.weight"], w.get(a + "v_proj.bias")).reshape(T, kv_heads, hd)
+        signal = 0.5 * np.sin(np.arange(T)[:, None] * 0.1 * (np.arange(hd)[None, :] + 1.0))
+        q, k = q + signal[:, None, :], k + signal[:, None, :]
+        x = x + P.linear(P.attention(q, k, v, window=0).reshape(T, heads * hd), w[a + "o_proj.weight"])
+        h = P.rms_norm(x, w["model.layers.0.post_attention_layernorm.weight"], cfg["rms_norm_eps"])
+        logits = h @ w["model.layers.0.moe.router.weight"].T
+        probs = np.exp(logits - logits.max(-1, keepdims=True))
+        probs /= probs.sum(-1, keepdims=True)
+        for t in range(T):
+            e = int(probs[t].argmax())
+            y = np.maximum(w[f"model.layers.0.moe.experts.{e}.up.weight"] @ h[t], 0.0)
+            x[t] = x[t] + probs[t, e] * (w[f"model.layers.0.moe.experts.{e}.down.weight"] @ y)
+        h = P.rms_norm(x, w["model.layers.1.input_layernorm.weight"], cfg["rms_norm_eps"])
+        x = x + P.attention_block(h, w, "model.layers.1.self_attn.", cfg, 0)
+        h = P.rms_norm(x, w["model.layers.1.post_attention_layernorm.weight"], cfg["rms_norm_eps"])
+        x = x + P.swiglu_mlp(h, *(w[f"model.layers.1.mlp.{n}_proj.weight"] for n in ("gate", "up", "down")))
+        return P.linear(P.rms_norm(x, w["model.norm.weight"], cfg["rms_norm_eps"]), w["model.embed_tokens.weight"])
+
+    register_ffn("top_one", TopOne)
+    register_position("tilt", Tilt)
+    register_architecture("ToyRoutedForCausalLM", MixedConfig, lambda config, runtime: DecoderModel(config, runtime))
+    try:
+        folder = make_folder(tmp_path / "routed", dict(CONFIG_A, architectures=["ToyRoutedForCausalLM"]), 8)
+        cfg, w = P.load_folder(folder)
+        assert "model.layers.0.moe.router.weight" in w and "model.layers.0.mlp.gate_proj.weight" not in w
+        tokens = random_tokens(256, 31, 4)
+        want = plain(cfg, w, tokens)
+        runner = ModelRunner.from_folder(folder, dtype="float32", block_size=8, num_blocks=16, num_slots=2)
+        rows, at = [], 0
+        for size in (9, 1, 1, 13, 2, 5):
+            runner.cache.reserve(0, at, at + size)
+            rows.append(runner.step([StepEntry(0, at, tokens[at:at + size], list(range(size)))]).cpu().numpy())
+            at += size
+        assert rel_err(np.concatenate(rows), want) < 1e-4
+    finally:
+        unregister_architecture("ToyRoutedForCausalLM")
+        unregister("ffn", "top_one")
+        unregister("position", "tilt")
+
+
 # --- the first tokens of a sequence --------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_first_tokens_of_a_sequence(tmp_path, dtype):
