@@ -16,7 +16,7 @@ import torch
 
 from ..errors import InfeasibleError, InvalidArgumentError, ViperaError
 from ..runtime import Runtime
-from ..sampling import BatchSampler, Rng, RowRequest, SamplingParams
+from ..sampling import RECENT_WINDOW, BatchSampler, Rng, RowRequest, SamplingParams
 from .batch import StepEntry
 from .runner import ModelRunner
 from .scheduler import FINISH_NAMES, NOT_FINISHED, Scheduler
@@ -62,6 +62,13 @@ class _Live:
     processed: int = 0
     preemptions: int = 0
     on_token: Optional[Callable[[int], None]] = None
+
+
+def _recent_tokens(live) -> List[int]:
+    """The last RECENT_WINDOW tokens of a request (prompt then generated): all that the penalties look at."""
+    generated = live.generated[-RECENT_WINDOW:]
+    missing = RECENT_WINDOW - len(generated)
+    return (live.prompt[-missing:] if missing > 0 else []) + generated
 
 
 class Engine:
@@ -195,7 +202,7 @@ class Engine:
             rows = []
             for e in wanting:
                 live = self._live[e.request]
-                rows.append(RowRequest(live.params, live.rng, live.prompt + live.generated))
+                rows.append(RowRequest(live.params, live.rng, _recent_tokens(live) if live.params.penalizes else ()))
             tokens = self.sampler.sample(logits, rows)
             for e, token in zip(wanting, tokens):
                 if token < 0:
