@@ -99,21 +99,25 @@ extern "C" int vk_rmsnorm(const float* x, const float* weight, const int* rows, 
 }
 
 // ---------------------------------------------------------------------------------------------
-// One workgroup of 64 threads per (token, head): grid (tokens, heads + 2 * kv_heads); the last
-// kv_heads of a row are the value heads. `qkv` row layout: [heads*hd | kv_heads*hd | kv_heads*hd].
+// One wave per (token, head), four heads to a workgroup: grid (tokens, ceil((heads + 2 * kv_heads) / 4));
+// the last kv_heads of a row are the value heads. `qkv` row layout: [heads*hd | kv_heads*hd | kv_heads*hd].
 // The first `rotary_dim` dims of every q and k head are rotated in place (angles in 32-bit:
 // float(pos) * inv_freq[i]); then the token's K and V rows go to the paged cache. K pages are
 // [page, kv_head, slot, hd]; V pages are transposed, [page, kv_head, hd, slot], so that the
 // attention kernels read consecutive positions of one output dim. A token whose page id is
 // negative writes nothing to the cache.
+constexpr int ROPE_HEADS_PER_BLOCK = 4;  // one wave per head
 template <typename T>
-__global__ __launch_bounds__(64) void rope_kvwrite_kernel(T* __restrict__ qkv, const int* __restrict__ positions,
+__global__ __launch_bounds__(ROPE_HEADS_PER_BLOCK * 64) void rope_kvwrite_kernel(
+    T* __restrict__ qkv, const int* __restrict__ positions,
                                                           const float* __restrict__ inv_freq, int rotary_dim,
                                                           T* __restrict__ k_cache, T* __restrict__ v_cache,
                                                           const int* __restrict__ entry_of_token,
                                                           const int* __restrict__ block_table, int table_width,
-                                                          int block_size, int heads, int kv_heads, int hd) {
-  const int t = blockIdx.x, head = blockIdx.y;
+                                                          int block_size, int heads, int kv_heads, int hd,
+                                                          int total_heads) {
+  const int t = blockIdx.x, head = blockIdx.y * ROPE_HEADS_PER_BLOCK + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (head >= total_heads) return;
   const int pos = positions[t];
   T* h = qkv + (size_t)t * (heads + 2 * kv_heads) * hd + (size_t)head * hd;
   const bool is_q = head < heads, is_k = !is_q && head < heads + kv_heads;
@@ -124,7 +128,7 @@ __global__ __launch_bounds__(64) void rope_kvwrite_kernel(T* __restrict__ qkv, c
   if (is_q || is_k) {
     const int kvh = head - heads;
     const size_t k_at = is_k && page >= 0 ? (((size_t)page * kv_heads + kvh) * block_size + slot) * hd : 0;
-    for (int i = threadIdx.x; i < hd; i += 64) {
+    for (int i = lane; i < hd; i += 64) {
       if (i < half) {
         float sn, cs;
         sincosf((float)pos * inv_freq[i], &sn, &cs);
@@ -143,7 +147,7 @@ __global__ __launch_bounds__(64) void rope_kvwrite_kernel(T* __restrict__ qkv, c
   } else if (page >= 0) {
     const int kvh = head - heads - kv_heads;
     const size_t v_at = (((size_t)page * kv_heads + kvh) * hd) * block_size + slot;
-    for (int i = threadIdx.x; i < hd; i += 64) v_cache[v_at + (size_t)i * block_size] = h[i];
+    for (int i = lane; i < hd; i += 64) v_cache[v_at + (size_t)i * block_size] = h[i];
   }
 }
 
@@ -157,15 +161,18 @@ extern "C" int vk_rope_kvwrite(void* qkv, int dtype, const int* positions, const
   if (k_cache && (block_size <= 0 || table_width <= 0)) return VK_BAD_ARGUMENT;
   if (heads + 2 * kv_heads > 65535) return VK_UNSUPPORTED_SIZE;
   hipStream_t s = (hipStream_t)stream;
-  const dim3 grid(num_tokens, heads + (k_cache ? 2 : 1) * kv_heads);  // without a cache the value heads have nothing to do
+  const int total_heads = heads + (k_cache ? 2 : 1) * kv_heads;  // without a cache the value heads have nothing to do
+  const dim3 grid(num_tokens, (total_heads + ROPE_HEADS_PER_BLOCK - 1) / ROPE_HEADS_PER_BLOCK);
+  constexpr int threads = ROPE_HEADS_PER_BLOCK * 64;
   if (dtype == DT_F32)
-    rope_kvwrite_kernel<float><<<grid, 64, 0, s>>>((float*)qkv, positions, inv_freq, rotary_dim,
-                                                           (float*)k_cache, (float*)v_cache, entry_of_token,
-                                                           block_table, table_width, block_size, heads, kv_heads, hd);
+    rope_kvwrite_kernel<float><<<grid, threads, 0, s>>>((float*)qkv, positions, inv_freq, rotary_dim, (float*)k_cache,
+                                                        (float*)v_cache, entry_of_token, block_table, table_width,
+                                                        block_size, heads, kv_heads, hd, total_heads);
   else if (dtype == DT_BF16)
-    rope_kvwrite_kernel<bf16_t><<<grid, 64, 0, s>>>((bf16_t*)qkv, positions, inv_freq, rotary_dim,
-                                                            (bf16_t*)k_cache, (bf16_t*)v_cache, entry_of_token,
-                                                            block_table, table_width, block_size, heads, kv_heads, hd);
+    rope_kvwrite_kernel<bf16_t><<<grid, threads, 0, s>>>((bf16_t*)qkv, positions, inv_freq, rotary_dim,
+                                                         (bf16_t*)k_cache, (bf16_t*)v_cache, entry_of_token,
+                                                         block_table, table_width, block_size, heads, kv_heads, hd,
+                                                         total_heads);
   else
     return VK_BAD_ARGUMENT;
   VK_LAUNCH_CHECK();
