@@ -9,7 +9,9 @@ width 128, feed-forward 18944, vocabulary 152064, rotary base 1e6, untied output
 random weights N(0, 0.02) in bfloat16; token ids are seeded uniform-random.  Every request is
 prefilled for real and then decoded up to a context of 4,096 tokens; the timed steps are the last K
 decode steps of that run, through the engine's scheduler, captured step and greedy sampler.  A step
-is one decode step of the whole batch.
+is one decode step of the whole batch.  The engine launches a step before the tokens of the step
+before have reached the host (`pipelined=True`; `--in-turn` switches that off): every timed call of
+`step()` launches one decode step and takes in the tokens of the one before.
 
 Bytes a decode step has to read: every weight it uses once (all layer matrices, norms and the output
 matrix; of the embedding table only the batch's rows) and the keys and values of the live requests.
@@ -65,6 +67,8 @@ def main() -> int:
     parser.add_argument("--prefill-tokens", type=int, default=2048)
     parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     parser.add_argument("--block-size", type=int, default=16)
+    parser.add_argument("--in-turn", action="store_true",
+                        help="wait for a step's tokens on the host before the next step is launched")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this engine runs on a single MI355X, so --gpus {args.gpus} is not run")
@@ -141,7 +145,7 @@ def main() -> int:
     def decode(batch, steps, warmup):
         # every prompt gets a portion in every prefill step, so that all requests start decoding together
         engine = Engine(None, runner=runner, max_num_seqs=batch, max_num_batched_tokens=batch * 2048, chunk_size=2048,
-                        max_model_len=ctx + 8)
+                        max_model_len=ctx + 8, pipelined=not args.in_turn)
         prompt_len = ctx - steps - warmup - 1
         for _ in range(batch):
             engine.add_request(tokens(prompt_len), max_new_tokens=steps + warmup + 4)
@@ -202,7 +206,7 @@ def main() -> int:
             "heads": config.num_attention_heads, "kv_heads": config.num_key_value_heads,
             "head_dim": config.head_dim, "intermediate": I, "vocab": V, "global_batch": args.batch,
             "seq_len": ctx, "prefill_tokens": T, "block_size": args.block_size, "parallelism": "single GPU",
-            "sampling": "greedy", "weights_gb": round(weight_bytes / 1e9, 2),
+            "sampling": "greedy", "weights_gb": round(weight_bytes / 1e9, 2), "steps_launched_ahead": not args.in_turn,
         },
         "prefill": prefill,
         "roofline": {"bound": "hbm", "achieved": round(head["gbs"], 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",

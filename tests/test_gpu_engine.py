@@ -196,3 +196,74 @@ def test_captured_decode_steps_equal_eager_steps_on_every_replay(folders):
                 runner.step([StepEntry(3, 0, prompts[3], [20])])
             lengths[3] = 21
     assert runners[1].graphs.replays == 24 and len(runners[1].graphs.graphs) >= 2
+
+
+# --- steps launched ahead of their tokens ---------------------------------------------------------------------------
+def test_steps_launched_ahead_generate_the_same_tokens(folders):
+    """``pipelined=True``: greedy and seeded generation, portions mixed with decoding, with and without
+    captured steps, give exactly the tokens of the engine that runs one step after the other."""
+    from vipera_rs_amd import SamplingParams
+    prompts = [random_tokens(CONFIG_B["vocab_size"], n, 70 + n) for n in (1, 7, 19, 33)]
+    for params in (None, [SamplingParams(temperature=0.8, seed=11 + k) for k in range(4)]):
+        kw = dict(block_size=8, num_blocks=40, max_num_seqs=4, chunk_size=6, max_num_batched_tokens=16)
+        want = [g.tokens for g in _engine(folders["B"], **kw).generate(prompts, 14, params)]
+        for graphs in (True, False):
+            engine = _engine(folders["B"], pipelined=True, use_graphs=graphs, **kw)
+            got = engine.generate(prompts, 14, params)
+            assert [g.tokens for g in got] == want, (params is None, graphs)
+            assert all(g.finish == "length" for g in got)
+            assert engine.runner.cache.check() == "" and engine.runner.cache.live_requests() == 0
+            assert not engine.has_work()
+
+
+def test_steps_launched_ahead_stop_at_end_of_sequence_and_drop_the_extra_token(folders):
+    cfg, weights = qwen2_plain.load_folder(folders["A"])
+    prompts = [random_tokens(CONFIG_A["vocab_size"], n, 3 + n) for n in (9, 12)]
+    free = [qwen2_plain.greedy_generate(cfg, weights, p, 9) for p in prompts]
+    eos = free[0][3]
+    engine = _engine(folders["A"], num_blocks=12, pipelined=True)
+    streamed = {0: [], 1: []}
+    ids = [engine.add_request(p, 9, eos_token_ids=[eos], on_token=streamed[k].append) for k, p in enumerate(prompts)]
+    done = {}
+    while engine.has_work():
+        for g in engine.step().finished:
+            done[g.request] = g
+    for k, rid in enumerate(ids):
+        stop_at = free[k].index(eos) if eos in free[k] else None
+        want = free[k] if stop_at is None else free[k][:stop_at + 1]
+        assert done[rid].tokens == want and done[rid].finish == ("length" if stop_at is None else "stop")
+        assert streamed[k] == (want if stop_at is None else want[:-1])
+    assert engine.runner.cache.check() == "" and engine.runner.cache.live_requests() == 0
+
+
+def test_steps_launched_ahead_survive_preemption_and_penalties(folders):
+    from vipera_rs_amd import SamplingParams
+    prompts = [random_tokens(CONFIG_A["vocab_size"], n, 90 + n) for n in (30, 28, 25, 31)]
+    kw = dict(block_size=16, num_blocks=10, max_num_seqs=4, chunk_size=16)
+    want = [g.tokens for g in _engine(folders["A"], **kw).generate(prompts, 40)]
+    engine = _engine(folders["A"], pipelined=True, **kw)
+    got = engine.generate(prompts, 40)
+    assert [g.tokens for g in got] == want and engine.stats()["preemptions"] > 0
+    assert engine.runner.cache.check() == "" and engine.runner.cache.free_blocks(0) == 10
+    # a request with penalties makes the engine run its steps in turn while it lives; the others are unchanged
+    params = [SamplingParams(temperature=0.7, seed=5, repetition_penalty=1.3), None, SamplingParams(temperature=0.9, seed=6)]
+    kw = dict(block_size=16, num_blocks=24, max_num_seqs=3)
+    want = [g.tokens for g in _engine(folders["A"], **kw).generate(prompts[:3], 12, params)]
+    got = _engine(folders["A"], pipelined=True, **kw).generate(prompts[:3], 12, params)
+    assert [g.tokens for g in got] == want
+
+
+def test_cancel_while_a_step_is_on_its_way(folders):
+    prompts = [random_tokens(CONFIG_A["vocab_size"], n, 20 + n) for n in (6, 7)]
+    want = _engine(folders["A"], num_blocks=12).generate([prompts[1]], 10)[0].tokens
+    engine = _engine(folders["A"], num_blocks=12, pipelined=True)
+    first, second = [engine.add_request(p, 10) for p in prompts]
+    for _ in range(4):
+        engine.step()
+    assert engine.cancel(first).finish == "cancelled"
+    done = {}
+    while engine.has_work():
+        for g in engine.step().finished:
+            done[g.request] = g
+    assert list(done) == [second] and done[second].tokens == want
+    assert engine.runner.cache.check() == "" and engine.runner.cache.live_requests() == 0

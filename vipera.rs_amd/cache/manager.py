@@ -55,6 +55,7 @@ def _host():
         "vk_sched_plan_read": ([p, up, ip, ip, ip, ip, up], None),
         "vk_sched_advance": ([p, u64], None),
         "vk_sched_append": ([p, u64, i, i], i),
+        "vk_sched_replace_token": ([p, u64, i, i], i),
         "vk_sched_cancel": ([p, u64], i),
         "vk_sched_has_work": ([p], i),
         "vk_sched_num_waiting": ([p], i),

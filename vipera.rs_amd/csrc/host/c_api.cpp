@@ -136,6 +136,10 @@ int vk_sched_append(void* handle, unsigned long long id, int token, int is_end_o
   return static_cast<SchedulerHandle*>(handle)->scheduler.append(id, token, is_end_of_sequence != 0);
 }
 
+int vk_sched_replace_token(void* handle, unsigned long long id, int back, int token) {
+  return static_cast<SchedulerHandle*>(handle)->scheduler.replace_token(id, back, token) ? 0 : 1;
+}
+
 int vk_sched_cancel(void* handle, unsigned long long id) {
   return static_cast<SchedulerHandle*>(handle)->scheduler.cancel(id) ? 0 : 1;
 }

@@ -137,6 +137,15 @@ FinishReason Scheduler::append(uint64_t id, int token, bool is_end_of_sequence) 
   return reason;
 }
 
+bool Scheduler::replace_token(uint64_t id, int back, int token) {
+  auto found = requests_.find(id);
+  if (found == requests_.end()) return false;
+  std::vector<int>& tokens = found->second.tokens;
+  if (back < 0 || back >= (int)tokens.size() - found->second.prompt_len) return false;  // generated tokens only
+  tokens[tokens.size() - 1 - (size_t)back] = token;
+  return true;
+}
+
 bool Scheduler::cancel(uint64_t id) {
   auto found = requests_.find(id);
   if (found == requests_.end()) return false;

@@ -61,6 +61,9 @@ class Scheduler {
   void advance(uint64_t id);
   // A token was sampled for `id`. Returns why the request ended, or NOT_FINISHED.
   FinishReason append(uint64_t id, int token, bool is_end_of_sequence);
+  // Overwrite the token `back` places before the request's last one (0: the last). For callers that
+  // append a placeholder before the sampled token has reached the host. False when unknown or out of range.
+  bool replace_token(uint64_t id, int back, int token);
   // Remove a request in any state and give back what it holds. False when unknown.
   bool cancel(uint64_t id);
   bool has_work() const { return !waiting_.empty() || !running_.empty(); }

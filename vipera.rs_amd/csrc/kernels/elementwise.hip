@@ -10,24 +10,34 @@
 #include "common.h"
 
 // ---------------------------------------------------------------------------------------------
+// `source` (may be null): where source[t] >= 0 the token is not tokens[t] but sampled[source[t]], an id
+// that an earlier kernel of the stream left on the device (the previous step's sampler), so that a
+// step can be launched before its input token has reached the host. An id outside the table reads row 0
+// (the sampler leaves -1 where a row of logits held no finite value; the host fails that request).
 template <typename TW>
 __global__ void embed_gather_kernel(const TW* __restrict__ table, const int* __restrict__ tokens,
-                                    float* __restrict__ out, int width) {
+                                    const int* __restrict__ source, const int* __restrict__ sampled,
+                                    float* __restrict__ out, int width, int vocab) {
   const int t = blockIdx.x;
-  const TW* row = table + (size_t)tokens[t] * width;
+  int token = tokens[t];
+  if (source != nullptr && source[t] >= 0) token = sampled[source[t]];
+  if (token < 0 || token >= vocab) token = 0;
+  const TW* row = table + (size_t)token * width;
   float* dst = out + (size_t)t * width;
   for (int i = threadIdx.x; i < width; i += blockDim.x) dst[i] = to_float<TW>(row[i]);
 }
 
-extern "C" int vk_embed_gather(const void* table, int table_dtype, const int* tokens, float* out,
-                               int num_tokens, int width, void* stream) {
+extern "C" int vk_embed_gather(const void* table, int table_dtype, const int* tokens, const int* source,
+                               const int* sampled, float* out, int num_tokens, int width, int vocab, void* stream) {
   if (num_tokens <= 0) return 0;
-  if (width <= 0) return VK_BAD_ARGUMENT;
+  if (width <= 0 || vocab <= 0 || (source != nullptr && sampled == nullptr)) return VK_BAD_ARGUMENT;
   hipStream_t s = (hipStream_t)stream;
   if (table_dtype == DT_F32)
-    embed_gather_kernel<float><<<num_tokens, 256, 0, s>>>((const float*)table, tokens, out, width);
+    embed_gather_kernel<float><<<num_tokens, 256, 0, s>>>((const float*)table, tokens, source, sampled, out, width,
+                                                          vocab);
   else if (table_dtype == DT_BF16)
-    embed_gather_kernel<bf16_t><<<num_tokens, 256, 0, s>>>((const bf16_t*)table, tokens, out, width);
+    embed_gather_kernel<bf16_t><<<num_tokens, 256, 0, s>>>((const bf16_t*)table, tokens, source, sampled, out, width,
+                                                           vocab);
   else
     return VK_BAD_ARGUMENT;
   VK_LAUNCH_CHECK();

@@ -32,6 +32,7 @@ class StepEntry:
     start: int
     tokens: Sequence[int]
     want: Sequence[int] = ()
+    source: int = -1   # >= 0 (single-token entries only): the token is row ``source`` of the sampler's last output on the device
 
 
 @dataclass
@@ -50,6 +51,8 @@ class StepBatch:
     prefill_tiles: torch.Tensor    # [tiles, 2] int32: (entry, first token within it) per 128 tokens of multi-token entries
     decode_entries: torch.Tensor   # [n] int32: entries that hold exactly one token
     block_tables: Dict[int, torch.Tensor]  # group -> [E, width] int32
+    token_source: Optional[torch.Tensor] = None    # [T] int32: -1, or the row of `sampled_tokens` that holds the token
+    sampled_tokens: Optional[torch.Tensor] = None  # the sampler's output buffer on the device (set by the runner)
     # host copies, for launch decisions
     host_counts: List[int] = field(default_factory=list)
     host_first_pos: List[int] = field(default_factory=list)
@@ -66,7 +69,7 @@ class StepBatch:
 class PackedStep:
     """Host side of a step: the sections in their fixed order, and what the launch decisions need."""
 
-    sections: List[np.ndarray]     # tokens, positions, entry_of, starts, first, kv_len, slots, rows, tiles, singles, tables...
+    sections: List[np.ndarray]     # tokens, positions, entry_of, starts, first, kv_len, slots, rows, tiles, singles, sources, tables...
     table_widths: List[int]
     num_tokens: int
     num_entries: int
@@ -132,6 +135,12 @@ def pack_entries(entries: Sequence[StepEntry], cache, vocab_size: int, min_table
                 raise InvalidArgumentError(
                     f"request {e.request}: wanted place {w} is outside its {counts[k]} tokens of this step")
             rows.append(int(starts[k]) + int(w))
+    sources = np.full(T, -1, dtype=np.int32)
+    for k, e in enumerate(entries):
+        if e.source >= 0:
+            if counts[k] != 1:
+                raise InvalidArgumentError(f"request {e.request}: only a single-token entry can take its token from the device")
+            sources[int(starts[k])] = e.source
     tile_list: List[tuple] = []
     singles: List[int] = []
     for k, n in enumerate(counts_all):
@@ -167,7 +176,8 @@ def pack_entries(entries: Sequence[StepEntry], cache, vocab_size: int, min_table
         tables.append(table)
         widths.append(width)
     sections = [tokens, positions, entry_of, starts, first, kv_len.astype(np.int32), slots,
-                np.array(rows, dtype=np.int32), np.array(tiles, dtype=np.int32), np.array(singles, dtype=np.int32)]
+                np.array(rows, dtype=np.int32), np.array(tiles, dtype=np.int32), np.array(singles, dtype=np.int32),
+                sources]
     sections += tables
     return PackedStep(sections, widths, T, E, len(rows), counts_all, [int(v) for v in first], [int(v) for v in slots],
                       int(kv_len.max()), max_decode_kv)
@@ -180,13 +190,14 @@ def batch_from_buffer(packed: PackedStep, dev: torch.Tensor) -> StepBatch:
         views.append(dev[at:at + section.size])
         at += section.size
     E = packed.num_entries
-    fixed = 10
+    fixed = 11
     block_tables = {g: views[fixed + g].view(E, packed.table_widths[g]) for g in range(len(packed.table_widths))}
     return StepBatch(
         num_tokens=packed.num_tokens, num_entries=E, num_logit_rows=packed.num_logit_rows,
         tokens=views[0], positions=views[1], entry_of_token=views[2], entry_start=views[3],
         entry_first_pos=views[4], entry_kv_len=views[5], slots=views[6], logit_rows=views[7],
         prefill_tiles=views[8].view(-1, 2), decode_entries=views[9], block_tables=block_tables,
+        token_source=views[10],
         host_counts=packed.counts, host_first_pos=packed.first, host_slots=packed.slots,
         max_count=max(packed.counts), max_kv_len=packed.max_kv_len, all_single=max(packed.counts) == 1,
         num_prefill_tiles=packed.sections[8].size // 2, num_decode_entries=packed.sections[9].size,

@@ -19,7 +19,7 @@ from ..runtime import Runtime
 from ..sampling import RECENT_WINDOW, BatchSampler, Rng, RowRequest, SamplingParams
 from .batch import StepEntry
 from .runner import ModelRunner
-from .scheduler import FINISH_NAMES, NOT_FINISHED, Scheduler
+from .scheduler import FINISH_NAMES, FINISH_STOP, NOT_FINISHED, Scheduler
 
 
 @dataclass
@@ -64,6 +64,17 @@ class _Live:
     on_token: Optional[Callable[[int], None]] = None
 
 
+@dataclass
+class _InFlight:
+    """A launched step whose sampled tokens are still on their way: per row the request, and why the
+    scheduler ended it when the placeholder was appended (NOT_FINISHED if it did not)."""
+
+    pending: object                      # sampling.PendingSample
+    requests: List[int]
+    reasons: List[int]
+    row_of: Dict[int, int]               # request -> its row of the sampler's output
+
+
 def _recent_tokens(live) -> List[int]:
     """The last RECENT_WINDOW tokens of a request (prompt then generated): all that the penalties look at."""
     generated = live.generated[-RECENT_WINDOW:]
@@ -79,13 +90,20 @@ class Engine:
     layers; when ``num_blocks`` is absent it is sized for ``max_num_seqs`` requests of
     ``max_model_len`` tokens, bounded by free device memory.  ``use_graphs`` (default on) replays
     steps of single tokens as captured HIP graphs.
+
+    ``pipelined``: a step is launched before the tokens of the step before have reached the host (they
+    are read on the device, where the sampler left them), and ``step()`` reports the tokens of the step
+    *before* the one it launches; the GPU then never waits for the host between steps.  What is generated
+    is the same.  A request that ends on an end-of-sequence token has one token more computed, which is
+    dropped.  While a live request uses penalties (they look at the last tokens on the host), steps run
+    one after the other as without the option.
     """
 
     def __init__(self, model: str, dtype: str = "bfloat16", device: str = "cuda:0", block_size: int = 16,
                  num_blocks: Optional[int] = None, max_num_seqs: int = 8, max_num_batched_tokens: int = 2048,
                  chunk_size: int = 512, max_model_len: Optional[int] = None,
                  eos_token_ids: Optional[Sequence[int]] = None, runner: Optional[ModelRunner] = None,
-                 use_graphs: Optional[bool] = None):
+                 use_graphs: Optional[bool] = None, pipelined: bool = False):
         if runner is None:
             runtime = Runtime(device, dtype)
             from ..config.registry import load_config
@@ -106,7 +124,9 @@ class Engine:
         self.config = config
         self.max_model_len = limit
         self.scheduler = Scheduler(runner.cache, max_num_seqs, max_num_batched_tokens, chunk_size, limit)
-        self.sampler = BatchSampler(runner.runtime.device)
+        self.sampler = BatchSampler(runner.runtime.device, out=runner.sampled_tokens)
+        self.pipelined = bool(pipelined) and runner.sampled_tokens is not None
+        self._inflight: Optional[_InFlight] = None   # the launched step whose tokens have not been collected
         default_eos = getattr(config, "eos_token_ids", ()) or ()
         self.eos_token_ids = frozenset(eos_token_ids if eos_token_ids is not None else default_eos)
         self._live: Dict[int, _Live] = {}
@@ -168,11 +188,101 @@ class Engine:
         return Generation(request, len(live.prompt), live.generated, "cancelled", live.processed, live.preemptions)
 
     def has_work(self) -> bool:
-        return self.scheduler.has_work()
+        return self.scheduler.has_work() or self._inflight is not None
 
     # --- one step -----------------------------------------------------------------------------------
     def step(self) -> StepReport:
+        if self.pipelined and not any(live.params.penalizes for live in self._live.values()):
+            return self._step_ahead()
         report = StepReport()
+        if self._inflight is not None:  # leaving the pipelined way: first take in what is on its way
+            self._collect(report)
+        return self._step_in_turn(report)
+
+    def _step_ahead(self) -> StepReport:
+        """Launch the next step, then take in the tokens of the step launched before it."""
+        report = StepReport()
+        started = time.perf_counter()
+        plan = self.scheduler.plan()
+        for request in plan.preempted:
+            if request in self._live:
+                self._live[request].preemptions += 1
+        report.preempted = list(plan.preempted)
+        scheduled = time.perf_counter()
+        self.micros["schedule"] += int((scheduled - started) * 1e6)
+        previous, launched = self._inflight, None
+        if plan.entries:
+            entries = []
+            for e in plan.entries:
+                # the last token of a request whose sample is still on its way is a placeholder on the host:
+                # the step reads it from the sampler's output on the device
+                source = -1
+                if previous is not None and len(e.tokens) == 1 and e.request in previous.row_of \
+                        and e.start + 1 == self.scheduler.length_of(e.request):
+                    source = previous.row_of[e.request]
+                entries.append(StepEntry(e.request, e.start, e.tokens, [len(e.tokens) - 1] if e.wants_logits else [],
+                                         source))
+            report.num_batched_tokens = plan.num_tokens
+            self.step_count += 1
+            try:
+                logits = self.runner.step(entries)
+            except ViperaError as err:
+                if previous is not None:
+                    self._collect(report)
+                for e in plan.entries:
+                    self._fail(e.request, str(err), report)
+                return report
+            for e in plan.entries:
+                self.scheduler.advance(e.request)
+                self._live[e.request].processed += len(e.tokens)
+            wanting = [e for e in plan.entries if e.wants_logits]
+            if wanting:
+                rows = [RowRequest(self._live[e.request].params, self._live[e.request].rng, ()) for e in wanting]
+                pending = self.sampler.launch(logits, rows)
+                # the scheduler goes on as if the token were known: a placeholder stands for it until it arrives
+                reasons = [self.scheduler.append(e.request, 0, False) for e in wanting]
+                launched = _InFlight(pending, [e.request for e in wanting], reasons,
+                                     {e.request: row for row, e in enumerate(wanting)})
+        computed = time.perf_counter()
+        self._inflight = previous
+        if previous is not None:
+            self._collect(report, newer=launched)
+        self._inflight = launched
+        done = time.perf_counter()
+        self.micros["compute"] += int((computed - scheduled) * 1e6)
+        self.micros["sample"] += int((done - computed) * 1e6)
+        return report
+
+    def _collect(self, report: StepReport, newer: Optional[_InFlight] = None) -> None:
+        """Take in the tokens of the step in flight. ``newer``: a step launched after it, in which the same
+        requests may already hold one more placeholder."""
+        flight, self._inflight = self._inflight, None
+        tokens = self.sampler.collect(flight.pending)
+        for request, reason, token in zip(flight.requests, flight.reasons, tokens):
+            live = self._live.get(request)
+            if live is None:  # ended, failed or cancelled since the launch: what was computed for it is dropped
+                continue
+            if token < 0:
+                self._fail(request, "the logits hold no finite value", report)
+                continue
+            live.generated.append(token)
+            is_eos = token in live.eos
+            report.tokens.append(StepToken(request, token))
+            if is_eos:
+                reason = FINISH_STOP
+                self.scheduler.cancel(request)   # a no-op if the scheduler ended it at its token budget already
+            else:
+                back = 1 if newer is not None and request in newer.row_of else 0
+                self.scheduler.replace_token(request, back, token)
+                if live.on_token is not None:
+                    live.on_token(token)
+            if reason != NOT_FINISHED:
+                self._live.pop(request)
+                self.generations += 1
+                report.finished.append(Generation(request, len(live.prompt), live.generated, FINISH_NAMES[reason],
+                                                  live.processed, live.preemptions))
+
+    def _step_in_turn(self, report: StepReport) -> StepReport:
         started = time.perf_counter()
         plan = self.scheduler.plan()
         for request in plan.preempted:

@@ -7,6 +7,7 @@ arithmetic are those of the eager step.  Nothing that clears memory is recorded 
 """
 from __future__ import annotations
 
+import gc
 from typing import Dict, Optional, Sequence, Tuple
 
 import numpy as np
@@ -27,6 +28,7 @@ def _bucket(value: int, buckets: Sequence[int]) -> Optional[int]:
 class _Captured:
     def __init__(self, graph, buffer, staging, batch, logits):
         self.graph, self.buffer, self.staging, self.batch, self.logits = graph, buffer, staging, batch, logits
+        self.turn = 0  # which of the two staging buffers the last step used
 
 
 class DecodeGraphs:
@@ -72,24 +74,40 @@ class DecodeGraphs:
         captured = self.graphs.get(key)
         if captured is None:
             device = runner.runtime.device
-            staging = torch.empty(flat.size, dtype=torch.int32).pin_memory()
+            # two pinned staging buffers, used in turn: with steps launched ahead of their results, the copy of
+            # the step before may still be waiting in the stream when the next step is packed
+            staging = [torch.empty(flat.size, dtype=torch.int32).pin_memory() for _ in range(2)]
             buffer = torch.empty(flat.size, dtype=torch.int32, device=device)
-            staging.numpy()[:] = flat
-            buffer.copy_(staging, non_blocking=True)
+            staging[0].numpy()[:] = flat
+            buffer.copy_(staging[0], non_blocking=True)
             batch = batch_from_buffer(packed, buffer)
+            batch.sampled_tokens = runner.sampled_tokens
             # an eager run first: it loads every kernel module the step needs, outside of the capture
             runner.model.forward(batch, runner.storage)
             torch.cuda.synchronize(device)
             graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph, pool=self.pool):
-                logits = runner.model.forward(batch, runner.storage)
+            # No garbage collection while the stream is capturing: a collected object that holds pinned or
+            # device memory, an event or another graph (an engine that is no longer used, say) would be
+            # freed through calls that are not allowed during a capture, and the process would abort.
+            # What is garbage now is collected before the capture starts.
+            gc.collect()
+            collecting = gc.isenabled()
+            gc.disable()
+            try:
+                with torch.cuda.graph(graph, pool=self.pool):
+                    logits = runner.model.forward(batch, runner.storage)
+            finally:
+                if collecting:
+                    gc.enable()
             if self.pool is None:
                 self.pool = graph.pool()
             captured = _Captured(graph, buffer, staging, batch, logits)
             self.graphs[key] = captured
         else:
-            captured.staging.numpy()[:] = flat
-            captured.buffer.copy_(captured.staging, non_blocking=True)
+            captured.turn ^= 1
+            staging = captured.staging[captured.turn]
+            staging.numpy()[:] = flat
+            captured.buffer.copy_(staging, non_blocking=True)
         captured.graph.replay()
         self.replays += 1
         rows = [k for k, e in enumerate(entries) if len(e.want)]

@@ -23,6 +23,9 @@ from ..weights import Checkpoint, load_tensors
 from .batch import StepBatch, StepEntry, build_batch
 
 
+SAMPLED_CAPACITY = 1024  # rows of logits one step may be sampled for with device-side feedback
+
+
 class ModelRunner:
     def __init__(self, model, runtime: Runtime, block_size: int, num_blocks: int, num_slots: int,
                  use_graphs: bool = False, max_context: int = 0):
@@ -38,6 +41,11 @@ class ModelRunner:
         self.storage = CacheStorage(self.needs, groups, num_slots, runtime)
         self.vocab_size = model.vocab_size
         self.steps = 0
+        # where a sampler may leave the ids it draws, for a next step that is launched before they reach the
+        # host (StepEntry.source); at a fixed address, because captured steps read it
+        self.sampled_tokens = None
+        if getattr(model.embedding, "reads_device_tokens", False):
+            self.sampled_tokens = torch.zeros(SAMPLED_CAPACITY, dtype=torch.int32, device=runtime.device)
         self.graphs = None
         if use_graphs:
             from .graphs import DecodeGraphs
@@ -60,7 +68,9 @@ class ModelRunner:
 
     # --- the step ---------------------------------------------------------------------------------
     def prepare(self, entries: Sequence[StepEntry]) -> StepBatch:
-        return build_batch(entries, self.cache, self.vocab_size, self.runtime.device)
+        batch = build_batch(entries, self.cache, self.vocab_size, self.runtime.device)
+        batch.sampled_tokens = self.sampled_tokens
+        return batch
 
     def run(self, batch: StepBatch) -> Optional[torch.Tensor]:
         self.steps += 1

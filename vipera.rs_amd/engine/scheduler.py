@@ -103,6 +103,11 @@ class Scheduler:
     def append(self, request: int, token: int, is_end_of_sequence: bool) -> int:
         return self._lib.vk_sched_append(self._handle, request, token, 1 if is_end_of_sequence else 0)
 
+    def replace_token(self, request: int, back: int, token: int) -> bool:
+        """Overwrite the generated token ``back`` places before the request's last one (a placeholder that
+        was appended before the sampled token reached the host)."""
+        return self._lib.vk_sched_replace_token(self._handle, request, back, token) == 0
+
     def cancel(self, request: int) -> bool:
         return self._lib.vk_sched_cancel(self._handle, request) == 0
 

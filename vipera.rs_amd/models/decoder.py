@@ -101,7 +101,10 @@ class DecoderModel:
 
     def forward(self, batch, storage) -> Optional[torch.Tensor]:
         """Run the step's tokens through the run order; returns ``[wanted rows, vocab]`` 32-bit logits."""
-        x = self.embedding.forward(batch.tokens, batch.num_tokens)
+        if batch.sampled_tokens is not None and batch.token_source is not None:  # ids the sampler left on the device
+            x = self.embedding.forward(batch.tokens, batch.num_tokens, batch.token_source, batch.sampled_tokens)
+        else:
+            x = self.embedding.forward(batch.tokens, batch.num_tokens)
         for index, entry in enumerate(self.schedule):
             owner = index if entry.cache_of is None else entry.cache_of
             self.layers[entry.layer].forward(x, batch, storage.kv[owner], storage.state[owner],

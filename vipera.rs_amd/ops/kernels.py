@@ -80,15 +80,25 @@ def _fn(module: str, name: str, argtypes, key: str = None):
 
 
 # ----------------------------------------------------------------------------------------------
-def embed_gather(table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor) -> None:
-    """``out[t, :] = table[tokens[t], :]`` widened to 32-bit.  The caller has checked the ids."""
-    _dev(table, tokens, out)
+def embed_gather(table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor,
+                 source: Optional[torch.Tensor] = None, sampled: Optional[torch.Tensor] = None) -> None:
+    """``out[t, :] = table[tokens[t], :]`` widened to 32-bit.  The caller has checked the ids.
+
+    With ``source`` and ``sampled``: where ``source[t] >= 0`` the id is ``sampled[source[t]]``, which an
+    earlier kernel of the stream left on the device."""
+    _dev(table, tokens, out, source, sampled)
     num_tokens, width = out.shape
     _need(table.dim() == 2 and table.shape[1] == width and table.is_contiguous(), "embed_gather: table shape")
     _need(tokens.dtype == torch.int32 and tokens.numel() >= num_tokens and tokens.is_contiguous(), "embed_gather: tokens")
     _need(out.dtype == torch.float32 and out.is_contiguous(), "embed_gather: out must be contiguous float32")
-    fn = _fn("elementwise", "vk_embed_gather", [_p, _i, _p, _p, _i, _i, _p])
-    _status(fn(_ptr(table), _dt(table, "table"), _ptr(tokens), _ptr(out), num_tokens, width, _stream()), "embed_gather")
+    if source is not None:
+        _need(sampled is not None and sampled.dtype == torch.int32 and sampled.is_contiguous(),
+              "embed_gather: sampled must be contiguous int32")
+        _need(source.dtype == torch.int32 and source.numel() >= num_tokens and source.is_contiguous(),
+              "embed_gather: source")
+    fn = _fn("elementwise", "vk_embed_gather", [_p, _i, _p, _p, _p, _p, _i, _i, _i, _p])
+    _status(fn(_ptr(table), _dt(table, "table"), _ptr(tokens), _ptr(source), _ptr(sampled if source is not None else None),
+               _ptr(out), num_tokens, width, table.shape[0], _stream()), "embed_gather")
 
 
 def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor,

@@ -18,6 +18,8 @@ from .base import Part, register_embedding, register_head
 
 
 class Embedding(Part):
+    reads_device_tokens = True  # forward() takes (source, sampled): ids may be read from the device
+
     def __init__(self, spec: PartSpec, prefix: str, runtime):
         super().__init__(spec, prefix, runtime)
         self.vocab = int(spec.params["vocab"])
@@ -32,9 +34,12 @@ class Embedding(Part):
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         self.table = tensors[f"{self.prefix}{self.spec.params['name']}.weight"]
 
-    def forward(self, tokens: torch.Tensor, count: int) -> torch.Tensor:
+    def forward(self, tokens: torch.Tensor, count: int, source: Optional[torch.Tensor] = None,
+                sampled: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Rows of the table for ``tokens``; where ``source`` is not negative the id is read from
+        ``sampled`` on the device instead (see ``kernels.embed_gather``)."""
         out = self.runtime.empty((count, self.width), torch.float32)
-        kernels.embed_gather(self.table, tokens, out)
+        kernels.embed_gather(self.table, tokens, out, source, sampled)
         return out
 
 

@@ -77,6 +77,13 @@ class RowRequest:
     recent: Sequence[int] = ()
 
 
+class PendingSample:
+    """Tokens that have been drawn on the device and are on their way to the host."""
+
+    def __init__(self, count: int, host: torch.Tensor, event):
+        self.count, self.host, self.event = count, host, event
+
+
 class BatchSampler:
     """Samples one token per row of ``[rows, vocab]`` logits on the device.
 
@@ -84,38 +91,66 @@ class BatchSampler:
     consumes exactly one uniform of its request's generator per token, so a request's stream does
     not depend on its company in the batch or on the order of arrival (the invariant of
     crates/vipera-runtime/src/engine.rs:665-670).
+
+    ``launch`` enqueues the work and returns at once, ``collect`` waits for the ids; ``out`` (optional,
+    int32 on the device) is where the ids are left for a next step that reads them there.
     """
 
-    def __init__(self, device):
+    def __init__(self, device, out: Optional[torch.Tensor] = None):
         self.device = torch.device(device)
-        self._staging = None        # pinned host words of the per-row options, reused by every call
-        self._device_words = None   # their place on the device
+        self.out = out
+        # pinned host words of the per-row options and of the ids, two of each used in turn (a launch may
+        # follow before the copies of the one before have run), and the options' place on the device
+        self._options = [None, None]
+        self._ids = [None, None]
+        self._device_words = None
+        self._turn = 0
 
     def sample(self, logits: torch.Tensor, rows: Sequence[RowRequest]) -> List[int]:
+        return self.collect(self.launch(logits, rows))
+
+    def launch(self, logits: torch.Tensor, rows: Sequence[RowRequest]) -> PendingSample:
         count, vocab = logits.shape
         if count != len(rows):
             raise InvalidArgumentError(f"{count} rows of logits for {len(rows)} requests")
         if logits.dtype != torch.float32 or not logits.is_contiguous():
             raise InvalidArgumentError("logits must be contiguous float32")
         self._penalize(logits, rows, vocab)
+        self._turn ^= 1
+        turn = self._turn
         # one pinned staging buffer, one copy: 4-byte columns first, then the 8-byte uniforms
         words = 6 * count
-        if self._staging is None or self._staging.numel() < words:
-            self._staging = torch.empty(max(words, 6 * 64), dtype=torch.int32).pin_memory()
-            self._device_words = torch.empty(self._staging.numel(), dtype=torch.int32, device=self.device)
-        host = self._staging.numpy()
+        if self._options[turn] is None or self._options[turn].numel() < words:
+            self._options[turn] = torch.empty(max(words, 6 * 64), dtype=torch.int32).pin_memory()
+            self._ids[turn] = torch.empty(max(count, 64), dtype=torch.int32).pin_memory()
+        if self._device_words is None or self._device_words.numel() < words:
+            self._device_words = torch.empty(max(words, 6 * 64), dtype=torch.int32, device=self.device)
+        host = self._options[turn].numpy()
         host[0:count].view(np.float32)[:] = [r.params.temperature for r in rows]
         host[count:2 * count] = [r.params.top_k for r in rows]
         host[2 * count:3 * count].view(np.float32)[:] = [r.params.top_p for r in rows]
         host[3 * count:4 * count].view(np.float32)[:] = [r.params.min_p for r in rows]
         host[4 * count:6 * count].view(np.float64)[:] = [0.0 if r.params.greedy else r.rng.next_f64() for r in rows]
         dev = self._device_words
-        dev[:words].copy_(self._staging[:words], non_blocking=True)
-        out = torch.empty(count, dtype=torch.int32, device=self.device)
+        dev[:words].copy_(self._options[turn][:words], non_blocking=True)
+        if self.out is not None:
+            if count > self.out.numel():
+                raise InvalidArgumentError(f"{count} rows to sample, the id buffer holds {self.out.numel()}")
+            out = self.out[:count]
+        else:
+            out = torch.empty(count, dtype=torch.int32, device=self.device)
         kernels.sample(logits, dev[0:count].view(torch.float32), dev[count:2 * count],
                        dev[2 * count:3 * count].view(torch.float32), dev[3 * count:4 * count].view(torch.float32),
                        dev[4 * count:6 * count].view(torch.float64), out)
-        return [int(t) for t in out.cpu().tolist()]
+        ids = self._ids[turn]
+        ids[:count].copy_(out, non_blocking=True)
+        event = torch.cuda.Event()
+        event.record()
+        return PendingSample(count, ids, event)
+
+    def collect(self, pending: PendingSample) -> List[int]:
+        pending.event.synchronize()
+        return pending.host[:pending.count].tolist()
 
     def _penalize(self, logits: torch.Tensor, rows: Sequence[RowRequest], vocab: int) -> None:
         pen_rows: List[int] = []
