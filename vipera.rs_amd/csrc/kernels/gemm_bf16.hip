@@ -7,15 +7,23 @@
 // them as one vector:
 //     lane l, register j of an accumulator  <->  C[token l % 16][column 4 * (l / 16) + j]
 //
-// Two kernels:
-//   gemm_tile    M large (prompts). 128x128 output tile per workgroup of four waves, K in steps of 64
+// Three kernels:
+//   gemm_tile    more than 64 tokens (prompts). An output tile per workgroup (256x256 on sixteen waves
+//                down to 128x128 on four, chosen by how many tiles the shape gives), K in steps of 64
 //                staged through LDS (rows padded to 144 bytes, which spreads the 16-byte reads of 16
 //                rows over all banks), double-buffered, one barrier per step. Workgroups are renumbered
 //                so that those running on one XCD (one L2) work on neighbouring tiles.
-//   gemm_skinny  M <= 64 (decoding). The product is a stream of the weights from HBM: a workgroup owns
-//                16 weight rows, its four waves split K in interleaved spans of 128 and read their span
-//                straight into the instruction's operand layout (no LDS), two spans in flight; the four
-//                partial sums are added in a fixed order.
+//   gemm_skinny  a few tokens (decoding). The product is a stream of the weights from HBM: a workgroup
+//                owns 16 weight rows, its waves split K in interleaved spans of 128 and read their span
+//                straight into the instruction's operand layout (no LDS); the waves' partial sums are
+//                added in a fixed order.
+//   gemm_mid     up to 64 tokens. The same stream of weights, with the activations of a 256-wide chunk
+//                of K fetched once per workgroup into LDS; K may be split over workgroups, whose partial
+//                sums a second kernel adds in a fixed order.
+// The two streaming kernels read through buffer descriptors, so that no load sits behind a branch, and
+// rotate their operand register sets at compile time (pipeline.h): a use waits for exactly its own
+// loads and the loads of the next spans stay in flight. The gated epilogue of gemm_tile and gemm_mid
+// turns the fused gate/up product into up * silu(gate).
 // Every sum has one fixed order for a given shape.
 //
 // Reference for what is computed: crates/vipera-backend-cpu/src/model.rs:1005-1031 (batched products,
@@ -379,114 +387,6 @@ int launch_skinny(const __bf16* A, const __bf16* W, const float* bias, TC* C, in
 }
 
 // ---------------------------------------------------------------------------------------------
-// M <= 16, activations stationary. A workgroup owns a range of weight rows and one slice of K
-// (SLICE_SPANS * 128 wide). Each wave loads the slice of the activations once into registers and then
-// streams the 16-row weight tiles of the range through them: no LDS, no barrier in the loop, the next
-// tile's loads in flight while the current one is multiplied. The slices' partial sums go to a
-// workspace, [slice, M, N] floats; the workgroup that finishes a row range last (an atomic counter per
-// range says who) adds the slices in ascending order, applies the epilogue and resets the counter. The
-// sum has one fixed order whoever is last. Workgroups of one row range run on different XCDs, whose L2
-// caches do not see each other's lines: the partial sums are therefore written and read with device-scope
-// accesses (they go through to memory), the writers wait for their stores to complete before the counter
-// is bumped, and no cache-wide fence is needed (one per workgroup would flush the L2 a thousand times).
-constexpr int SLICE_SPANS = 4;
-constexpr int SLICE_K = SLICE_SPANS * SPAN;
-
-template <typename TC, bool ACCUMULATE>
-__global__ __launch_bounds__(256) void gemm_stationary_kernel(const __bf16* __restrict__ A,
-                                                              const __bf16* __restrict__ W,
-                                                              const float* __restrict__ bias, TC* __restrict__ C,
-                                                              float* __restrict__ partial,
-                                                              int* __restrict__ counters, int M, int N, int K,
-                                                              long long lda, long long ldc, int rows_per_group,
-                                                              int vector_ok) {
-  __shared__ int is_last;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int lr = lane & 15, lg = lane >> 4;
-  const int group = blockIdx.x, slice = blockIdx.y, slices = gridDim.y;
-  const int row0 = group * rows_per_group, row_end = min(N, row0 + rows_per_group);
-  const int k0 = slice * SLICE_K;
-
-  // the slice of the activations: lane (m = lr, g = lg), step i holds A[m][k0 + 32 i + 8 g .. + 8]
-  bf16x8 act[SLICE_SPANS * 4];
-  {
-    const bool a_ok = lr < M;
-    const __bf16* ap = A + (size_t)(a_ok ? lr : 0) * lda + k0 + lg * 8;
-#pragma unroll
-    for (int i = 0; i < SLICE_SPANS * 4; ++i)
-      act[i] = (a_ok && k0 + i * 32 + lg * 8 < K) ? *(const bf16x8*)(ap + i * 32) : zero8();
-  }
-  const int tiles = (row_end - row0 + 15) / 16;
-  bf16x8 w_cur[SLICE_SPANS * 4], w_next[SLICE_SPANS * 4];
-  auto load_tile = [&](int tile, bf16x8* dst) {
-    const int wrow = min(row0 + tile * 16 + lr, N - 1);
-    const __bf16* wp = W + (size_t)wrow * K + k0 + lg * 8;
-#pragma unroll
-    for (int i = 0; i < SLICE_SPANS * 4; ++i)
-      dst[i] = (tile < tiles && k0 + i * 32 + lg * 8 < K) ? *(const bf16x8*)(wp + i * 32) : zero8();
-  };
-  load_tile(wave, w_cur);
-  for (int tile = wave; tile < tiles; tile += 4) {
-    load_tile(tile + 4, w_next);
-    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int i = 0; i < SLICE_SPANS * 4; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_cur[i], act[i], acc, 0, 0, 0);
-    const int n = row0 + tile * 16 + lg * 4;
-    if (lr < M && n < N) {
-      float* dst = partial + ((size_t)slice * M + lr) * N + n;
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        if (n + j < N) __hip_atomic_store(dst + j, acc[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-#pragma unroll
-    for (int i = 0; i < SLICE_SPANS * 4; ++i) w_cur[i] = w_next[i];
-  }
-  // who is last for this row range? every store above has completed before the counter moves
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-  __syncthreads();
-  if (tid == 0) {
-    const int before = __hip_atomic_fetch_add(&counters[group], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    is_last = before == slices - 1;
-  }
-  __syncthreads();
-  if (!is_last) return;
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-  const int width = row_end - row0;
-  for (int idx = tid * 4; idx < M * ((width + 3) & ~3); idx += 256 * 4) {
-    const int per_row = (width + 3) & ~3;
-    const int m = idx / per_row, n = row0 + (idx - m * per_row);
-    if (n >= N) continue;
-    f32x4 sum = {0.f, 0.f, 0.f, 0.f};
-    for (int sl = 0; sl < slices; ++sl) {
-      const float* src = partial + ((size_t)sl * M + m) * N + n;
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        if (n + j < N) sum[j] += __hip_atomic_load(src + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    store4<TC, ACCUMULATE>(C, ldc, m, n, M, N, sum, bias, vector_ok != 0);
-  }
-  if (tid == 0) __hip_atomic_store(&counters[group], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next product
-}
-
-template <typename TC, bool ACC>
-int launch_stationary(const __bf16* A, const __bf16* W, const float* bias, TC* C, float* partial, int* counters,
-                      int max_groups, long long partial_floats, int M, int N, int K, long long lda, long long ldc,
-                      int vector_ok, hipStream_t s) {
-  const int slices = (K + SLICE_K - 1) / SLICE_K;
-  // about a thousand workgroups, at least one tile per wave
-  long long rows = ((long long)N * slices / 1024 + 63) / 64 * 64;
-  if (rows < 64) rows = 64;
-  if (rows > 512) rows = 512;
-  const int groups = (int)((N + rows - 1) / rows);
-  if (groups > max_groups || (long long)slices * M * N > partial_floats || slices > 65535) return VK_UNSUPPORTED_SIZE;
-  dim3 grid(groups, slices);
-  gemm_stationary_kernel<TC, ACC><<<grid, 256, 0, s>>>(A, W, bias, C, partial, counters, M, N, K, lda, ldc, (int)rows,
-                                                         vector_ok);
-  VK_LAUNCH_CHECK();
-  return 0;
-}
-
-// ---------------------------------------------------------------------------------------------
 // M <= 64, activations shared through LDS. A workgroup owns 64 * RT weight rows (16 * RT per wave)
 // and a range of K; all four waves walk that range together in chunks of 256. A chunk's activations
 // (16 * CB tokens x 256) are fetched once per workgroup into LDS, double-buffered, one barrier per
@@ -782,34 +682,6 @@ extern "C" int vk_gemm_bf16(const void* A, const void* W, const float* bias, voi
   if (c_dtype == DT_BF16)
     return skinny ? launch_skinny<__bf16, false>(a, w, bias, (__bf16*)C, M, N, K, lda, ldc, vector_ok, skinny_shape, s)
                   : launch_tile<__bf16, false>(a, w, bias, (__bf16*)C, M, N, K, lda, ldc, vector_ok, s);
-  return VK_BAD_ARGUMENT;
-}
-
-// The same product for M <= 16 with the activations held in registers and K split over workgroups.
-// partial: workspace of `partial_floats` floats, at least ceil(K / 512) * M * N. counters: `max_groups`
-// ints that are zero before the first call; every call leaves them zero. Calls that share a workspace
-// must not overlap (one stream).
-extern "C" int vk_gemm_bf16_stationary(const void* A, const void* W, const float* bias, void* C, int c_dtype, int M,
-                                       int N, int K, long long lda, long long ldc, int accumulate, float* partial,
-                                       long long partial_floats, int* counters, int max_groups, void* stream) {
-  if (M <= 0 || N <= 0) return 0;
-  if (M > 16) return VK_UNSUPPORTED_SIZE;
-  if (K <= 0 || (K & 7) || (lda & 7) || lda < K || ldc < N) return VK_BAD_ARGUMENT;
-  if (((uintptr_t)A & 15) || ((uintptr_t)W & 15) || ((uintptr_t)partial & 15) || !partial || !counters) return VK_BAD_ARGUMENT;
-  if (accumulate && c_dtype != DT_F32) return VK_BAD_ARGUMENT;
-  const int elem = c_dtype == DT_F32 ? 4 : 2;
-  const int vector_ok = ((ldc & 3) == 0 && ((uintptr_t)C & (4 * elem - 1)) == 0 &&
-                         (bias == nullptr || ((uintptr_t)bias & 15) == 0)) ? 1 : 0;
-  hipStream_t s = (hipStream_t)stream;
-  const __bf16* a = (const __bf16*)A;
-  const __bf16* w = (const __bf16*)W;
-  if (c_dtype == DT_F32) {
-    if (accumulate)
-      return launch_stationary<float, true>(a, w, bias, (float*)C, partial, counters, max_groups, partial_floats, M, N, K, lda, ldc, vector_ok, s);
-    return launch_stationary<float, false>(a, w, bias, (float*)C, partial, counters, max_groups, partial_floats, M, N, K, lda, ldc, vector_ok, s);
-  }
-  if (c_dtype == DT_BF16)
-    return launch_stationary<__bf16, false>(a, w, bias, (__bf16*)C, partial, counters, max_groups, partial_floats, M, N, K, lda, ldc, vector_ok, s);
   return VK_BAD_ARGUMENT;
 }
 

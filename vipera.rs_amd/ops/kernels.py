@@ -363,49 +363,19 @@ def attn_bf16_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
             "attn_bf16_decode")
 
 
-_STATIONARY_SLICE = 512      # k per slice of the activation-stationary product (SLICE_K in gemm_bf16.hip)
-_STATIONARY_GROUPS = 8192    # counters kept per device
 _workspaces = {}
 
 
-def _stationary_workspace(device: torch.device, floats: int):
-    """Partial-sum workspace and counters of a device; grown when a product needs more, never shrunk.
+def _split_k_workspace(device: torch.device, floats: int) -> torch.Tensor:
+    """Partial-sum workspace of a device; grown when a product needs more, never shrunk.
 
-    Every product on the device shares them, which is safe because products run on one stream.
+    Every product on the device shares it, which is safe because products run on one stream.
     """
     entry = _workspaces.get(device)
-    if entry is None or entry[0].numel() < floats:
-        counters = entry[1] if entry else torch.zeros(_STATIONARY_GROUPS, dtype=torch.int32, device=device)
-        entry = (torch.empty(floats, dtype=torch.float32, device=device), counters)
+    if entry is None or entry.numel() < floats:
+        entry = torch.empty(floats, dtype=torch.float32, device=device)
         _workspaces[device] = entry
     return entry
-
-
-def gemm_bf16_stationary(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
-                         accumulate: bool = False) -> None:
-    """``out (+)= a @ w.T + bias`` for at most 16 rows of ``a``: activations held in registers, K split
-    over workgroups, the slices' partial sums added in a fixed order by the last workgroup of a row range."""
-    _dev(a, w, bias, out)
-    _need(a.dim() == 2 and w.dim() == 2 and out.dim() == 2, "gemm: operands must be matrices")
-    m, k = a.shape
-    n = w.shape[0]
-    _need(m <= 16, "gemm_bf16_stationary takes at most 16 rows")
-    _need(w.shape[1] == k and out.shape == (m, n), f"gemm: shapes {tuple(a.shape)} x {tuple(w.shape)}^T -> {tuple(out.shape)}")
-    _need(gemm_bf16_supported(a, w, out), "gemm_bf16: operands must be bfloat16, K a multiple of 8, rows 16-byte aligned")
-    if bias is not None:
-        _need(bias.dtype == torch.float32 and bias.numel() == n and bias.is_contiguous(), "gemm: bias must be float32 [n]")
-    if accumulate:
-        _need(out.dtype == torch.float32, "gemm: accumulation needs a float32 output")
-    lda = a.stride(0) if m > 1 else max(a.stride(0), k)
-    lda = lda if lda % 8 == 0 else k
-    ldc = out.stride(0) if m > 1 else max(out.stride(0), n)
-    _need(ldc >= n, "gemm: out's row stride")
-    slices = (k + _STATIONARY_SLICE - 1) // _STATIONARY_SLICE
-    partial, counters = _stationary_workspace(a.device, slices * 16 * n)
-    fn = _fn("gemm_bf16", "vk_gemm_bf16_stationary",
-             [_p, _p, _p, _p, _i, _i, _i, _i, _ll, _ll, _i, _p, _ll, _p, _i, _p])
-    _status(fn(_ptr(a), _ptr(w), _ptr(bias), _ptr(out), _dt(out, "out"), m, n, k, lda, ldc, 1 if accumulate else 0,
-               _ptr(partial), partial.numel(), _ptr(counters), counters.numel(), _stream()), "gemm_bf16_stationary")
 
 
 def gemm_bf16_mid(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
@@ -430,7 +400,7 @@ def gemm_bf16_mid(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor]
     _need(ldc >= n, "gemm: out's row stride")
     partial = None
     if ranges > 1:
-        partial, _ = _stationary_workspace(a.device, ranges * 64 * n)
+        partial = _split_k_workspace(a.device, ranges * 64 * n)
     fn = _fn("gemm_bf16", "vk_gemm_bf16_mid", [_p, _p, _p, _p, _i, _i, _i, _i, _ll, _ll, _i, _i, _i, _p, _ll, _p])
     _status(fn(_ptr(a), _ptr(w), _ptr(bias), _ptr(out), _dt(out, "out"), m, n, k, lda, ldc, 1 if accumulate else 0,
                int(ranges), int(rows_per_wave), _ptr(partial), partial.numel() if partial is not None else 0, _stream()),

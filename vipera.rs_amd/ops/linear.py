@@ -18,8 +18,6 @@ import torch
 
 from . import kernels
 
-STATIONARY = False   # the register-stationary split-K product is measured slower than the others; kept for tests
-
 
 def mid_plan(m: int, n: int, k: int) -> Tuple[int, int]:
     """``(ranges of K, 16-row tiles per wave)`` for the LDS-shared kernel."""
@@ -39,10 +37,7 @@ def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: 
         m, k = a.shape
         n = w.shape[0]
         if m > 64 or m <= 4 or (m <= 16 and n < 16_384 and k < 8_192):
-            if m <= 16 and STATIONARY:
-                kernels.gemm_bf16_stationary(a, w, bias, out, accumulate)
-            else:
-                kernels.gemm_bf16(a, w, bias, out, accumulate)
+            kernels.gemm_bf16(a, w, bias, out, accumulate)
         else:
             ranges, rows_per_wave = mid_plan(m, n, k)
             kernels.gemm_bf16_mid(a, w, bias, out, accumulate, ranges, rows_per_wave)
