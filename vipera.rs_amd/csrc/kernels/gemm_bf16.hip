@@ -367,9 +367,6 @@ int launch_skinny_cb(const __bf16* A, const __bf16* W, const float* bias, TC* C,
   switch (shape) {
     case 1: return launch_skinny_as<CB, 1, 4, TC, ACC>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, s);
     case 2: return launch_skinny_as<CB, 2, 4, TC, ACC>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, s);
-    case 3: return launch_skinny_as<CB, 1, 16, TC, ACC>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, s);
-    case 4: return launch_skinny_as<CB, 1, 8, TC, ACC>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, s);
-    case 5: return launch_skinny_as<CB, 2, 8, TC, ACC>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, s);
   }
   return VK_BAD_ARGUMENT;
 }
@@ -629,7 +626,7 @@ int launch_tile_as(const __bf16* A, const __bf16* W, const float* bias, TC* C, i
   return 0;
 }
 
-int g_tile_config = -1;  // -1: chosen by shape; 0..5 force a tiling (vk_gemm_bf16_tile_config, for measurements)
+int g_tile_config = -1;  // -1: chosen by shape; 0, 2, 3, 4 force a tiling (vk_gemm_bf16_tile_config, for measurements)
 
 // Measured on the 7B shapes at 2,048 tokens: 256x256 tiles with sixteen waves are fastest when there are
 // enough of them to fill the GPU (about 1 PFLOP/s), 256x128 with eight waves otherwise; few tokens keep
@@ -644,11 +641,9 @@ template <typename TC, bool ACC, bool GATED = false>
 int launch_tile(const __bf16* A, const __bf16* W, const float* bias, TC* C, int M, int N, int K, long long lda,
                 long long ldc, int vector_ok, hipStream_t s) {
   switch (g_tile_config >= 0 ? g_tile_config : choose_tile_config(M, N)) {
-    case 1: return launch_tile_as<128, 128, 2, 4, TC, ACC, GATED>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, s);
     case 2: return launch_tile_as<256, 128, 4, 2, TC, ACC, GATED>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, s);
     case 3: return launch_tile_as<128, 256, 2, 4, TC, ACC, GATED>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, s);
     case 4: return launch_tile_as<256, 256, 4, 4, TC, ACC, GATED>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, s);
-    case 5: return launch_tile_as<256, 256, 2, 4, TC, ACC, GATED>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, s);
     default: return launch_tile_as<128, 128, 2, 2, TC, ACC, GATED>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, s);
   }
 }
@@ -657,7 +652,7 @@ int launch_tile(const __bf16* A, const __bf16* W, const float* bias, TC* C, int 
 // A, W: bfloat16. c_dtype: 0 float, 1 bfloat16. accumulate needs a float C. Requirements (checked here):
 // K a multiple of 8 and lda a multiple of 8 (16-byte chunks); A and W 16-byte aligned.
 // `skinny_limit`: M at or below it takes the weight-streaming kernel (at most 64).
-// `skinny_shape`: 0 lets the launcher choose rows per wave and waves per workgroup; 1..5 force a choice.
+// `skinny_shape`: 0 lets the launcher choose the row tiles per wave; 1 or 2 force one or two.
 extern "C" int vk_gemm_bf16(const void* A, const void* W, const float* bias, void* C, int c_dtype, int M, int N, int K,
                             long long lda, long long ldc, int accumulate, int skinny_limit, int skinny_shape, void* stream) {
   if (M <= 0 || N <= 0) return 0;
