@@ -42,11 +42,24 @@ __device__ __forceinline__ bf16x8 zero8() {
   return z;
 }
 
+// Position -> (page index, slot in the page). Page sizes are almost always powers of two: then a shift
+// and a mask stand for the division, which would otherwise cost some thirty instructions per use, on
+// the path to every load address.
+struct PageSize {
+  int size, shift;  // shift < 0: not a power of two
+  __device__ __forceinline__ explicit PageSize(int block_size)
+      : size(block_size), shift((block_size & (block_size - 1)) == 0 ? __ffs(block_size) - 1 : -1) {}
+  __device__ __forceinline__ int page(int p) const { return shift >= 0 ? p >> shift : p / size; }
+  __device__ __forceinline__ int slot(int p) const { return shift >= 0 ? p & (size - 1) : p % size; }
+};
+
 struct CacheView {
   const __bf16* k;
   const __bf16* v;
   const int* table;  // this request's row of the block table
-  int table_width, block_size, kv_heads, hd, kvh;
+  int table_width;
+  PageSize ps;
+  int kv_heads, hd, kvh;
   int page0, pages;  // REGS: lane i of `pages` holds the id of page page0 + i of the request
 };
 
@@ -55,7 +68,7 @@ struct CacheView {
 // K and V reads can be issued.
 template <bool REGS>
 __device__ __forceinline__ int page_of(const CacheView& cv, int p) {
-  const int index = p / cv.block_size;
+  const int index = cv.ps.page(p);
   if (REGS) return __shfl(cv.pages, (index - cv.page0) & 63, 64);
   return cv.table[min(max(index, 0), cv.table_width - 1)];
 }
@@ -76,12 +89,12 @@ struct StepOperands {
 template <bool REGS>
 __device__ __forceinline__ void load_step(int kb, int begin, int end, const CacheView& cv, StepOperands& r) {
   const int lane = threadIdx.x & 63, lr = lane & 15, lg = lane >> 4;
-  const int bs = cv.block_size, hd = cv.hd;
+  const int bs = cv.ps.size, hd = cv.hd;
 #pragma unroll
   for (int sub = 0; sub < 2; ++sub) {
     const int p = min(max(kb + sub * 16 + lr, begin), end - 1);
     const int page = max(page_of<REGS>(cv, p), 0);
-    const __bf16* row = cv.k + (((size_t)page * cv.kv_heads + cv.kvh) * bs + (p % bs)) * hd;
+    const __bf16* row = cv.k + (((size_t)page * cv.kv_heads + cv.kvh) * bs + cv.ps.slot(p)) * hd;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const int dim = ks * 32 + lg * 8;
@@ -94,7 +107,7 @@ __device__ __forceinline__ void load_step(int kb, int begin, int end, const Cach
     // groups of four positions start at multiples of 4 and lie in one page (4 divides the page size)
     const int p = min(max(kb + half * 16 + lg * 4, begin & ~3), (end - 1) & ~3);
     const int page = max(page_of<REGS>(cv, p), 0);
-    vrow[half] = cv.v + (((size_t)page * cv.kv_heads + cv.kvh) * hd) * bs + (p % bs);
+    vrow[half] = cv.v + (((size_t)page * cv.kv_heads + cv.kvh) * hd) * bs + cv.ps.slot(p);
   }
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) {
@@ -224,6 +237,7 @@ __global__ __launch_bounds__(PT_THREADS) void attn_prefill_kernel(
   const int first_pos = entry_first_pos[entry];
   const int* table = block_table + (size_t)entry * table_width;
   const int bs = block_size;
+  const PageSize ps(block_size);
 
   // the workgroup's range of positions
   const int tile_cols = min(PT_TOKENS, count - tile_off);
@@ -257,9 +271,9 @@ __global__ __launch_bounds__(PT_THREADS) void attn_prefill_kernel(
     for (int i = 0; i < PT_PER_THREAD; ++i) {
       const int id = tid + PT_THREADS * i;
       const int pk = p0 + id / (HDP / 8);
-      k_page[i] = (id < PT_PIECES && pk >= begin && pk < end) ? table[pk / bs] : -1;
+      k_page[i] = (id < PT_PIECES && pk >= begin && pk < end) ? table[ps.page(pk)] : -1;
       const int pv = p0 + (id % (PT_KV / 8)) * 8;  // eight positions of one page (8 divides the page size)
-      v_page[i] = (id < PT_PIECES && pv + 7 >= begin && pv < end) ? table[pv / bs] : -1;
+      v_page[i] = (id < PT_PIECES && pv + 7 >= begin && pv < end) ? table[ps.page(pv)] : -1;
     }
   };
   auto fetch = [&](int p0) {
@@ -269,12 +283,12 @@ __global__ __launch_bounds__(PT_THREADS) void attn_prefill_kernel(
       const int r = id / (HDP / 8), ck = id % (HDP / 8);
       const int pk = p0 + r;
       k_stage[i] = (k_page[i] >= 0 && ck * 8 < hd)
-                       ? *(const bf16x8*)(k_cache + (((size_t)k_page[i] * kv_heads + kvh) * bs + (pk % bs)) * hd + ck * 8)
+                       ? *(const bf16x8*)(k_cache + (((size_t)k_page[i] * kv_heads + kvh) * bs + ps.slot(pk)) * hd + ck * 8)
                        : zero8();
       const int d = id / (PT_KV / 8), cv = id % (PT_KV / 8);
       const int pv = p0 + cv * 8;
       v_stage[i] = (v_page[i] >= 0 && d < hd)
-                       ? *(const bf16x8*)(v_cache + (((size_t)v_page[i] * kv_heads + kvh) * hd + d) * bs + (pv % bs))
+                       ? *(const bf16x8*)(v_cache + (((size_t)v_page[i] * kv_heads + kvh) * hd + d) * bs + ps.slot(pv))
                        : zero8();
     }
   };
@@ -418,11 +432,12 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void at
   }
   bf16x8 qf[KS];
   load_q(col_ok ? q + (size_t)token * q_stride + (size_t)h * hd : nullptr, hd, qf);
-  CacheView cv{k_cache, v_cache, block_table + (size_t)entry * table_width, table_width, block_size,
-               kv_heads, hd, kvh, begin / block_size, -1};
+  const PageSize ps(block_size);
+  CacheView cv{k_cache, v_cache, block_table + (size_t)entry * table_width, table_width, ps,
+               kv_heads, hd, kvh, ps.page(begin), -1};
   if (REGS) {
     const int index = cv.page0 + lane;
-    if (index <= (end - 1) / block_size && index < table_width) cv.pages = cv.table[index];
+    if (index <= ps.page(end - 1) && index < table_width) cv.pages = cv.table[index];
   }
   f32x4 o[DT];
 #pragma unroll
