@@ -67,6 +67,10 @@ def main() -> int:
     parser.add_argument("--prefill-tokens", type=int, default=2048)
     parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     parser.add_argument("--block-size", type=int, default=16)
+    parser.add_argument("--serving", action="store_true",
+                        help="instead of the headline measurement: a continuous batch of 64 requests, prompts of 128 to "
+                             "8,192 random tokens in portions of 512, 256 new tokens each (the 1.5B workload; use with "
+                             "--shape 1.5b --ctx 32768)")
     parser.add_argument("--in-turn", action="store_true",
                         help="wait for a step's tokens on the host before the next step is launched")
     args = parser.parse_args()
@@ -99,6 +103,8 @@ def main() -> int:
     torch.cuda.synchronize()
     log(f"random weights for {args.layers} layers on the device in {time.perf_counter() - started:.1f} s")
 
+    if args.serving:
+        return serving(args, config, runtime, model, shape_name, layers_full, dtype_key)
     batches = [args.batch] + [int(b) for b in args.points.split(",") if b.strip()]
     largest = max(batches)
     ctx = args.ctx
@@ -215,6 +221,58 @@ def main() -> int:
         "points_ms": {f"decode_b{b}": round(r["ms"], 4) for b, r in results.items() if b != args.batch},
     }
     print(json.dumps(line), flush=True)
+    return 0
+
+
+def serving(args, config, runtime, model, shape_name, layers_full, dtype_key) -> int:
+    """Continuous batching under load: every request is queued at once, prompts run in portions of 512 beside the
+    decode tokens of the requests that are further on, and the run ends when all have their 256 new tokens."""
+    import torch
+
+    from vipera_rs_amd import Engine
+    from vipera_rs_amd.engine.runner import ModelRunner
+
+    requests, new_tokens, chunk, budget = 64, 256, 512, 2048
+    gen = torch.Generator().manual_seed(1)
+    lengths = torch.randint(128, 8193, (requests,), generator=gen).tolist()
+    prompts = [torch.randint(0, config.vocab_size, (n,), generator=gen).tolist() for n in lengths]
+    pages = sum((n + new_tokens + args.block_size - 1) // args.block_size + 1 for n in lengths)
+    runner = ModelRunner(model, runtime, args.block_size, pages, requests + 1, use_graphs=True, max_context=args.ctx)
+    engine = Engine(None, runner=runner, max_num_seqs=requests, max_num_batched_tokens=budget, chunk_size=chunk,
+                    max_model_len=args.ctx, pipelined=not args.in_turn)
+    # a short run first: kernel modules are compiled and loaded, decode graphs of the small buckets captured
+    engine.generate([prompts[0][:600], prompts[1][:300]], 8)
+    for prompt in prompts:
+        engine.add_request(prompt, new_tokens)
+    torch.cuda.synchronize()
+    started = time.perf_counter()
+    steps = generated = 0
+    last = started
+    while engine.has_work():
+        report = engine.step()
+        steps += 1
+        generated += len(report.tokens)
+        if time.perf_counter() - last > 20:
+            log(f"  serving: {steps} steps, {generated} tokens generated, {engine.scheduler.num_waiting} requests waiting")
+            last = time.perf_counter()
+    torch.cuda.synchronize()
+    seconds = time.perf_counter() - started
+    assert generated == requests * new_tokens and runner.cache.live_requests() == 0
+    prompt_tokens = sum(lengths)
+    log(f"serving: {requests} requests, {prompt_tokens} prompt tokens and {generated} new tokens in {seconds:.2f} s "
+        f"over {steps} steps; {engine.stats()['preemptions']} preemptions")
+    print(json.dumps({
+        "metric": "tokens per second (prompt and generated) of a continuous batch of 64 requests",
+        "value": round((prompt_tokens + generated) / seconds, 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps,
+        "warmup": 0, "ms_per_step": round(seconds / steps * 1e3, 3), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": dtype_key,
+        "data": "synthetic: seeded random weights N(0, 0.02) and uniform-random token ids",
+        "config": {"model": shape_name, "layers": args.layers, "layers_full": layers_full, "requests": requests,
+                   "prompt_tokens": prompt_tokens, "new_tokens_each": new_tokens, "chunk_size": chunk,
+                   "max_num_batched_tokens": budget, "seq_len": args.ctx, "block_size": args.block_size,
+                   "steps_launched_ahead": not args.in_turn},
+        "generated_per_second": round(generated / seconds, 1), "seconds": round(seconds, 3),
+    }), flush=True)
     return 0
 
 

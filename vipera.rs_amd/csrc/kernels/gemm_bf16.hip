@@ -133,7 +133,12 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_tile_kernel(const __bf16* _
                                                                    const __bf16* __restrict__ W,
                                                                    const float* __restrict__ bias, TC* __restrict__ C,
                                                                    int M, int N, int K, long long lda, long long ldc,
-                                                                   int tiles_m, int tiles_n, int vector_ok) {
+                                                                   int tiles_m, int tiles_n, int vector_ok,
+                                                                   int k_per_range, long long range_stride) {
+  // gridDim.y > 1: K is split into ranges of k_per_range (a multiple of 64); range r writes its partial
+  // sums to C + r * range_stride and a second kernel adds the ranges
+  const int k_begin = blockIdx.y * k_per_range, k_end = min(K, k_begin + k_per_range);
+  C += (size_t)blockIdx.y * range_stride;
   constexpr int THREADS = WM * WN * 64;
   constexpr int TM = BM / WM / 16, TN = BN / WN / 16;
   constexpr int A_PIECES = BM * 8 / THREADS, W_PIECES = BN * 8 / THREADS;  // 16-byte pieces per thread and step
@@ -181,13 +186,13 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_tile_kernel(const __bf16* _
     for (int i = 0; i < A_PIECES; ++i) ra[i] = a_view.load(a_off[i] + (unsigned)k0 * 2);
 #pragma unroll
     for (int i = 0; i < W_PIECES; ++i) rw[i] = w_view.load(w_off[i] + (unsigned)k0 * 2);
-    if (k0 + BK > K) {  // the last step of a K that is no multiple of 64: pieces past K are zero
+    if (k0 + BK > k_end) {  // the last step of a range that is no multiple of 64 long: pieces past its end are zero
 #pragma unroll
       for (int i = 0; i < A_PIECES; ++i)
-        if (k0 + ((tid + THREADS * i) & 7) * 8 >= K) ra[i] = zero8();
+        if (k0 + ((tid + THREADS * i) & 7) * 8 >= k_end) ra[i] = zero8();
 #pragma unroll
       for (int i = 0; i < W_PIECES; ++i)
-        if (k0 + ((tid + THREADS * i) & 7) * 8 >= K) rw[i] = zero8();
+        if (k0 + ((tid + THREADS * i) & 7) * 8 >= k_end) rw[i] = zero8();
     }
   };
   auto store_lds = [&](int buf) {
@@ -203,13 +208,13 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_tile_kernel(const __bf16* _
     }
   };
 
-  const int steps = (K + BK - 1) / BK;
-  load_global(0);
+  const int steps = (k_end - k_begin + BK - 1) / BK;
+  load_global(k_begin);
   store_lds(0);
   __syncthreads();
   for (int s = 0; s < steps; ++s) {
     const int buf = s & 1;
-    if (s + 1 < steps) load_global((s + 1) * BK);
+    if (s + 1 < steps) load_global(k_begin + (s + 1) * BK);
     const __bf16* tA = sA + buf * BM * ROW + (wm * TM * 16 + lr) * ROW + lg * 8;
     const __bf16* tW = sW + buf * BN * ROW + (wn * TN * 16 + lr) * ROW + lg * 8;
 #pragma unroll
@@ -608,43 +613,104 @@ int launch_mid(const __bf16* A, const __bf16* W, const float* bias, TC* C, float
 
 template <int BM, int BN, int WM, int WN, typename TC, bool ACC, bool GATED>
 int launch_tile_as(const __bf16* A, const __bf16* W, const float* bias, TC* C, int M, int N, int K, long long lda,
-                   long long ldc, int vector_ok, hipStream_t s) {
-  static bool configured = false;
+                   long long ldc, int vector_ok, int ranges, float* partial, hipStream_t s) {
   constexpr int lds_bytes = 2 * (BM + BN) * ROW * (int)sizeof(__bf16);
-  auto kernel = gemm_tile_kernel<BM, BN, WM, WN, TC, ACC, GATED>;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-    if (e != hipSuccess) return (int)e;
-    configured = true;
-  }
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
   const long long total = (long long)tiles_m * tiles_n;
   const long long grid = (total + XCDS - 1) / XCDS * XCDS;
   if (grid > 0x7fffffffLL) return VK_UNSUPPORTED_SIZE;
-  kernel<<<(int)grid, WM * WN * 64, lds_bytes, s>>>(A, W, bias, C, M, N, K, lda, ldc, tiles_m, tiles_n, vector_ok);
-  VK_LAUNCH_CHECK();
+  if (ranges <= 1 || GATED) {
+    static bool configured = false;
+    auto kernel = gemm_tile_kernel<BM, BN, WM, WN, TC, ACC, GATED>;
+    if (!configured) {
+      hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+      if (e != hipSuccess) return (int)e;
+      configured = true;
+    }
+    kernel<<<(int)grid, WM * WN * 64, lds_bytes, s>>>(A, W, bias, C, M, N, K, lda, ldc, tiles_m, tiles_n, vector_ok, K,
+                                                      0);
+    VK_LAUNCH_CHECK();
+    return 0;
+  }
+  // K split over workgroups: float partial sums [range, M, N], then the ranges are added in ascending order
+  if constexpr (!GATED) {
+    static bool configured_partial = false;
+    auto kernel = gemm_tile_kernel<BM, BN, WM, WN, float, false, false>;
+    if (!configured_partial) {
+      hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+      if (e != hipSuccess) return (int)e;
+      configured_partial = true;
+    }
+    const int k_per_range = ((K + ranges - 1) / ranges + BK - 1) / BK * BK;
+    const int used = (K + k_per_range - 1) / k_per_range;
+    kernel<<<dim3((unsigned)grid, used), WM * WN * 64, lds_bytes, s>>>(A, W, nullptr, partial, M, N, K, lda, N, tiles_m,
+                                                                       tiles_n, (N & 3) == 0 ? 1 : 0, k_per_range,
+                                                                       (long long)M * N);
+    VK_LAUNCH_CHECK();
+    const long long threads = (long long)M * ((N + 3) / 4);
+    gemm_reduce_kernel<TC, ACC><<<(int)((threads + 255) / 256), 256, 0, s>>>(partial, bias, C, M, N, ldc, used, vector_ok);
+    VK_LAUNCH_CHECK();
+  }
   return 0;
 }
 
-int g_tile_config = -1;  // -1: chosen by shape; 0, 2, 3, 4 force a tiling (vk_gemm_bf16_tile_config, for measurements)
+int g_tile_config = -1;  // -1: chosen by shape; else 10 * ranges + tiling (0, 2, 3, 4) forces a plan, for measurements
 
-// Measured on the 7B shapes at 2,048 tokens: 256x256 tiles with sixteen waves are fastest when there are
-// enough of them to fill the GPU (about 1 PFLOP/s), 256x128 with eight waves otherwise; few tokens keep
-// the token side of the tile at 128.
-int choose_tile_config(int M, int N) {
-  if (M <= 128) return N >= 8192 ? 3 : 0;
-  const long long big = (long long)((M + 255) / 256) * ((N + 255) / 256);
-  return big >= 128 ? 4 : 2;
+// Which tiling, and into how many ranges K is split: the pair with the shortest estimated time. A full GPU
+// of 256x256 tiles on sixteen waves runs at about 1 PFLOP/s (measured on the 7B shapes at 2,048 tokens),
+// 256x128 and 128x256 on eight waves at 0.8, 128x128 on four at 0.75 of that; workgroups run in whole
+// rounds of one per CU (two for the small tile, whose LDS lets two share a CU), so a launch that fills
+// the last round badly loses that share. Splitting K multiplies the workgroups, at the price of writing
+// and re-reading float partial sums (they mostly stay in the caches: about 6 TB/s) and one more launch;
+// each range keeps at least 512 of K. The estimate ranks the plans as measurements at 256 to 2,048 tokens do. Few tokens keep the token side of the tile at
+// 128. Ties go to the larger tile and to fewer ranges.
+struct TilePlan { int config, ranges; };
+int g_compute_units = 0;
+TilePlan choose_tile_plan(int M, int N, int K, long long partial_floats) {
+  if (g_compute_units == 0) {
+    int device = 0, count = 0;
+    if (hipGetDevice(&device) != hipSuccess ||
+        hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || count <= 0)
+      count = 256;
+    g_compute_units = count;
+  }
+  struct Tiling { int config, tokens, rows, resident; double speed; };
+  static const Tiling tilings[] = {{4, 256, 256, 1, 1.0}, {2, 256, 128, 1, 0.8}, {3, 128, 256, 1, 0.8}, {0, 128, 128, 2, 0.75}};
+  TilePlan best{0, 1};
+  double best_time = 1e30;
+  const double flops = 2.0 * M * N * (double)K, output_bytes = 4.0 * M * N;
+  for (const Tiling& t : tilings) {
+    if (M <= 128 && t.tokens > 128) continue;
+    if (M > 128 && t.config == 3) continue;  // with many tokens the wide side goes to the tokens
+    const long long groups = (long long)((M + t.tokens - 1) / t.tokens) * ((N + t.rows - 1) / t.rows);
+    for (int ranges = 1; ranges <= 8; ranges *= 2) {
+      if (ranges > 1 && (K / ranges < 512 || (long long)ranges * M * N > partial_floats)) break;
+      const long long slots = (long long)g_compute_units * t.resident;
+      const long long rounds = (groups * ranges + slots - 1) / slots;
+      const double fill = (double)(groups * ranges) / ((double)rounds * slots);
+      double time = flops / (1e15 * t.speed * fill);
+      if (ranges > 1) time += (2.0 * ranges + 1.0) * output_bytes / 6e12 + 4e-6;
+      if (time < best_time * (1.0 - 1e-9)) {
+        best_time = time;
+        best = TilePlan{t.config, ranges};
+      }
+    }
+  }
+  return best;
 }
 
 template <typename TC, bool ACC, bool GATED = false>
 int launch_tile(const __bf16* A, const __bf16* W, const float* bias, TC* C, int M, int N, int K, long long lda,
-                long long ldc, int vector_ok, hipStream_t s) {
-  switch (g_tile_config >= 0 ? g_tile_config : choose_tile_config(M, N)) {
-    case 2: return launch_tile_as<256, 128, 4, 2, TC, ACC, GATED>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, s);
-    case 3: return launch_tile_as<128, 256, 2, 4, TC, ACC, GATED>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, s);
-    case 4: return launch_tile_as<256, 256, 4, 4, TC, ACC, GATED>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, s);
-    default: return launch_tile_as<128, 128, 2, 2, TC, ACC, GATED>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, s);
+                long long ldc, int vector_ok, float* partial, long long partial_floats, hipStream_t s) {
+  TilePlan plan = choose_tile_plan(M, N, K, (GATED || !partial) ? 0 : partial_floats);
+  if (g_tile_config >= 0) plan = TilePlan{g_tile_config % 10, g_tile_config >= 10 && !GATED && partial ? g_tile_config / 10 : 1};
+  if (plan.ranges > 1 && (long long)plan.ranges * M * N > partial_floats) plan.ranges = 1;
+  const int r = plan.ranges;
+  switch (plan.config) {
+    case 2: return launch_tile_as<256, 128, 4, 2, TC, ACC, GATED>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, r, partial, s);
+    case 3: return launch_tile_as<128, 256, 2, 4, TC, ACC, GATED>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, r, partial, s);
+    case 4: return launch_tile_as<256, 256, 4, 4, TC, ACC, GATED>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, r, partial, s);
+    default: return launch_tile_as<128, 128, 2, 2, TC, ACC, GATED>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, r, partial, s);
   }
 }
 }  // namespace
@@ -653,8 +719,10 @@ int launch_tile(const __bf16* A, const __bf16* W, const float* bias, TC* C, int 
 // K a multiple of 8 and lda a multiple of 8 (16-byte chunks); A and W 16-byte aligned.
 // `skinny_limit`: M at or below it takes the weight-streaming kernel (at most 64).
 // `skinny_shape`: 0 lets the launcher choose the row tiles per wave; 1 or 2 force one or two.
+// `partial` (may be null): a float workspace of `partial_floats` floats that the tiled kernel may split K into.
 extern "C" int vk_gemm_bf16(const void* A, const void* W, const float* bias, void* C, int c_dtype, int M, int N, int K,
-                            long long lda, long long ldc, int accumulate, int skinny_limit, int skinny_shape, void* stream) {
+                            long long lda, long long ldc, int accumulate, int skinny_limit, int skinny_shape,
+                            float* partial, long long partial_floats, void* stream) {
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0 || (K & 7) || (lda & 7) || lda < K || ldc < N) return VK_BAD_ARGUMENT;
   if (((uintptr_t)A & 15) || ((uintptr_t)W & 15)) return VK_BAD_ARGUMENT;
@@ -670,13 +738,13 @@ extern "C" int vk_gemm_bf16(const void* A, const void* W, const float* bias, voi
   if (c_dtype == DT_F32) {
     if (accumulate)
       return skinny ? launch_skinny<float, true>(a, w, bias, (float*)C, M, N, K, lda, ldc, vector_ok, skinny_shape, s)
-                    : launch_tile<float, true>(a, w, bias, (float*)C, M, N, K, lda, ldc, vector_ok, s);
+                    : launch_tile<float, true>(a, w, bias, (float*)C, M, N, K, lda, ldc, vector_ok, partial, partial_floats, s);
     return skinny ? launch_skinny<float, false>(a, w, bias, (float*)C, M, N, K, lda, ldc, vector_ok, skinny_shape, s)
-                  : launch_tile<float, false>(a, w, bias, (float*)C, M, N, K, lda, ldc, vector_ok, s);
+                  : launch_tile<float, false>(a, w, bias, (float*)C, M, N, K, lda, ldc, vector_ok, partial, partial_floats, s);
   }
   if (c_dtype == DT_BF16)
     return skinny ? launch_skinny<__bf16, false>(a, w, bias, (__bf16*)C, M, N, K, lda, ldc, vector_ok, skinny_shape, s)
-                  : launch_tile<__bf16, false>(a, w, bias, (__bf16*)C, M, N, K, lda, ldc, vector_ok, s);
+                  : launch_tile<__bf16, false>(a, w, bias, (__bf16*)C, M, N, K, lda, ldc, vector_ok, partial, partial_floats, s);
   return VK_BAD_ARGUMENT;
 }
 
@@ -721,7 +789,7 @@ extern "C" int vk_gemm_bf16_gated(const void* A, const void* W, void* C, int M, 
   const __bf16* a = (const __bf16*)A;
   const __bf16* w = (const __bf16*)W;
   __bf16* c = (__bf16*)C;
-  if (M > 64) return launch_tile<__bf16, false, true>(a, w, nullptr, c, M, N, K, lda, ldc, 0, s);
+  if (M > 64) return launch_tile<__bf16, false, true>(a, w, nullptr, c, M, N, K, lda, ldc, 0, nullptr, 0, s);
   const int cb = (M + 15) / 16;
 #define VK_GATED(CBV, RTV)                                                                                         \
   {                                                                                                                \

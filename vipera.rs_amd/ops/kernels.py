@@ -299,9 +299,13 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], ou
     lda = lda if lda % 8 == 0 else k
     ldc = out.stride(0) if m > 1 else max(out.stride(0), n)
     _need(ldc >= n, "gemm: out's row stride")
-    fn = _fn("gemm_bf16", "vk_gemm_bf16", [_p, _p, _p, _p, _i, _i, _i, _i, _ll, _ll, _i, _i, _i, _p])
+    partial = None
+    if m > skinny_limit or m > 64:  # the tiled kernel may split K into a workspace of at most eight ranges
+        partial = _split_k_workspace(a.device, min(8 * m * n, _TILE_WORKSPACE_FLOATS), "tile")
+    fn = _fn("gemm_bf16", "vk_gemm_bf16", [_p, _p, _p, _p, _i, _i, _i, _i, _ll, _ll, _i, _i, _i, _p, _ll, _p])
     _status(fn(_ptr(a), _ptr(w), _ptr(bias), _ptr(out), _dt(out, "out"), m, n, k, lda, ldc, 1 if accumulate else 0,
-               int(skinny_limit), int(skinny_shape), _stream()), "gemm_bf16")
+               int(skinny_limit), int(skinny_shape), _ptr(partial), partial.numel() if partial is not None else 0,
+               _stream()), "gemm_bf16")
 
 
 # ----------------------------------------------------------------------------------------------
@@ -364,17 +368,22 @@ def attn_bf16_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
 
 
 _workspaces = {}
+_retired = []  # outgrown workspaces: kept alive, since a captured graph may still write to them
+_TILE_WORKSPACE_FLOATS = 64 * 1024 * 1024   # 256 MB: the most the tiled kernel's K ranges may take
 
 
-def _split_k_workspace(device: torch.device, floats: int) -> torch.Tensor:
-    """Partial-sum workspace of a device; grown when a product needs more, never shrunk.
+def _split_k_workspace(device: torch.device, floats: int, kind: str) -> torch.Tensor:
+    """Partial-sum workspace of a device and a kind of product; grown when a product needs more, never shrunk.
 
-    Every product on the device shares it, which is safe because products run on one stream.
+    Every product of the kind on the device shares it, which is safe because products run on one stream.
     """
-    entry = _workspaces.get(device)
+    key = (device, kind)
+    entry = _workspaces.get(key)
     if entry is None or entry.numel() < floats:
+        if entry is not None:
+            _retired.append(entry)
         entry = torch.empty(floats, dtype=torch.float32, device=device)
-        _workspaces[device] = entry
+        _workspaces[key] = entry
     return entry
 
 
@@ -400,7 +409,7 @@ def gemm_bf16_mid(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor]
     _need(ldc >= n, "gemm: out's row stride")
     partial = None
     if ranges > 1:
-        partial = _split_k_workspace(a.device, ranges * 64 * n)
+        partial = _split_k_workspace(a.device, ranges * 64 * n, "mid")
     fn = _fn("gemm_bf16", "vk_gemm_bf16_mid", [_p, _p, _p, _p, _i, _i, _i, _i, _ll, _ll, _i, _i, _i, _p, _ll, _p])
     _status(fn(_ptr(a), _ptr(w), _ptr(bias), _ptr(out), _dt(out, "out"), m, n, k, lda, ldc, 1 if accumulate else 0,
                int(ranges), int(rows_per_wave), _ptr(partial), partial.numel() if partial is not None else 0, _stream()),
