@@ -40,6 +40,52 @@ def test_gemm_bf16_against_float64(m, n, k, out_dtype):
         assert _rel(acc, base.double() + a.double() @ w.double().T) < 1e-5
 
 
+@pytest.mark.parametrize("tiling", [0, 2, 3, 4, 9, 7, 8, 5])
+@pytest.mark.parametrize("ranges", [1, 2, 8])
+def test_gemm_bf16_every_tiling_of_the_tiled_kernel(tiling, ranges):
+    """Each tiling of both tiled kernels, forced: tails in both directions, one to many K steps (an odd
+    number too, so both LDS stages end a run), K split into ranges, and a K that the direct kernel passes on."""
+    from vipera_rs_amd.ops import kernels
+    shapes = [(257, 520, 1024), (129, 1028, 128), (300, 264, 64), (513, 300, 1600), (65, 2100, 4608), (200, 257, 136)]
+    try:
+        kernels.gemm_bf16_force_tiling(tiling, ranges)
+        for m, n, k in shapes:
+            g = torch.Generator().manual_seed(m + n + k)
+            a = torch.randn(m, k, generator=g).to(torch.bfloat16).to(DEV)
+            w = torch.randn(n, k, generator=g).to(torch.bfloat16).to(DEV)
+            bias = torch.randn(n, generator=g).to(DEV)
+            product = a.double() @ w.double().T
+            for out_dtype, tol in ((torch.float32, 1e-5), (torch.bfloat16, 6e-3)):
+                out = torch.full((m, n), 7.0, dtype=out_dtype, device=DEV)
+                kernels.gemm_bf16(a, w, bias, out)
+                assert _rel(out, product + bias.double()) < tol, (m, n, k, out_dtype)
+            base = torch.randn(m, n, generator=g).to(DEV)
+            acc = base.clone()
+            kernels.gemm_bf16(a, w, None, acc, accumulate=True)
+            assert _rel(acc, base.double() + product) < 1e-5, (m, n, k, "accumulate")
+    finally:
+        kernels.gemm_bf16_force_tiling(-1)
+
+
+@pytest.mark.parametrize("tiling", [0, 2, 3, 4, 9, 7, 8, 5])
+def test_gated_product_with_every_tiling(tiling):
+    from vipera_rs_amd.ops import kernels
+    from vipera_rs_amd.ops.linear import interleave_gate_up
+    try:
+        kernels.gemm_bf16_force_tiling(tiling)
+        for m, inter, k in [(300, 208, 192), (2048, 528, 128), (130, 1008, 640), (70, 48, 72)]:
+            g = torch.Generator().manual_seed(m + inter + k)
+            a = torch.randn(m, k, generator=g).to(torch.bfloat16).to(DEV)
+            gate = torch.randn(inter, k, generator=g).to(torch.bfloat16).to(DEV)
+            up = torch.randn(inter, k, generator=g).to(torch.bfloat16).to(DEV)
+            gd, ud = a.double() @ gate.double().T, a.double() @ up.double().T
+            out = torch.full((m, inter), 7.0, dtype=torch.bfloat16, device=DEV)
+            kernels.gemm_bf16_gated(a, interleave_gate_up(gate, up), out)
+            assert _rel(out, ud * (gd / (1 + torch.exp(-gd)))) < 8e-3, (m, inter, k)
+    finally:
+        kernels.gemm_bf16_force_tiling(-1)
+
+
 def test_gemm_bf16_tile_and_skinny_kernels_agree():
     from vipera_rs_amd.ops import kernels
     g = torch.Generator().manual_seed(5)

@@ -7,12 +7,15 @@
 // them as one vector:
 //     lane l, register j of an accumulator  <->  C[token l % 16][column 4 * (l / 16) + j]
 //
-// Three kernels:
-//   gemm_tile    more than 64 tokens (prompts). An output tile per workgroup (256x256 on sixteen waves
-//                down to 128x128 on four, chosen by how many tiles the shape gives), K in steps of 64
-//                staged through LDS (rows padded to 144 bytes, which spreads the 16-byte reads of 16
-//                rows over all banks), double-buffered, one barrier per step. Workgroups are renumbered
-//                so that those running on one XCD (one L2) work on neighbouring tiles.
+// Kernels:
+//   gemm_tile    more than 64 tokens (prompts). An output tile per workgroup (256x256 down to 128x128,
+//                chosen with a split of K by an estimate of the time), K in steps of 64 through two LDS
+//                stages, one barrier per step. Workgroups are renumbered so that those running on one XCD
+//                (one L2) work on neighbouring tiles. Two kernels: gemm_tile_direct_kernel loads both
+//                operands straight into LDS (unpadded rows, chunks swizzled) and pipelines the LDS reads
+//                against the products inside each wave; it takes K in multiples of 64. gemm_tile_kernel
+//                stages the operands through registers into rows padded to 144 bytes and takes any K that
+//                is a multiple of 8.
 //   gemm_skinny  a few tokens (decoding). The product is a stream of the weights from HBM: a workgroup
 //                owns 16 weight rows, its waves split K in interleaved spans of 128 and read their span
 //                straight into the instruction's operand layout (no LDS); the waves' partial sums are
@@ -237,6 +240,150 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_tile_kernel(const __bf16* _
   const int wave_m = m0 + wm * TM * 16, wave_n = n0 + wn * TN * 16;
   if constexpr (GATED) {
     // N counts fused rows (pairs of 16-row tiles: gate, up); the output has N / 2 columns
+    static_assert(!GATED || TN % 2 == 0, "a wave must own whole gate/up pairs");
+#pragma unroll
+    for (int pair = 0; pair < TN / 2; ++pair)
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm)
+        store_gated((__bf16*)C, ldc, wave_m + tm * 16 + lr, (wave_n + pair * 32) / 2 + lg * 4, M, N / 2,
+                    acc[2 * pair][tm], acc[2 * pair + 1][tm]);
+  } else {
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm)
+        store4<TC, ACCUMULATE>(C, ldc, wave_m + tm * 16 + lr, wave_n + tn * 16 + lg * 4, M, N, acc[tn][tm], bias,
+                               vector_ok != 0);
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// The tiled product with both operands loaded straight into LDS (buffer loads with the lds modifier: no
+// staging registers, no LDS store instructions) and a software pipeline inside each wave: two register
+// sets of operand fragments, one being read from LDS while the other is multiplied, so that a wave keeps
+// the matrix core busy by itself and a wave tile of 64 x 128 (eight waves per 256 x 256 tile) fits the
+// register file. Per K step of 64 a CU then reads 192 KB of fragments from LDS, against 256 KB with
+// sixteen waves of 64 x 64.
+//
+// LDS rows are 128 bytes, unpadded (a load instruction fills 1 KB: 8 rows, lane L the 16 bytes at 16 L).
+// The 16-byte chunk c of row r sits in slot c ^ (r % 8); the loading lane picks the global chunk that
+// belongs in its slot, the reading lane the slot of its chunk, and 16 rows read the same chunk from
+// different banks.
+//
+// Step s works on stage s % 2, the fragments of its first half (k 0..31 of the step) already in registers:
+//   read the fragments of the second half; multiply the first half;
+//   wait for the own loads of step s + 1, barrier (now nobody reads stage s % 2 any more);
+//   issue the loads of step s + 2 into stage s % 2; read the first-half fragments of step s + 1;
+//   multiply the second half.
+// K ranges must be multiples of 64 (the launcher sends other shapes to gemm_tile_kernel). Four stages of
+// 32 k, which give a load three short steps to arrive instead of one long one, were slower.
+constexpr int DIRECT_ROW = BK * 2;  // bytes per LDS row
+
+// Until none of the wave's vector memory loads is in flight (s_waitcnt vmcnt(0), the other counters left
+// alone). A barrier alone does not wait for loads that write LDS: the compiler's fence only waits for the
+// wave's LDS instructions.
+__device__ __forceinline__ void wait_own_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
+template <int BM, int BN, int WM, int WN, typename TC, bool ACCUMULATE, bool GATED>
+__global__ __launch_bounds__(WM * WN * 64) void gemm_tile_direct_kernel(const __bf16* __restrict__ A,
+                                                                          const __bf16* __restrict__ W,
+                                                                          const float* __restrict__ bias,
+                                                                          TC* __restrict__ C, int M, int N, int K,
+                                                                          long long lda, long long ldc, int tiles_m,
+                                                                          int tiles_n, int vector_ok, int k_per_range,
+                                                                          long long range_stride) {
+  typedef __attribute__((address_space(3))) void* lds_ptr;
+  const int k_begin = blockIdx.y * k_per_range, k_end = min(K, k_begin + k_per_range);
+  C += (size_t)blockIdx.y * range_stride;
+  constexpr int WAVES = WM * WN;
+  constexpr int TM = BM / WM / 16, TN = BN / WN / 16;
+  constexpr int A_LOADS = BM / 8 / WAVES, W_LOADS = BN / 8 / WAVES;  // load instructions per wave and step
+  static_assert(BM % (8 * WAVES) == 0 && BN % (8 * WAVES) == 0, "tile rows must divide among the waves' loads");
+  constexpr int STAGE = (BM + BN) * DIRECT_ROW;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];  // [2][BM + BN][128]
+
+  const int total = tiles_m * tiles_n;
+  const int per_xcd = (total + XCDS - 1) / XCDS;
+  const int logical = (blockIdx.x % XCDS) * per_xcd + blockIdx.x / XCDS;
+  if (logical >= total) return;
+  const int tile_n = logical / tiles_m, tile_m = logical % tiles_m;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WN, wn = wave % WN;
+  const int lr = lane & 15, lg = lane >> 4;
+
+  f32x4 acc[TN][TM];
+#pragma unroll
+  for (int i = 0; i < TN; ++i)
+#pragma unroll
+    for (int j = 0; j < TM; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // rows past M or N read zero through the buffer descriptors
+  const BufferView a_view = buffer_view(A + (size_t)m0 * lda, ((unsigned long long)(M - m0 - 1) * lda + K) * 2);
+  const BufferView w_view = buffer_view(W + (size_t)n0 * K, (unsigned long long)(N - n0) * K * 2);
+  // a load instruction covers 8 rows: lane L fills slot L % 8 of row L / 8 with chunk (L % 8) ^ (L / 8)
+  const int ld_row = lane >> 3, ld_chunk = (lane & 7) ^ (lane >> 3);
+  unsigned a_off[A_LOADS], w_off[W_LOADS];
+#pragma unroll
+  for (int i = 0; i < A_LOADS; ++i)
+    a_off[i] = (unsigned)((((wave * A_LOADS + i) * 8 + ld_row) * lda + ld_chunk * 8 + k_begin) * 2);
+#pragma unroll
+  for (int i = 0; i < W_LOADS; ++i)
+    w_off[i] = (unsigned)((((size_t)(wave * W_LOADS + i) * 8 + ld_row) * K + ld_chunk * 8 + k_begin) * 2);
+  auto issue_loads = [&](int stage, int step) {
+    unsigned char* to_a = lds_raw + stage * STAGE + wave * A_LOADS * 1024;
+    unsigned char* to_w = lds_raw + stage * STAGE + BM * DIRECT_ROW + wave * W_LOADS * 1024;
+    const unsigned kb = (unsigned)step * (BK * 2);
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(a_view.rsrc, (lds_ptr)(to_a + i * 1024), 16, (int)(a_off[i] + kb), 0, 0, 0);
+#pragma unroll
+    for (int i = 0; i < W_LOADS; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(w_view.rsrc, (lds_ptr)(to_w + i * 1024), 16, (int)(w_off[i] + kb), 0, 0, 0);
+  };
+  // a lane's fragment chunks within a stage: row lr of each 16-row tile, chunk lg (first half of the step)
+  // or lg + 4 (second half), which differ in bit 6 of the byte offset
+  const unsigned frag_a = (unsigned)((wm * TM * 16 + lr) * DIRECT_ROW + ((lg ^ (lr & 7)) * 16));
+  const unsigned frag_w = (unsigned)(BM * DIRECT_ROW + (wn * TN * 16 + lr) * DIRECT_ROW + ((lg ^ (lr & 7)) * 16));
+  auto read_fragments = [&](int stage, int half, bf16x8 (&fa)[TM], bf16x8 (&fw)[TN]) {
+    const unsigned char* base = lds_raw + stage * STAGE;
+#pragma unroll
+    for (int t = 0; t < TN; ++t) fw[t] = *(const bf16x8*)(base + (frag_w ^ (half * 64)) + t * 16 * DIRECT_ROW);
+#pragma unroll
+    for (int t = 0; t < TM; ++t) fa[t] = *(const bf16x8*)(base + (frag_a ^ (half * 64)) + t * 16 * DIRECT_ROW);
+  };
+  auto multiply = [&](const bf16x8 (&fa)[TM], const bf16x8 (&fw)[TN]) {
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm)
+        acc[tn][tm] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[tn], fa[tm], acc[tn][tm], 0, 0, 0);
+  };
+
+  const int steps = (k_end - k_begin) / BK;
+  bf16x8 fa0[TM], fw0[TN], fa1[TM], fw1[TN];
+  issue_loads(0, 0);
+  if (steps > 1) issue_loads(1, 1);
+  wait_own_loads();
+  __syncthreads();
+  read_fragments(0, 0, fa0, fw0);
+  for (int s = 0; s < steps; ++s) {
+    const int stage = s & 1;
+    read_fragments(stage, 1, fa1, fw1);
+    multiply(fa0, fw0);
+    __builtin_amdgcn_sched_barrier(0);  // the products stay on this side: they cover the reads above
+    wait_own_loads();
+    __syncthreads();
+    if (s + 2 < steps) issue_loads(stage, s + 2);
+    if (s + 1 < steps) read_fragments(stage ^ 1, 0, fa0, fw0);
+    multiply(fa1, fw1);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+
+  const int wave_m = m0 + wm * TM * 16, wave_n = n0 + wn * TN * 16;
+  if constexpr (GATED) {
     static_assert(!GATED || TN % 2 == 0, "a wave must own whole gate/up pairs");
 #pragma unroll
     for (int pair = 0; pair < TN / 2; ++pair)
@@ -611,17 +758,24 @@ int launch_mid(const __bf16* A, const __bf16* W, const float* bias, TC* C, float
   return VK_UNSUPPORTED_SIZE;
 }
 
-template <int BM, int BN, int WM, int WN, typename TC, bool ACC, bool GATED>
+template <bool DIRECT, int BM, int BN, int WM, int WN, typename TC, bool ACC, bool GATED>
+constexpr auto tile_kernel() {
+  if constexpr (DIRECT) return gemm_tile_direct_kernel<BM, BN, WM, WN, TC, ACC, GATED>;
+  else return gemm_tile_kernel<BM, BN, WM, WN, TC, ACC, GATED>;
+}
+
+// DIRECT: the kernel that loads straight into LDS; K must be a multiple of 64.
+template <int BM, int BN, int WM, int WN, typename TC, bool ACC, bool GATED, bool DIRECT = false>
 int launch_tile_as(const __bf16* A, const __bf16* W, const float* bias, TC* C, int M, int N, int K, long long lda,
                    long long ldc, int vector_ok, int ranges, float* partial, hipStream_t s) {
-  constexpr int lds_bytes = 2 * (BM + BN) * ROW * (int)sizeof(__bf16);
+  constexpr int lds_bytes = DIRECT ? 2 * (BM + BN) * DIRECT_ROW : 2 * (BM + BN) * ROW * (int)sizeof(__bf16);
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
   const long long total = (long long)tiles_m * tiles_n;
   const long long grid = (total + XCDS - 1) / XCDS * XCDS;
   if (grid > 0x7fffffffLL) return VK_UNSUPPORTED_SIZE;
   if (ranges <= 1 || GATED) {
     static bool configured = false;
-    auto kernel = gemm_tile_kernel<BM, BN, WM, WN, TC, ACC, GATED>;
+    auto kernel = tile_kernel<DIRECT, BM, BN, WM, WN, TC, ACC, GATED>();
     if (!configured) {
       hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
       if (e != hipSuccess) return (int)e;
@@ -635,7 +789,7 @@ int launch_tile_as(const __bf16* A, const __bf16* W, const float* bias, TC* C, i
   // K split over workgroups: float partial sums [range, M, N], then the ranges are added in ascending order
   if constexpr (!GATED) {
     static bool configured_partial = false;
-    auto kernel = gemm_tile_kernel<BM, BN, WM, WN, float, false, false>;
+    auto kernel = tile_kernel<DIRECT, BM, BN, WM, WN, float, false, false>();
     if (!configured_partial) {
       hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
       if (e != hipSuccess) return (int)e;
@@ -654,19 +808,20 @@ int launch_tile_as(const __bf16* A, const __bf16* W, const float* bias, TC* C, i
   return 0;
 }
 
-int g_tile_config = -1;  // -1: chosen by shape; else 10 * ranges + tiling (0, 2, 3, 4) forces a plan, for measurements
+int g_tile_config = -1;  // -1: chosen by shape; else 10 * ranges + tiling (see launch_tile) forces a plan, for measurements
 
 // Which tiling, and into how many ranges K is split: the pair with the shortest estimated time. A full GPU
-// of 256x256 tiles on sixteen waves runs at about 1 PFLOP/s (measured on the 7B shapes at 2,048 tokens),
-// 256x128 and 128x256 on eight waves at 0.8, 128x128 on four at 0.75 of that; workgroups run in whole
-// rounds of one per CU (two for the small tile, whose LDS lets two share a CU), so a launch that fills
-// the last round badly loses that share. Splitting K multiplies the workgroups, at the price of writing
-// and re-reading float partial sums (they mostly stay in the caches: about 6 TB/s) and one more launch;
-// each range keeps at least 512 of K. The estimate ranks the plans as measurements at 256 to 2,048 tokens do. Few tokens keep the token side of the tile at
-// 128. Ties go to the larger tile and to fewer ranges.
+// of 256x256 tiles runs at about 1.15 PFLOP/s with the kernel that loads straight into LDS and at 1.0
+// with the staged one (measured on the 7B shapes at 2,048 tokens); the smaller tiles reach 0.75 to 0.8 of
+// their kernel's best. Workgroups run in whole rounds of one per CU (two for the 128x128 tile, whose LDS
+// lets two share a CU), so a launch that fills the last round badly loses that share. Splitting K
+// multiplies the workgroups, at the price of writing and re-reading float partial sums (they mostly stay
+// in the caches: about 6 TB/s) and one more launch; each range keeps at least 512 of K. The estimate ranks
+// the plans as measurements at 128 to 2,048 tokens do. Few tokens keep the token side of the tile at 128.
+// Ties go to the larger tile and to fewer ranges.
 struct TilePlan { int config, ranges; };
 int g_compute_units = 0;
-TilePlan choose_tile_plan(int M, int N, int K, long long partial_floats) {
+TilePlan choose_tile_plan(int M, int N, int K, long long partial_floats, bool direct) {
   if (g_compute_units == 0) {
     int device = 0, count = 0;
     if (hipGetDevice(&device) != hipSuccess ||
@@ -675,13 +830,16 @@ TilePlan choose_tile_plan(int M, int N, int K, long long partial_floats) {
     g_compute_units = count;
   }
   struct Tiling { int config, tokens, rows, resident; double speed; };
-  static const Tiling tilings[] = {{4, 256, 256, 1, 1.0}, {2, 256, 128, 1, 0.8}, {3, 128, 256, 1, 0.8}, {0, 128, 128, 2, 0.75}};
-  TilePlan best{0, 1};
+  static const Tiling staged[] = {{4, 256, 256, 1, 1.0}, {2, 256, 128, 1, 0.8}, {3, 128, 256, 1, 0.8}, {0, 128, 128, 2, 0.75}};
+  static const Tiling straight[] = {{5, 256, 256, 1, 1.15}, {7, 256, 128, 1, 0.92}, {8, 128, 256, 1, 0.88}, {9, 128, 128, 2, 0.9}};
+  const Tiling* tilings = direct ? straight : staged;
+  TilePlan best{tilings[3].config, 1};
   double best_time = 1e30;
   const double flops = 2.0 * M * N * (double)K, output_bytes = 4.0 * M * N;
-  for (const Tiling& t : tilings) {
+  for (int i = 0; i < 4; ++i) {
+    const Tiling& t = tilings[i];
     if (M <= 128 && t.tokens > 128) continue;
-    if (M > 128 && t.config == 3) continue;  // with many tokens the wide side goes to the tokens
+    if (M > 128 && t.tokens == 128 && t.rows == 256) continue;  // with many tokens the wide side goes to the tokens
     const long long groups = (long long)((M + t.tokens - 1) / t.tokens) * ((N + t.rows - 1) / t.rows);
     for (int ranges = 1; ranges <= 8; ranges *= 2) {
       if (ranges > 1 && (K / ranges < 512 || (long long)ranges * M * N > partial_floats)) break;
@@ -699,19 +857,32 @@ TilePlan choose_tile_plan(int M, int N, int K, long long partial_floats) {
   return best;
 }
 
+// Tilings: 0, 2, 3, 4 the staged kernel at 128x128, 256x128, 128x256, 256x256; 9, 7, 8, 5 the same tiles
+// with the kernel that loads straight into LDS, which needs K to be a multiple of 64.
 template <typename TC, bool ACC, bool GATED = false>
 int launch_tile(const __bf16* A, const __bf16* W, const float* bias, TC* C, int M, int N, int K, long long lda,
                 long long ldc, int vector_ok, float* partial, long long partial_floats, hipStream_t s) {
-  TilePlan plan = choose_tile_plan(M, N, K, (GATED || !partial) ? 0 : partial_floats);
+  const bool direct = (K & 63) == 0;
+  TilePlan plan = choose_tile_plan(M, N, K, (GATED || !partial) ? 0 : partial_floats, direct);
   if (g_tile_config >= 0) plan = TilePlan{g_tile_config % 10, g_tile_config >= 10 && !GATED && partial ? g_tile_config / 10 : 1};
   if (plan.ranges > 1 && (long long)plan.ranges * M * N > partial_floats) plan.ranges = 1;
-  const int r = plan.ranges;
-  switch (plan.config) {
-    case 2: return launch_tile_as<256, 128, 4, 2, TC, ACC, GATED>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, r, partial, s);
-    case 3: return launch_tile_as<128, 256, 2, 4, TC, ACC, GATED>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, r, partial, s);
-    case 4: return launch_tile_as<256, 256, 4, 4, TC, ACC, GATED>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, r, partial, s);
-    default: return launch_tile_as<128, 128, 2, 2, TC, ACC, GATED>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, r, partial, s);
+  if (!direct) {
+    switch (plan.config) { case 5: plan.config = 4; break; case 7: plan.config = 2; break; case 8: plan.config = 3; break; case 9: plan.config = 0; break; }
   }
+  const int r = plan.ranges;
+#define VK_TILE(BMV, BNV, WMV, WNV, DIRECTV) \
+  return launch_tile_as<BMV, BNV, WMV, WNV, TC, ACC, GATED, DIRECTV>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, r, partial, s)
+  switch (plan.config) {
+    case 5: VK_TILE(256, 256, 4, 2, true);
+    case 7: VK_TILE(256, 128, 4, 2, true);
+    case 8: VK_TILE(128, 256, 2, 4, true);
+    case 9: VK_TILE(128, 128, 2, 2, true);
+    case 2: VK_TILE(256, 128, 4, 2, false);
+    case 3: VK_TILE(128, 256, 2, 4, false);
+    case 4: VK_TILE(256, 256, 4, 4, false);
+    default: VK_TILE(128, 128, 2, 2, false);
+  }
+#undef VK_TILE
 }
 }  // namespace
 
@@ -726,7 +897,7 @@ extern "C" int vk_gemm_bf16(const void* A, const void* W, const float* bias, voi
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0 || (K & 7) || (lda & 7) || lda < K || ldc < N) return VK_BAD_ARGUMENT;
   if (((uintptr_t)A & 15) || ((uintptr_t)W & 15)) return VK_BAD_ARGUMENT;
-  if (K >= (1 << 24) || lda >= (1 << 24)) return VK_UNSUPPORTED_SIZE;  // byte offsets inside a tile of rows are 32-bit
+  if (K >= (1 << 23) || lda >= (1 << 23)) return VK_UNSUPPORTED_SIZE;  // byte offsets inside a tile of 256 rows are 32-bit
   if (accumulate && c_dtype != DT_F32) return VK_BAD_ARGUMENT;
   const int elem = c_dtype == DT_F32 ? 4 : 2;
   const int vector_ok = ((ldc & 3) == 0 && ((uintptr_t)C & (4 * elem - 1)) == 0 &&
@@ -784,7 +955,7 @@ extern "C" int vk_gemm_bf16_gated(const void* A, const void* W, void* C, int M, 
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0 || (K & 7) || (lda & 7) || lda < K || (N & 31) || ldc < N / 2) return VK_BAD_ARGUMENT;
   if (((uintptr_t)A & 15) || ((uintptr_t)W & 15)) return VK_BAD_ARGUMENT;
-  if (K >= (1 << 24) || lda >= (1 << 24)) return VK_UNSUPPORTED_SIZE;  // byte offsets inside a tile of rows are 32-bit
+  if (K >= (1 << 23) || lda >= (1 << 23)) return VK_UNSUPPORTED_SIZE;  // byte offsets inside a tile of 256 rows are 32-bit
   hipStream_t s = (hipStream_t)stream;
   const __bf16* a = (const __bf16*)A;
   const __bf16* w = (const __bf16*)W;

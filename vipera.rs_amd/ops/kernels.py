@@ -308,6 +308,20 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], ou
                _stream()), "gemm_bf16")
 
 
+TILE_TILINGS = {0: "128x128 staged", 2: "256x128 staged", 3: "128x256 staged", 4: "256x256 staged",
+                9: "128x128 direct", 7: "256x128 direct", 8: "128x256 direct", 5: "256x256 direct"}
+
+
+def gemm_bf16_force_tiling(tiling: int = -1, ranges: int = 1) -> None:
+    """For tests and measurements: make the tiled kernel of :func:`gemm_bf16` and :func:`gemm_bf16_gated`
+    use one tiling (a key of ``TILE_TILINGS``) and split K into ``ranges``; ``-1`` gives the choice back
+    to the launcher.  A "direct" tiling falls back to its staged twin when K is no multiple of 64."""
+    if tiling >= 0:
+        _need(tiling in TILE_TILINGS and 1 <= ranges <= 8, "gemm_bf16_force_tiling: unknown tiling or ranges")
+    fn = _fn("gemm_bf16", "vk_gemm_bf16_tile_config", [_i])
+    _status(fn(-1 if tiling < 0 else (10 * ranges if ranges > 1 else 0) + tiling), "gemm_bf16_force_tiling")
+
+
 # ----------------------------------------------------------------------------------------------
 def attn_bf16_padded_width(head_dim: int) -> int:
     """The padded head width a matrix-core attention module is compiled for (a multiple of 32)."""
