@@ -369,18 +369,39 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_tile_direct_kernel(const __
   wait_own_loads();
   __syncthreads();
   read_fragments(0, 0, fa0, fw0);
-  for (int s = 0; s < steps; ++s) {
+  // Hints for the instruction order within a half step: the LDS reads and the loads go out one by one
+  // between products, so that their issue hides behind the matrix core's work instead of stalling it.
+  auto interleave = [](auto lds_reads, auto loads) {
+    constexpr int READS = decltype(lds_reads)::value, LOADS = decltype(loads)::value;
+    static_for<LOADS>([](auto) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one matrix instruction
+      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one load
+    });
+    static_for<READS>([](auto) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
+    });
+    __builtin_amdgcn_sched_group_barrier(0x008, TM * TN, 0);
+  };
+  auto step = [&](int s, auto with_loads, auto with_next) {
     const int stage = s & 1;
     read_fragments(stage, 1, fa1, fw1);
     multiply(fa0, fw0);
+    interleave(std::integral_constant<int, TM + TN>{}, std::integral_constant<int, 0>{});
     __builtin_amdgcn_sched_barrier(0);  // the products stay on this side: they cover the reads above
     wait_own_loads();
     __syncthreads();
-    if (s + 2 < steps) issue_loads(stage, s + 2);
-    if (s + 1 < steps) read_fragments(stage ^ 1, 0, fa0, fw0);
+    if constexpr (decltype(with_loads)::value) issue_loads(stage, s + 2);
+    if constexpr (decltype(with_next)::value) read_fragments(stage ^ 1, 0, fa0, fw0);
     multiply(fa1, fw1);
+    interleave(std::integral_constant<int, decltype(with_next)::value ? TM + TN : 0>{},
+               std::integral_constant<int, decltype(with_loads)::value ? A_LOADS + W_LOADS : 0>{});
     __builtin_amdgcn_sched_barrier(0);
-  }
+  };
+  int s = 0;
+  for (; s + 2 < steps; ++s) step(s, std::true_type{}, std::true_type{});
+  if (s + 1 < steps) step(s++, std::false_type{}, std::true_type{});
+  step(s, std::false_type{}, std::false_type{});
 
   const int wave_m = m0 + wm * TM * 16, wave_n = n0 + wn * TN * 16;
   if constexpr (GATED) {
