@@ -257,6 +257,8 @@ __global__ __launch_bounds__(PT_THREADS) void attn_prefill_kernel(
   const int wave_end = wave_cols > 0 ? first_pos + q_off + wave_cols : 0;  // nothing at or past it is visible
   const int wave_first = first_pos + q_off;
   const int wave_begin = (window > 0 && wave_first + 1 > window) ? wave_first + 1 - window : 0;
+  const int wave_last = wave_end - 1;  // position of the wave's last column
+  const int wave_lo_max = (window > 0 && wave_last + 1 > window) ? wave_last + 1 - window : 0;
 
   f32x4 o[DT];
   float m = -INFINITY, l = 0.f;
@@ -314,6 +316,81 @@ __global__ __launch_bounds__(PT_THREADS) void attn_prefill_kernel(
     }
   };
 
+  // One tile of 64 positions for this wave's 16 columns. The running maximum m is kept in units of the raw
+  // score (the scale is positive, so it commutes with the maximum) and a weight is one fused multiply-add
+  // and one exp2: exp2(s * c - m * c) with c = scale * log2(e). `masked`: some column of the wave does not
+  // see all 64 positions (the tiles on the diagonal and at a window's edge); the other tiles skip the
+  // comparisons. The sums are rescaled only when some column's maximum moved, which is rare after the
+  // first tiles.
+  const float c2 = scale * 1.44269504088896341f;
+  auto tile_body = [&](bool masked, int p0) {
+    // ---- scores of four 16-position tiles
+    f32x4 s[4];
+#pragma unroll
+    for (int sub = 0; sub < 4; ++sub) {
+      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const bf16x8 kf = *(const bf16x8*)(sK + (sub * 16 + lr) * PT_KROW + ks * 32 + lg * 8);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[ks], acc, 0, 0, 0);
+      }
+      s[sub] = acc;
+    }
+    // ---- mask, running max, weights
+    if (masked) {
+#pragma unroll
+      for (int sub = 0; sub < 4; ++sub)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int p = p0 + sub * 16 + lg * 4 + j;
+          if (!(p >= col_lo && p <= col_pos)) s[sub][j] = -INFINITY;
+        }
+    }
+    float tile_max = -INFINITY;
+#pragma unroll
+    for (int sub = 0; sub < 4; ++sub)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) tile_max = fmaxf(tile_max, s[sub][j]);
+    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, 64));
+    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
+    const float m_new = fmaxf(m, tile_max);
+    bf16x8 pf[2] = {zero8(), zero8()};
+    if (__builtin_amdgcn_ballot_w64(m_new > m) != 0) {
+      const float alpha = (m_new > m && m > -INFINITY) ? __builtin_amdgcn_exp2f((m - m_new) * c2) : 1.f;
+      l *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) o[dt] *= alpha;
+      m = m_new;
+    }
+    if (m_new > -INFINITY) {   // a masked tile may hold nothing for this column yet
+      const float mc = m_new * c2;
+      float sum = 0.f;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const float w = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i >> 2][i & 3], c2, -mc));
+        sum += w;
+        pf[i >> 3][i & 7] = (__bf16)w;   // step 0: tiles 0 and 1; step 1: tiles 2 and 3
+      }
+      l += sum;
+    }
+    // ---- output: V^T operands from LDS
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+#pragma unroll
+      for (int step = 0; step < 2; ++step) {
+        const __bf16* vrow = sV + (dt * 16 + lr) * PT_VROW + step * 32 + lg * 4;
+        const bf16x4 v0 = *(const bf16x4*)vrow, v1 = *(const bf16x4*)(vrow + 16);
+        bf16x8 vf;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          vf[i] = v0[i];
+          vf[4 + i] = v1[i];
+        }
+        o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[step], o[dt], 0, 0, 0);
+      }
+    }
+  };
+
   const int first_tile = begin & ~(PT_KV - 1);
   lookup(first_tile);
   fetch(first_tile);
@@ -326,67 +403,8 @@ __global__ __launch_bounds__(PT_THREADS) void attn_prefill_kernel(
       fetch(p0 + PT_KV);        // with the page ids looked up one tile ago
       lookup(p0 + 2 * PT_KV);
     }
-    if (p0 < wave_end && p0 + PT_KV > wave_begin) {  // some of this tile is visible to this wave
-      // ---- scores of four 16-position tiles
-      f32x4 s[4];
-#pragma unroll
-      for (int sub = 0; sub < 4; ++sub) {
-        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          const bf16x8 kf = *(const bf16x8*)(sK + (sub * 16 + lr) * PT_KROW + ks * 32 + lg * 8);
-          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[ks], acc, 0, 0, 0);
-        }
-        s[sub] = acc;
-      }
-      // ---- mask, running max, weights
-      float sv[16];
-      float tile_max = -INFINITY;
-#pragma unroll
-      for (int sub = 0; sub < 4; ++sub)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const int p = p0 + sub * 16 + lg * 4 + j;
-          const bool visible = p >= col_lo && p <= col_pos;
-          const float x = visible ? s[sub][j] * scale : -INFINITY;
-          sv[sub * 4 + j] = x;
-          tile_max = fmaxf(tile_max, x);
-        }
-      tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, 64));
-      tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
-      const float m_new = fmaxf(m, tile_max);
-      float alpha = 1.f;
-      bf16x8 pf[2] = {zero8(), zero8()};
-      if (m_new > -INFINITY) {
-        alpha = __expf(m - m_new);
-        float sum = 0.f;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const float w = __expf(sv[i] - m_new);
-          sum += w;
-          pf[i >> 3][i & 7] = (__bf16)w;   // step 0: tiles 0 and 1; step 1: tiles 2 and 3
-        }
-        l = l * alpha + sum;
-        m = m_new;
-      }
-      // ---- output: V^T operands from LDS
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
-        o[dt] *= alpha;
-#pragma unroll
-        for (int step = 0; step < 2; ++step) {
-          const __bf16* vrow = sV + (dt * 16 + lr) * PT_VROW + step * 32 + lg * 4;
-          const bf16x4 v0 = *(const bf16x4*)vrow, v1 = *(const bf16x4*)(vrow + 16);
-          bf16x8 vf;
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            vf[i] = v0[i];
-            vf[4 + i] = v1[i];
-          }
-          o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[step], o[dt], 0, 0, 0);
-        }
-      }
-    }
+    if (p0 < wave_end && p0 + PT_KV > wave_begin)   // some of this tile is visible to this wave
+      tile_body(!(p0 + PT_KV - 1 <= wave_first && p0 >= wave_lo_max), p0);
     __syncthreads();  // everyone is done with this tile
     if (more) {
       stash();
