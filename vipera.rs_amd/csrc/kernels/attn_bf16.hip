@@ -203,14 +203,14 @@ __device__ __forceinline__ void load_q(const __bf16* qrow, int hd, bf16x8 (&qf)[
 // are fetched once per workgroup into LDS and read from there by all eight waves: while a tile is being
 // multiplied the next one's loads are in flight in registers, and the page ids of the tile after that
 // are already being looked up. Two workgroups fit a CU, so one's barriers and loads hide behind the
-// other's arithmetic. LDS rows are padded (K by 16 bytes, V^T by 8) so that the 16 rows of an operand read
-// fall into different banks.
+// other's arithmetic. LDS rows are padded by 16 bytes so that the 16 rows of an operand read fall into
+// different banks.
 constexpr int PT_WAVES = 8;
 constexpr int PT_THREADS = PT_WAVES * 64;
 constexpr int PT_TOKENS = PT_WAVES * 16;   // tokens of a tile
 constexpr int PT_KV = 64;                  // positions of a K/V tile
 constexpr int PT_KROW = HDP + 8;           // elements of a K row in LDS
-constexpr int PT_VROW = PT_KV + 4;         // elements of a V^T row in LDS: 136 bytes, see below
+constexpr int PT_VROW = PT_KV + 8;         // elements of a V^T row in LDS: 144 bytes
 constexpr int PT_PIECES = PT_KV * HDP / 8; // 16-byte pieces of a K tile, and of a V^T tile
 constexpr int PT_PER_THREAD = (PT_PIECES + PT_THREADS - 1) / PT_THREADS;
 
@@ -300,10 +300,12 @@ __global__ __launch_bounds__(PT_THREADS) void attn_prefill_kernel(
       const int id = tid + PT_THREADS * i;
       if (id < PT_PIECES) {
         *(bf16x8*)(sK + (id / (HDP / 8)) * PT_KROW + (id % (HDP / 8)) * 8) = k_stage[i];
-        // V^T rows are 136 bytes apart: the 8-byte reads of 16 rows then fall into 16 different pairs of
-        // banks (with 144 bytes rows r and r + 8 met in one; measured 11 % slower). A row is therefore
-        // only 8-byte aligned and a piece goes in as two halves.
-        __bf16* dst_v = sV + (id / (PT_KV / 8)) * PT_VROW + (id % (PT_KV / 8)) * 8;
+        // Within each group of 32 positions a V^T row is stored in the order in which the weights sit in
+        // the matrix instruction's operand: four positions of one 16-position tile, then the four at the
+        // same place in the next tile. A lane's operand is then one 16-byte read. A piece of 8 positions
+        // goes in as two halves, 16 bytes apart.
+        const int cv8 = (id % (PT_KV / 8)) * 8;   // first position of the piece within the tile
+        __bf16* dst_v = sV + (id / (PT_KV / 8)) * PT_VROW + (cv8 & 32) + ((cv8 & 8) ? 16 : 0) + ((cv8 & 16) ? 4 : 0);
         bf16x4 lo, hi;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -311,7 +313,7 @@ __global__ __launch_bounds__(PT_THREADS) void attn_prefill_kernel(
           hi[j] = v_stage[i][4 + j];
         }
         *(bf16x4*)dst_v = lo;
-        *(bf16x4*)(dst_v + 4) = hi;
+        *(bf16x4*)(dst_v + 8) = hi;
       }
     }
   };
@@ -378,14 +380,7 @@ __global__ __launch_bounds__(PT_THREADS) void attn_prefill_kernel(
     for (int dt = 0; dt < DT; ++dt) {
 #pragma unroll
       for (int step = 0; step < 2; ++step) {
-        const __bf16* vrow = sV + (dt * 16 + lr) * PT_VROW + step * 32 + lg * 4;
-        const bf16x4 v0 = *(const bf16x4*)vrow, v1 = *(const bf16x4*)(vrow + 16);
-        bf16x8 vf;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          vf[i] = v0[i];
-          vf[4 + i] = v1[i];
-        }
+        const bf16x8 vf = *(const bf16x8*)(sV + (dt * 16 + lr) * PT_VROW + step * 32 + lg * 8);
         o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[step], o[dt], 0, 0, 0);
       }
     }
