@@ -237,9 +237,10 @@ def serving(args, config, runtime, model, shape_name, layers_full, dtype_key) ->
     lengths = torch.randint(128, 8193, (requests,), generator=gen).tolist()
     prompts = [torch.randint(0, config.vocab_size, (n,), generator=gen).tolist() for n in lengths]
     pages = sum((n + new_tokens + args.block_size - 1) // args.block_size + 1 for n in lengths)
-    runner = ModelRunner(model, runtime, args.block_size, pages, requests + 1, use_graphs=True, max_context=args.ctx)
+    context = max(args.ctx, max(lengths) + new_tokens)   # the longest request has to fit
+    runner = ModelRunner(model, runtime, args.block_size, pages, requests + 1, use_graphs=True, max_context=context)
     engine = Engine(None, runner=runner, max_num_seqs=requests, max_num_batched_tokens=budget, chunk_size=chunk,
-                    max_model_len=args.ctx, pipelined=not args.in_turn)
+                    max_model_len=context, pipelined=not args.in_turn)
     # a short run first: kernel modules are compiled and loaded, decode graphs of the small buckets captured
     engine.generate([prompts[0][:600], prompts[1][:300]], 8)
     for prompt in prompts:
@@ -269,7 +270,7 @@ def serving(args, config, runtime, model, shape_name, layers_full, dtype_key) ->
         "data": "synthetic: seeded random weights N(0, 0.02) and uniform-random token ids",
         "config": {"model": shape_name, "layers": args.layers, "layers_full": layers_full, "requests": requests,
                    "prompt_tokens": prompt_tokens, "new_tokens_each": new_tokens, "chunk_size": chunk,
-                   "max_num_batched_tokens": budget, "seq_len": args.ctx, "block_size": args.block_size,
+                   "max_num_batched_tokens": budget, "seq_len": context, "block_size": args.block_size,
                    "steps_launched_ahead": not args.in_turn},
         "generated_per_second": round(generated / seconds, 1), "seconds": round(seconds, 3),
     }), flush=True)
