@@ -72,6 +72,14 @@ def test_rope_and_cache_write(dtype, hd, rotary_dim):
     kernels.rope_kvwrite(qkv_d, dev(torch.tensor(positions, dtype=torch.int32)), dev(inv), rotary_dim, k_d, v_d,
                          dev(torch.tensor(entry_of, dtype=torch.int32)), dev(table), heads, kv_heads, hd)
     got = qkv_d.float().cpu().numpy()
+    if rotary_dim:  # with the step's table of sines and cosines: the same bits in q, k and the cache
+        pos_d = dev(torch.tensor(positions, dtype=torch.int32))
+        angles = kernels.rope_angles(pos_d, dev(inv), len(positions))
+        assert angles.shape == (len(positions), rotary_dim // 2, 2)
+        qkv_t, k_t, v_t = dev(qkv.clone()), dev(k_cache), dev(v_cache)
+        kernels.rope_kvwrite(qkv_t, pos_d, dev(inv), rotary_dim, k_t, v_t, dev(torch.tensor(entry_of, dtype=torch.int32)),
+                             dev(table), heads, kv_heads, hd, angles)
+        assert torch.equal(qkv_t, qkv_d) and torch.equal(k_t, k_d) and torch.equal(v_t, v_d)
     tol = 2e-6 if dtype == torch.float32 else 8e-3
     for t, pos in enumerate(positions):
         # 32-bit rows make the plain rotation round the angle to 32-bit as the reference does (model.rs:4199-4201);

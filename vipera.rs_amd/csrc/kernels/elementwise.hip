@@ -116,11 +116,37 @@ extern "C" int vk_rmsnorm(const float* x, const float* weight, const int* rows, 
 // [page, kv_head, slot, hd]; V pages are transposed, [page, kv_head, hd, slot], so that the
 // attention kernels read consecutive positions of one output dim. A token whose page id is
 // negative writes nothing to the cache.
+// Sines and cosines of a step's rotation angles, once for all heads and all layers that share the
+// frequencies: out[t * half + i] = (sin, cos)(float(pos_t) * inv_freq[i]), the same expression in the same
+// precision as rope_kvwrite_kernel evaluates without a table (the reference keeps one table per position for
+// all layers, crates/vipera-backend-cpu/src/model.rs:4174-4181).
+__global__ void rope_angles_kernel(const int* __restrict__ positions, const float* __restrict__ inv_freq,
+                                   float2* __restrict__ out, int num_tokens, int half) {
+  const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (long long)num_tokens * half) return;
+  const int t = (int)(idx / half), i = (int)(idx % half);
+  float sn, cs;
+  sincosf((float)positions[t] * inv_freq[i], &sn, &cs);
+  out[idx] = make_float2(sn, cs);
+}
+
+extern "C" int vk_rope_angles(const int* positions, const float* inv_freq, int half, int num_tokens, float* out,
+                              void* stream) {
+  if (num_tokens <= 0 || half <= 0) return 0;
+  const long long total = (long long)num_tokens * half;
+  if (total > 0x7fffffffLL * 256) return VK_UNSUPPORTED_SIZE;
+  rope_angles_kernel<<<(unsigned)((total + 255) / 256), 256, 0, (hipStream_t)stream>>>(positions, inv_freq,
+                                                                                        (float2*)out, num_tokens, half);
+  VK_LAUNCH_CHECK();
+  return 0;
+}
+
 constexpr int ROPE_HEADS_PER_BLOCK = 4;  // one wave per head
 template <typename T>
 __global__ __launch_bounds__(ROPE_HEADS_PER_BLOCK * 64) void rope_kvwrite_kernel(
     T* __restrict__ qkv, const int* __restrict__ positions,
-                                                          const float* __restrict__ inv_freq, int rotary_dim,
+                                                          const float* __restrict__ inv_freq,
+                                                          const float2* __restrict__ angles, int rotary_dim,
                                                           T* __restrict__ k_cache, T* __restrict__ v_cache,
                                                           const int* __restrict__ entry_of_token,
                                                           const int* __restrict__ block_table, int table_width,
@@ -141,7 +167,13 @@ __global__ __launch_bounds__(ROPE_HEADS_PER_BLOCK * 64) void rope_kvwrite_kernel
     for (int i = lane; i < hd; i += 64) {
       if (i < half) {
         float sn, cs;
-        sincosf((float)pos * inv_freq[i], &sn, &cs);
+        if (angles) {
+          const float2 sc = angles[(size_t)t * half + i];
+          sn = sc.x;
+          cs = sc.y;
+        } else {
+          sincosf((float)pos * inv_freq[i], &sn, &cs);
+        }
         const float lo = to_float<T>(h[i]), hi = to_float<T>(h[i + half]);
         const T a = from_float<T>(lo * cs - hi * sn), b = from_float<T>(lo * sn + hi * cs);
         h[i] = a;
@@ -161,8 +193,9 @@ __global__ __launch_bounds__(ROPE_HEADS_PER_BLOCK * 64) void rope_kvwrite_kernel
   }
 }
 
-extern "C" int vk_rope_kvwrite(void* qkv, int dtype, const int* positions, const float* inv_freq, int rotary_dim,
-                               void* k_cache, void* v_cache, const int* entry_of_token, const int* block_table,
+// `angles` (may be null): the step's table from vk_rope_angles, [num_tokens, rotary_dim / 2] pairs.
+extern "C" int vk_rope_kvwrite(void* qkv, int dtype, const int* positions, const float* inv_freq, const float* angles,
+                               int rotary_dim, void* k_cache, void* v_cache, const int* entry_of_token, const int* block_table,
                                int table_width, int block_size, int num_tokens, int heads, int kv_heads, int hd,
                                void* stream) {
   if (num_tokens <= 0) return 0;
@@ -175,11 +208,13 @@ extern "C" int vk_rope_kvwrite(void* qkv, int dtype, const int* positions, const
   const dim3 grid(num_tokens, (total_heads + ROPE_HEADS_PER_BLOCK - 1) / ROPE_HEADS_PER_BLOCK);
   constexpr int threads = ROPE_HEADS_PER_BLOCK * 64;
   if (dtype == DT_F32)
-    rope_kvwrite_kernel<float><<<grid, threads, 0, s>>>((float*)qkv, positions, inv_freq, rotary_dim, (float*)k_cache,
+    rope_kvwrite_kernel<float><<<grid, threads, 0, s>>>((float*)qkv, positions, inv_freq, (const float2*)angles,
+                                                        rotary_dim, (float*)k_cache,
                                                         (float*)v_cache, entry_of_token, block_table, table_width,
                                                         block_size, heads, kv_heads, hd, total_heads);
   else if (dtype == DT_BF16)
-    rope_kvwrite_kernel<bf16_t><<<grid, threads, 0, s>>>((bf16_t*)qkv, positions, inv_freq, rotary_dim,
+    rope_kvwrite_kernel<bf16_t><<<grid, threads, 0, s>>>((bf16_t*)qkv, positions, inv_freq, (const float2*)angles,
+                                                         rotary_dim,
                                                          (bf16_t*)k_cache, (bf16_t*)v_cache, entry_of_token,
                                                          block_table, table_width, block_size, heads, kv_heads, hd,
                                                          total_heads);

@@ -53,6 +53,7 @@ class StepBatch:
     block_tables: Dict[int, torch.Tensor]  # group -> [E, width] int32
     token_source: Optional[torch.Tensor] = None    # [T] int32: -1, or the row of `sampled_tokens` that holds the token
     sampled_tokens: Optional[torch.Tensor] = None  # the sampler's output buffer on the device (set by the runner)
+    shared: Dict[object, torch.Tensor] = field(default_factory=dict)  # what parts compute once per step for all layers
     # host copies, for launch decisions
     host_counts: List[int] = field(default_factory=list)
     host_first_pos: List[int] = field(default_factory=list)

@@ -118,10 +118,24 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor
             "rmsnorm")
 
 
+def rope_angles(positions: torch.Tensor, inv_freq: torch.Tensor, num_tokens: int) -> torch.Tensor:
+    """``[num_tokens, len(inv_freq), 2]`` floats: sine and cosine of ``float(pos) * inv_freq`` for a step's
+    tokens, computed once where many heads and layers would each compute them again."""
+    _dev(positions, inv_freq)
+    _need(positions.dtype == torch.int32 and positions.numel() >= num_tokens, "rope_angles: positions")
+    _need(inv_freq.dtype == torch.float32 and inv_freq.is_contiguous(), "rope_angles: inv_freq must be float32")
+    out = torch.empty((num_tokens, inv_freq.numel(), 2), dtype=torch.float32, device=positions.device)
+    fn = _fn("elementwise", "vk_rope_angles", [_p, _p, _i, _i, _p, _p])
+    _status(fn(_ptr(positions), _ptr(inv_freq), inv_freq.numel(), num_tokens, _ptr(out), _stream()), "rope_angles")
+    return out
+
+
 def rope_kvwrite(qkv: torch.Tensor, positions: torch.Tensor, inv_freq: Optional[torch.Tensor], rotary_dim: int,
                  k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor], entry_of_token: torch.Tensor,
-                 block_table: Optional[torch.Tensor], heads: int, kv_heads: int, head_dim: int) -> None:
+                 block_table: Optional[torch.Tensor], heads: int, kv_heads: int, head_dim: int,
+                 angles: Optional[torch.Tensor] = None) -> None:
     """Rotate the q and k heads of ``qkv`` in place, then store the tokens' K and V in their pages.
+    ``angles``: the step's table from :func:`rope_angles`, used instead of computing sines and cosines here.
 
     ``k_cache``: ``[pages, kv_heads, block_size, head_dim]``; ``v_cache`` is transposed,
     ``[pages, kv_heads, head_dim, block_size]``; ``block_table``: ``[entries, width]``.
@@ -144,8 +158,12 @@ def rope_kvwrite(qkv: torch.Tensor, positions: torch.Tensor, inv_freq: Optional[
               "rope_kvwrite: block table")
         _need(entry_of_token.dtype == torch.int32 and entry_of_token.numel() >= num_tokens, "rope_kvwrite: entries")
         table_width, block_size = block_table.shape[1], k_cache.shape[2]
-    fn = _fn("elementwise", "vk_rope_kvwrite", [_p, _i, _p, _p, _i, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p])
-    _status(fn(_ptr(qkv), _dt(qkv, "qkv"), _ptr(positions), _ptr(inv_freq), rotary_dim, _ptr(k_cache), _ptr(v_cache),
+    if angles is not None:
+        _dev(angles)
+        _need(rotary_dim > 0 and angles.dtype == torch.float32 and angles.is_contiguous()
+              and angles.shape == (num_tokens, rotary_dim // 2, 2), "rope_kvwrite: angles must be [tokens, rotary_dim / 2, 2]")
+    fn = _fn("elementwise", "vk_rope_kvwrite", [_p, _i, _p, _p, _p, _i, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p])
+    _status(fn(_ptr(qkv), _dt(qkv, "qkv"), _ptr(positions), _ptr(inv_freq), _ptr(angles), rotary_dim, _ptr(k_cache), _ptr(v_cache),
                _ptr(entry_of_token), _ptr(block_table), table_width, block_size, num_tokens, heads, kv_heads,
                head_dim, _stream()), "rope_kvwrite")
 

@@ -87,13 +87,14 @@ class Attention(Mixer):
             inv_freq, rotary_dim = None, 0
         else:
             inv_freq, rotary_dim = fused
+        angles = position.step_angles(batch) if rotary_dim else None
         if reads_only:
             if rotary_dim:
                 kernels.rope_kvwrite(qkv, batch.positions, inv_freq, rotary_dim, None, None, batch.entry_of_token,
-                                     None, self.heads, self.kv_heads, self.head_dim)
+                                     None, self.heads, self.kv_heads, self.head_dim, angles)
         else:
             kernels.rope_kvwrite(qkv, batch.positions, inv_freq, rotary_dim, cache.k, cache.v, batch.entry_of_token,
-                                 table, self.heads, self.kv_heads, self.head_dim)
+                                 table, self.heads, self.kv_heads, self.head_dim, angles)
         attn = self.runtime.empty((tokens, self.q_width))
         paged_attention(qkv, cache.k, cache.v, attn, batch, table, self.heads, self.kv_heads, self.head_dim,
                         self.scale, self.window)

@@ -76,6 +76,11 @@ class PositionEncoding(Part):
     def fused_rotary(self):
         return None
 
+    def step_angles(self, batch):
+        """With ``fused_rotary``: a table of the step's sines and cosines that the rotation kernel may read
+        instead of computing them (shared by the layers of a step), or None."""
+        return None
+
     def apply(self, qkv: torch.Tensor, batch, heads: int, kv_heads: int, head_dim: int) -> None:
         raise NotImplementedError
 
