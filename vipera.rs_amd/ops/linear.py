@@ -56,6 +56,20 @@ def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     return fused.reshape(2 * inter, width).contiguous()
 
 
+def gated_rows_per_wave(m: int, n: int) -> int:
+    """One or two 16-row tiles per wave for the LDS-shared gated product (64 or 128 weight rows per workgroup).
+    A workgroup reads its weight rows and all of the activations; a CU's time goes with the bytes it pulls,
+    so what counts is how many workgroups the busiest CU gets (whole rounds over 256 CUs while they are few;
+    with three rounds or more the dispatcher evens them out) times the rows and padded tokens of each.
+    Measured at the 1.5B, 7B and 32B widths with 8 to 64 tokens; ties go to one tile."""
+    padded = (m + 15) // 16 * 16
+    def cost(rows: int) -> float:
+        groups = (n + rows - 1) // rows
+        rounds = groups / 256 if groups >= 768 else (groups + 255) // 256
+        return rounds * (rows + padded)
+    return 2 if cost(128) < cost(64) else 1
+
+
 def linear_gated(a: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor, interleaved: bool) -> torch.Tensor:
     """``out = up(a) * silu(gate(a))`` with the fused weight ``w_gate_up`` (``interleaved`` or ``[gate; up]``)."""
     m, k = a.shape
@@ -64,7 +78,7 @@ def linear_gated(a: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor, in
                and out.dtype == torch.bfloat16 and kernels.gemm_bf16_supported(a, w_gate_up, out))
     if fusable and m > 4:
         # the epilogue of the tiled kernel, or of the LDS-shared kernel with one K range, applies the gate
-        kernels.gemm_bf16_gated(a, w_gate_up, out, rows_per_wave=1)
+        kernels.gemm_bf16_gated(a, w_gate_up, out, rows_per_wave=gated_rows_per_wave(m, n))
         return out
     gate_up = torch.empty((m, n), dtype=out.dtype, device=out.device)
     linear(a, w_gate_up, None, gate_up)
