@@ -1,0 +1,191 @@
+"""Each kernel beside its plain C++ twin: the same parameter list goes to ``vk_*`` with device pointers and to
+``plain_*`` with host pointers, and the outputs are compared.  Sizes are not the engine's."""
+import ctypes
+import math
+
+import pytest
+import torch
+
+from helpers import rel_err
+from plain_cpp import DT, SIGNATURES, call
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _kernel(module: str, name: str):
+    from vipera_rs_amd.ops.build import load_module
+    fn = getattr(load_module(module), "vk_" + name)
+    fn.argtypes, fn.restype = SIGNATURES["plain_" + name], ctypes.c_int
+    return fn
+
+
+def both(module: str, name: str, args, outputs):
+    """Run kernel and twin on copies of ``args``; returns ``[(kernel output, twin output), ...]`` for the argument
+    indices in ``outputs``."""
+    host = [a.clone() if isinstance(a, torch.Tensor) else a for a in args]
+    dev = [a.to(DEV) if isinstance(a, torch.Tensor) else a for a in args]
+    call("plain_" + name, *host)
+    status = _kernel(module, name)(*[a.data_ptr() if isinstance(a, torch.Tensor) else a for a in dev])
+    torch.cuda.synchronize()
+    assert status == 0, f"vk_{name} returned {status}"
+    return [(dev[i].cpu(), host[i]) for i in outputs]
+
+
+def i32(values):
+    return torch.tensor(values, dtype=torch.int32)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_row_wise_kernels_beside_their_twins(dtype):
+    g = torch.Generator().manual_seed(7)
+    table = torch.randn(37, 50, generator=g).to(dtype)
+    (got, want), = both("elementwise", "embed_gather",
+                        [table, DT[dtype], i32([5, 36, 0, 99]), i32([-1, -1, 1, -1]), i32([7, 20]), torch.empty(4, 50), 4, 50,
+                         37, None], [5])
+    assert torch.equal(got, want) and torch.equal(got[2], table[20].float()) and torch.equal(got[3], table[0].float())
+    x, w = torch.randn(6, 1000, generator=g) * 3, 1 + 0.1 * torch.randn(1000, generator=g)
+    (got, want), = both("elementwise", "rmsnorm", [x, w, i32([4, 1, 5]), torch.empty(3, 1000, dtype=dtype), DT[dtype], 3, 1000,
+                                                   1e-5, None], [3])
+    assert rel_err(got.float().numpy(), want.double().numpy()) < (2e-6 if dtype == torch.float32 else 4e-3)
+    gate_up = (torch.randn(5, 2 * 208, generator=g) * 4).to(dtype)
+    for interleaved in (0, 1):
+        (got, want), = both("elementwise", "swiglu", [gate_up, torch.empty(5, 208, dtype=dtype), DT[dtype], 5, 208, interleaved,
+                                                      None], [1])
+        assert rel_err(got.float().numpy(), want.double().numpy()) < (2e-6 if dtype == torch.float32 else 4e-3)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("hd,rotary_dim", [(48, 48), (128, 128), (64, 32)])
+def test_rotation_and_cache_write_beside_its_twin(dtype, hd, rotary_dim):
+    heads, kv_heads, bs = 5, 2, 8
+    positions, entry_of = [0, 3, 8, 9, 1000, 41], [0, 0, 0, 0, 1, 1]
+    g = torch.Generator().manual_seed(hd + rotary_dim)
+    qkv = torch.randn(6, (heads + 2 * kv_heads) * hd, generator=g).to(dtype)
+    half = rotary_dim // 2
+    inv = (1.0 / torch.pow(torch.tensor(1e6), torch.arange(half).float() * 2 / rotary_dim)).float()
+    table = torch.full((2, 130), -1, dtype=torch.int32)
+    table[0, 0], table[0, 1], table[1, 1000 // bs], table[1, 41 // bs] = 5, 2, 7, 3
+    k_cache, v_cache = torch.zeros(9, kv_heads, bs, hd, dtype=dtype), torch.zeros(9, kv_heads, hd, bs, dtype=dtype)
+    (angles_d, angles_h), = both("elementwise", "rope_angles", [i32(positions), inv, half, 6, torch.empty(6, half, 2), None], [4])
+    assert rel_err(angles_d.numpy(), angles_h.double().numpy()) < 1e-6
+    for angles in (None, angles_d):
+        outs = both("elementwise", "rope_kvwrite",
+                    [qkv, DT[dtype], i32(positions), inv, angles, rotary_dim, k_cache, v_cache, i32(entry_of), table, 130, bs, 6,
+                     heads, kv_heads, hd, None], [0, 6, 7])
+        tol = 3e-6 if dtype == torch.float32 else 8e-3
+        for got, want in outs:
+            assert rel_err(got.float().numpy(), want.double().numpy()) < tol
+        assert torch.equal(outs[2][0], outs[2][1])                       # values are copied, not computed
+
+
+PRODUCTS = [(1, 48, 64), (7, 300, 96), (33, 1000, 264), (65, 130, 72), (200, 257, 136), (300, 520, 1024), (515, 384, 192)]
+
+
+@pytest.mark.parametrize("m,n,k", PRODUCTS)
+def test_products_beside_their_twins(m, n, k):
+    g = torch.Generator().manual_seed(m + n + k)
+    a, w, bias = torch.randn(m, k, generator=g), torch.randn(n, k, generator=g), torch.randn(n, generator=g)
+    (got, want), = both("gemm_generic", "gemm_generic", [a, 0, w, 0, bias, torch.empty(m, n), 0, m, n, k, k, n, 0, None], [5])
+    assert rel_err(got.numpy(), want.double().numpy()) < 2e-6
+    ab, wb = a.to(torch.bfloat16), w.to(torch.bfloat16)
+    for out_dtype, tol in ((torch.float32, 1e-5), (torch.bfloat16, 6e-3)):
+        (got, want), = both("gemm_bf16", "gemm_bf16", [ab, wb, bias, torch.empty(m, n, dtype=out_dtype), DT[out_dtype], m, n, k, k,
+                                                       n, 0, 64, 0, None, 0, None], [3])
+        assert rel_err(got.float().numpy(), want.double().numpy()) < tol
+    base = torch.randn(m, n, generator=g)
+    (got, want), = both("gemm_bf16", "gemm_bf16", [ab, wb, None, base, 0, m, n, k, k, n, 1, 64, 0, None, 0, None], [3])
+    assert rel_err(got.numpy(), want.double().numpy()) < 1e-5
+    if m <= 64:
+        partial = torch.empty(3 * m * n)
+        (got, want), = both("gemm_bf16", "gemm_bf16_mid", [ab, wb, bias, torch.empty(m, n), 0, m, n, k, k, n, 0, 3, 1, partial,
+                                                           partial.numel(), None], [3])
+        assert rel_err(got.numpy(), want.double().numpy()) < 1e-5
+
+
+@pytest.mark.parametrize("m,inter,k", [(5, 48, 96), (33, 128, 264), (64, 1024, 256), (300, 208, 192), (130, 1008, 640)])
+def test_gated_product_beside_its_twin(m, inter, k):
+    g = torch.Generator().manual_seed(m + inter + k)
+    a = torch.randn(m, k, generator=g).to(torch.bfloat16)
+    fused = torch.randn(2 * inter, k, generator=g).to(torch.bfloat16)
+    (got, want), = both("gemm_bf16", "gemm_bf16_gated", [a, fused, torch.empty(m, inter, dtype=torch.bfloat16), m, 2 * inter, k, k,
+                                                         inter, 1, None], [2])
+    assert rel_err(got.float().numpy(), want.double().numpy()) < 8e-3
+
+
+def _paged(T, kv_heads, hd, bs, dtype, seed, entries=1):
+    """A cache whose pages are dealt out in a shuffled order, and its table: [entries, pages per entry]."""
+    g = torch.Generator().manual_seed(seed)
+    per = (T + bs - 1) // bs
+    order = torch.randperm(entries * per + 3, generator=g)[: entries * per]
+    table = order.view(entries, per).to(torch.int32).contiguous()
+    k = torch.randn(entries * per + 3, kv_heads, bs, hd, generator=g).to(dtype)
+    v = torch.randn(entries * per + 3, kv_heads, hd, bs, generator=g).to(dtype)
+    return k, v, table
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("window", [0, 37])
+def test_generic_attention_beside_its_twin(dtype, window):
+    heads, kv_heads, hd, bs, T = 6, 3, 48, 8, 301
+    k, v, table = _paged(T, kv_heads, hd, bs, dtype, 11)
+    g = torch.Generator().manual_seed(12)
+    qkv = torch.randn(9, (heads + 2 * kv_heads) * hd, generator=g).to(dtype)
+    positions = i32([0, 1, 7, 8, 36, 37, 38, 255, 300])
+    (got, want), = both("attn_generic", "attn_generic",
+                        [qkv, qkv.shape[1], k, v, torch.empty(9, heads * hd, dtype=dtype), DT[dtype], positions, i32([0] * 9), table,
+                         table.shape[1], bs, 9, heads, kv_heads, hd, 1 / math.sqrt(hd), window, None], [4])
+    assert rel_err(got.float().numpy(), want.double().numpy()) < (3e-6 if dtype == torch.float32 else 8e-3)
+
+
+@pytest.mark.parametrize("hd", [64, 128, 80])
+@pytest.mark.parametrize("window", [0, 150])
+def test_matrix_core_attention_beside_its_twins(hd, window):
+    from vipera_rs_amd.ops import kernels
+    heads, kv_heads, bs = 6, 2, 16
+    module = f"attn_bf16_hd{kernels.attn_bf16_padded_width(hd)}"
+    first, count = 200, 300                       # a portion of 300 tokens after 200 cached ones, and a second entry of one token
+    k, v, table = _paged(first + count, kv_heads, hd, bs, torch.bfloat16, hd, entries=2)
+    g = torch.Generator().manual_seed(hd + 1)
+    T = count + 1
+    qkv = torch.randn(T, (heads + 2 * kv_heads) * hd, generator=g).to(torch.bfloat16)
+    entry_start, first_pos = i32([0, count, count + 1]), i32([first, 499])
+    tiles = i32([0, 256, 0, 0, 0, 128])           # any order of the tiles
+    (got, want), = both(module, "attn_bf16_prefill",
+                        [qkv, qkv.shape[1], k, v, torch.zeros(T, heads * hd, dtype=torch.bfloat16), tiles, 3, entry_start, first_pos,
+                         table, table.shape[1], bs, heads, kv_heads, hd, 1 / math.sqrt(hd), window, None], [4])
+    assert rel_err(got[:count].float().numpy(), want[:count].double().numpy()) < 8e-3
+    chunk, chunks = 128, 4
+    partial = torch.empty(1 * heads * chunks * (hd + 2))
+    (got, want), = both(module, "attn_bf16_decode",
+                        [qkv, qkv.shape[1], k, v, torch.zeros(T, heads * hd, dtype=torch.bfloat16), partial, i32([1]), 1, entry_start,
+                         first_pos, table, table.shape[1], bs, heads, kv_heads, hd, 1 / math.sqrt(hd), window, chunk, chunks, None],
+                        [4])
+    assert rel_err(got[count:].float().numpy(), want[count:].double().numpy()) < 8e-3
+
+
+def test_sampling_kernels_beside_their_twins():
+    g = torch.Generator().manual_seed(5)
+    rows, vocab = 40, 3001
+    logits = torch.randn(rows, vocab, generator=g) * 3
+    logits[3, 17] = float("inf")
+    logits[4, :] = float("nan")
+    logits[5, 100] = logits[5, 2000] = logits[5].max() + 1
+    temperature = torch.where(torch.arange(rows) < 8, torch.zeros(rows), 0.5 + torch.rand(rows, generator=g))
+    top_k = torch.where(torch.arange(rows) % 3 == 0, torch.full((rows,), 40), torch.zeros(rows)).to(torch.int32)
+    top_p = torch.where(torch.arange(rows) % 2 == 0, torch.full((rows,), 0.9), torch.ones(rows))
+    min_p = torch.where(torch.arange(rows) % 5 == 0, torch.full((rows,), 0.02), torch.zeros(rows))
+    uniform = torch.rand(rows, generator=g, dtype=torch.float64)
+    (got, want), = both("sampling", "sample", [logits, rows, vocab, temperature, top_k, top_p, min_p, uniform,
+                                               torch.empty(rows, dtype=torch.int32), None], [8])
+    assert torch.equal(got[:8], want[:8]) and got[4] == -1 and got[5] == 100
+    # a sampled row could differ where u * mass falls within rounding of a boundary between two kept tokens, or where a
+    # cut's edge rounds the other way; none of these seeded rows does
+    assert torch.equal(got, want)
+    pen = torch.randn(3, 500, generator=g)
+    args = [pen, 500, i32([0, 0, 2]), i32([3, 499, 3]), i32([2, 1, 4]), torch.tensor([1.3, 1.0, 0.7]), torch.tensor([0.2, 0.0, 0.1]),
+            torch.tensor([0.1, 0.5, 0.0]), 3, None]
+    (got, want), = both("sampling", "penalize", args, [0])
+    assert torch.allclose(got, want, rtol=1e-6, atol=1e-6)
+    (got, want), = both("sampling", "logit_bias", [pen, 500, i32([1, 2]), i32([4, 499]), torch.tensor([2.5, -1.0]), 2, None], [0])
+    assert torch.equal(got, want)
