@@ -1,10 +1,11 @@
-"""Plain C++ twins of the engine's kernels (``plain_kernels.cpp``), compiled with the host compiler into a
-temporary folder and called through ctypes.  A twin takes the parameter list of its ``vk_*`` kernel, with host
+"""Plain C++ twins of the engine's kernels (``plain_kernels.cpp``), compiled with the host compiler and called
+through ctypes.  A twin takes the parameter list of its ``vk_*`` kernel, with host
 pointers and the stream ignored.  Nothing of the engine is used here."""
 from __future__ import annotations
 
 import atexit
 import ctypes
+import hashlib
 import os
 import shutil
 import subprocess
@@ -35,15 +36,36 @@ SIGNATURES = {
 }
 
 
+def build() -> str:
+    """Compile the twins if no library of the current source is there; returns its path.  The library is named
+    after a hash of the source and lives beside it (``_build/``), or in a temporary folder where that cannot be
+    written."""
+    here = os.path.dirname(os.path.abspath(__file__))
+    source = os.path.join(here, "plain_kernels.cpp")
+    with open(source, "rb") as handle:
+        digest = hashlib.sha256(handle.read()).hexdigest()[:12]
+    folder = os.path.join(here, "_build")
+    target = os.path.join(folder, f"plain_kernels-{digest}.so")
+    if os.path.exists(target):
+        return target
+    try:
+        os.makedirs(folder, exist_ok=True)
+        probe = tempfile.NamedTemporaryFile(dir=folder, delete=True)
+        probe.close()
+    except OSError:
+        folder = tempfile.mkdtemp(prefix="plain_cpp_")
+        atexit.register(shutil.rmtree, folder, ignore_errors=True)
+        target = os.path.join(folder, f"plain_kernels-{digest}.so")
+    partial = target + f".{os.getpid()}.tmp"
+    subprocess.run(["g++", "-O2", "-std=c++17", "-shared", "-fPIC", "-Wall", "-o", partial, source], check=True)
+    os.replace(partial, target)
+    return target
+
+
 def library() -> ctypes.CDLL:
     global _lib
     if _lib is None:
-        folder = tempfile.mkdtemp(prefix="plain_cpp_")
-        atexit.register(shutil.rmtree, folder, ignore_errors=True)
-        target = os.path.join(folder, "plain_kernels.so")
-        source = os.path.join(os.path.dirname(os.path.abspath(__file__)), "plain_kernels.cpp")
-        subprocess.run(["g++", "-O2", "-std=c++17", "-shared", "-fPIC", "-Wall", "-o", target, source], check=True)
-        _lib = ctypes.CDLL(target)
+        _lib = ctypes.CDLL(build())
         for name, argtypes in SIGNATURES.items():
             fn = getattr(_lib, name)
             fn.argtypes, fn.restype = argtypes, I
