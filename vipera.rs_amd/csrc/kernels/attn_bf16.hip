@@ -214,6 +214,7 @@ constexpr int PT_VROW = PT_KV + 8;         // elements of a V^T row in LDS: 144 
 constexpr int PT_PIECES = PT_KV * HDP / 8; // 16-byte pieces of a K tile, and of a V^T tile
 constexpr int PT_PER_THREAD = (PT_PIECES + PT_THREADS - 1) / PT_THREADS;
 
+template <bool FAST>
 __global__ __launch_bounds__(PT_THREADS) void attn_prefill_kernel(
     const __bf16* __restrict__ q, long long q_stride, const __bf16* __restrict__ k_cache,
     const __bf16* __restrict__ v_cache, __bf16* __restrict__ out, const int* __restrict__ tiles,
@@ -268,30 +269,68 @@ __global__ __launch_bounds__(PT_THREADS) void attn_prefill_kernel(
   // per thread: PT_PER_THREAD pieces of the K tile (row r, 8 dims) and of the V^T tile (dim d, 8 positions)
   bf16x8 k_stage[PT_PER_THREAD], v_stage[PT_PER_THREAD];
   int k_page[PT_PER_THREAD], v_page[PT_PER_THREAD];
-  auto lookup = [&](int p0) {  // page ids of the tile at p0 (-1: nothing to read)
+  // FAST: the page size is a power of two that divides 64. Tiles start at multiples of 64, so which page of
+  // a tile a piece lies in, and where in that page, is the same for every tile: the thread keeps both, a tile's
+  // page id is one table read at a clamped index, and an address is one multiply-add. Nothing is loaded
+  // conditionally: a piece outside [begin, end) reads a page of the same request inside that range (finite
+  // numbers: the pool starts zeroed), and its positions are masked, or weigh zero, for every column.
+  int k_tab[PT_PER_THREAD], v_tab[PT_PER_THREAD];          // page of the piece within a tile
+  unsigned k_in[PT_PER_THREAD], v_in[PT_PER_THREAD];       // byte offset of the piece within its page
+  const unsigned page_bytes = (unsigned)(kv_heads * bs * hd * 2);
+  const int page_lo = ps.page(begin), page_hi = ps.page(end - 1);
+  if constexpr (FAST) {
 #pragma unroll
     for (int i = 0; i < PT_PER_THREAD; ++i) {
-      const int id = tid + PT_THREADS * i;
-      const int pk = p0 + id / (HDP / 8);
-      k_page[i] = (id < PT_PIECES && pk >= begin && pk < end) ? table[ps.page(pk)] : -1;
-      const int pv = p0 + (id % (PT_KV / 8)) * 8;  // eight positions of one page (8 divides the page size)
-      v_page[i] = (id < PT_PIECES && pv + 7 >= begin && pv < end) ? table[ps.page(pv)] : -1;
+      const int id = min(tid + PT_THREADS * i, PT_PIECES - 1);
+      const int r = id / (HDP / 8), ck = id % (HDP / 8);
+      k_tab[i] = r >> ps.shift;
+      k_in[i] = (unsigned)((((kvh * bs + (r & (bs - 1))) * hd) + min(ck * 8, hd - 8)) * 2);
+      const int d = id / (PT_KV / 8), cv = id % (PT_KV / 8);
+      v_tab[i] = (cv * 8) >> ps.shift;
+      v_in[i] = (unsigned)((((kvh * hd + min(d, hd - 1)) * bs) + ((cv * 8) & (bs - 1))) * 2);
+    }
+  }
+  auto lookup = [&](int p0) {  // page ids of the tile at p0 (without FAST, -1: nothing to read)
+    if constexpr (FAST) {
+      const int tp = p0 >> ps.shift;
+#pragma unroll
+      for (int i = 0; i < PT_PER_THREAD; ++i) {
+        k_page[i] = table[min(max(tp + k_tab[i], page_lo), page_hi)];
+        v_page[i] = table[min(max(tp + v_tab[i], page_lo), page_hi)];
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < PT_PER_THREAD; ++i) {
+        const int id = tid + PT_THREADS * i;
+        const int pk = p0 + id / (HDP / 8);
+        k_page[i] = (id < PT_PIECES && pk >= begin && pk < end) ? table[ps.page(pk)] : -1;
+        const int pv = p0 + (id % (PT_KV / 8)) * 8;  // eight positions of one page (8 divides the page size)
+        v_page[i] = (id < PT_PIECES && pv + 7 >= begin && pv < end) ? table[ps.page(pv)] : -1;
+      }
     }
   };
   auto fetch = [&](int p0) {
+    if constexpr (FAST) {
 #pragma unroll
-    for (int i = 0; i < PT_PER_THREAD; ++i) {
-      const int id = tid + PT_THREADS * i;
-      const int r = id / (HDP / 8), ck = id % (HDP / 8);
-      const int pk = p0 + r;
-      k_stage[i] = (k_page[i] >= 0 && ck * 8 < hd)
-                       ? *(const bf16x8*)(k_cache + (((size_t)k_page[i] * kv_heads + kvh) * bs + ps.slot(pk)) * hd + ck * 8)
-                       : zero8();
-      const int d = id / (PT_KV / 8), cv = id % (PT_KV / 8);
-      const int pv = p0 + cv * 8;
-      v_stage[i] = (v_page[i] >= 0 && d < hd)
-                       ? *(const bf16x8*)(v_cache + (((size_t)v_page[i] * kv_heads + kvh) * hd + d) * bs + ps.slot(pv))
-                       : zero8();
+      for (int i = 0; i < PT_PER_THREAD; ++i) {
+        k_stage[i] = *(const bf16x8*)((const char*)k_cache + ((size_t)(unsigned)k_page[i] * page_bytes + k_in[i]));
+        v_stage[i] = *(const bf16x8*)((const char*)v_cache + ((size_t)(unsigned)v_page[i] * page_bytes + v_in[i]));
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < PT_PER_THREAD; ++i) {
+        const int id = tid + PT_THREADS * i;
+        const int r = id / (HDP / 8), ck = id % (HDP / 8);
+        const int pk = p0 + r;
+        k_stage[i] = (k_page[i] >= 0 && ck * 8 < hd)
+                         ? *(const bf16x8*)(k_cache + (((size_t)k_page[i] * kv_heads + kvh) * bs + ps.slot(pk)) * hd + ck * 8)
+                         : zero8();
+        const int d = id / (PT_KV / 8), cv = id % (PT_KV / 8);
+        const int pv = p0 + cv * 8;
+        v_stage[i] = (v_page[i] >= 0 && d < hd)
+                         ? *(const bf16x8*)(v_cache + (((size_t)v_page[i] * kv_heads + kvh) * hd + d) * bs + ps.slot(pv))
+                         : zero8();
+      }
     }
   };
   auto stash = [&]() {
@@ -567,12 +606,15 @@ extern "C" int vk_attn_bf16_prefill(const void* q, long long q_stride, const voi
       heads % kv_heads || (q_stride & 7) || window < 0)
     return VK_UNSUPPORTED_SIZE;
   constexpr int lds_bytes = (PT_KV * PT_KROW + HDP * PT_VROW) * (int)sizeof(__bf16);
-  static bool configured = false;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute((const void*)attn_prefill_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       lds_bytes);
+  // page sizes that are powers of two dividing 64 take the kernel with fixed piece addresses
+  const bool fast = (block_size & (block_size - 1)) == 0 && block_size <= PT_KV &&
+                    (long long)kv_heads * block_size * hd * 2 < (1ll << 32);
+  auto kernel = fast ? attn_prefill_kernel<true> : attn_prefill_kernel<false>;
+  static bool configured[2] = {false, false};
+  if (!configured[fast]) {
+    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
     if (e != hipSuccess) return (int)e;
-    configured = true;
+    configured[fast] = true;
   }
   static int cus = 0;  // compute units of the device, for the pairing of long and short tiles
   if (cus == 0) {
@@ -583,7 +625,7 @@ extern "C" int vk_attn_bf16_prefill(const void* q, long long q_stride, const voi
     cus = count > 0 ? count : 1;
   }
   if ((long long)num_tiles * heads > 0x7fffffffLL) return VK_UNSUPPORTED_SIZE;
-  attn_prefill_kernel<<<num_tiles * heads, PT_THREADS, lds_bytes, (hipStream_t)stream>>>(
+  kernel<<<num_tiles * heads, PT_THREADS, lds_bytes, (hipStream_t)stream>>>(
       (const __bf16*)q, q_stride, (const __bf16*)k_cache, (const __bf16*)v_cache, (__bf16*)out, tiles, entry_start,
       entry_first_pos, block_table, table_width, block_size, heads, kv_heads, hd, scale, window, cus);
   VK_LAUNCH_CHECK();
