@@ -51,7 +51,7 @@ def test_rmsnorm_kernel(width, out_dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("hd,rotary_dim", [(16, 16), (48, 48), (128, 128), (64, 32), (32, 0)])
+@pytest.mark.parametrize("hd,rotary_dim", [(16, 16), (48, 48), (128, 128), (64, 32), (32, 0), (24, 12), (40, 20)])  # the last two: one element per lane
 def test_rope_and_cache_write(dtype, hd, rotary_dim):
     from vipera_rs_amd.ops import kernels
     from vipera_rs_amd.parts.rotary import neox_inverse_frequencies

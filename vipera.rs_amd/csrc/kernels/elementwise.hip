@@ -193,6 +193,67 @@ __global__ __launch_bounds__(ROPE_HEADS_PER_BLOCK * 64) void rope_kvwrite_kernel
   }
 }
 
+// The same work with 16 bytes per thread: a thread owns V consecutive dims of one head (V = 8 bfloat16 or 4 floats).
+// A chunk in the first half of the rotated dims rotates with its partner half a rotation width further on; a chunk
+// past the rotated dims of a key head is copied to the cache; a chunk of a value head is scattered into the
+// transposed page. Per element the arithmetic is that of rope_kvwrite_kernel. Needs head width, rotated width and
+// its half to be multiples of V.
+template <typename T>
+__global__ __launch_bounds__(256) void rope_kvwrite_vector_kernel(
+    T* __restrict__ qkv, const int* __restrict__ positions, const float* __restrict__ inv_freq,
+    const float2* __restrict__ angles, int rotary_dim, T* __restrict__ k_cache, T* __restrict__ v_cache,
+    const int* __restrict__ entry_of_token, const int* __restrict__ block_table, int table_width, int block_size,
+    int heads, int kv_heads, int hd, int total_heads) {
+  constexpr int V = 16 / (int)sizeof(T);
+  typedef T vec_t __attribute__((ext_vector_type(V)));
+  const int chunks = hd / V;
+  const int unit = blockIdx.y * blockDim.x + threadIdx.x;
+  if (unit >= total_heads * chunks) return;
+  const int t = blockIdx.x, head = unit / chunks, i0 = (unit % chunks) * V;
+  const int pos = positions[t];
+  T* h = qkv + (size_t)t * (heads + 2 * kv_heads) * hd + (size_t)head * hd;
+  const bool is_q = head < heads, is_k = !is_q && head < heads + kv_heads;
+  const int half = rotary_dim / 2;
+  int page = -1;
+  if (!is_q && k_cache != nullptr) page = block_table[(size_t)entry_of_token[t] * table_width + pos / block_size];
+  const int slot = pos % block_size;
+  if (is_q || is_k) {
+    const size_t k_at = is_k && page >= 0 ? (((size_t)page * kv_heads + (head - heads)) * block_size + slot) * hd : 0;
+    if (i0 < half) {
+      const vec_t lo = *(const vec_t*)(h + i0), hi = *(const vec_t*)(h + i0 + half);
+      vec_t a, b;
+#pragma unroll
+      for (int j = 0; j < V; ++j) {
+        float sn, cs;
+        if (angles) {
+          const float2 sc = angles[(size_t)t * half + i0 + j];
+          sn = sc.x;
+          cs = sc.y;
+        } else {
+          sincosf((float)pos * inv_freq[i0 + j], &sn, &cs);
+        }
+        const float l = to_float<T>(lo[j]), u = to_float<T>(hi[j]);
+        a[j] = from_float<T>(l * cs - u * sn);
+        b[j] = from_float<T>(l * sn + u * cs);
+      }
+      *(vec_t*)(h + i0) = a;
+      *(vec_t*)(h + i0 + half) = b;
+      if (is_k && page >= 0) {
+        *(vec_t*)(k_cache + k_at + i0) = a;
+        *(vec_t*)(k_cache + k_at + i0 + half) = b;
+      }
+    } else if (i0 >= rotary_dim && is_k && page >= 0) {
+      *(vec_t*)(k_cache + k_at + i0) = *(const vec_t*)(h + i0);
+    }
+  } else if (page >= 0) {
+    const int kvh = head - heads - kv_heads;
+    const size_t v_at = (((size_t)page * kv_heads + kvh) * hd + i0) * block_size + slot;
+    const vec_t v = *(const vec_t*)(h + i0);
+#pragma unroll
+    for (int j = 0; j < V; ++j) v_cache[v_at + (size_t)j * block_size] = v[j];
+  }
+}
+
 // `angles` (may be null): the step's table from vk_rope_angles, [num_tokens, rotary_dim / 2] pairs.
 extern "C" int vk_rope_kvwrite(void* qkv, int dtype, const int* positions, const float* inv_freq, const float* angles,
                                int rotary_dim, void* k_cache, void* v_cache, const int* entry_of_token, const int* block_table,
@@ -205,6 +266,26 @@ extern "C" int vk_rope_kvwrite(void* qkv, int dtype, const int* positions, const
   if (heads + 2 * kv_heads > 65535) return VK_UNSUPPORTED_SIZE;
   hipStream_t s = (hipStream_t)stream;
   const int total_heads = heads + (k_cache ? 2 : 1) * kv_heads;  // without a cache the value heads have nothing to do
+  {  // 16 bytes per thread where the widths allow it and the sines come from the step's table (a step of many
+     // tokens); computing eight sines in a row per thread is slower than one per lane (measured with 8 tokens)
+    const int v = dtype == DT_F32 ? 4 : 8;
+    const bool aligned = ((uintptr_t)qkv & 15) == 0 && ((uintptr_t)k_cache & 15) == 0;
+    if ((dtype == DT_F32 || dtype == DT_BF16) && angles != nullptr && aligned && hd % v == 0 && rotary_dim % v == 0 &&
+        (rotary_dim / 2) % v == 0) {
+      const int units = total_heads * (hd / v);
+      const dim3 vgrid(num_tokens, (units + 255) / 256);
+      if (dtype == DT_F32)
+        rope_kvwrite_vector_kernel<float><<<vgrid, 256, 0, s>>>(
+            (float*)qkv, positions, inv_freq, (const float2*)angles, rotary_dim, (float*)k_cache, (float*)v_cache,
+            entry_of_token, block_table, table_width, block_size, heads, kv_heads, hd, total_heads);
+      else
+        rope_kvwrite_vector_kernel<bf16_t><<<vgrid, 256, 0, s>>>(
+            (bf16_t*)qkv, positions, inv_freq, (const float2*)angles, rotary_dim, (bf16_t*)k_cache, (bf16_t*)v_cache,
+            entry_of_token, block_table, table_width, block_size, heads, kv_heads, hd, total_heads);
+      VK_LAUNCH_CHECK();
+      return 0;
+    }
+  }
   const dim3 grid(num_tokens, (total_heads + ROPE_HEADS_PER_BLOCK - 1) / ROPE_HEADS_PER_BLOCK);
   constexpr int threads = ROPE_HEADS_PER_BLOCK * 64;
   if (dtype == DT_F32)
