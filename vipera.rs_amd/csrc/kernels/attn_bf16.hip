@@ -534,6 +534,22 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(const float* __restric
   const int slot = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const size_t stride = hd + 2;
   const float* src = partial + ((size_t)slot * heads + h) * chunks * stride;
+  // lane -> (part, four output dims); part p sums the chunks c = p, p + parts, ... ; parts are added in order
+  const int quads = hd / 4;                         // hd is a multiple of 8
+  const int parts = quads >= 64 ? 1 : 64 / quads;
+  // Everything this wave reads is requested before anything is computed: the token's row, the chunks' (max, sum)
+  // and the first four chunks of each lane's sums. With a few chunks that is all of them, and the kernel is one
+  // round trip to memory instead of one per chunk behind the weights.
+  constexpr int AHEAD = 4;
+  const int token = entry_start[entries[slot]];
+  const int quad0 = parts > 1 ? lane % quads : lane, part0 = parts > 1 ? lane / quads : 0;
+  const bool active0 = quad0 < quads && part0 < parts;
+  f32x4 ahead[AHEAD];
+#pragma unroll
+  for (int u = 0; u < AHEAD; ++u) {
+    const int c = min(part0 + u * parts, chunks - 1);   // a clamped chunk's value is not used
+    ahead[u] = *(const f32x4*)(src + (size_t)c * stride + min(quad0, quads - 1) * 4);
+  }
   float mc[MAX_CHUNKS / 64], lc[MAX_CHUNKS / 64];
   float best = -INFINITY;
 #pragma unroll
@@ -555,20 +571,26 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(const float* __restric
   total = wave_sum(total);
   __syncthreads();
   const float inv = 1.f / total;
-  // lane -> (part, four output dims); part p sums the chunks c = p, p + parts, ... ; parts are added in order
-  const int quads = hd / 4;                         // hd is a multiple of 8
-  const int parts = quads >= 64 ? 1 : 64 / quads;
-  const int token = entry_start[entries[slot]];
   __bf16* dst = out + (size_t)token * heads * hd + (size_t)h * hd;
   for (int q0 = 0; q0 < quads; q0 += 64) {
-    const int quad = q0 + (parts > 1 ? lane % quads : lane);
-    const int part = parts > 1 ? lane / quads : 0;
+    const int quad = q0 + quad0;
+    const int part = part0;
     const bool active = quad < quads && part < parts;
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
     if (active) {
-      for (int c = part; c < chunks; c += parts) {
+      int c = part;
+      if (q0 == 0 && active0) {   // the chunks requested ahead
+#pragma unroll
+        for (int u = 0; u < AHEAD; ++u, c += parts) {
+          if (c >= chunks) break;
+          const float w = weight[c];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) acc[j] += w != 0.f ? ahead[u][j] * w : 0.f;   // an empty chunk holds stale numbers
+        }
+      }
+      for (; c < chunks; c += parts) {
         const float w = weight[c];
-        const f32x4 v = *(const f32x4*)(src + (size_t)c * stride + quad * 4);  // an empty chunk holds stale numbers
+        const f32x4 v = *(const f32x4*)(src + (size_t)c * stride + quad * 4);
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[j] += w != 0.f ? v[j] * w : 0.f;
       }

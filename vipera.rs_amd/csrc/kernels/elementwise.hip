@@ -60,15 +60,22 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ 
   TO* dst = out + (size_t)r * width;
   constexpr int MAXV = 8;  // up to 8 * 4 * 256 = 8192 columns stay in registers
   if ((width & 3) == 0 && width <= MAXV * 4 * 256) {
-    f32x4_t v[MAXV];
+    // the weights are requested together with the row, not after the sum: a row of a few tokens is all latency,
+    // and a second round trip to memory behind the barrier would be a third of it
+    f32x4_t v[MAXV], w[MAXV];
     float sum = 0.f;
 #pragma unroll
     for (int i = 0; i < MAXV; ++i) {
       const int c = (threadIdx.x + 256 * i) * 4;
       if (c < width) {
         v[i] = *(const f32x4_t*)(src + c);
-        sum += v[i][0] * v[i][0] + v[i][1] * v[i][1] + v[i][2] * v[i][2] + v[i][3] * v[i][3];
+        w[i] = *(const f32x4_t*)(weight + c);
       }
+    }
+#pragma unroll
+    for (int i = 0; i < MAXV; ++i) {
+      const int c = (threadIdx.x + 256 * i) * 4;
+      if (c < width) sum += v[i][0] * v[i][0] + v[i][1] * v[i][1] + v[i][2] * v[i][2] + v[i][3] * v[i][3];
     }
     sum = block_sum(sum, scratch);
     const float inv = 1.0f / sqrtf(sum / (float)width + eps);
@@ -76,9 +83,8 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ 
     for (int i = 0; i < MAXV; ++i) {
       const int c = (threadIdx.x + 256 * i) * 4;
       if (c < width) {
-        const f32x4_t w = *(const f32x4_t*)(weight + c);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) dst[c + j] = from_float<TO>(v[i][j] * inv * w[j]);
+        for (int j = 0; j < 4; ++j) dst[c + j] = from_float<TO>(v[i][j] * inv * w[i][j]);
       }
     }
     return;
