@@ -452,6 +452,18 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const __bf16* _
 #pragma unroll
     for (int cb = 0; cb < CB; ++cb) acc[rt][cb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+  // What the epilogue adds to the first tile this wave will store (bias, and the old C when accumulating) is
+  // requested now: read after the last product it would be one more round trip to memory at the end of a
+  // kernel that takes a few of them in all. Clamped addresses, so the loads are unconditional.
+  f32x4 early_bias = {0.f, 0.f, 0.f, 0.f}, early_c = {0.f, 0.f, 0.f, 0.f};
+  const bool early = vector_ok && wave < RT * CB && N >= 4;
+  const int early_m = (wave % CB) * 16 + lr, early_n = n0 + (wave / CB) * 16 + lg * 4;
+  if (early) {
+    const int m = min(early_m, M - 1), n = min(early_n, N - 4);
+    if (bias) early_bias = *(const f32x4*)(bias + n);
+    if constexpr (ACCUMULATE) early_c = *(const f32x4*)((const float*)C + (size_t)m * ldc + n);
+  }
+
   // SETS register sets of operands rotate through run_pipeline: the loads of SETS - 1 spans are in flight
   // while one span is multiplied (three sets with one block of tokens, two with more).
   bf16x8 wf[SETS][RT][4], af[SETS][CB][4];
@@ -516,6 +528,21 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const __bf16* _
 #pragma unroll
     for (int w = 1; w < WAVES; ++w) sum += partial[w][t][lane];
     const int rt = t / CB, cb = t % CB;
+    if (early && t == wave && early_m < M && early_n + 3 < N) {
+      // the same sums in the same order as store4, with the operands read at the start
+      if (bias) sum += early_bias;
+      TC* dst = C + (size_t)early_m * ldc + early_n;
+      if constexpr (sizeof(TC) == 4) {
+        if (ACCUMULATE) sum += early_c;
+        *(f32x4*)dst = sum;
+      } else {
+        bf16x4 o;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) o[j] = (__bf16)sum[j];
+        *(bf16x4*)dst = o;
+      }
+      continue;
+    }
     store4<TC, ACCUMULATE>(C, ldc, cb * 16 + lr, n0 + rt * 16 + lg * 4, M, N, sum, bias, vector_ok != 0);
   }
 }
