@@ -333,10 +333,14 @@ def test_gemm_mid_against_float64(m, n, k, ranges, rows_per_wave):
 
 
 @pytest.mark.parametrize("m,inter,k", [(1, 32, 64), (5, 48, 96), (8, 18944, 512), (16, 176, 200), (33, 128, 264), (64, 1024, 256),
-                                       (65, 64, 72), (300, 208, 136), (2048, 512, 128), (2048, 8208, 72), (100, 4608, 64)])
+                                       (65, 64, 72), (300, 208, 136), (2048, 512, 128), (2048, 8208, 72), (100, 4608, 64),
+                                       # the resident kernel: one pair on four waves, fewer units than waves, runs of
+                                       # uneven length, a wave's stretch inside one pair, many pairs per workgroup
+                                       (1, 16, 256), (3, 48, 256), (16, 16 * 37, 512), (5, 16 * 1000, 1024), (8, 16 * 257, 3584),
+                                       (16, 16 * 300, 4352), (2, 16 * 4111, 768), (7, 32, 2048)])
 def test_gated_product_and_interleaved_swiglu(m, inter, k):
     from vipera_rs_amd.ops import kernels
-    from vipera_rs_amd.ops.linear import interleave_gate_up, linear_gated
+    from vipera_rs_amd.ops.linear import gated_resident_fits, interleave_gate_up, linear_gated
     g = torch.Generator().manual_seed(m + inter + k)
     a = torch.randn(m, k, generator=g).to(torch.bfloat16).to(DEV)
     gate = torch.randn(inter, k, generator=g).to(torch.bfloat16).to(DEV)
@@ -349,6 +353,10 @@ def test_gated_product_and_interleaved_swiglu(m, inter, k):
         out = torch.full((m, inter), 7.0, dtype=torch.bfloat16, device=DEV)
         kernels.gemm_bf16_gated(a, fused, out, rows_per_wave)
         assert _rel(out, want) < 8e-3, f"fused epilogue, {rows_per_wave} tiles per wave"
+    if gated_resident_fits(m, 2 * inter, k):
+        out = torch.full((m, inter), 7.0, dtype=torch.bfloat16, device=DEV)
+        kernels.gemm_bf16_gated(a, fused, out, 0)
+        assert _rel(out, want) < 8e-3, "resident activations"
     out = torch.empty(m, inter, dtype=torch.bfloat16, device=DEV)
     linear_gated(a, fused, out, True)                       # whichever path the dispatch takes
     assert _rel(out, want) < 1.2e-2

@@ -103,13 +103,14 @@ def test_products_beside_their_twins(m, n, k):
         assert rel_err(got.numpy(), want.double().numpy()) < 1e-5
 
 
-@pytest.mark.parametrize("m,inter,k", [(5, 48, 96), (33, 128, 264), (64, 1024, 256), (300, 208, 192), (130, 1008, 640)])
-def test_gated_product_beside_its_twin(m, inter, k):
+@pytest.mark.parametrize("m,inter,k,plan", [(5, 48, 96, 1), (33, 128, 264, 1), (64, 1024, 256, 2), (300, 208, 192, 1),
+                                            (130, 1008, 640, 1), (6, 16 * 270, 768, 0), (16, 80, 1280, 0)])
+def test_gated_product_beside_its_twin(m, inter, k, plan):
     g = torch.Generator().manual_seed(m + inter + k)
     a = torch.randn(m, k, generator=g).to(torch.bfloat16)
     fused = torch.randn(2 * inter, k, generator=g).to(torch.bfloat16)
     (got, want), = both("gemm_bf16", "gemm_bf16_gated", [a, fused, torch.empty(m, inter, dtype=torch.bfloat16), m, 2 * inter, k, k,
-                                                         inter, 1, None], [2])
+                                                         inter, plan, None], [2])
     assert rel_err(got.float().numpy(), want.double().numpy()) < 8e-3
 
 

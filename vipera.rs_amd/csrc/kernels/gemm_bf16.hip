@@ -732,6 +732,203 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const __bf16* __restrict_
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// The gated product of up to 16 tokens with the activations resident in LDS. The launch has one workgroup
+// per CU (its LDS request keeps a second one away) and cuts the weight's pairs of 16 gate and 16 up rows
+// into as many contiguous runs, so every CU pulls the same number of bytes to within one pair: with a
+// fixed tile per workgroup the CUs that get one workgroup more than the others set the time. A workgroup
+// copies the activations into LDS once (all of K), and from then on its four waves do not meet: the run's
+// (pair, chunk of 256 k) units are cut into four equal stretches, a wave streams its stretch of weights
+// from HBM straight into operand registers, SETS register sets deep (two, three and four measured the
+// same), across pair boundaries without draining. Where a stretch begins or ends inside a pair the wave leaves its partial sums in LDS, and the
+// wave that holds the pair's first unit adds the parts in wave order: the order of the sums depends on N,
+// K and the number of workgroups only. K must be a multiple of 256.
+#ifndef VK_RESIDENT_SETS
+#define VK_RESIDENT_SETS 3
+#endif
+constexpr int RES_CHUNK = 256;
+constexpr int RES_PARTIAL_BYTES = 4 * 2 * 2 * 64 * 16;  // [wave][first or last pair of its stretch][gate, up][lane]
+
+template <int SETS>
+__global__ __launch_bounds__(256) void gemm_resident_gated_kernel(const __bf16* __restrict__ A,
+                                                                  const __bf16* __restrict__ W,
+                                                                  __bf16* __restrict__ C, int M, int N, int K,
+                                                                  long long lda, long long ldc) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char res_lds[];
+  f32x4* partial = (f32x4*)res_lds;
+  __bf16* acts = (__bf16*)(res_lds + RES_PARTIAL_BYTES);  // [M][K + 8]: 16 rows start in 16 different 16-byte slots
+  const int row_elems = K + 8;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lr = lane & 15, lg = lane >> 4;
+  const int chunks = K / RES_CHUNK, pairs = N / 32;
+  const int p_begin = (int)((long long)pairs * blockIdx.x / gridDim.x);
+  const int p_end = (int)((long long)pairs * (blockIdx.x + 1) / gridDim.x);
+  const int units = (p_end - p_begin) * chunks;
+  auto bound = [&](int w) { return (int)((long long)units * w / 4); };
+  const int u0 = bound(wave), u1 = bound(wave + 1), count = u1 - u0;
+  const int first_pair = u0 / chunks, first_chunk = u0 % chunks;  // within the workgroup's run
+
+  const size_t w_first_row = (size_t)(p_begin + first_pair) * 32;
+  const BufferView w_view = buffer_view(W + w_first_row * K, (unsigned long long)(N - w_first_row) * K * 2);
+  unsigned w_off[2];
+#pragma unroll
+  for (int rt = 0; rt < 2; ++rt) w_off[rt] = (unsigned)(((rt * 16 + lr) * K + lg * 8) * 2);
+  unsigned load_off = (unsigned)first_chunk * RES_CHUNK * 2;
+  int load_c = first_chunk;
+  const unsigned pair_skip = 62u * (unsigned)K;  // from the end of a pair's first row to the start of the next pair
+  bf16x8 w[SETS][2][8];
+  auto load_next = [&](bf16x8 (&dst)[2][8]) {
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) dst[rt][i] = w_view.load(w_off[rt] + load_off + i * 64);
+    load_off += RES_CHUNK * 2;
+    if (++load_c == chunks) {
+      load_c = 0;
+      load_off += pair_skip;
+    }
+  };
+
+  {  // Activations: 16-byte pieces in row-major order, 256 a pass, BATCH passes requested together. The weights
+     // of the first SETS - 1 units are requested right after the first batch: loads return in order, so the
+     // copy into LDS waits for its own loads only and the weights stay on their way through the barrier.
+    const BufferView a_view = buffer_view(A, ((unsigned long long)(M - 1) * lda + K) * 2);
+    const int k8 = K / 8, pieces = M * k8;
+    const int row_step = 256 / k8, col_step = 256 % k8;
+    int row = tid / k8, col = tid % k8;
+    constexpr int BATCH = 16;
+    bf16x8 stage[BATCH];
+    int at[BATCH];
+    auto request = [&]() {
+#pragma unroll
+      for (int j = 0; j < BATCH; ++j) {
+        at[j] = row < M ? row * row_elems + col * 8 : -1;
+        stage[j] = a_view.load((unsigned)((row * lda + col * 8) * 2));  // a row past the last reads zero
+        row += row_step;
+        col += col_step;
+        if (col >= k8) {
+          col -= k8;
+          ++row;
+        }
+      }
+    };
+    auto copy = [&]() {
+#pragma unroll
+      for (int j = 0; j < BATCH; ++j)
+        if (at[j] >= 0) *(bf16x8*)(acts + at[j]) = stage[j];
+    };
+    request();
+    static_for<SETS - 1>([&](auto j) {
+      if (j.value < count) load_next(w[j.value]);
+    });
+    copy();
+    for (int base = 256 * BATCH; base < pieces; base += 256 * BATCH) {
+      request();
+      copy();
+    }
+  }
+  __syncthreads();
+
+  // a token past M gives a column of the instruction that is never stored: its lanes read the last row
+  const __bf16* a_lane = acts + min(lr, M - 1) * row_elems + lg * 8;
+  f32x4 acc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
+  int mul_c = first_chunk, mul_p = first_pair;
+  bool first_part = true, from_start = first_chunk == 0;
+  auto flush = [&](bool to_end) {  // the sums of units [from_start ? 0 : first_chunk, mul_c) of pair mul_p
+    if (from_start && to_end) {
+      store_gated(C, ldc, lr, (p_begin + mul_p) * 16 + lg * 4, M, N / 2, acc[0], acc[1]);
+    } else {
+      f32x4* dst = partial + (wave * 2 + (first_part ? 0 : 1)) * 2 * 64;
+      dst[lane] = acc[0];
+      dst[64 + lane] = acc[1];
+    }
+    acc[0] = acc[1] = f32x4{0.f, 0.f, 0.f, 0.f};
+    first_part = false;
+    from_start = true;
+    mul_c = 0;
+    ++mul_p;
+  };
+  auto multiply = [&](const bf16x8 (&wf)[2][8]) {
+    const __bf16* a = a_lane + mul_c * RES_CHUNK;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const bf16x8 av = *(const bf16x8*)(a + i * 32);
+      acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[0][i], av, acc[0], 0, 0, 0);
+      acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[1][i], av, acc[1], 0, 0, 0);
+    }
+    ++mul_c;
+  };
+  auto step = [&](auto set_, auto rem_, int) {
+    constexpr int SET = decltype(set_)::value, REM = decltype(rem_)::value;
+    if constexpr (REM >= SETS - 1) load_next(w[(SET + SETS - 1) % SETS]);
+    multiply(w[SET]);
+    if constexpr (REM == 0) {
+      flush(mul_c == chunks);
+    } else {
+      if (mul_c == chunks) flush(true);
+    }
+  };
+  if (count >= SETS - 1) {
+    run_pipeline<SETS, SETS - 1>(step, count);
+  } else {  // fewer units than the pipeline is deep: all of them were requested above
+    static_for<SETS - 1>([&](auto j) {
+      if (j.value < count) {
+        multiply(w[j.value]);
+        if (j.value == count - 1 || mul_c == chunks) flush(mul_c == chunks);
+      }
+    });
+  }
+  __syncthreads();
+  // A pair that a stretch boundary cuts is finished by the wave that holds its first unit: its own part,
+  // then the first parts of the waves that follow, while they begin inside the pair.
+  if (wave < 3 && u1 % chunks != 0) {
+    const int p = u1 / chunks;
+    if (p * chunks >= u0 && count > 0) {
+      const f32x4* mine = partial + (wave * 2 + (p == first_pair ? 0 : 1)) * 2 * 64;
+      f32x4 gate = mine[lane], up = mine[64 + lane];
+      for (int w2 = wave + 1; w2 < 4 && bound(w2) < (p + 1) * chunks; ++w2) {
+        if (bound(w2 + 1) == bound(w2)) continue;
+        const f32x4* theirs = partial + w2 * 2 * 2 * 64;
+        gate += theirs[lane];
+        up += theirs[64 + lane];
+      }
+      store_gated(C, ldc, lr, (p_begin + p) * 16 + lg * 4, M, N / 2, gate, up);
+    }
+  }
+}
+
+// Whether the resident kernel takes the shape, and the LDS it asks for (0: it does not).
+int resident_lds_bytes(int M, int N, int K) {
+  if (M > 16 || (K % RES_CHUNK) || (N & 31)) return 0;
+  const long long need = RES_PARTIAL_BYTES + (long long)M * (K + 8) * 2;
+  if (need > 160 * 1024) return 0;
+  return (int)(need > 82 * 1024 ? need : 82 * 1024);  // more than half a CU's LDS: one workgroup per CU
+}
+
+int launch_resident_gated(const __bf16* A, const __bf16* W, __bf16* C, int M, int N, int K, long long lda,
+                          long long ldc, hipStream_t s) {
+  const int lds_bytes = resident_lds_bytes(M, N, K);
+  if (!lds_bytes) return VK_UNSUPPORTED_SIZE;
+  static int cus = 0;
+  auto kernel = gemm_resident_gated_kernel<VK_RESIDENT_SETS>;
+  if (!cus) {
+    int device = 0, count = 0;
+    hipError_t e = hipGetDevice(&device);
+    if (e == hipSuccess) e = hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, device);
+    if (e == hipSuccess) e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (e != hipSuccess) return (int)e;
+    cus = count > 0 ? count : 1;
+  }
+  const int pairs = N / 32;
+  const int groups = pairs < cus ? pairs : cus;
+  // byte offsets from a wave's first pair are 32-bit
+  if (((long long)(pairs / groups) + 2) * 64 * K >= (1ll << 31)) return VK_UNSUPPORTED_SIZE;
+  kernel<<<groups, 256, lds_bytes, s>>>(A, W, C, M, N, K, lda, ldc);
+  VK_LAUNCH_CHECK();
+  return 0;
+}
+
 // C (+)= sum over ranges of partial[range] (+ bias): ranges in ascending order, four columns per thread.
 template <typename TC, bool ACCUMULATE>
 __global__ void gemm_reduce_kernel(const float* __restrict__ partial, const float* __restrict__ bias,
@@ -997,7 +1194,9 @@ extern "C" int vk_gemm_bf16_mid(const void* A, const void* W, const float* bias,
 
 // out[M, N / 2] = up * silu(gate) of the product with a fused gate/up weight W[N, K] whose rows are
 // interleaved in groups of 16 (see store_gated). bfloat16 in and out; N a multiple of 32.
-// More than 64 tokens: the tiled kernel; up to 64: the LDS-shared kernel with one K range.
+// More than 64 tokens: the tiled kernel; up to 64: the LDS-shared kernel with one K range and `rows_per_wave`
+// (1 or 2) tiles of 16 rows per wave, or with `rows_per_wave` 0 the kernel that keeps the activations resident
+// in LDS (up to 16 tokens, K a multiple of 256, tokens x K within LDS; anything else is refused).
 extern "C" int vk_gemm_bf16_gated(const void* A, const void* W, void* C, int M, int N, int K, long long lda,
                                   long long ldc, int rows_per_wave, void* stream) {
   if (M <= 0 || N <= 0) return 0;
@@ -1009,6 +1208,7 @@ extern "C" int vk_gemm_bf16_gated(const void* A, const void* W, void* C, int M, 
   const __bf16* w = (const __bf16*)W;
   __bf16* c = (__bf16*)C;
   if (M > 64) return launch_tile<__bf16, false, true>(a, w, nullptr, c, M, N, K, lda, ldc, 0, nullptr, 0, s);
+  if (rows_per_wave == 0) return launch_resident_gated(a, w, c, M, N, K, lda, ldc, s);
   const int cb = (M + 15) / 16;
 #define VK_GATED(CBV, RTV)                                                                                         \
   {                                                                                                                \

@@ -448,9 +448,22 @@ def gemm_bf16_mid(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor]
             "gemm_bf16_mid")
 
 
+_COMPUTE_UNITS: dict = {}
+
+
+def compute_units(device: torch.device) -> int:
+    """CUs of the device (cached; what the launchers with one workgroup per CU use as their grid)."""
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    if index not in _COMPUTE_UNITS:
+        _COMPUTE_UNITS[index] = int(torch.cuda.get_device_properties(index).multi_processor_count)
+    return _COMPUTE_UNITS[index]
+
+
 def gemm_bf16_gated(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, rows_per_wave: int = 1) -> None:
     """``out = up * silu(gate)`` where ``[gate, up] = a @ w.T`` and ``w`` interleaves gate and up rows in
-    groups of 16.  ``out``: ``[tokens, w.shape[0] / 2]`` bfloat16."""
+    groups of 16.  ``out``: ``[tokens, w.shape[0] / 2]`` bfloat16.  ``rows_per_wave`` (up to 64 tokens): 1 or
+    2 tiles per wave of the LDS-shared kernel, or 0 for the kernel with resident activations (up to 16
+    tokens, K a multiple of 256, ``tokens x K`` within LDS; refused otherwise)."""
     _dev(a, w, out)
     m, k = a.shape
     n = w.shape[0]

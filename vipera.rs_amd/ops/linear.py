@@ -8,7 +8,8 @@ combination (the 32-bit run, or a matrix kept in 32-bit inside a bfloat16 run) g
 * up to 64 (decoding): the product is a stream of the weights.  Up to four tokens, or a small weight
   at up to 16 tokens, use the kernel whose waves split K inside a workgroup; otherwise the kernel that
   shares the activations through LDS, with K split over workgroups where the weight has too few rows
-  to fill the GPU otherwise.  The thresholds were measured on the 7B shapes on an MI355X.
+  to fill the GPU otherwise.  The thresholds were measured on the 7B shapes on an MI355X.  The gated
+  product of up to 16 tokens keeps all activations in LDS and gives every CU the same share of rows.
 """
 from __future__ import annotations
 
@@ -56,6 +57,15 @@ def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     return fused.reshape(2 * inter, width).contiguous()
 
 
+RESIDENT_LDS_BYTES = 160 * 1024 - 16 * 1024   # what the resident kernel may fill with activations
+
+
+def gated_resident_fits(m: int, n: int, k: int) -> bool:
+    """Whether the gated kernel that keeps all activations in LDS takes the shape: up to 16 tokens, K in
+    whole chunks of 256, and ``tokens x (K + 8)`` bfloat16 values within a CU's LDS."""
+    return m <= 16 and k % 256 == 0 and n % 32 == 0 and m * (k + 8) * 2 <= RESIDENT_LDS_BYTES
+
+
 def gated_rows_per_wave(m: int, n: int) -> int:
     """One or two 16-row tiles per wave for the LDS-shared gated product (64 or 128 weight rows per workgroup).
     A workgroup reads its weight rows and all of the activations; a CU's time goes with the bytes it pulls,
@@ -70,16 +80,31 @@ def gated_rows_per_wave(m: int, n: int) -> int:
     return 2 if cost(128) < cost(64) else 1
 
 
+def gated_plan(m: int, n: int, k: int, cus: int = 256) -> int:
+    """What :func:`kernels.gemm_bf16_gated` is asked for at up to 64 tokens: 0, the kernel with resident
+    activations and one workgroup per CU, where it takes the shape and the pairs of 16 gate and 16 up rows
+    divide evenly enough over the ``cus`` workgroups (the busiest within 15 % of the mean: at 7B and 32B
+    widths it measured 2 to 7 % faster than the LDS-shared kernel, at the 1.5B width, 2 or 3 pairs a
+    workgroup, 5 % slower); else the LDS-shared kernel with one or two tiles per wave."""
+    pairs = n // 32
+    if gated_resident_fits(m, n, k) and -(-pairs // cus) * cus <= 1.15 * pairs:
+        return 0
+    return gated_rows_per_wave(m, n)
+
+
 def linear_gated(a: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor, interleaved: bool) -> torch.Tensor:
     """``out = up(a) * silu(gate(a))`` with the fused weight ``w_gate_up`` (``interleaved`` or ``[gate; up]``)."""
     m, k = a.shape
     n = w_gate_up.shape[0]
     fusable = (interleaved and a.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16
                and out.dtype == torch.bfloat16 and kernels.gemm_bf16_supported(a, w_gate_up, out))
-    if fusable and m > 4:
-        # the epilogue of the tiled kernel, or of the LDS-shared kernel with one K range, applies the gate
-        kernels.gemm_bf16_gated(a, w_gate_up, out, rows_per_wave=gated_rows_per_wave(m, n))
-        return out
+    if fusable:
+        # the epilogue of the tiled kernel, of the resident kernel, or of the LDS-shared kernel with one K
+        # range applies the gate
+        plan = gated_plan(m, n, k, kernels.compute_units(a.device)) if m <= 64 else 1
+        if m > 4 or plan == 0:
+            kernels.gemm_bf16_gated(a, w_gate_up, out, rows_per_wave=plan)
+            return out
     gate_up = torch.empty((m, n), dtype=out.dtype, device=out.device)
     linear(a, w_gate_up, None, gate_up)
     kernels.swiglu(gate_up, out, interleaved)
