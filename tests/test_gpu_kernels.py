@@ -86,6 +86,32 @@ def test_gated_product_with_every_tiling(tiling):
         kernels.gemm_bf16_force_tiling(-1)
 
 
+@pytest.mark.parametrize("m,n,k", [(1, 100, 64), (8, 4608, 256), (16, 333, 520), (3, 9, 128), (5, 47, 72)])
+def test_skinny_product_with_every_number_of_rows_per_workgroup(m, n, k):
+    """A workgroup of the weight-streaming kernel may own 8 to 16 weight rows; the launcher picks the number
+    that divides N evenly over the CUs.  Every choice gives the same sums (the order within a row's sum does
+    not depend on it), beside bias, accumulation and both output types."""
+    from vipera_rs_amd.ops import kernels
+    g = torch.Generator().manual_seed(m + n + k)
+    a = torch.randn(m, k, generator=g).to(torch.bfloat16).to(DEV)
+    w = torch.randn(n, k, generator=g).to(torch.bfloat16).to(DEV)
+    bias = torch.randn(n, generator=g).to(DEV)
+    base = torch.randn(m, n, generator=g).to(DEV)
+    want = a.double() @ w.double().T + bias.double()
+    first = {}
+    for shape in [0] + list(range(108, 117)):
+        out = torch.full((m, n), 7.0, dtype=torch.bfloat16, device=DEV)
+        kernels.gemm_bf16(a, w, bias, out, skinny_shape=shape)
+        assert _rel(out, want) < 6e-3, shape
+        acc = base.clone()
+        kernels.gemm_bf16(a, w, bias, acc, accumulate=True, skinny_shape=shape)
+        assert _rel(acc, base.double() + want) < 1e-5, shape
+        if first:
+            assert torch.equal(out, first["out"]) and torch.equal(acc, first["acc"]), shape
+        first = first or {"out": out, "acc": acc}
+
+
+
 def test_gemm_bf16_tile_and_skinny_kernels_agree():
     from vipera_rs_amd.ops import kernels
     g = torch.Generator().manual_seed(5)
@@ -314,7 +340,7 @@ def test_attention_finds_one_far_key_among_hundreds(dtype):
 
 @pytest.mark.parametrize("m,n,k", [(1, 48, 64), (7, 300, 96), (8, 3584, 512), (16, 200, 1544), (17, 331, 520), (33, 1000, 264),
                                    (64, 520, 1024), (48, 130, 72), (64, 4608, 3584)])
-@pytest.mark.parametrize("ranges,rows_per_wave", [(1, 1), (1, 2), (3, 1), (8, 2)])
+@pytest.mark.parametrize("ranges,rows_per_wave", [(1, 1), (1, 2), (3, 1), (8, 2), (2, 110), (1, 114), (3, 109)])
 def test_gemm_mid_against_float64(m, n, k, ranges, rows_per_wave):
     from vipera_rs_amd.ops import kernels
     g = torch.Generator().manual_seed(m * 1000 + n + k)

@@ -72,11 +72,52 @@ __device__ __forceinline__ BufferView buffer_view(const void* base, unsigned lon
   return BufferView{__builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)range, 0x00020000)};
 }
 
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+// Four consecutive outputs of row m from column n on, columns at or past N left out. `align`: 4 when the
+// four may go as one vector (C, its row stride and the bias aligned to four elements and n a multiple of
+// four), 2 when pairs may (n even), else element by element.
+template <typename TC, bool ACCUMULATE>
+__device__ __forceinline__ void store4_aligned(TC* __restrict__ C, long long ldc, int m, int n, int M, int N, f32x4 v,
+                                               const float* __restrict__ bias, int align);
+
 template <typename TC, bool ACCUMULATE>
 __device__ __forceinline__ void store4(TC* __restrict__ C, long long ldc, int m, int n, int M, int N, f32x4 v,
                                        const float* __restrict__ bias, bool vector_ok) {
+  store4_aligned<TC, ACCUMULATE>(C, ldc, m, n, M, N, v, bias, vector_ok ? 4 : 1);
+}
+
+template <typename TC, bool ACCUMULATE>
+__device__ __forceinline__ void store4_aligned(TC* __restrict__ C, long long ldc, int m, int n, int M, int N, f32x4 v,
+                                               const float* __restrict__ bias, int align) {
   if (m >= M || n >= N) return;
   TC* dst = C + (size_t)m * ldc + n;
+  if (align == 2) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int nn = n + 2 * h;
+      if (nn + 1 < N) {
+        f32x2 x = {v[2 * h], v[2 * h + 1]};
+        if (bias) x += *(const f32x2*)(bias + nn);
+        if constexpr (sizeof(TC) == 4) {
+          f32x2* p = (f32x2*)(dst + 2 * h);
+          if (ACCUMULATE) x += *p;
+          *p = x;
+        } else {
+          bf16x2 o = {(__bf16)x[0], (__bf16)x[1]};
+          *(bf16x2*)(dst + 2 * h) = o;
+        }
+      } else if (nn < N) {
+        float x = v[2 * h];
+        if (bias) x += bias[nn];
+        if (ACCUMULATE) x += to_float<TC>(dst[2 * h]);
+        dst[2 * h] = from_float<TC>(x);
+      }
+    }
+    return;
+  }
+  const bool vector_ok = align == 4;
   if (vector_ok && n + 3 < N) {
     if (bias) {
       const f32x4 b = *(const f32x4*)(bias + n);
@@ -432,14 +473,20 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const __bf16* _
                                                                   const __bf16* __restrict__ W,
                                                                   const float* __restrict__ bias,
                                                                   TC* __restrict__ C, int M, int N, int K,
-                                                                  long long lda, long long ldc, int vector_ok) {
+                                                                  long long lda, long long ldc, int vector_ok,
+                                                                  int rows) {
   __shared__ f32x4 partial[WAVES][RT * CB][64];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lr = lane & 15, lg = lane >> 4;
-  const int n0 = blockIdx.x * 16 * RT;
-  // reads past the last weight row or the last token return zero and fetch nothing (see BufferView)
-  const BufferView w_view = buffer_view(W + (size_t)n0 * K, (unsigned long long)(N - n0) * K * 2);
+  // The workgroup owns weight rows [n0, n_end): `rows` of them, at most 16 * RT. Fewer than a full tile lets
+  // the launch cut N into as many equal workgroups as fill the CUs evenly; the instruction's other rows
+  // lie past the view's end.
+  const int n0 = blockIdx.x * rows, n_end = min(N, n0 + rows);
+  const int align = !vector_ok ? 1 : (n0 & 3) == 0 ? 4 : (n0 & 1) == 0 ? 2 : 1;
+  vector_ok = align == 4;
+  // reads past the workgroup's last weight row or the last token return zero and fetch nothing (see BufferView)
+  const BufferView w_view = buffer_view(W + (size_t)n0 * K, (unsigned long long)(n_end - n0) * K * 2);
   const BufferView a_view = buffer_view(A, ((unsigned long long)(M - 1) * lda + K) * 2);
   unsigned w_off[RT], a_off[CB];
 #pragma unroll
@@ -456,10 +503,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const __bf16* _
   // requested now: read after the last product it would be one more round trip to memory at the end of a
   // kernel that takes a few of them in all. Clamped addresses, so the loads are unconditional.
   f32x4 early_bias = {0.f, 0.f, 0.f, 0.f}, early_c = {0.f, 0.f, 0.f, 0.f};
-  const bool early = vector_ok && wave < RT * CB && N >= 4;
+  const bool early = vector_ok && wave < RT * CB && n_end - n0 >= 4;
   const int early_m = (wave % CB) * 16 + lr, early_n = n0 + (wave / CB) * 16 + lg * 4;
   if (early) {
-    const int m = min(early_m, M - 1), n = min(early_n, N - 4);
+    const int m = min(early_m, M - 1), n = min(early_n, n_end - 4);
     if (bias) early_bias = *(const f32x4*)(bias + n);
     if constexpr (ACCUMULATE) early_c = *(const f32x4*)((const float*)C + (size_t)m * ldc + n);
   }
@@ -528,7 +575,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const __bf16* _
 #pragma unroll
     for (int w = 1; w < WAVES; ++w) sum += partial[w][t][lane];
     const int rt = t / CB, cb = t % CB;
-    if (early && t == wave && early_m < M && early_n + 3 < N) {
+    if (early && t == wave && early_m < M && early_n + 3 < n_end) {
       // the same sums in the same order as store4, with the operands read at the start
       if (bias) sum += early_bias;
       TC* dst = C + (size_t)early_m * ldc + early_n;
@@ -543,15 +590,51 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const __bf16* _
       }
       continue;
     }
-    store4<TC, ACCUMULATE>(C, ldc, cb * 16 + lr, n0 + rt * 16 + lg * 4, M, N, sum, bias, vector_ok != 0);
+    store4_aligned<TC, ACCUMULATE>(C, ldc, cb * 16 + lr, n0 + rt * 16 + lg * 4, M, n_end, sum, bias, align);
   }
+}
+
+// CUs of the current device (asked once).
+int compute_units() {
+  static int cus = 0;
+  if (!cus) {
+    int device = 0, count = 0;
+    if (hipGetDevice(&device) != hipSuccess ||
+        hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess)
+      count = 0;
+    cus = count > 0 ? count : 256;
+  }
+  return cus;
+}
+
+// Weight rows per tile, 8 to 16 and even (outputs go out in pairs at least), for a launch of
+// `ranges` x ceil(N / (tiles * rows)) workgroups with `tiles` tiles each. A CU's time goes with the bytes it
+// pulls: the rounds of workgroups over the CUs (whole rounds while they are few; with three or more the
+// dispatcher evens them out) times a workgroup's rows, the activations counted as half a row per token (they
+// come from L2) and eight rows for what a workgroup costs before and after its stream. Fitted to sweeps of the
+// 7B and 32B products at 8 to 64 tokens. N = 3584 on 256 CUs: 256 workgroups of 14 rows instead of 224 of 16.
+int balanced_rows(int M, int N, int tiles, int ranges) {
+  const int cus = compute_units();
+  int best = 16;
+  double best_cost = 0.0;
+  for (int rows = 16; rows >= 8; rows -= 2) {
+    const long long groups = (long long)((N + tiles * rows - 1) / (tiles * rows)) * ranges;
+    const double rounds = groups >= 3 * cus ? (double)groups / cus : (double)((groups + cus - 1) / cus);
+    const double cost = rounds * (tiles * rows + 0.5 * M + 8.0);
+    if (rows == 16 || cost < best_cost * 0.97) {
+      best = rows;
+      best_cost = cost;
+    }
+  }
+  return best;
 }
 
 template <int CB, int RT, int WAVES, typename TC, bool ACC>
 int launch_skinny_as(const __bf16* A, const __bf16* W, const float* bias, TC* C, int M, int N, int K, long long lda,
-                     long long ldc, int vector_ok, hipStream_t s) {
-  const int blocks = (N + 16 * RT - 1) / (16 * RT);
-  gemm_skinny_kernel<CB, RT, WAVES, TC, ACC><<<blocks, WAVES * 64, 0, s>>>(A, W, bias, C, M, N, K, lda, ldc, vector_ok);
+                     long long ldc, int vector_ok, int rows, hipStream_t s) {
+  if (rows <= 0 || rows > 16 * RT) rows = RT == 1 ? balanced_rows(M, N, 1, 1) : 16 * RT;
+  const int blocks = (N + rows - 1) / rows;
+  gemm_skinny_kernel<CB, RT, WAVES, TC, ACC><<<blocks, WAVES * 64, 0, s>>>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, rows);
   VK_LAUNCH_CHECK();
   return 0;
 }
@@ -565,9 +648,11 @@ int launch_skinny_cb(const __bf16* A, const __bf16* W, const float* bias, TC* C,
   const int tiles = (N + 15) / 16;
   if (shape == 0) shape = (CB >= 2 && tiles >= 1024) ? 2 : 1;
   switch (shape) {
-    case 1: return launch_skinny_as<CB, 1, 4, TC, ACC>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, s);
-    case 2: return launch_skinny_as<CB, 2, 4, TC, ACC>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, s);
+    case 1: return launch_skinny_as<CB, 1, 4, TC, ACC>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, 0, s);
+    case 2: return launch_skinny_as<CB, 2, 4, TC, ACC>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, 0, s);
   }
+  if (shape >= 108 && shape <= 116)  // one tile per wave with a forced number of rows per workgroup
+    return launch_skinny_as<CB, 1, 4, TC, ACC>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, shape - 100, s);
   return VK_BAD_ARGUMENT;
 }
 
@@ -584,8 +669,8 @@ int launch_skinny(const __bf16* A, const __bf16* W, const float* bias, TC* C, in
 }
 
 // ---------------------------------------------------------------------------------------------
-// M <= 64, activations shared through LDS. A workgroup owns 64 * RT weight rows (16 * RT per wave)
-// and a range of K; all four waves walk that range together in chunks of 256. A chunk's activations
+// M <= 64, activations shared through LDS. A workgroup owns 64 * RT weight rows (16 * RT per wave; with
+// RT 1 the launcher may give a wave fewer rows, see balanced_rows) and a range of K; all four waves walk that range together in chunks of 256. A chunk's activations
 // (16 * CB tokens x 256) are fetched once per workgroup into LDS, double-buffered, one barrier per
 // chunk; the weights go from HBM straight into the instruction's operand layout, the next chunk's
 // loads in flight while the current one is multiplied. With several K ranges (gridDim.y > 1) every
@@ -599,21 +684,23 @@ template <int CB, int RT, typename TC, bool ACCUMULATE, bool GATED = false,
 __global__ __launch_bounds__(256) void gemm_mid_kernel(const __bf16* __restrict__ A, const __bf16* __restrict__ W,
                                                        const float* __restrict__ bias, TC* __restrict__ C, int M,
                                                        int N, int K, long long lda, long long ldc, int k_per_range,
-                                                       long long range_stride, int vector_ok) {
+                                                       long long range_stride, int vector_ok, int rows) {
   extern __shared__ __attribute__((aligned(16))) __bf16 lds[];  // [2][CB * 16][MID_ROW]
   constexpr int BUF = CB * 16 * MID_ROW;
   constexpr int A_LOADS = CB * 2;  // 16-byte pieces of a chunk per thread
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lr = lane & 15, lg = lane >> 4;
-  const int n0 = blockIdx.x * 64 * RT + wave * 16 * RT;
+  // a wave owns weight rows [n0, n_end): `rows` of them, at most 16 * RT (fewer than the tiles hold lets the
+  // launch cut N into as many equal workgroups as fill the CUs evenly; the other rows lie past the view's end)
+  const int n0 = (blockIdx.x * 4 + wave) * rows, n_end = min(N, n0 + rows);
   const int k_begin = blockIdx.y * k_per_range, k_end = min(K, k_begin + k_per_range);
   C += (size_t)blockIdx.y * range_stride;
 
   // Reads go through buffer descriptors: one past the end (a weight row past N, a token past M) returns
   // zero and fetches nothing, so no load of the pipeline below sits behind a branch, the compiler can
   // count exactly which loads a use waits for, and the later ones stay in flight.
-  const BufferView w_view = buffer_view(W + (size_t)min(n0, N - 1) * K, n0 < N ? (unsigned long long)(N - n0) * K * 2 : 0);
+  const BufferView w_view = buffer_view(W + (size_t)min(n0, N - 1) * K, n0 < N ? (unsigned long long)(n_end - n0) * K * 2 : 0);
   const BufferView a_view = buffer_view(A, ((unsigned long long)(M - 1) * lda + K) * 2);
   unsigned w_off[RT], a_off[A_LOADS];
 #pragma unroll
@@ -724,11 +811,12 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const __bf16* __restrict_
       }
     }
   } else {
+    const int align = !vector_ok ? 1 : (n0 & 3) == 0 ? 4 : (n0 & 1) == 0 ? 2 : 1;
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
       for (int cb = 0; cb < CB; ++cb)
-        store4<TC, ACCUMULATE>(C, ldc, cb * 16 + lr, n0 + rt * 16 + lg * 4, M, N, acc[rt][cb], bias, vector_ok != 0);
+        store4_aligned<TC, ACCUMULATE>(C, ldc, cb * 16 + lr, n0 + rt * 16 + lg * 4, M, n_end, acc[rt][cb], bias, align);
   }
 }
 
@@ -910,16 +998,14 @@ int launch_resident_gated(const __bf16* A, const __bf16* W, __bf16* C, int M, in
                           long long ldc, hipStream_t s) {
   const int lds_bytes = resident_lds_bytes(M, N, K);
   if (!lds_bytes) return VK_UNSUPPORTED_SIZE;
-  static int cus = 0;
   auto kernel = gemm_resident_gated_kernel<VK_RESIDENT_SETS>;
-  if (!cus) {
-    int device = 0, count = 0;
-    hipError_t e = hipGetDevice(&device);
-    if (e == hipSuccess) e = hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, device);
-    if (e == hipSuccess) e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (e != hipSuccess) return (int)e;
-    cus = count > 0 ? count : 1;
+    configured = true;
   }
+  const int cus = compute_units();
   const int pairs = N / 32;
   const int groups = pairs < cus ? pairs : cus;
   // byte offsets from a wave's first pair are 32-bit
@@ -954,9 +1040,11 @@ __global__ void gemm_reduce_kernel(const float* __restrict__ partial, const floa
 
 template <int CB, int RT, typename TC, bool ACC>
 int launch_mid_as(const __bf16* A, const __bf16* W, const float* bias, TC* C, float* partial, long long partial_floats,
-                  int ranges, int M, int N, int K, long long lda, long long ldc, int vector_ok, hipStream_t s) {
+                  int ranges, int forced_rows, int M, int N, int K, long long lda, long long ldc, int vector_ok,
+                  hipStream_t s) {
   constexpr int lds_bytes = 2 * CB * 16 * MID_ROW * (int)sizeof(__bf16);
-  const int blocks = (N + 64 * RT - 1) / (64 * RT);
+  const int rows = RT == 2 ? 32 : forced_rows ? forced_rows : balanced_rows(M, N, 4, ranges < 1 ? 1 : ranges);  // per wave
+  const int blocks = (N + 4 * rows - 1) / (4 * rows);
   if (ranges <= 1) {
     auto kernel = gemm_mid_kernel<CB, RT, TC, ACC>;
     static bool configured = false;
@@ -965,7 +1053,7 @@ int launch_mid_as(const __bf16* A, const __bf16* W, const float* bias, TC* C, fl
       if (e != hipSuccess) return (int)e;
       configured = true;
     }
-    kernel<<<dim3(blocks, 1), 256, lds_bytes, s>>>(A, W, bias, C, M, N, K, lda, ldc, K, 0, vector_ok);
+    kernel<<<dim3(blocks, 1), 256, lds_bytes, s>>>(A, W, bias, C, M, N, K, lda, ldc, K, 0, vector_ok, rows);
     VK_LAUNCH_CHECK();
     return 0;
   }
@@ -980,7 +1068,7 @@ int launch_mid_as(const __bf16* A, const __bf16* W, const float* bias, TC* C, fl
   const int k_per_range = ((K + ranges - 1) / ranges + MID_CHUNK - 1) / MID_CHUNK * MID_CHUNK;
   const int used = (K + k_per_range - 1) / k_per_range;
   kernel<<<dim3(blocks, used), 256, lds_bytes, s>>>(A, W, nullptr, partial, M, N, K, lda, N, k_per_range,
-                                                    (long long)M * N, (N & 3) == 0 ? 1 : 0);
+                                                    (long long)M * N, (N & 3) == 0 ? 1 : 0, rows);
   VK_LAUNCH_CHECK();
   const long long threads = (long long)M * ((N + 3) / 4);
   gemm_reduce_kernel<TC, ACC><<<(int)((threads + 255) / 256), 256, 0, s>>>(partial, bias, C, M, N, ldc, used, vector_ok);
@@ -993,7 +1081,9 @@ int launch_mid(const __bf16* A, const __bf16* W, const float* bias, TC* C, float
                int ranges, int rows_per_wave, int M, int N, int K, long long lda, long long ldc, int vector_ok,
                hipStream_t s) {
   const int cb = (M + 15) / 16;
-#define VK_MID(CBV, RTV) return launch_mid_as<CBV, RTV, TC, ACC>(A, W, bias, C, partial, partial_floats, ranges, M, N, K, lda, ldc, vector_ok, s)
+  // 108 to 116: one tile per wave with a forced number of rows (8 to 16), for tests and measurements
+  const int forced = rows_per_wave >= 108 && rows_per_wave <= 116 ? rows_per_wave - 100 : 0;
+#define VK_MID(CBV, RTV) return launch_mid_as<CBV, RTV, TC, ACC>(A, W, bias, C, partial, partial_floats, ranges, forced, M, N, K, lda, ldc, vector_ok, s)
   if (rows_per_wave == 2) {
     switch (cb) { case 1: VK_MID(1, 2); case 2: VK_MID(2, 2); case 3: VK_MID(3, 2); case 4: VK_MID(4, 2); }
   } else {
@@ -1134,7 +1224,8 @@ int launch_tile(const __bf16* A, const __bf16* W, const float* bias, TC* C, int 
 // A, W: bfloat16. c_dtype: 0 float, 1 bfloat16. accumulate needs a float C. Requirements (checked here):
 // K a multiple of 8 and lda a multiple of 8 (16-byte chunks); A and W 16-byte aligned.
 // `skinny_limit`: M at or below it takes the weight-streaming kernel (at most 64).
-// `skinny_shape`: 0 lets the launcher choose the row tiles per wave; 1 or 2 force one or two.
+// `skinny_shape`: 0 lets the launcher choose the row tiles per wave and the rows per workgroup; 1 or 2 force one
+// or two tiles; 108 to 116 force one tile and 8 to 16 rows per workgroup.
 // `partial` (may be null): a float workspace of `partial_floats` floats that the tiled kernel may split K into.
 extern "C" int vk_gemm_bf16(const void* A, const void* W, const float* bias, void* C, int c_dtype, int M, int N, int K,
                             long long lda, long long ldc, int accumulate, int skinny_limit, int skinny_shape,
@@ -1166,7 +1257,8 @@ extern "C" int vk_gemm_bf16(const void* A, const void* W, const float* bias, voi
 
 // The same product for M <= 64 with the activations shared through LDS. `ranges` > 1 splits K over
 // workgroups: partial sums go to `partial` (at least ranges * M * N floats) and a second kernel adds them.
-// rows_per_wave: 1 or 2 tiles of 16 weight rows per wave.
+// rows_per_wave: 1 or 2 tiles of 16 weight rows per wave; with 1 the launcher may give a wave fewer than 16 rows
+// (balanced_rows), and 108 to 116 force one tile with 8 to 16 rows.
 extern "C" int vk_gemm_bf16_mid(const void* A, const void* W, const float* bias, void* C, int c_dtype, int M, int N,
                                 int K, long long lda, long long ldc, int accumulate, int ranges, int rows_per_wave,
                                 float* partial, long long partial_floats, void* stream) {
@@ -1220,7 +1312,7 @@ extern "C" int vk_gemm_bf16_gated(const void* A, const void* W, void* C, int M, 
       if (e != hipSuccess) return (int)e;                                                                          \
       configured = true;                                                                                           \
     }                                                                                                              \
-    kernel<<<dim3((N + 64 * RTV - 1) / (64 * RTV), 1), 256, lds_bytes, s>>>(a, w, nullptr, c, M, N, K, lda, ldc, K, 0, 0); \
+    kernel<<<dim3((N + 64 * RTV - 1) / (64 * RTV), 1), 256, lds_bytes, s>>>(a, w, nullptr, c, M, N, K, lda, ldc, K, 0, 0, 16 * RTV); \
     VK_LAUNCH_CHECK();                                                                                             \
     return 0;                                                                                                      \
   }

@@ -430,7 +430,8 @@ def gemm_bf16_mid(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor]
     _need(m <= 64, "gemm_bf16_mid takes at most 64 rows")
     _need(w.shape[1] == k and out.shape == (m, n), f"gemm: shapes {tuple(a.shape)} x {tuple(w.shape)}^T -> {tuple(out.shape)}")
     _need(gemm_bf16_supported(a, w, out), "gemm_bf16: operands must be bfloat16, K a multiple of 8, rows 16-byte aligned")
-    _need(rows_per_wave in (1, 2) and ranges >= 1, "gemm_bf16_mid: rows_per_wave is 1 or 2, ranges at least 1")
+    _need((rows_per_wave in (1, 2) or 108 <= rows_per_wave <= 116) and ranges >= 1,
+          "gemm_bf16_mid: rows_per_wave is 1 or 2 (or 108 to 116: one tile with 8 to 16 rows), ranges at least 1")
     if bias is not None:
         _need(bias.dtype == torch.float32 and bias.numel() == n and bias.is_contiguous(), "gemm: bias must be float32 [n]")
     if accumulate:
