@@ -1288,7 +1288,8 @@ extern "C" int vk_gemm_bf16_mid(const void* A, const void* W, const float* bias,
 // interleaved in groups of 16 (see store_gated). bfloat16 in and out; N a multiple of 32.
 // More than 64 tokens: the tiled kernel; up to 64: the LDS-shared kernel with one K range and `rows_per_wave`
 // (1 or 2) tiles of 16 rows per wave, or with `rows_per_wave` 0 the kernel that keeps the activations resident
-// in LDS (up to 16 tokens, K a multiple of 256, tokens x K within LDS; anything else is refused).
+// in LDS (up to 16 tokens, K a multiple of 256, tokens x K within LDS; anything else is refused), or with
+// `rows_per_wave` 3 the tiled kernel.
 extern "C" int vk_gemm_bf16_gated(const void* A, const void* W, void* C, int M, int N, int K, long long lda,
                                   long long ldc, int rows_per_wave, void* stream) {
   if (M <= 0 || N <= 0) return 0;
@@ -1299,7 +1300,7 @@ extern "C" int vk_gemm_bf16_gated(const void* A, const void* W, void* C, int M, 
   const __bf16* a = (const __bf16*)A;
   const __bf16* w = (const __bf16*)W;
   __bf16* c = (__bf16*)C;
-  if (M > 64) return launch_tile<__bf16, false, true>(a, w, nullptr, c, M, N, K, lda, ldc, 0, nullptr, 0, s);
+  if (M > 64 || rows_per_wave == 3) return launch_tile<__bf16, false, true>(a, w, nullptr, c, M, N, K, lda, ldc, 0, nullptr, 0, s);
   if (rows_per_wave == 0) return launch_resident_gated(a, w, c, M, N, K, lda, ldc, s);
   const int cb = (M + 15) / 16;
 #define VK_GATED(CBV, RTV)                                                                                         \

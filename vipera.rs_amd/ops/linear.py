@@ -89,6 +89,10 @@ def gated_plan(m: int, n: int, k: int, cus: int = 256) -> int:
     pairs = n // 32
     if gated_resident_fits(m, n, k) and -(-pairs // cus) * cus <= 1.15 * pairs:
         return 0
+    if m * n * k >= 6.5e9:
+        # many tokens on a large weight: the tiled kernel (3), which reads a tile's activations once for 256
+        # weight rows, passes the LDS-shared one (7B widths from about 52 tokens, 32B from about 20, 1.5B never)
+        return 3
     return gated_rows_per_wave(m, n)
 
 
