@@ -1148,8 +1148,9 @@ int g_tile_config = -1;  // -1: chosen by shape; else 10 * ranges + tiling (see 
 // Which tiling, and into how many ranges K is split: the pair with the shortest estimated time. A full GPU
 // of 256x256 tiles runs at about 1.15 PFLOP/s with the kernel that loads straight into LDS and at 1.0
 // with the staged one (measured on the 7B shapes at 2,048 tokens); the smaller tiles reach 0.75 to 0.8 of
-// their kernel's best. Workgroups run in whole rounds of one per CU (two for the 128x128 tile, whose LDS
-// lets two share a CU), so a launch that fills the last round badly loses that share. Splitting K
+// their kernel's best, 256x192 about 0.9. Workgroups run in whole rounds of one per CU (two for the 128x128
+// tile, whose LDS lets two share a CU, unless every workgroup finds a CU of its own), so a launch that fills
+// the last round badly loses that share. Splitting K
 // multiplies the workgroups, at the price of writing and re-reading float partial sums (they mostly stay
 // in the caches: about 6 TB/s) and one more launch; each range keeps at least 512 of K. The estimate ranks
 // the plans as measurements at 128 to 2,048 tokens do. Few tokens keep the token side of the tile at 128.
@@ -1166,19 +1167,21 @@ TilePlan choose_tile_plan(int M, int N, int K, long long partial_floats, bool di
   }
   struct Tiling { int config, tokens, rows, resident; double speed; };
   static const Tiling staged[] = {{4, 256, 256, 1, 1.0}, {2, 256, 128, 1, 0.8}, {3, 128, 256, 1, 0.8}, {0, 128, 128, 2, 0.75}};
-  static const Tiling straight[] = {{5, 256, 256, 1, 1.15}, {7, 256, 128, 1, 0.92}, {8, 128, 256, 1, 0.88}, {9, 128, 128, 2, 0.9}};
+  static const Tiling straight[] = {{5, 256, 256, 1, 1.15}, {7, 256, 128, 1, 0.92}, {8, 128, 256, 1, 0.88}, {9, 128, 128, 2, 0.9},
+                                    {6, 256, 192, 1, 1.05}};
   const Tiling* tilings = direct ? straight : staged;
   TilePlan best{tilings[3].config, 1};
   double best_time = 1e30;
   const double flops = 2.0 * M * N * (double)K, output_bytes = 4.0 * M * N;
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < (direct ? 5 : 4); ++i) {
     const Tiling& t = tilings[i];
     if (M <= 128 && t.tokens > 128) continue;
     if (M > 128 && t.tokens == 128 && t.rows == 256) continue;  // with many tokens the wide side goes to the tokens
     const long long groups = (long long)((M + t.tokens - 1) / t.tokens) * ((N + t.rows - 1) / t.rows);
     for (int ranges = 1; ranges <= 8; ranges *= 2) {
       if (ranges > 1 && (K / ranges < 512 || (long long)ranges * M * N > partial_floats)) break;
-      const long long slots = (long long)g_compute_units * t.resident;
+      // workgroups that all find a CU of their own do not share one, however many would fit
+      const long long slots = groups * ranges <= g_compute_units ? g_compute_units : (long long)g_compute_units * t.resident;
       const long long rounds = (groups * ranges + slots - 1) / slots;
       const double fill = (double)(groups * ranges) / ((double)rounds * slots);
       double time = flops / (1e15 * t.speed * fill);
@@ -1193,7 +1196,8 @@ TilePlan choose_tile_plan(int M, int N, int K, long long partial_floats, bool di
 }
 
 // Tilings: 0, 2, 3, 4 the staged kernel at 128x128, 256x128, 128x256, 256x256; 9, 7, 8, 5 the same tiles
-// with the kernel that loads straight into LDS, which needs K to be a multiple of 64.
+// with the kernel that loads straight into LDS, which needs K to be a multiple of 64, and 6 that kernel at
+// 256x192 (2,048 tokens x 4,608 rows are 192 such tiles for 256 CUs, against 144 of 256x256).
 template <typename TC, bool ACC, bool GATED = false>
 int launch_tile(const __bf16* A, const __bf16* W, const float* bias, TC* C, int M, int N, int K, long long lda,
                 long long ldc, int vector_ok, float* partial, long long partial_floats, hipStream_t s) {
@@ -1202,13 +1206,14 @@ int launch_tile(const __bf16* A, const __bf16* W, const float* bias, TC* C, int 
   if (g_tile_config >= 0) plan = TilePlan{g_tile_config % 10, g_tile_config >= 10 && !GATED && partial ? g_tile_config / 10 : 1};
   if (plan.ranges > 1 && (long long)plan.ranges * M * N > partial_floats) plan.ranges = 1;
   if (!direct) {
-    switch (plan.config) { case 5: plan.config = 4; break; case 7: plan.config = 2; break; case 8: plan.config = 3; break; case 9: plan.config = 0; break; }
+    switch (plan.config) { case 5: case 6: plan.config = 4; break; case 7: plan.config = 2; break; case 8: plan.config = 3; break; case 9: plan.config = 0; break; }
   }
   const int r = plan.ranges;
 #define VK_TILE(BMV, BNV, WMV, WNV, DIRECTV) \
   return launch_tile_as<BMV, BNV, WMV, WNV, TC, ACC, GATED, DIRECTV>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, r, partial, s)
   switch (plan.config) {
     case 5: VK_TILE(256, 256, 4, 2, true);
+    case 6: VK_TILE(256, 192, 4, 2, true);
     case 7: VK_TILE(256, 128, 4, 2, true);
     case 8: VK_TILE(128, 256, 2, 4, true);
     case 9: VK_TILE(128, 128, 2, 2, true);

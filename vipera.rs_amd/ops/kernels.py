@@ -327,7 +327,7 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], ou
 
 
 TILE_TILINGS = {0: "128x128 staged", 2: "256x128 staged", 3: "128x256 staged", 4: "256x256 staged",
-                9: "128x128 direct", 7: "256x128 direct", 8: "128x256 direct", 5: "256x256 direct"}
+                9: "128x128 direct", 7: "256x128 direct", 8: "128x256 direct", 5: "256x256 direct", 6: "256x192 direct"}
 
 
 def gemm_bf16_force_tiling(tiling: int = -1, ranges: int = 1) -> None:
