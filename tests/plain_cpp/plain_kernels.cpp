@@ -231,6 +231,18 @@ extern "C" int plain_gemm_bf16_gated(const void* A, const void* W, void* C, int 
   return 0;
 }
 
+// The fused q/k/v product: the product in bfloat16, then the rotation and the cache write on its output.
+extern "C" int plain_gemm_bf16_qkv_rope(const void* A, const void* W, const float* bias, void* C, int M, int N, int K,
+                                        long long lda, long long ldc, const int* positions, const float* inv_freq,
+                                        void* k_cache, void* v_cache, const int* entry_of_token, const int* block_table,
+                                        int table_width, int block_size, int heads, int kv_heads, int hd, void*) {
+  if (M <= 0 || N <= 0) return 0;
+  if (K <= 0 || lda < K || ldc != N || (long long)(heads + 2 * kv_heads) * hd != N) return BAD_ARGUMENT;
+  product(A, DT_BF16, W, DT_BF16, bias, C, DT_BF16, M, N, K, lda, ldc, false);
+  return plain_rope_kvwrite(C, DT_BF16, positions, inv_freq, nullptr, hd, k_cache, v_cache, entry_of_token, block_table,
+                            table_width, block_size, M, heads, kv_heads, hd, nullptr);
+}
+
 // --- attention over the paged cache ----------------------------------------------------------------------------
 extern "C" int plain_attn_generic(const void* q, long long q_stride, const void* k_cache, const void* v_cache,
                                   void* out, int dtype, const int* positions, const int* entry_of_token,

@@ -79,6 +79,48 @@ def test_rotation_and_cache_write_beside_its_twin(dtype, hd, rotary_dim):
         assert torch.equal(outs[2][0], outs[2][1])                       # values are copied, not computed
 
 
+@pytest.mark.parametrize("m,heads,kv_heads,hd,k,with_bias,with_cache", [(6, 5, 2, 48, 96, True, True), (1, 4, 4, 128, 256, False, True),
+                                                                        (16, 3, 1, 16, 72, True, True), (3, 7, 1, 64, 520, True, False)])
+def test_fused_qkv_product_beside_its_twin_and_the_two_kernels(m, heads, kv_heads, hd, k, with_bias, with_cache):
+    """Product, rotation and cache write in one kernel: beside its twin, and bit for bit what the product followed
+    by the rotation kernel leaves in the q/k/v rows and in both caches (other pages untouched)."""
+    bs, n = 8, (heads + 2 * kv_heads) * hd
+    g = torch.Generator().manual_seed(m + n + k)
+    a = torch.randn(m, k, generator=g).to(torch.bfloat16)
+    w = (torch.randn(n, k, generator=g) / math.sqrt(k)).to(torch.bfloat16)
+    bias = torch.randn(n, generator=g) if with_bias else None
+    positions = [0, 3, 8, 9, 1000, 41, 7, 15, 16, 17, 100, 5, 2, 1, 63, 64][:m]
+    entry_of = [0, 0, 0, 0, 1, 1, 2, 2, 2, 2, 3, 3, 3, 3, 3, 3][:m]
+    inv = (1.0 / torch.pow(torch.tensor(1e6), torch.arange(hd // 2).float() * 2 / hd)).float()
+    table = torch.full((4, 130), -1, dtype=torch.int32)
+    pages = iter(torch.randperm(40, generator=g).tolist())
+    for e, pos in zip(entry_of, positions):
+        if table[e, pos // bs] < 0:
+            table[e, pos // bs] = next(pages)
+    table[0, 0] = -1                                     # a token without a page writes nothing to the cache
+    k_cache = torch.full((40, kv_heads, bs, hd), 9.0, dtype=torch.bfloat16) if with_cache else None
+    v_cache = torch.full((40, kv_heads, hd, bs), 9.0, dtype=torch.bfloat16) if with_cache else None
+    args = [a, w, bias, torch.empty(m, n, dtype=torch.bfloat16), m, n, k, k, n, i32(positions), inv, k_cache, v_cache,
+            i32(entry_of), table, 130, bs, heads, kv_heads, hd, None]
+    outs = both("gemm_bf16", "gemm_bf16_qkv_rope", args, [3, 11, 12] if with_cache else [3])
+    for got, want in outs:
+        assert rel_err(got.float().numpy(), want.double().numpy()) < 8e-3
+    # the same through the two kernels, on the device
+    from vipera_rs_amd.ops import kernels
+    dev = [x.to(DEV) if isinstance(x, torch.Tensor) else x for x in args]
+    qkv = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
+    kernels.gemm_bf16(dev[0], dev[1], dev[2], qkv)
+    kernels.rope_kvwrite(qkv, dev[9], dev[10], hd, dev[11], dev[12], dev[13], dev[14] if with_cache else None, heads, kv_heads, hd)
+    fused = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
+    kc, vc = (torch.full_like(dev[11], 9.0), torch.full_like(dev[12], 9.0)) if with_cache else (None, None)
+    kernels.gemm_bf16_qkv_rope(dev[0], dev[1], dev[2], fused, dev[9], dev[10], kc, vc, dev[13], dev[14] if with_cache else None,
+                               heads, kv_heads, hd)
+    assert torch.equal(fused, qkv)
+    if with_cache:
+        assert torch.equal(kc, dev[11]) and torch.equal(vc, dev[12])
+        assert torch.equal(kc.cpu(), outs[1][0]) and float((kc == 9.0).float().mean()) > 0.5
+
+
 PRODUCTS = [(1, 48, 64), (7, 300, 96), (33, 1000, 264), (65, 130, 72), (200, 257, 136), (300, 520, 1024), (515, 384, 192)]
 
 

@@ -466,51 +466,13 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_tile_direct_kernel(const __
 // ---------------------------------------------------------------------------------------------
 constexpr int SPAN = 128;  // k per wave per step: four instructions of 32
 
-// CB: blocks of 16 tokens (M <= 16 * CB). RT: tiles of 16 weight rows per wave. WAVES: waves of a
-// workgroup, which split K in interleaved spans. A workgroup owns 16 * RT weight rows.
-template <int CB, int RT, int WAVES, typename TC, bool ACCUMULATE, int SETS = (CB == 1 ? VK_SKINNY_SETS : 2)>
-__global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const __bf16* __restrict__ A,
-                                                                  const __bf16* __restrict__ W,
-                                                                  const float* __restrict__ bias,
-                                                                  TC* __restrict__ C, int M, int N, int K,
-                                                                  long long lda, long long ldc, int vector_ok,
-                                                                  int rows) {
-  __shared__ f32x4 partial[WAVES][RT * CB][64];
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int lr = lane & 15, lg = lane >> 4;
-  // The workgroup owns weight rows [n0, n_end): `rows` of them, at most 16 * RT. Fewer than a full tile lets
-  // the launch cut N into as many equal workgroups as fill the CUs evenly; the instruction's other rows
-  // lie past the view's end.
-  const int n0 = blockIdx.x * rows, n_end = min(N, n0 + rows);
-  const int align = !vector_ok ? 1 : (n0 & 3) == 0 ? 4 : (n0 & 1) == 0 ? 2 : 1;
-  vector_ok = align == 4;
-  // reads past the workgroup's last weight row or the last token return zero and fetch nothing (see BufferView)
-  const BufferView w_view = buffer_view(W + (size_t)n0 * K, (unsigned long long)(n_end - n0) * K * 2);
-  const BufferView a_view = buffer_view(A, ((unsigned long long)(M - 1) * lda + K) * 2);
-  unsigned w_off[RT], a_off[CB];
-#pragma unroll
-  for (int rt = 0; rt < RT; ++rt) w_off[rt] = (unsigned)(((rt * 16 + lr) * K + lg * 8) * 2);
-#pragma unroll
-  for (int cb = 0; cb < CB; ++cb) a_off[cb] = (unsigned)(((cb * 16 + lr) * lda + lg * 8) * 2);
-  f32x4 acc[RT][CB];
-#pragma unroll
-  for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-    for (int cb = 0; cb < CB; ++cb) acc[rt][cb] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-  // What the epilogue adds to the first tile this wave will store (bias, and the old C when accumulating) is
-  // requested now: read after the last product it would be one more round trip to memory at the end of a
-  // kernel that takes a few of them in all. Clamped addresses, so the loads are unconditional.
-  f32x4 early_bias = {0.f, 0.f, 0.f, 0.f}, early_c = {0.f, 0.f, 0.f, 0.f};
-  const bool early = vector_ok && wave < RT * CB && n_end - n0 >= 4;
-  const int early_m = (wave % CB) * 16 + lr, early_n = n0 + (wave / CB) * 16 + lg * 4;
-  if (early) {
-    const int m = min(early_m, M - 1), n = min(early_n, n_end - 4);
-    if (bias) early_bias = *(const f32x4*)(bias + n);
-    if constexpr (ACCUMULATE) early_c = *(const f32x4*)((const float*)C + (size_t)m * ldc + n);
-  }
-
+// The K loop of the weight-streaming kernels: wave `wave` of WAVES multiplies the spans wave, wave + WAVES, ...
+// of K (and the rest of K, less than a span, falls to one of them) into acc. w_off / a_off: a lane's byte offsets
+// of its operand rows at k = 0.
+template <int CB, int RT, int WAVES, int SETS>
+__device__ __forceinline__ void skinny_products(const BufferView& w_view, const BufferView& a_view,
+                                                const unsigned (&w_off)[RT], const unsigned (&a_off)[CB], int K, int wave,
+                                                int lg, f32x4 (&acc)[RT][CB]) {
   // SETS register sets of operands rotate through run_pipeline: the loads of SETS - 1 spans are in flight
   // while one span is multiplied (three sets with one block of tokens, two with more).
   bf16x8 wf[SETS][RT][4], af[SETS][CB][4];
@@ -564,6 +526,54 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const __bf16* _
       }
     multiply(wf[0], af[0]);
   }
+}
+
+// CB: blocks of 16 tokens (M <= 16 * CB). RT: tiles of 16 weight rows per wave. WAVES: waves of a
+// workgroup, which split K in interleaved spans. A workgroup owns 16 * RT weight rows.
+template <int CB, int RT, int WAVES, typename TC, bool ACCUMULATE, int SETS = (CB == 1 ? VK_SKINNY_SETS : 2)>
+__global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const __bf16* __restrict__ A,
+                                                                  const __bf16* __restrict__ W,
+                                                                  const float* __restrict__ bias,
+                                                                  TC* __restrict__ C, int M, int N, int K,
+                                                                  long long lda, long long ldc, int vector_ok,
+                                                                  int rows) {
+  __shared__ f32x4 partial[WAVES][RT * CB][64];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lr = lane & 15, lg = lane >> 4;
+  // The workgroup owns weight rows [n0, n_end): `rows` of them, at most 16 * RT. Fewer than a full tile lets
+  // the launch cut N into as many equal workgroups as fill the CUs evenly; the instruction's other rows
+  // lie past the view's end.
+  const int n0 = blockIdx.x * rows, n_end = min(N, n0 + rows);
+  const int align = !vector_ok ? 1 : (n0 & 3) == 0 ? 4 : (n0 & 1) == 0 ? 2 : 1;
+  vector_ok = align == 4;
+  // reads past the workgroup's last weight row or the last token return zero and fetch nothing (see BufferView)
+  const BufferView w_view = buffer_view(W + (size_t)n0 * K, (unsigned long long)(n_end - n0) * K * 2);
+  const BufferView a_view = buffer_view(A, ((unsigned long long)(M - 1) * lda + K) * 2);
+  unsigned w_off[RT], a_off[CB];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) w_off[rt] = (unsigned)(((rt * 16 + lr) * K + lg * 8) * 2);
+#pragma unroll
+  for (int cb = 0; cb < CB; ++cb) a_off[cb] = (unsigned)(((cb * 16 + lr) * lda + lg * 8) * 2);
+  f32x4 acc[RT][CB];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb) acc[rt][cb] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // What the epilogue adds to the first tile this wave will store (bias, and the old C when accumulating) is
+  // requested now: read after the last product it would be one more round trip to memory at the end of a
+  // kernel that takes a few of them in all. Clamped addresses, so the loads are unconditional.
+  f32x4 early_bias = {0.f, 0.f, 0.f, 0.f}, early_c = {0.f, 0.f, 0.f, 0.f};
+  const bool early = vector_ok && wave < RT * CB && n_end - n0 >= 4;
+  const int early_m = (wave % CB) * 16 + lr, early_n = n0 + (wave / CB) * 16 + lg * 4;
+  if (early) {
+    const int m = min(early_m, M - 1), n = min(early_n, n_end - 4);
+    if (bias) early_bias = *(const f32x4*)(bias + n);
+    if constexpr (ACCUMULATE) early_c = *(const f32x4*)((const float*)C + (size_t)m * ldc + n);
+  }
+
+  skinny_products<CB, RT, WAVES, SETS>(w_view, a_view, w_off, a_off, K, wave, lg, acc);
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
@@ -666,6 +676,97 @@ int launch_skinny(const __bf16* A, const __bf16* W, const float* bias, TC* C, in
     case 4: return launch_skinny_cb<4, TC, ACC>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, shape, s);
   }
   return VK_UNSUPPORTED_SIZE;
+}
+
+// ---------------------------------------------------------------------------------------------
+// The q/k/v product of up to 16 tokens with the rotation and the cache write in its epilogue, which saves the
+// launch between the product and the attention of a decode step. The streaming is gemm_skinny_kernel's (four
+// waves split K). A workgroup owns 16 outputs of one head: for a q or k head eight dims of the first half and
+// their eight partners half a head further on (rows 0-7 and 8-15 of the instruction's tile, so a lane finds a
+// dim's partner in lane ^ 32), for a v head 16 consecutive dims. The sums take the bias, are rounded to bfloat16
+// as the product alone would leave them, and are then rotated and stored exactly as rope_kvwrite_kernel does
+// (crates/vipera-backend-cpu/src/model.rs:4192-4251, 1495-1542): what the cache and the attention see does not
+// depend on which of the two paths a token took. Full rotation only (rotary width = head width, a multiple of 16).
+struct QkvRope {
+  const int* positions;
+  const float* inv_freq;
+  __bf16* k_cache;  // null: rotate only (a layer that reads another layer's cache)
+  __bf16* v_cache;
+  const int* entry_of_token;
+  const int* block_table;
+  int table_width, block_size, heads, kv_heads, hd;
+};
+
+__global__ __launch_bounds__(256) void gemm_qkv_rope_kernel(const __bf16* __restrict__ A, const __bf16* __restrict__ W,
+                                                            const float* __restrict__ bias, __bf16* __restrict__ C,
+                                                            int M, int N, int K, long long lda, long long ldc, QkvRope r) {
+  constexpr int WAVES = 4;
+  __shared__ f32x4 partial[WAVES][64];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lr = lane & 15, lg = lane >> 4;
+  const int hd = r.hd, half = hd / 2, groups = hd / 16;
+  const int head = blockIdx.x / groups, g = blockIdx.x % groups;
+  const bool is_q = head < r.heads, is_v = head >= r.heads + r.kv_heads;
+  // the weight row of the tile's row `i`, and the dim within the head of the lane's first output
+  auto dim_of = [&](int i) { return is_v ? 16 * g + i : (i < 8 ? 8 * g + i : half + 8 * g + i - 8); };
+  const int d0 = dim_of(lg * 4), n0 = head * hd + d0;
+  const BufferView w_view = buffer_view(W, (unsigned long long)N * K * 2);
+  const BufferView a_view = buffer_view(A, ((unsigned long long)(M - 1) * lda + K) * 2);
+  const unsigned w_off[1] = {(unsigned)((((size_t)head * hd + dim_of(lr)) * K + lg * 8) * 2)};
+  const unsigned a_off[1] = {(unsigned)((lr * lda + lg * 8) * 2)};
+  // what the epilogue needs from memory is requested now (clamped, so the loads are unconditional); the page id,
+  // which depends on two of them, after the products
+  const int token = min(lr, M - 1);
+  const int pos = r.positions[token];
+  const int entry = r.k_cache ? r.entry_of_token[token] : 0;
+  const f32x4 b = bias ? *(const f32x4*)(bias + n0) : f32x4{0.f, 0.f, 0.f, 0.f};
+  const int angle0 = 8 * g + (lg & 1) * 4;  // index of the first of the lane's four angles
+  const f32x4 freq = is_v ? f32x4{0.f, 0.f, 0.f, 0.f} : *(const f32x4*)(r.inv_freq + angle0);
+
+  f32x4 acc[1][1] = {{f32x4{0.f, 0.f, 0.f, 0.f}}};
+  skinny_products<1, 1, WAVES, VK_SKINNY_SETS>(w_view, a_view, w_off, a_off, K, wave, lg, acc);
+  partial[wave][lane] = acc[0][0];
+  int page = -1;
+  if (!is_q && r.k_cache) page = r.block_table[(size_t)entry * r.table_width + pos / r.block_size];
+  __syncthreads();
+  if (wave != 0) return;
+  f32x4 sum = partial[0][lane];
+#pragma unroll
+  for (int w = 1; w < WAVES; ++w) sum += partial[w][lane];
+  sum += b;
+  float x[4], y[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    x[j] = (float)(__bf16)sum[j];
+    y[j] = __shfl_xor(x[j], 32);  // the partner dim's value of the same token
+  }
+  bf16x4 out;
+  if (is_v) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) out[j] = (__bf16)x[j];
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float sn, cs;
+      sincosf((float)pos * freq[j], &sn, &cs);
+      const float lo = lg < 2 ? x[j] : y[j], hi = lg < 2 ? y[j] : x[j];
+      out[j] = (__bf16)(lg < 2 ? lo * cs - hi * sn : lo * sn + hi * cs);
+    }
+  }
+  if (lr >= M) return;
+  *(bf16x4*)(C + (size_t)lr * ldc + n0) = out;
+  if (page < 0) return;
+  const int slot = pos % r.block_size;
+  if (!is_v) {
+    const int kvh = head - r.heads;
+    *(bf16x4*)(r.k_cache + (((size_t)page * r.kv_heads + kvh) * r.block_size + slot) * hd + d0) = out;
+  } else {
+    const int kvh = head - r.heads - r.kv_heads;
+    __bf16* dst = r.v_cache + (((size_t)page * r.kv_heads + kvh) * hd + d0) * r.block_size + slot;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) dst[(size_t)j * r.block_size] = out[j];
+  }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1329,6 +1430,33 @@ extern "C" int vk_gemm_bf16_gated(const void* A, const void* W, void* C, int M, 
   }
 #undef VK_GATED
   return VK_UNSUPPORTED_SIZE;
+}
+
+// qkv[M, N] = A W^T + bias in bfloat16 for up to 16 tokens, its q and k heads rotated (full rotation: inv_freq
+// holds hd / 2 floats) and the tokens' K and V stored in their pages, as vk_gemm_bf16 followed by vk_rope_kvwrite
+// would leave them. N = (heads + 2 kv_heads) hd, hd a multiple of 16. k_cache null: no cache is written.
+// K pages [page, kv_head, slot, hd], V pages [page, kv_head, hd, slot]; a negative page id writes nothing.
+extern "C" int vk_gemm_bf16_qkv_rope(const void* A, const void* W, const float* bias, void* C, int M, int N, int K,
+                                     long long lda, long long ldc, const int* positions, const float* inv_freq,
+                                     void* k_cache, void* v_cache, const int* entry_of_token, const int* block_table,
+                                     int table_width, int block_size, int heads, int kv_heads, int hd, void* stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (M > 16) return VK_UNSUPPORTED_SIZE;
+  if (K <= 0 || (K & 7) || (lda & 7) || lda < K || ldc < N || (ldc & 3)) return VK_BAD_ARGUMENT;
+  if (((uintptr_t)A & 15) || ((uintptr_t)W & 15) || ((uintptr_t)C & 7) || ((uintptr_t)bias & 15) ||
+      ((uintptr_t)inv_freq & 15) || ((uintptr_t)k_cache & 7))
+    return VK_BAD_ARGUMENT;
+  if (heads <= 0 || kv_heads <= 0 || hd <= 0 || (hd & 15) || (long long)(heads + 2 * kv_heads) * hd != N || !positions ||
+      !inv_freq)
+    return VK_BAD_ARGUMENT;
+  if (k_cache && (!v_cache || !entry_of_token || !block_table || table_width <= 0 || block_size <= 0)) return VK_BAD_ARGUMENT;
+  if ((long long)N * K * 2 >= (1ll << 32) || lda >= (1 << 23)) return VK_UNSUPPORTED_SIZE;  // 32-bit byte offsets
+  const QkvRope r{positions, inv_freq, (__bf16*)k_cache, (__bf16*)v_cache, entry_of_token, block_table,
+                  table_width, block_size, heads, kv_heads, hd};
+  gemm_qkv_rope_kernel<<<N / 16, 256, 0, (hipStream_t)stream>>>((const __bf16*)A, (const __bf16*)W, bias, (__bf16*)C, M,
+                                                                N, K, lda, ldc, r);
+  VK_LAUNCH_CHECK();
+  return 0;
 }
 
 extern "C" int vk_gemm_bf16_tile_config(int config) {

@@ -326,6 +326,48 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], ou
                _stream()), "gemm_bf16")
 
 
+def gemm_bf16_qkv_rope_supported(a: torch.Tensor, w: torch.Tensor, qkv: torch.Tensor, head_dim: int) -> bool:
+    """Whether :func:`gemm_bf16_qkv_rope` takes the operands: all bfloat16, at most 16 tokens, a head width that is
+    a multiple of 16, a contiguous output."""
+    return (qkv.dtype == torch.bfloat16 and 1 <= a.shape[0] <= 16 and head_dim % 16 == 0 and qkv.is_contiguous()
+            and qkv.shape[1] % 4 == 0 and gemm_bf16_supported(a, w, qkv) and w.shape[0] * w.shape[1] * 2 < 2 ** 32)
+
+
+def gemm_bf16_qkv_rope(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], qkv: torch.Tensor,
+                       positions: torch.Tensor, inv_freq: torch.Tensor, k_cache: Optional[torch.Tensor],
+                       v_cache: Optional[torch.Tensor], entry_of_token: torch.Tensor, block_table: Optional[torch.Tensor],
+                       heads: int, kv_heads: int, head_dim: int) -> None:
+    """``qkv = a @ w.T + bias`` for up to 16 tokens with the full rotation of its q and k heads and the write of
+    the tokens' K and V into their pages in the product's epilogue: what :func:`gemm_bf16` followed by
+    :func:`rope_kvwrite` (without a table of angles) leaves, in one launch."""
+    _dev(a, w, bias, qkv, positions, inv_freq, k_cache, v_cache, entry_of_token, block_table)
+    m, k = a.shape
+    n = w.shape[0]
+    _need(w.shape[1] == k and qkv.shape == (m, n) and n == (heads + 2 * kv_heads) * head_dim, "gemm_bf16_qkv_rope: shapes")
+    _need(gemm_bf16_qkv_rope_supported(a, w, qkv, head_dim), "gemm_bf16_qkv_rope: bfloat16 operands, at most 16 tokens, "
+          "a head width that is a multiple of 16")
+    if bias is not None:
+        _need(bias.dtype == torch.float32 and bias.numel() == n and bias.is_contiguous(), "gemm: bias must be float32 [n]")
+    _need(positions.dtype == torch.int32 and positions.numel() >= m, "gemm_bf16_qkv_rope: positions")
+    _need(inv_freq.dtype == torch.float32 and inv_freq.numel() == head_dim // 2 and inv_freq.is_contiguous(),
+          "gemm_bf16_qkv_rope: inv_freq must hold head_dim / 2 floats")
+    table_width = block_size = 0
+    if k_cache is not None:
+        _need(v_cache is not None and block_table is not None, "gemm_bf16_qkv_rope: cache without table")
+        _need(_cache_ok(k_cache, v_cache, kv_heads, head_dim, qkv.dtype), "gemm_bf16_qkv_rope: cache shape or dtype")
+        _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(),
+              "gemm_bf16_qkv_rope: block table")
+        _need(entry_of_token.dtype == torch.int32 and entry_of_token.numel() >= m, "gemm_bf16_qkv_rope: entries")
+        table_width, block_size = block_table.shape[1], k_cache.shape[2]
+    lda = a.stride(0) if m > 1 else max(a.stride(0), k)
+    lda = lda if lda % 8 == 0 else k
+    fn = _fn("gemm_bf16", "vk_gemm_bf16_qkv_rope",
+             [_p, _p, _p, _p, _i, _i, _i, _ll, _ll, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _p])
+    _status(fn(_ptr(a), _ptr(w), _ptr(bias), _ptr(qkv), m, n, k, lda, n, _ptr(positions), _ptr(inv_freq), _ptr(k_cache),
+               _ptr(v_cache), _ptr(entry_of_token), _ptr(block_table), table_width, block_size, heads, kv_heads, head_dim,
+               _stream()), "gemm_bf16_qkv_rope")
+
+
 TILE_TILINGS = {0: "128x128 staged", 2: "256x128 staged", 3: "128x256 staged", 4: "256x256 staged",
                 9: "128x128 direct", 7: "256x128 direct", 8: "128x256 direct", 5: "256x256 direct", 6: "256x192 direct"}
 

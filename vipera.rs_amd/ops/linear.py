@@ -34,12 +34,17 @@ def mid_plan(m: int, n: int, k: int) -> Tuple[int, int]:
     return max(1, min(k // 512, 256 // row_blocks)), rows_per_wave
 
 
+def streams_in_wave_order(m: int, n: int, k: int) -> bool:
+    """Whether a bfloat16 product of ``m`` tokens runs on the kernel whose waves split K inside a workgroup."""
+    return m <= 4 or (m <= 16 and n < 16_384 and k < 8_192)
+
+
 def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
            accumulate: bool = False) -> torch.Tensor:
     if a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and kernels.gemm_bf16_supported(a, w, out):
         m, k = a.shape
         n = w.shape[0]
-        if m > 64 or m <= 4 or (m <= 16 and n < 16_384 and k < 8_192):
+        if m > 64 or streams_in_wave_order(m, n, k):
             kernels.gemm_bf16(a, w, bias, out, accumulate)
         else:
             ranges, rows_per_wave = mid_plan(m, n, k)

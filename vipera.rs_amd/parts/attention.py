@@ -17,7 +17,7 @@ from ..config.base import PartSpec
 from ..errors import InvalidArgumentError
 from ..ops import kernels
 from ..ops.attention import paged_attention
-from ..ops.linear import linear
+from ..ops.linear import linear, streams_in_wave_order
 from ..weights.checkpoint import MATRIX, VECTOR, TensorSpec
 from .base import KVCacheSpec, Mixer, register_mixer
 
@@ -79,22 +79,28 @@ class Attention(Mixer):
     def forward(self, h, batch, cache, state, position, residual, reads_only: bool = False) -> None:
         tokens = h.shape[0]
         qkv = self.runtime.empty((tokens, self.q_width + 2 * self.kv_width))
-        linear(h, self.w_qkv, self.b_qkv, qkv)
         table = batch.block_tables[cache.group]
         fused = position.fused_rotary()
-        if fused is None:
-            position.apply(qkv, batch, self.heads, self.kv_heads, self.head_dim)
-            inv_freq, rotary_dim = None, 0
-        else:
-            inv_freq, rotary_dim = fused
+        inv_freq, rotary_dim = fused if fused is not None else (None, 0)
         angles = position.step_angles(batch) if rotary_dim else None
-        if reads_only:
-            if rotary_dim:
+        if (rotary_dim == self.head_dim and angles is None and h.dtype == torch.bfloat16
+                and self.w_qkv.dtype == torch.bfloat16 and streams_in_wave_order(tokens, *self.w_qkv.shape)
+                and kernels.gemm_bf16_qkv_rope_supported(h, self.w_qkv, qkv, self.head_dim)):
+            # a few tokens with a full rotation: product, rotation and cache write are one kernel
+            kernels.gemm_bf16_qkv_rope(h, self.w_qkv, self.b_qkv, qkv, batch.positions, inv_freq,
+                                       None if reads_only else cache.k, None if reads_only else cache.v,
+                                       batch.entry_of_token, None if reads_only else table, self.heads, self.kv_heads,
+                                       self.head_dim)
+        else:
+            linear(h, self.w_qkv, self.b_qkv, qkv)
+            if fused is None:
+                position.apply(qkv, batch, self.heads, self.kv_heads, self.head_dim)
+            if not reads_only:
+                kernels.rope_kvwrite(qkv, batch.positions, inv_freq, rotary_dim, cache.k, cache.v, batch.entry_of_token,
+                                     table, self.heads, self.kv_heads, self.head_dim, angles)
+            elif rotary_dim:
                 kernels.rope_kvwrite(qkv, batch.positions, inv_freq, rotary_dim, None, None, batch.entry_of_token,
                                      None, self.heads, self.kv_heads, self.head_dim, angles)
-        else:
-            kernels.rope_kvwrite(qkv, batch.positions, inv_freq, rotary_dim, cache.k, cache.v, batch.entry_of_token,
-                                 table, self.heads, self.kv_heads, self.head_dim, angles)
         attn = self.runtime.empty((tokens, self.q_width))
         paged_attention(qkv, cache.k, cache.v, attn, batch, table, self.heads, self.kv_heads, self.head_dim,
                         self.scale, self.window)
