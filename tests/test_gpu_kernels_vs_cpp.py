@@ -80,7 +80,9 @@ def test_rotation_and_cache_write_beside_its_twin(dtype, hd, rotary_dim):
 
 
 @pytest.mark.parametrize("m,heads,kv_heads,hd,k,with_bias,with_cache", [(6, 5, 2, 48, 96, True, True), (1, 4, 4, 128, 256, False, True),
-                                                                        (16, 3, 1, 16, 72, True, True), (3, 7, 1, 64, 520, True, False)])
+                                                                        (16, 3, 1, 16, 72, True, True), (3, 7, 1, 64, 520, True, False),
+                                                                        (8, 28, 4, 128, 256, True, True), (5, 9, 3, 40, 64, True, True),
+                                                                        (2, 40, 8, 128, 128, False, True)])
 def test_fused_qkv_product_beside_its_twin_and_the_two_kernels(m, heads, kv_heads, hd, k, with_bias, with_cache):
     """Product, rotation and cache write in one kernel: beside its twin, and bit for bit what the product followed
     by the rotation kernel leaves in the q/k/v rows and in both caches (other pages untouched)."""

@@ -681,12 +681,16 @@ int launch_skinny(const __bf16* A, const __bf16* W, const float* bias, TC* C, in
 // ---------------------------------------------------------------------------------------------
 // The q/k/v product of up to 16 tokens with the rotation and the cache write in its epilogue, which saves the
 // launch between the product and the attention of a decode step. The streaming is gemm_skinny_kernel's (four
-// waves split K). A workgroup owns 16 outputs of one head: for a q or k head eight dims of the first half and
-// their eight partners half a head further on (rows 0-7 and 8-15 of the instruction's tile, so a lane finds a
-// dim's partner in lane ^ 32), for a v head 16 consecutive dims. The sums take the bias, are rounded to bfloat16
-// as the product alone would leave them, and are then rotated and stored exactly as rope_kvwrite_kernel does
-// (crates/vipera-backend-cpu/src/model.rs:4192-4251, 1495-1542): what the cache and the attention see does not
-// depend on which of the two paths a token took. Full rotation only (rotary width = head width, a multiple of 16).
+// waves split K) with two tiles per workgroup. The first tile holds `pairs` (at most 8) rotation pairs of the q
+// and k heads, taken from the list of all (head, dim below half the head width): the dims in the tile's rows
+// 0-7 and their partners half a head further on in rows 8-15, so a lane finds a dim's partner in lane ^ 32. The
+// second tile holds `values` (at most 16) dims of the v heads. The launcher picks the two numbers so that the
+// workgroups fill the CUs evenly (28 + 4 heads of 128 and 4 v heads: 256 workgroups of 8 pairs and 2 values,
+// 18 weight rows each; a tile's unused rows lie past the end of the buffer view and fetch nothing). The sums take
+// the bias, are rounded to bfloat16 as the product alone would leave them, and are then rotated and stored exactly
+// as rope_kvwrite_kernel does (crates/vipera-backend-cpu/src/model.rs:4192-4251, 1495-1542): what the cache and
+// the attention see does not depend on which of the two paths a token took. Full rotation only (rotary width =
+// head width).
 struct QkvRope {
   const int* positions;
   const float* inv_freq;
@@ -694,78 +698,110 @@ struct QkvRope {
   __bf16* v_cache;
   const int* entry_of_token;
   const int* block_table;
-  int table_width, block_size, heads, kv_heads, hd;
+  int table_width, block_size, heads, kv_heads, hd, pairs, values;
 };
 
 __global__ __launch_bounds__(256) void gemm_qkv_rope_kernel(const __bf16* __restrict__ A, const __bf16* __restrict__ W,
                                                             const float* __restrict__ bias, __bf16* __restrict__ C,
                                                             int M, int N, int K, long long lda, long long ldc, QkvRope r) {
   constexpr int WAVES = 4;
-  __shared__ f32x4 partial[WAVES][64];
+  constexpr unsigned NO_ROW = 0x80000000u;  // past the end of the weight's view (the launcher checks its size)
+  __shared__ f32x4 partial[WAVES][2][64];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lr = lane & 15, lg = lane >> 4;
-  const int hd = r.hd, half = hd / 2, groups = hd / 16;
-  const int head = blockIdx.x / groups, g = blockIdx.x % groups;
-  const bool is_q = head < r.heads, is_v = head >= r.heads + r.kv_heads;
-  // the weight row of the tile's row `i`, and the dim within the head of the lane's first output
-  auto dim_of = [&](int i) { return is_v ? 16 * g + i : (i < 8 ? 8 * g + i : half + 8 * g + i - 8); };
-  const int d0 = dim_of(lg * 4), n0 = head * hd + d0;
+  const int hd = r.hd, half = hd / 2;
+  const int all_pairs = (r.heads + r.kv_heads) * half, all_values = r.kv_heads * hd, first_value_row = (r.heads + r.kv_heads) * hd;
+  // row i of the first tile -> its output column (head * hd + dim), or -1
+  auto rotated_column = [&](int i) {
+    const int slot = i & 7, pair = blockIdx.x * r.pairs + slot;
+    if (slot >= r.pairs || pair >= all_pairs) return -1;
+    return (pair / half) * hd + pair % half + (i >= 8 ? half : 0);
+  };
+  // row i of the second tile -> its output column among the value heads, or -1
+  auto value_column = [&](int i) {
+    const int v = blockIdx.x * r.values + i;
+    return i < r.values && v < all_values ? first_value_row + v : -1;
+  };
   const BufferView w_view = buffer_view(W, (unsigned long long)N * K * 2);
   const BufferView a_view = buffer_view(A, ((unsigned long long)(M - 1) * lda + K) * 2);
-  const unsigned w_off[1] = {(unsigned)((((size_t)head * hd + dim_of(lr)) * K + lg * 8) * 2)};
+  const int row0 = rotated_column(lr), row1 = value_column(lr);
+  const unsigned w_off[2] = {row0 >= 0 ? (unsigned)(((size_t)row0 * K + lg * 8) * 2) : NO_ROW,
+                             row1 >= 0 ? (unsigned)(((size_t)row1 * K + lg * 8) * 2) : NO_ROW};
   const unsigned a_off[1] = {(unsigned)((lr * lda + lg * 8) * 2)};
-  // what the epilogue needs from memory is requested now (clamped, so the loads are unconditional); the page id,
-  // which depends on two of them, after the products
+  // What the epilogue needs from memory is requested now (clamped, so the loads are unconditional); the page id,
+  // which depends on two of them, after the products. Wave 0 finishes the first tile, wave 1 the second.
   const int token = min(lr, M - 1);
   const int pos = r.positions[token];
   const int entry = r.k_cache ? r.entry_of_token[token] : 0;
-  const f32x4 b = bias ? *(const f32x4*)(bias + n0) : f32x4{0.f, 0.f, 0.f, 0.f};
-  const int angle0 = 8 * g + (lg & 1) * 4;  // index of the first of the lane's four angles
-  const f32x4 freq = is_v ? f32x4{0.f, 0.f, 0.f, 0.f} : *(const f32x4*)(r.inv_freq + angle0);
-
-  f32x4 acc[1][1] = {{f32x4{0.f, 0.f, 0.f, 0.f}}};
-  skinny_products<1, 1, WAVES, VK_SKINNY_SETS>(w_view, a_view, w_off, a_off, K, wave, lg, acc);
-  partial[wave][lane] = acc[0][0];
-  int page = -1;
-  if (!is_q && r.k_cache) page = r.block_table[(size_t)entry * r.table_width + pos / r.block_size];
-  __syncthreads();
-  if (wave != 0) return;
-  f32x4 sum = partial[0][lane];
-#pragma unroll
-  for (int w = 1; w < WAVES; ++w) sum += partial[w][lane];
-  sum += b;
-  float x[4], y[4];
+  int column[4];
+  float b[4], freq[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    x[j] = (float)(__bf16)sum[j];
-    y[j] = __shfl_xor(x[j], 32);  // the partner dim's value of the same token
+    column[j] = wave == 0 ? rotated_column(lg * 4 + j) : value_column(lg * 4 + j);
+    b[j] = bias ? bias[max(column[j], 0)] : 0.f;
+    freq[j] = r.inv_freq[wave == 0 ? max(column[j], 0) % hd % half : 0];
   }
-  bf16x4 out;
-  if (is_v) {
+
+  f32x4 acc[2][1] = {{f32x4{0.f, 0.f, 0.f, 0.f}}, {f32x4{0.f, 0.f, 0.f, 0.f}}};
+  skinny_products<1, 2, WAVES, VK_SKINNY_SETS>(w_view, a_view, w_off, a_off, K, wave, lg, acc);
+  partial[wave][0][lane] = acc[0][0];
+  partial[wave][1][lane] = acc[1][0];
+  int page = -1;
+  if (r.k_cache) page = r.block_table[(size_t)entry * r.table_width + pos / r.block_size];
+  __syncthreads();
+  if (wave > 1) return;
+  f32x4 sum = partial[0][wave][lane];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) out[j] = (__bf16)x[j];
+  for (int w = 1; w < WAVES; ++w) sum += partial[w][wave][lane];
+  const int slot = pos % r.block_size;
+  if (wave == 0) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float x = (float)(__bf16)(sum[j] + b[j]);
+      const float y = __shfl_xor(x, 32);  // the partner dim's value of the same token
+      float sn, cs;
+      sincosf((float)pos * freq[j], &sn, &cs);
+      const float lo = lg < 2 ? x : y, hi = lg < 2 ? y : x;
+      const __bf16 out = (__bf16)(lg < 2 ? lo * cs - hi * sn : lo * sn + hi * cs);
+      if (lr < M && column[j] >= 0) {
+        C[(size_t)lr * ldc + column[j]] = out;
+        const int kvh = column[j] / hd - r.heads;
+        if (kvh >= 0 && page >= 0)
+          r.k_cache[(((size_t)page * r.kv_heads + kvh) * r.block_size + slot) * hd + column[j] % hd] = out;
+      }
+    }
   } else {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      float sn, cs;
-      sincosf((float)pos * freq[j], &sn, &cs);
-      const float lo = lg < 2 ? x[j] : y[j], hi = lg < 2 ? y[j] : x[j];
-      out[j] = (__bf16)(lg < 2 ? lo * cs - hi * sn : lo * sn + hi * cs);
+      const __bf16 out = (__bf16)(sum[j] + b[j]);
+      if (lr < M && column[j] >= 0) {
+        C[(size_t)lr * ldc + column[j]] = out;
+        const int v = column[j] - first_value_row;
+        if (page >= 0) r.v_cache[(((size_t)page * r.kv_heads + v / hd) * hd + v % hd) * r.block_size + slot] = out;
+      }
     }
   }
-  if (lr >= M) return;
-  *(bf16x4*)(C + (size_t)lr * ldc + n0) = out;
-  if (page < 0) return;
-  const int slot = pos % r.block_size;
-  if (!is_v) {
-    const int kvh = head - r.heads;
-    *(bf16x4*)(r.k_cache + (((size_t)page * r.kv_heads + kvh) * r.block_size + slot) * hd + d0) = out;
-  } else {
-    const int kvh = head - r.heads - r.kv_heads;
-    __bf16* dst = r.v_cache + (((size_t)page * r.kv_heads + kvh) * hd + d0) * r.block_size + slot;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) dst[(size_t)j * r.block_size] = out[j];
+}
+
+// Pairs and values per workgroup of gemm_qkv_rope_kernel: as in balanced_rows, the workgroups' rounds over the CUs
+// times a workgroup's rows, tokens and fixed cost.
+void qkv_rope_plan(int M, int heads, int kv_heads, int hd, int* pairs, int* values, int* groups) {
+  const int cus = compute_units();
+  const int all_pairs = (heads + kv_heads) * (hd / 2), all_values = kv_heads * hd;
+  double best_cost = 0.0;
+  for (int p = 8; p >= 4; --p) {
+    const int by_pairs = (all_pairs + p - 1) / p, by_values = (all_values + 15) / 16;
+    const int g = by_pairs > by_values ? by_pairs : by_values;
+    const int v = (all_values + g - 1) / g;
+    const double rounds = g >= 3 * cus ? (double)g / cus : (double)((g + cus - 1) / cus);
+    const double cost = rounds * (2 * p + v + 0.5 * M + 8.0);
+    if (p == 8 || cost < best_cost * 0.97) {
+      best_cost = cost;
+      *pairs = p;
+      *values = v;
+      *groups = g;
+    }
   }
 }
 
@@ -1434,7 +1470,7 @@ extern "C" int vk_gemm_bf16_gated(const void* A, const void* W, void* C, int M, 
 
 // qkv[M, N] = A W^T + bias in bfloat16 for up to 16 tokens, its q and k heads rotated (full rotation: inv_freq
 // holds hd / 2 floats) and the tokens' K and V stored in their pages, as vk_gemm_bf16 followed by vk_rope_kvwrite
-// would leave them. N = (heads + 2 kv_heads) hd, hd a multiple of 16. k_cache null: no cache is written.
+// would leave them. N = (heads + 2 kv_heads) hd, hd even. k_cache null: no cache is written.
 // K pages [page, kv_head, slot, hd], V pages [page, kv_head, hd, slot]; a negative page id writes nothing.
 extern "C" int vk_gemm_bf16_qkv_rope(const void* A, const void* W, const float* bias, void* C, int M, int N, int K,
                                      long long lda, long long ldc, const int* positions, const float* inv_freq,
@@ -1442,18 +1478,19 @@ extern "C" int vk_gemm_bf16_qkv_rope(const void* A, const void* W, const float* 
                                      int table_width, int block_size, int heads, int kv_heads, int hd, void* stream) {
   if (M <= 0 || N <= 0) return 0;
   if (M > 16) return VK_UNSUPPORTED_SIZE;
-  if (K <= 0 || (K & 7) || (lda & 7) || lda < K || ldc < N || (ldc & 3)) return VK_BAD_ARGUMENT;
-  if (((uintptr_t)A & 15) || ((uintptr_t)W & 15) || ((uintptr_t)C & 7) || ((uintptr_t)bias & 15) ||
-      ((uintptr_t)inv_freq & 15) || ((uintptr_t)k_cache & 7))
-    return VK_BAD_ARGUMENT;
-  if (heads <= 0 || kv_heads <= 0 || hd <= 0 || (hd & 15) || (long long)(heads + 2 * kv_heads) * hd != N || !positions ||
+  if (K <= 0 || (K & 7) || (lda & 7) || lda < K || ldc < N) return VK_BAD_ARGUMENT;
+  if (((uintptr_t)A & 15) || ((uintptr_t)W & 15)) return VK_BAD_ARGUMENT;
+  if (heads <= 0 || kv_heads <= 0 || hd <= 0 || (hd & 1) || (long long)(heads + 2 * kv_heads) * hd != N || !positions ||
       !inv_freq)
     return VK_BAD_ARGUMENT;
   if (k_cache && (!v_cache || !entry_of_token || !block_table || table_width <= 0 || block_size <= 0)) return VK_BAD_ARGUMENT;
-  if ((long long)N * K * 2 >= (1ll << 32) || lda >= (1 << 23)) return VK_UNSUPPORTED_SIZE;  // 32-bit byte offsets
+  // byte offsets are 32-bit, and bit 31 switches a lane's row off
+  if ((long long)N * K * 2 >= (1ll << 31) || lda >= (1 << 23)) return VK_UNSUPPORTED_SIZE;
+  int pairs = 8, values = 16, groups = 1;
+  qkv_rope_plan(M, heads, kv_heads, hd, &pairs, &values, &groups);
   const QkvRope r{positions, inv_freq, (__bf16*)k_cache, (__bf16*)v_cache, entry_of_token, block_table,
-                  table_width, block_size, heads, kv_heads, hd};
-  gemm_qkv_rope_kernel<<<N / 16, 256, 0, (hipStream_t)stream>>>((const __bf16*)A, (const __bf16*)W, bias, (__bf16*)C, M,
+                  table_width, block_size, heads, kv_heads, hd, pairs, values};
+  gemm_qkv_rope_kernel<<<groups, 256, 0, (hipStream_t)stream>>>((const __bf16*)A, (const __bf16*)W, bias, (__bf16*)C, M,
                                                                 N, K, lda, ldc, r);
   VK_LAUNCH_CHECK();
   return 0;

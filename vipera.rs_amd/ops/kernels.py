@@ -327,10 +327,10 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], ou
 
 
 def gemm_bf16_qkv_rope_supported(a: torch.Tensor, w: torch.Tensor, qkv: torch.Tensor, head_dim: int) -> bool:
-    """Whether :func:`gemm_bf16_qkv_rope` takes the operands: all bfloat16, at most 16 tokens, a head width that is
-    a multiple of 16, a contiguous output."""
-    return (qkv.dtype == torch.bfloat16 and 1 <= a.shape[0] <= 16 and head_dim % 16 == 0 and qkv.is_contiguous()
-            and qkv.shape[1] % 4 == 0 and gemm_bf16_supported(a, w, qkv) and w.shape[0] * w.shape[1] * 2 < 2 ** 32)
+    """Whether :func:`gemm_bf16_qkv_rope` takes the operands: all bfloat16, at most 16 tokens, an even head
+    width, a contiguous output, a weight of less than 2 GiB."""
+    return (qkv.dtype == torch.bfloat16 and 1 <= a.shape[0] <= 16 and head_dim % 2 == 0 and qkv.is_contiguous()
+            and gemm_bf16_supported(a, w, qkv) and w.shape[0] * w.shape[1] * 2 < 2 ** 31)
 
 
 def gemm_bf16_qkv_rope(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], qkv: torch.Tensor,
@@ -345,7 +345,7 @@ def gemm_bf16_qkv_rope(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Te
     n = w.shape[0]
     _need(w.shape[1] == k and qkv.shape == (m, n) and n == (heads + 2 * kv_heads) * head_dim, "gemm_bf16_qkv_rope: shapes")
     _need(gemm_bf16_qkv_rope_supported(a, w, qkv, head_dim), "gemm_bf16_qkv_rope: bfloat16 operands, at most 16 tokens, "
-          "a head width that is a multiple of 16")
+          "an even head width")
     if bias is not None:
         _need(bias.dtype == torch.float32 and bias.numel() == n and bias.is_contiguous(), "gemm: bias must be float32 [n]")
     _need(positions.dtype == torch.int32 and positions.numel() >= m, "gemm_bf16_qkv_rope: positions")
