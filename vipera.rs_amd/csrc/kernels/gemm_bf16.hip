@@ -468,11 +468,15 @@ constexpr int SPAN = 128;  // k per wave per step: four instructions of 32
 
 // The K loop of the weight-streaming kernels: wave `wave` of WAVES multiplies the spans wave, wave + WAVES, ...
 // of K (and the rest of K, less than a span, falls to one of them) into acc. w_off / a_off: a lane's byte offsets
-// of its operand rows at k = 0.
-template <int CB, int RT, int WAVES, int SETS>
+// of its operand rows at k = 0. `between` runs once the first spans are requested and before the first product:
+// work that waits for earlier loads costs nothing there, the weights are on their way meanwhile.
+struct Nothing {
+  __device__ __forceinline__ void operator()() const {}
+};
+template <int CB, int RT, int WAVES, int SETS, typename Between = Nothing>
 __device__ __forceinline__ void skinny_products(const BufferView& w_view, const BufferView& a_view,
                                                 const unsigned (&w_off)[RT], const unsigned (&a_off)[CB], int K, int wave,
-                                                int lg, f32x4 (&acc)[RT][CB]) {
+                                                int lg, f32x4 (&acc)[RT][CB], Between between = Between()) {
   // SETS register sets of operands rotate through run_pipeline: the loads of SETS - 1 spans are in flight
   // while one span is multiplied (three sets with one block of tokens, two with more).
   bf16x8 wf[SETS][RT][4], af[SETS][CB][4];
@@ -505,11 +509,13 @@ __device__ __forceinline__ void skinny_products(const BufferView& w_view, const 
   };
   if (count >= SETS - 1) {
     static_for<SETS - 1>([&](auto j) { load_span(wave + j.value * WAVES, wf[j.value], af[j.value]); });
+    between();
     run_pipeline<SETS, SETS - 1>(step, count);
   } else {  // fewer spans than the pipeline is deep: request them all, then multiply
     static_for<SETS - 1>([&](auto j) {
       if (j.value < count) load_span(wave + j.value * WAVES, wf[j.value], af[j.value]);
     });
+    between();
     static_for<SETS - 1>([&](auto j) {
       if (j.value < count) multiply(wf[j.value], af[j.value]);
     });
@@ -681,12 +687,14 @@ int launch_skinny(const __bf16* A, const __bf16* W, const float* bias, TC* C, in
 // ---------------------------------------------------------------------------------------------
 // The q/k/v product of up to 16 tokens with the rotation and the cache write in its epilogue, which saves the
 // launch between the product and the attention of a decode step. The streaming is gemm_skinny_kernel's (four
-// waves split K) with two tiles per workgroup. The first tile holds `pairs` (at most 8) rotation pairs of the q
-// and k heads, taken from the list of all (head, dim below half the head width): the dims in the tile's rows
-// 0-7 and their partners half a head further on in rows 8-15, so a lane finds a dim's partner in lane ^ 32. The
-// second tile holds `values` (at most 16) dims of the v heads. The launcher picks the two numbers so that the
-// workgroups fill the CUs evenly (28 + 4 heads of 128 and 4 v heads: 256 workgroups of 8 pairs and 2 values,
-// 18 weight rows each; a tile's unused rows lie past the end of the buffer view and fetch nothing). The sums take
+// waves split K). A workgroup's tile holds `pairs` (at most 8) rotation pairs of the q and k heads, taken from the
+// list of all (head, dim below half the head width): the dims in the tile's rows 0-7 and their partners half a head
+// further on in rows 8-15, so a lane finds a dim's partner in lane ^ 32. Its `values` (at most 16) dims of the v
+// heads sit in the rows that the pairs leave free, or, where those are too few, in a second tile (RT 2). The
+// launcher picks the two numbers so that the workgroups fill the CUs evenly (28 + 4 heads of 128 and 4 v heads: 256
+// workgroups of 8 pairs and, in a second tile, 2 values, 18 weight rows each; 40 + 8 and 8 heads: 512 workgroups of
+// 6 pairs and 2 values in one tile; a tile's unused rows lie past the end of the buffer view and fetch nothing, but
+// every load instruction costs the same, which is why one tile is preferred). The sums take
 // the bias, are rounded to bfloat16 as the product alone would leave them, and are then rotated and stored exactly
 // as rope_kvwrite_kernel does (crates/vipera-backend-cpu/src/model.rs:4192-4251, 1495-1542): what the cache and
 // the attention see does not depend on which of the two paths a token took. Full rotation only (rotary width =
@@ -701,84 +709,99 @@ struct QkvRope {
   int table_width, block_size, heads, kv_heads, hd, pairs, values;
 };
 
+template <int RT>
 __global__ __launch_bounds__(256) void gemm_qkv_rope_kernel(const __bf16* __restrict__ A, const __bf16* __restrict__ W,
                                                             const float* __restrict__ bias, __bf16* __restrict__ C,
                                                             int M, int N, int K, long long lda, long long ldc, QkvRope r) {
   constexpr int WAVES = 4;
   constexpr unsigned NO_ROW = 0x80000000u;  // past the end of the weight's view (the launcher checks its size)
-  __shared__ f32x4 partial[WAVES][2][64];
+  __shared__ f32x4 partial[WAVES][RT][64];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lr = lane & 15, lg = lane >> 4;
   const int hd = r.hd, half = hd / 2;
   const int all_pairs = (r.heads + r.kv_heads) * half, all_values = r.kv_heads * hd, first_value_row = (r.heads + r.kv_heads) * hd;
-  // row i of the first tile -> its output column (head * hd + dim), or -1
-  auto rotated_column = [&](int i) {
-    const int slot = i & 7, pair = blockIdx.x * r.pairs + slot;
-    if (slot >= r.pairs || pair >= all_pairs) return -1;
-    return (pair / half) * hd + pair % half + (i >= 8 ? half : 0);
+  // Row i of the first tile -> its output column, or -1: slots 0 .. pairs - 1 of each half of the tile hold the
+  // pairs (head * hd + dim, the partner in the other half); with one tile (RT 1) the slots behind them hold
+  // the workgroup's values, the first 8 - pairs in rows pairs .. 7, the rest in rows 8 + pairs .. 15.
+  auto value_of = [&](int index) {  // the workgroup's value number `index` -> column, or -1
+    const int v = blockIdx.x * r.values + index;
+    return index < r.values && v < all_values ? first_value_row + v : -1;
   };
-  // row i of the second tile -> its output column among the value heads, or -1
-  auto value_column = [&](int i) {
-    const int v = blockIdx.x * r.values + i;
-    return i < r.values && v < all_values ? first_value_row + v : -1;
+  auto first_tile_column = [&](int i, bool& rotated) {
+    const int slot = i & 7, pair = blockIdx.x * r.pairs + slot;
+    rotated = slot < r.pairs;
+    if (rotated) return pair < all_pairs ? (pair / half) * hd + pair % half + (i >= 8 ? half : 0) : -1;
+    return RT == 1 ? value_of(slot - r.pairs + (i >= 8 ? 8 - r.pairs : 0)) : -1;
   };
   const BufferView w_view = buffer_view(W, (unsigned long long)N * K * 2);
   const BufferView a_view = buffer_view(A, ((unsigned long long)(M - 1) * lda + K) * 2);
-  const int row0 = rotated_column(lr), row1 = value_column(lr);
-  const unsigned w_off[2] = {row0 >= 0 ? (unsigned)(((size_t)row0 * K + lg * 8) * 2) : NO_ROW,
-                             row1 >= 0 ? (unsigned)(((size_t)row1 * K + lg * 8) * 2) : NO_ROW};
+  unsigned w_off[RT];
+  {
+    bool unused;
+    const int row0 = first_tile_column(lr, unused);
+    w_off[0] = row0 >= 0 ? (unsigned)(((size_t)row0 * K + lg * 8) * 2) : NO_ROW;
+    if constexpr (RT == 2) {
+      const int row1 = value_of(lr);
+      w_off[1] = row1 >= 0 ? (unsigned)(((size_t)row1 * K + lg * 8) * 2) : NO_ROW;
+    }
+  }
   const unsigned a_off[1] = {(unsigned)((lr * lda + lg * 8) * 2)};
-  // What the epilogue needs from memory is requested now (clamped, so the loads are unconditional); the page id,
-  // which depends on two of them, after the products. Wave 0 finishes the first tile, wave 1 the second.
+  // What the epilogue needs from memory is requested now (clamped, so the loads are unconditional). Wave 0 finishes
+  // the first tile, wave 1 the second.
   const int token = min(lr, M - 1);
   const int pos = r.positions[token];
   const int entry = r.k_cache ? r.entry_of_token[token] : 0;
   int column[4];
+  bool rotated[4];
   float b[4], freq[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    column[j] = wave == 0 ? rotated_column(lg * 4 + j) : value_column(lg * 4 + j);
+    rotated[j] = false;
+    column[j] = wave == 0 ? first_tile_column(lg * 4 + j, rotated[j]) : value_of(lg * 4 + j);
     b[j] = bias ? bias[max(column[j], 0)] : 0.f;
-    freq[j] = r.inv_freq[wave == 0 ? max(column[j], 0) % hd % half : 0];
+    freq[j] = r.inv_freq[rotated[j] ? max(column[j], 0) % hd % half : 0];
   }
 
-  f32x4 acc[2][1] = {{f32x4{0.f, 0.f, 0.f, 0.f}}, {f32x4{0.f, 0.f, 0.f, 0.f}}};
-  skinny_products<1, 2, WAVES, VK_SKINNY_SETS>(w_view, a_view, w_off, a_off, K, wave, lg, acc);
-  partial[wave][0][lane] = acc[0][0];
-  partial[wave][1][lane] = acc[1][0];
+  f32x4 acc[RT][1];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) acc[rt][0] = f32x4{0.f, 0.f, 0.f, 0.f};
+  // the page id and the sines wait for the position, which was requested before the weights: they are worked out
+  // while the first weights are on their way, not between the last product and the stores
   int page = -1;
-  if (r.k_cache) page = r.block_table[(size_t)entry * r.table_width + pos / r.block_size];
+  float sn[4], cs[4];
+  auto lookups = [&]() {
+    if (r.k_cache) page = r.block_table[(size_t)entry * r.table_width + pos / r.block_size];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) sincosf((float)pos * freq[j], &sn[j], &cs[j]);
+  };
+  skinny_products<1, RT, WAVES, VK_SKINNY_SETS>(w_view, a_view, w_off, a_off, K, wave, lg, acc, lookups);
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) partial[wave][rt][lane] = acc[rt][0];
   __syncthreads();
-  if (wave > 1) return;
+  if (wave >= RT) return;
   f32x4 sum = partial[0][wave][lane];
 #pragma unroll
   for (int w = 1; w < WAVES; ++w) sum += partial[w][wave][lane];
   const int slot = pos % r.block_size;
-  if (wave == 0) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const float x = (float)(__bf16)(sum[j] + b[j]);
-      const float y = __shfl_xor(x, 32);  // the partner dim's value of the same token
-      float sn, cs;
-      sincosf((float)pos * freq[j], &sn, &cs);
+  for (int j = 0; j < 4; ++j) {
+    const float x = (float)(__bf16)(sum[j] + b[j]);
+    const float y = __shfl_xor(x, 32);  // in the first tile: the partner dim's value of the same token
+    __bf16 out = (__bf16)x;
+    if (rotated[j]) {
       const float lo = lg < 2 ? x : y, hi = lg < 2 ? y : x;
-      const __bf16 out = (__bf16)(lg < 2 ? lo * cs - hi * sn : lo * sn + hi * cs);
-      if (lr < M && column[j] >= 0) {
-        C[(size_t)lr * ldc + column[j]] = out;
-        const int kvh = column[j] / hd - r.heads;
-        if (kvh >= 0 && page >= 0)
-          r.k_cache[(((size_t)page * r.kv_heads + kvh) * r.block_size + slot) * hd + column[j] % hd] = out;
-      }
+      out = (__bf16)(lg < 2 ? lo * cs[j] - hi * sn[j] : lo * sn[j] + hi * cs[j]);
     }
-  } else {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const __bf16 out = (__bf16)(sum[j] + b[j]);
-      if (lr < M && column[j] >= 0) {
-        C[(size_t)lr * ldc + column[j]] = out;
+    if (lr < M && column[j] >= 0) {
+      C[(size_t)lr * ldc + column[j]] = out;
+      if (page < 0) continue;
+      if (rotated[j]) {
+        const int kvh = column[j] / hd - r.heads;
+        if (kvh >= 0) r.k_cache[(((size_t)page * r.kv_heads + kvh) * r.block_size + slot) * hd + column[j] % hd] = out;
+      } else {
         const int v = column[j] - first_value_row;
-        if (page >= 0) r.v_cache[(((size_t)page * r.kv_heads + v / hd) * hd + v % hd) * r.block_size + slot] = out;
+        r.v_cache[(((size_t)page * r.kv_heads + v / hd) * hd + v % hd) * r.block_size + slot] = out;
       }
     }
   }
@@ -795,7 +818,8 @@ void qkv_rope_plan(int M, int heads, int kv_heads, int hd, int* pairs, int* valu
     const int g = by_pairs > by_values ? by_pairs : by_values;
     const int v = (all_values + g - 1) / g;
     const double rounds = g >= 3 * cus ? (double)g / cus : (double)((g + cus - 1) / cus);
-    const double cost = rounds * (2 * p + v + 0.5 * M + 8.0);
+    const int tiles = v <= 2 * (8 - p) ? 1 : 2;
+    const double cost = rounds * (2 * p + v + 0.5 * M + 8.0 + 2.0 * (tiles - 1));
     if (p == 8 || cost < best_cost * 0.97) {
       best_cost = cost;
       *pairs = p;
@@ -1490,8 +1514,12 @@ extern "C" int vk_gemm_bf16_qkv_rope(const void* A, const void* W, const float* 
   qkv_rope_plan(M, heads, kv_heads, hd, &pairs, &values, &groups);
   const QkvRope r{positions, inv_freq, (__bf16*)k_cache, (__bf16*)v_cache, entry_of_token, block_table,
                   table_width, block_size, heads, kv_heads, hd, pairs, values};
-  gemm_qkv_rope_kernel<<<groups, 256, 0, (hipStream_t)stream>>>((const __bf16*)A, (const __bf16*)W, bias, (__bf16*)C, M,
-                                                                N, K, lda, ldc, r);
+  if (values <= 2 * (8 - pairs))
+    gemm_qkv_rope_kernel<1><<<groups, 256, 0, (hipStream_t)stream>>>((const __bf16*)A, (const __bf16*)W, bias, (__bf16*)C,
+                                                                     M, N, K, lda, ldc, r);
+  else
+    gemm_qkv_rope_kernel<2><<<groups, 256, 0, (hipStream_t)stream>>>((const __bf16*)A, (const __bf16*)W, bias, (__bf16*)C,
+                                                                     M, N, K, lda, ldc, r);
   VK_LAUNCH_CHECK();
   return 0;
 }
