@@ -243,6 +243,52 @@ extern "C" int plain_gemm_bf16_qkv_rope(const void* A, const void* W, const floa
                             table_width, block_size, M, heads, kv_heads, hd, nullptr);
 }
 
+// The residual product that also prepares the norm after it: C += A W^T + bias; scaled = bfloat16(C * gain); the
+// sums of squares of the rows of C as one group.
+extern "C" int plain_gemm_bf16_follow(const void* A, const void* W, const float* bias, float* C, int M, int N, int K,
+                                      long long lda, long long ldc, const float* gain, void* scaled, long long ld_scaled,
+                                      float* sumsq, long long sumsq_floats, int* groups, void*) {
+  if (M <= 0 || N <= 0 || M > 16 || K <= 0 || lda < K || ldc < N || ld_scaled < N || sumsq_floats < 16) return BAD_ARGUMENT;
+  product(A, DT_BF16, W, DT_BF16, bias, C, DT_F32, M, N, K, lda, ldc, true);
+  for (int m = 0; m < 16; ++m) sumsq[m] = 0.f;
+  for (int m = 0; m < M; ++m) {
+    double sum = 0.0;
+    for (int n = 0; n < N; ++n) {
+      const float x = C[(size_t)m * ldc + n];
+      sum += (double)x * (double)x;
+      ((uint16_t*)scaled)[(size_t)m * ld_scaled + n] = float_to_bf16(x * gain[n]);
+    }
+    sumsq[m] = (float)sum;
+  }
+  *groups = 1;
+  return 0;
+}
+
+// The gated product on such a scaled input: gate and up divided by the root mean square first.
+extern "C" int plain_gemm_bf16_gated_scaled(const void* A, const void* W, void* C, int M, int N, int K, long long lda,
+                                            long long ldc, const float* sumsq, int groups, float eps, void*) {
+  if (M <= 0 || N <= 0) return 0;
+  if (K <= 0 || lda < K || (N & 31) || ldc < N / 2 || groups <= 0) return BAD_ARGUMENT;
+  for (int m = 0; m < M; ++m) {
+    double squares = 0.0;
+    for (int g = 0; g < groups; ++g) squares += (double)sumsq[(size_t)g * 16 + m];
+    const double inv = 1.0 / std::sqrt(squares / (double)K + (double)eps);
+    for (int i = 0; i < N / 2; ++i) {
+      const int gate_row = (i / 16) * 32 + i % 16, up_row = gate_row + 16;
+      double gate = 0.0, up = 0.0;
+      for (int k = 0; k < K; ++k) {
+        const double a = load(A, DT_BF16, (size_t)m * lda + k);
+        gate += a * (double)load(W, DT_BF16, (size_t)gate_row * K + k);
+        up += a * (double)load(W, DT_BF16, (size_t)up_row * K + k);
+      }
+      gate *= inv;
+      up *= inv;
+      store(C, DT_BF16, (size_t)m * ldc + i, (float)(up * (gate / (1.0 + std::exp(-gate)))));
+    }
+  }
+  return 0;
+}
+
 // --- attention over the paged cache ----------------------------------------------------------------------------
 extern "C" int plain_attn_generic(const void* q, long long q_stride, const void* k_cache, const void* v_cache,
                                   void* out, int dtype, const int* positions, const int* entry_of_token,

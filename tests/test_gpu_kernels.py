@@ -358,6 +358,50 @@ def test_gemm_mid_against_float64(m, n, k, ranges, rows_per_wave):
     assert _rel(acc, base.double() + a.double() @ w.double().T) < 1e-5
 
 
+@pytest.mark.parametrize("m,width,k_in,inter", [(8, 3584, 512, 18944), (1, 256, 64, 32), (16, 512, 1024, 16 * 1000),
+                                               (5, 768, 264, 16 * 41), (3, 1024, 3584, 16 * 300)])
+def test_the_norm_split_between_the_products_around_it(m, width, k_in, inter):
+    """x += a Wo^T, h = rms_norm(x) * g, out = up(h) * silu(gate(h)) as two kernels: the first also leaves
+    bfloat16(x * g) and its workgroups' sums of squares, the second adds those and divides gate and up by the
+    root mean square.  Against 64-bit, and against residual product, norm kernel and gated product."""
+    from vipera_rs_amd.ops import kernels
+    from vipera_rs_amd.ops.linear import interleave_gate_up
+    g = torch.Generator().manual_seed(m + width + k_in)
+    a = torch.randn(m, k_in, generator=g).to(torch.bfloat16).to(DEV)
+    w_o = (torch.randn(width, k_in, generator=g) / k_in ** 0.5).to(torch.bfloat16).to(DEV)
+    x0 = (torch.randn(m, width, generator=g) * 2).to(DEV)
+    x0[0, 0] = 60.0                                          # one row with a far larger mean square
+    gain = (1 + 0.2 * torch.randn(width, generator=g)).to(DEV)
+    gate = (torch.randn(inter, width, generator=g) / width ** 0.5).to(torch.bfloat16).to(DEV)
+    up = (torch.randn(inter, width, generator=g) / width ** 0.5).to(torch.bfloat16).to(DEV)
+    fused = interleave_gate_up(gate, up)
+    eps = 1e-5
+    x = x0.clone()
+    scaled = torch.empty(m, width, dtype=torch.bfloat16, device=DEV)
+    sumsq = torch.full((kernels.follow_sumsq_floats(width),), 7.0, device=DEV)
+    groups = kernels.gemm_bf16_follow(a, w_o, None, x, gain, scaled, sumsq)
+    want_x = x0.double() + a.double() @ w_o.double().T
+    assert _rel(x, want_x) < 1e-5
+    assert _rel(scaled, want_x * gain.double()) < 6e-3
+    squares = sumsq[: groups * 16].view(groups, 16).double().sum(0)[:m]
+    assert _rel(squares, (want_x ** 2).sum(-1)) < 1e-5
+    out = torch.full((m, inter), 7.0, dtype=torch.bfloat16, device=DEV)
+    kernels.gemm_bf16_gated_scaled(scaled, fused, out, sumsq, groups, eps)
+    h = want_x * torch.rsqrt((want_x ** 2).mean(-1, keepdim=True) + eps) * gain.double()
+    gd, ud = h @ gate.double().T, h @ up.double().T
+    want = ud * (gd / (1 + torch.exp(-gd)))
+    assert _rel(out, want) < 1.2e-2
+    # the three kernels it replaces
+    x3 = x0.clone()
+    kernels.gemm_bf16(a, w_o, None, x3, accumulate=True)
+    assert torch.equal(x3, x)
+    h3 = torch.empty(m, width, dtype=torch.bfloat16, device=DEV)
+    kernels.rmsnorm(x3, gain, eps, h3)
+    out3 = torch.empty(m, inter, dtype=torch.bfloat16, device=DEV)
+    kernels.gemm_bf16_gated(h3, fused, out3, 0)
+    assert _rel(out, out3.double()) < 1.2e-2
+
+
 @pytest.mark.parametrize("m,inter,k", [(1, 32, 64), (5, 48, 96), (8, 18944, 512), (16, 176, 200), (33, 128, 264), (64, 1024, 256),
                                        (65, 64, 72), (300, 208, 136), (2048, 512, 128), (2048, 8208, 72), (100, 4608, 64),
                                        # the resident kernel: one pair on four waves, fewer units than waves, runs of

@@ -536,13 +536,28 @@ __device__ __forceinline__ void skinny_products(const BufferView& w_view, const 
 
 // CB: blocks of 16 tokens (M <= 16 * CB). RT: tiles of 16 weight rows per wave. WAVES: waves of a
 // workgroup, which split K in interleaved spans. A workgroup owns 16 * RT weight rows.
-template <int CB, int RT, int WAVES, typename TC, bool ACCUMULATE, int SETS = (CB == 1 ? VK_SKINNY_SETS : 2)>
+// What the product that adds into the residual leaves for the RMS norm that follows it (FOLLOW): beside the new
+// residual x, scaled[m][n] = bfloat16(x * gain[n]) and sumsq[workgroup][m] = the sum of x^2 over the workgroup's
+// columns, 16 floats per workgroup. The product after the norm adds the workgroups' sums in a fixed order, takes
+// 1 / sqrt(mean + eps) and scales its own 32-bit sums with it: the norm costs no launch and no workgroup waits
+// for a whole row (crates/vipera-backend-cpu/src/model.rs:4282-4288 is the formula; the rounding to bfloat16 falls
+// on x * gain instead of x * inv * gain).
+struct FollowNorm {
+  const float* gain;
+  __bf16* scaled;
+  float* sumsq;
+  long long ld_scaled;
+};
+
+template <int CB, int RT, int WAVES, typename TC, bool ACCUMULATE, int SETS = (CB == 1 ? VK_SKINNY_SETS : 2),
+          bool FOLLOW = false>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const __bf16* __restrict__ A,
                                                                   const __bf16* __restrict__ W,
                                                                   const float* __restrict__ bias,
                                                                   TC* __restrict__ C, int M, int N, int K,
                                                                   long long lda, long long ldc, int vector_ok,
-                                                                  int rows) {
+                                                                  int rows, FollowNorm follow) {
+  static_assert(!FOLLOW || (CB == 1 && RT == 1 && ACCUMULATE && sizeof(TC) == 4), "the norm follows a residual product");
   __shared__ f32x4 partial[WAVES][RT * CB][64];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -570,13 +585,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const __bf16* _
   // What the epilogue adds to the first tile this wave will store (bias, and the old C when accumulating) is
   // requested now: read after the last product it would be one more round trip to memory at the end of a
   // kernel that takes a few of them in all. Clamped addresses, so the loads are unconditional.
-  f32x4 early_bias = {0.f, 0.f, 0.f, 0.f}, early_c = {0.f, 0.f, 0.f, 0.f};
+  f32x4 early_bias = {0.f, 0.f, 0.f, 0.f}, early_c = {0.f, 0.f, 0.f, 0.f}, early_gain = {0.f, 0.f, 0.f, 0.f};
   const bool early = vector_ok && wave < RT * CB && n_end - n0 >= 4;
   const int early_m = (wave % CB) * 16 + lr, early_n = n0 + (wave / CB) * 16 + lg * 4;
   if (early) {
     const int m = min(early_m, M - 1), n = min(early_n, n_end - 4);
     if (bias) early_bias = *(const f32x4*)(bias + n);
     if constexpr (ACCUMULATE) early_c = *(const f32x4*)((const float*)C + (size_t)m * ldc + n);
+    if constexpr (FOLLOW) early_gain = *(const f32x4*)(follow.gain + n);
   }
 
   skinny_products<CB, RT, WAVES, SETS>(w_view, a_view, w_off, a_off, K, wave, lg, acc);
@@ -591,6 +607,38 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const __bf16* _
 #pragma unroll
     for (int w = 1; w < WAVES; ++w) sum += partial[w][t][lane];
     const int rt = t / CB, cb = t % CB;
+    if constexpr (FOLLOW) {  // one tile, wave 0: the new residual, its gained bfloat16 copy, its squares
+      float squares = 0.f;
+      if (lr < M) {
+        if (early && early_n + 3 < n_end) {
+          if (bias) sum += early_bias;
+          sum += early_c;
+          *(f32x4*)((float*)C + (size_t)lr * ldc + early_n) = sum;
+          bf16x4 o;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            o[j] = (__bf16)(sum[j] * early_gain[j]);
+            squares += sum[j] * sum[j];
+          }
+          *(bf16x4*)(follow.scaled + (size_t)lr * follow.ld_scaled + early_n) = o;
+        } else {
+          const int n = n0 + lg * 4;
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            if (n + j < n_end) {
+              float* at = (float*)C + (size_t)lr * ldc + n + j;
+              const float x = sum[j] + (bias ? bias[n + j] : 0.f) + *at;
+              *at = x;
+              follow.scaled[(size_t)lr * follow.ld_scaled + n + j] = (__bf16)(x * follow.gain[n + j]);
+              squares += x * x;
+            }
+        }
+      }
+      squares += __shfl_xor(squares, 16);
+      squares += __shfl_xor(squares, 32);
+      if (lg == 0) follow.sumsq[(size_t)blockIdx.x * 16 + lr] = squares;
+      continue;
+    }
     if (early && t == wave && early_m < M && early_n + 3 < n_end) {
       // the same sums in the same order as store4, with the operands read at the start
       if (bias) sum += early_bias;
@@ -650,7 +698,8 @@ int launch_skinny_as(const __bf16* A, const __bf16* W, const float* bias, TC* C,
                      long long ldc, int vector_ok, int rows, hipStream_t s) {
   if (rows <= 0 || rows > 16 * RT) rows = RT == 1 ? balanced_rows(M, N, 1, 1) : 16 * RT;
   const int blocks = (N + rows - 1) / rows;
-  gemm_skinny_kernel<CB, RT, WAVES, TC, ACC><<<blocks, WAVES * 64, 0, s>>>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, rows);
+  gemm_skinny_kernel<CB, RT, WAVES, TC, ACC><<<blocks, WAVES * 64, 0, s>>>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, rows,
+                                                                           FollowNorm{});
   VK_LAUNCH_CHECK();
   return 0;
 }
@@ -997,15 +1046,22 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const __bf16* __restrict_
 #endif
 constexpr int RES_CHUNK = 256;
 constexpr int RES_PARTIAL_BYTES = 4 * 2 * 2 * 64 * 16;  // [wave][first or last pair of its stretch][gate, up][lane]
+constexpr int RES_NORM_BYTES = 4 * 16 * 4;               // [wave][token]: sums of squares (SCALED)
+constexpr int RES_HEAD_BYTES = RES_PARTIAL_BYTES + RES_NORM_BYTES;
 
-template <int SETS>
+// SCALED: the activations are x * gain of a norm whose division is still to come (see FollowNorm): the sums of
+// squares of `groups` workgroups, 16 floats each, are added here in a fixed order (a thread takes every 256th
+// workgroup, then the block's tree), and 1 / sqrt(mean + eps) scales gate and up before the activation.
+template <int SETS, bool SCALED>
 __global__ __launch_bounds__(256) void gemm_resident_gated_kernel(const __bf16* __restrict__ A,
                                                                   const __bf16* __restrict__ W,
                                                                   __bf16* __restrict__ C, int M, int N, int K,
-                                                                  long long lda, long long ldc) {
+                                                                  long long lda, long long ldc,
+                                                                  const float* __restrict__ sumsq, int groups, float eps) {
   extern __shared__ __attribute__((aligned(16))) unsigned char res_lds[];
   f32x4* partial = (f32x4*)res_lds;
-  __bf16* acts = (__bf16*)(res_lds + RES_PARTIAL_BYTES);  // [M][K + 8]: 16 rows start in 16 different 16-byte slots
+  float* norm_part = (float*)(res_lds + RES_PARTIAL_BYTES);
+  __bf16* acts = (__bf16*)(res_lds + RES_HEAD_BYTES);  // [M][K + 8]: 16 rows start in 16 different 16-byte slots
   const int row_elems = K + 8;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1067,10 +1123,44 @@ __global__ __launch_bounds__(256) void gemm_resident_gated_kernel(const __bf16* 
       for (int j = 0; j < BATCH; ++j)
         if (at[j] >= 0) *(bf16x8*)(acts + at[j]) = stage[j];
     };
+    // The sums of squares are requested first of all and used after the other requests, so that adding them
+    // waits for nothing else: two groups per thread (at most 512 groups), unconditionally at clamped addresses,
+    // because a load behind a branch would make the compiler wait for every load in flight.
+    f32x4 squares[4], more[4];
+    if constexpr (SCALED) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        squares[q] = *(const f32x4*)(sumsq + (size_t)min(tid, groups - 1) * 16 + q * 4);
+        more[q] = *(const f32x4*)(sumsq + (size_t)min(tid + 256, groups - 1) * 16 + q * 4);
+      }
+    }
     request();
-    static_for<SETS - 1>([&](auto j) {
-      if (j.value < count) load_next(w[j.value]);
-    });
+    // unconditionally (a stretch shorter than the pipeline requests units past its end, which it does not use:
+    // memory of the next pairs, or nothing past the weight's end): behind a branch these loads would make the
+    // copy below wait for them, since the compiler could not tell how many are in flight
+    static_for<SETS - 1>([&](auto j) { load_next(w[j.value]); });
+    if constexpr (SCALED) {
+      const float has = tid < groups ? 1.f : 0.f, has_more = tid + 256 < groups ? 1.f : 0.f;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) squares[q] = squares[q] * has + more[q] * has_more;
+      // 16 sums over the wave's 64 lanes with 17 exchanges: at each of four steps a lane keeps one half of its
+      // values and adds the partner's copy of that half (the lane bit chooses which), then two full steps; lane
+      // l ends with the wave's sum of token 8 b0 + 4 b1 + 2 b2 + b3 (b: the bits of l)
+      float v[16];
+#pragma unroll
+      for (int m = 0; m < 16; ++m) v[m] = squares[m / 4][m % 4];
+      static_for<4>([&](auto step) {  // every index a compile-time constant: the values stay in registers
+        constexpr int bit = 1 << step.value, n = 8 >> step.value;
+        const bool upper = (lane & bit) != 0;
+        static_for<n>([&](auto i) {
+          const float got = __shfl_xor(upper ? v[i.value] : v[i.value + n], bit);
+          v[i.value] = (upper ? v[i.value + n] : v[i.value]) + got;
+        });
+      });
+      v[0] += __shfl_xor(v[0], 16);
+      v[0] += __shfl_xor(v[0], 32);
+      if (lane < 16) norm_part[wave * 16 + ((lane & 1) * 8 + (lane & 2) * 2 + (lane & 4) / 2 + (lane & 8) / 8)] = v[0];
+    }
     copy();
     for (int base = 256 * BATCH; base < pieces; base += 256 * BATCH) {
       request();
@@ -1080,13 +1170,19 @@ __global__ __launch_bounds__(256) void gemm_resident_gated_kernel(const __bf16* 
   __syncthreads();
 
   // a token past M gives a column of the instruction that is never stored: its lanes read the last row
-  const __bf16* a_lane = acts + min(lr, M - 1) * row_elems + lg * 8;
+  const int token = min(lr, M - 1);
+  float inv = 1.f;
+  if constexpr (SCALED) {
+    const float sum = norm_part[token] + norm_part[16 + token] + norm_part[32 + token] + norm_part[48 + token];
+    inv = 1.0f / sqrtf(sum / (float)K + eps);
+  }
+  const __bf16* a_lane = acts + token * row_elems + lg * 8;
   f32x4 acc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
   int mul_c = first_chunk, mul_p = first_pair;
   bool first_part = true, from_start = first_chunk == 0;
   auto flush = [&](bool to_end) {  // the sums of units [from_start ? 0 : first_chunk, mul_c) of pair mul_p
     if (from_start && to_end) {
-      store_gated(C, ldc, lr, (p_begin + mul_p) * 16 + lg * 4, M, N / 2, acc[0], acc[1]);
+      store_gated(C, ldc, lr, (p_begin + mul_p) * 16 + lg * 4, M, N / 2, acc[0] * inv, acc[1] * inv);
     } else {
       f32x4* dst = partial + (wave * 2 + (first_part ? 0 : 1)) * 2 * 64;
       dst[lane] = acc[0];
@@ -1142,7 +1238,7 @@ __global__ __launch_bounds__(256) void gemm_resident_gated_kernel(const __bf16* 
         gate += theirs[lane];
         up += theirs[64 + lane];
       }
-      store_gated(C, ldc, lr, (p_begin + p) * 16 + lg * 4, M, N / 2, gate, up);
+      store_gated(C, ldc, lr, (p_begin + p) * 16 + lg * 4, M, N / 2, gate * inv, up * inv);
     }
   }
 }
@@ -1150,16 +1246,17 @@ __global__ __launch_bounds__(256) void gemm_resident_gated_kernel(const __bf16* 
 // Whether the resident kernel takes the shape, and the LDS it asks for (0: it does not).
 int resident_lds_bytes(int M, int N, int K) {
   if (M > 16 || (K % RES_CHUNK) || (N & 31)) return 0;
-  const long long need = RES_PARTIAL_BYTES + (long long)M * (K + 8) * 2;
+  const long long need = RES_HEAD_BYTES + (long long)M * (K + 8) * 2;
   if (need > 160 * 1024) return 0;
   return (int)(need > 82 * 1024 ? need : 82 * 1024);  // more than half a CU's LDS: one workgroup per CU
 }
 
+template <bool SCALED>
 int launch_resident_gated(const __bf16* A, const __bf16* W, __bf16* C, int M, int N, int K, long long lda,
-                          long long ldc, hipStream_t s) {
+                          long long ldc, const float* sumsq, int norm_groups, float eps, hipStream_t s) {
   const int lds_bytes = resident_lds_bytes(M, N, K);
   if (!lds_bytes) return VK_UNSUPPORTED_SIZE;
-  auto kernel = gemm_resident_gated_kernel<VK_RESIDENT_SETS>;
+  auto kernel = gemm_resident_gated_kernel<VK_RESIDENT_SETS, SCALED>;
   static bool configured = false;
   if (!configured) {
     hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
@@ -1171,7 +1268,7 @@ int launch_resident_gated(const __bf16* A, const __bf16* W, __bf16* C, int M, in
   const int groups = pairs < cus ? pairs : cus;
   // byte offsets from a wave's first pair are 32-bit
   if (((long long)(pairs / groups) + 2) * 64 * K >= (1ll << 31)) return VK_UNSUPPORTED_SIZE;
-  kernel<<<groups, 256, lds_bytes, s>>>(A, W, C, M, N, K, lda, ldc);
+  kernel<<<groups, 256, lds_bytes, s>>>(A, W, C, M, N, K, lda, ldc, sumsq, norm_groups, eps);
   VK_LAUNCH_CHECK();
   return 0;
 }
@@ -1467,7 +1564,7 @@ extern "C" int vk_gemm_bf16_gated(const void* A, const void* W, void* C, int M, 
   const __bf16* w = (const __bf16*)W;
   __bf16* c = (__bf16*)C;
   if (M > 64 || rows_per_wave == 3) return launch_tile<__bf16, false, true>(a, w, nullptr, c, M, N, K, lda, ldc, 0, nullptr, 0, s);
-  if (rows_per_wave == 0) return launch_resident_gated(a, w, c, M, N, K, lda, ldc, s);
+  if (rows_per_wave == 0) return launch_resident_gated<false>(a, w, c, M, N, K, lda, ldc, nullptr, 0, 0.f, s);
   const int cb = (M + 15) / 16;
 #define VK_GATED(CBV, RTV)                                                                                         \
   {                                                                                                                \
@@ -1522,6 +1619,44 @@ extern "C" int vk_gemm_bf16_qkv_rope(const void* A, const void* W, const float* 
                                                                      M, N, K, lda, ldc, r);
   VK_LAUNCH_CHECK();
   return 0;
+}
+
+// C += A W^T + bias for up to 16 tokens (C float: the residual), and what the RMS norm after it needs (see
+// FollowNorm): scaled[M, N] = bfloat16(C * gain) with row stride ld_scaled, and the workgroups' sums of squares,
+// sumsq[*groups][16] floats (`sumsq_floats`: the room there is). *groups receives the number of workgroups.
+extern "C" int vk_gemm_bf16_follow(const void* A, const void* W, const float* bias, float* C, int M, int N, int K,
+                                   long long lda, long long ldc, const float* gain, void* scaled, long long ld_scaled,
+                                   float* sumsq, long long sumsq_floats, int* groups, void* stream) {
+  if (M <= 0 || N <= 0 || M > 16) return VK_UNSUPPORTED_SIZE;
+  if (K <= 0 || (K & 7) || (lda & 7) || lda < K || ldc < N || ld_scaled < N || !gain || !scaled || !sumsq || !groups)
+    return VK_BAD_ARGUMENT;
+  if (((uintptr_t)A & 15) || ((uintptr_t)W & 15)) return VK_BAD_ARGUMENT;
+  if (K >= (1 << 23) || lda >= (1 << 23)) return VK_UNSUPPORTED_SIZE;
+  const int vector_ok = ((ldc & 3) == 0 && ((uintptr_t)C & 15) == 0 && (bias == nullptr || ((uintptr_t)bias & 15) == 0) &&
+                         ((uintptr_t)gain & 15) == 0 && (ld_scaled & 3) == 0 && ((uintptr_t)scaled & 7) == 0) ? 1 : 0;
+  int rows = balanced_rows(M, N, 1, 1);
+  if ((N + rows - 1) / rows > 512) rows = 16;  // the product after the norm adds at most 512 groups
+  const int blocks = (N + rows - 1) / rows;
+  if (blocks > 512 || (long long)blocks * 16 > sumsq_floats) return VK_UNSUPPORTED_SIZE;
+  *groups = blocks;
+  gemm_skinny_kernel<1, 1, 4, float, true, VK_SKINNY_SETS, true><<<blocks, 256, 0, (hipStream_t)stream>>>(
+      (const __bf16*)A, (const __bf16*)W, bias, C, M, N, K, lda, ldc, vector_ok, rows,
+      FollowNorm{gain, (__bf16*)scaled, sumsq, ld_scaled});
+  VK_LAUNCH_CHECK();
+  return 0;
+}
+
+// vk_gemm_bf16_gated with resident activations (rows_per_wave 0) on the output of vk_gemm_bf16_follow: A = scaled,
+// and gate and up are divided by the root mean square that `sumsq[groups][16]` and `eps` give before the activation.
+extern "C" int vk_gemm_bf16_gated_scaled(const void* A, const void* W, void* C, int M, int N, int K, long long lda,
+                                         long long ldc, const float* sumsq, int groups, float eps, void* stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (K <= 0 || (K & 7) || (lda & 7) || lda < K || (N & 31) || ldc < N / 2 || !sumsq || groups <= 0) return VK_BAD_ARGUMENT;
+  if (((uintptr_t)A & 15) || ((uintptr_t)W & 15) || ((uintptr_t)sumsq & 15)) return VK_BAD_ARGUMENT;
+  if (K >= (1 << 23) || lda >= (1 << 23)) return VK_UNSUPPORTED_SIZE;
+  if (groups > 512) return VK_UNSUPPORTED_SIZE;  // a thread adds two groups
+  return launch_resident_gated<true>((const __bf16*)A, (const __bf16*)W, (__bf16*)C, M, N, K, lda, ldc, sumsq, groups, eps,
+                                     (hipStream_t)stream);
 }
 
 extern "C" int vk_gemm_bf16_tile_config(int config) {

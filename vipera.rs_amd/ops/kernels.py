@@ -368,6 +368,64 @@ def gemm_bf16_qkv_rope(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Te
                _stream()), "gemm_bf16_qkv_rope")
 
 
+def gemm_bf16_follow_supported(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> bool:
+    """Whether :func:`gemm_bf16_follow` takes the operands: bfloat16 product of up to 16 tokens into a float32
+    residual whose width is a multiple of four and at most 8,192 (512 workgroups of 16 columns)."""
+    return (out.dtype == torch.float32 and 1 <= a.shape[0] <= 16 and out.shape[1] % 4 == 0 and out.shape[1] <= 8192
+            and out.is_contiguous() and gemm_bf16_supported(a, w, out))
+
+
+def follow_sumsq_floats(n: int) -> int:
+    """Floats that the sums of squares of :func:`gemm_bf16_follow` may take for an output of ``n`` columns
+    (16 per workgroup, a workgroup owns at least 8 columns)."""
+    return ((n + 7) // 8) * 16
+
+
+def gemm_bf16_follow(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
+                     gain: torch.Tensor, scaled: torch.Tensor, sumsq: torch.Tensor) -> int:
+    """``out += a @ w.T + bias`` (``out`` float32: the residual) for up to 16 tokens, and the first half of the RMS
+    norm that follows: ``scaled = bfloat16(out * gain)`` and per workgroup the sums of squares of its columns
+    (``sumsq[groups, 16]``).  Returns ``groups``; :func:`gemm_bf16_gated_scaled` does the other half."""
+    _dev(a, w, bias, out, gain, scaled, sumsq)
+    m, k = a.shape
+    n = w.shape[0]
+    _need(w.shape[1] == k and out.shape == (m, n) and scaled.shape == (m, n), "gemm_bf16_follow: shapes")
+    _need(gemm_bf16_follow_supported(a, w, out), "gemm_bf16_follow: bfloat16 operands, a float32 output, at most 16 tokens")
+    _need(scaled.dtype == torch.bfloat16 and scaled.is_contiguous(), "gemm_bf16_follow: scaled must be bfloat16 [m, n]")
+    _need(gain.dtype == torch.float32 and gain.numel() == n and gain.is_contiguous(), "gemm_bf16_follow: gain must be float32 [n]")
+    _need(sumsq.dtype == torch.float32 and sumsq.is_contiguous() and sumsq.numel() >= follow_sumsq_floats(n),
+          "gemm_bf16_follow: sumsq is too small")
+    if bias is not None:
+        _need(bias.dtype == torch.float32 and bias.numel() == n and bias.is_contiguous(), "gemm: bias must be float32 [n]")
+    lda = a.stride(0) if m > 1 else max(a.stride(0), k)
+    lda = lda if lda % 8 == 0 else k
+    groups = ctypes.c_int(0)
+    fn = _fn("gemm_bf16", "vk_gemm_bf16_follow", [_p, _p, _p, _p, _i, _i, _i, _ll, _ll, _p, _p, _ll, _p, _ll,
+                                                  ctypes.POINTER(ctypes.c_int), _p])
+    _status(fn(_ptr(a), _ptr(w), _ptr(bias), _ptr(out), m, n, k, lda, n, _ptr(gain), _ptr(scaled), n, _ptr(sumsq),
+               sumsq.numel(), ctypes.byref(groups), _stream()), "gemm_bf16_follow")
+    return int(groups.value)
+
+
+def gemm_bf16_gated_scaled(scaled: torch.Tensor, w: torch.Tensor, out: torch.Tensor, sumsq: torch.Tensor, groups: int,
+                           eps: float) -> None:
+    """:func:`gemm_bf16_gated` with resident activations on what :func:`gemm_bf16_follow` left: ``scaled`` is
+    ``x * gain`` in bfloat16, and gate and up are divided by the root mean square of ``x`` (from the ``groups``
+    sums of squares and ``eps``) before the activation."""
+    _dev(scaled, w, out, sumsq)
+    m, k = scaled.shape
+    n = w.shape[0]
+    _need(w.shape[1] == k and out.shape == (m, n // 2) and n % 32 == 0, "gemm_gated: shapes")
+    _need(gemm_bf16_supported(scaled, w, out) and out.dtype == torch.bfloat16, "gemm_gated: operands must be bfloat16")
+    _need(sumsq.dtype == torch.float32 and sumsq.numel() >= groups * 16 and groups >= 1, "gemm_bf16_gated_scaled: sumsq")
+    lda = scaled.stride(0) if m > 1 else max(scaled.stride(0), k)
+    lda = lda if lda % 8 == 0 else k
+    ldc = out.stride(0) if m > 1 else max(out.stride(0), n // 2)
+    fn = _fn("gemm_bf16", "vk_gemm_bf16_gated_scaled", [_p, _p, _p, _i, _i, _i, _ll, _ll, _p, _i, _f, _p])
+    _status(fn(_ptr(scaled), _ptr(w), _ptr(out), m, n, k, lda, ldc, _ptr(sumsq), int(groups), float(eps), _stream()),
+            "gemm_bf16_gated_scaled")
+
+
 TILE_TILINGS = {0: "128x128 staged", 2: "256x128 staged", 3: "128x256 staged", 4: "256x256 staged",
                 9: "128x128 direct", 7: "256x128 direct", 8: "128x256 direct", 5: "256x256 direct", 6: "256x192 direct"}
 

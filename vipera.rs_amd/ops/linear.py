@@ -62,7 +62,7 @@ def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     return fused.reshape(2 * inter, width).contiguous()
 
 
-RESIDENT_LDS_BYTES = 160 * 1024 - 16 * 1024   # what the resident kernel may fill with activations
+RESIDENT_LDS_BYTES = 160 * 1024 - (16 * 1024 + 256)   # what the resident kernel may fill with activations
 
 
 def gated_resident_fits(m: int, n: int, k: int) -> bool:

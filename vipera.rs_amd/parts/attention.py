@@ -76,7 +76,9 @@ class Attention(Mixer):
     def cache_spec(self) -> Optional[KVCacheSpec]:
         return KVCacheSpec(self.kv_heads, self.head_dim, self.window)
 
-    def forward(self, h, batch, cache, state, position, residual, reads_only: bool = False) -> None:
+    fills_handoff = True
+
+    def forward(self, h, batch, cache, state, position, residual, reads_only: bool = False, handoff=None) -> None:
         tokens = h.shape[0]
         qkv = self.runtime.empty((tokens, self.q_width + 2 * self.kv_width))
         table = batch.block_tables[cache.group]
@@ -104,7 +106,14 @@ class Attention(Mixer):
         attn = self.runtime.empty((tokens, self.q_width))
         paged_attention(qkv, cache.k, cache.v, attn, batch, table, self.heads, self.kv_heads, self.head_dim,
                         self.scale, self.window)
-        linear(attn, self.w_o, self.b_o, residual, accumulate=True)
+        if (handoff is not None and attn.dtype == torch.bfloat16 and self.w_o.dtype == torch.bfloat16
+                and streams_in_wave_order(tokens, *self.w_o.shape)
+                and kernels.gemm_bf16_follow_supported(attn, self.w_o, residual)):
+            # the output product also prepares the norm that follows (its gained copy of the residual, its squares)
+            handoff.groups = kernels.gemm_bf16_follow(attn, self.w_o, self.b_o, residual, handoff.gain, handoff.scaled,
+                                                      handoff.sumsq)
+        else:
+            linear(attn, self.w_o, self.b_o, residual, accumulate=True)
 
 
 register_mixer("attention", Attention)

@@ -66,10 +66,28 @@ class Part:
         """Take the declared tensors (already on the device in their kept dtype)."""
 
 
+@dataclass
+class NormHandoff:
+    """A norm whose work is split between the products around it (few tokens, see
+    ``kernels.gemm_bf16_follow``): the part before the norm, while it adds into the residual ``x``, fills
+    ``scaled = x * gain`` and the workgroups' sums of squares and sets ``groups``; the part after the norm takes
+    ``scaled`` as its input and divides by the root mean square itself.  ``groups`` 0: not filled (the part before
+    could not), and the norm runs as a kernel of its own."""
+    gain: torch.Tensor
+    eps: float
+    scaled: torch.Tensor
+    sumsq: torch.Tensor
+    groups: int = 0
+
+
 class Norm(Part):
     def forward(self, x: torch.Tensor, out: Optional[torch.Tensor] = None,
                 rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         raise NotImplementedError
+
+    def handoff(self, tokens: int) -> Optional[NormHandoff]:
+        """A :class:`NormHandoff` for ``tokens`` rows if this norm can be split between its neighbours, else None."""
+        return None
 
 
 class PositionEncoding(Part):
@@ -92,11 +110,18 @@ class Mixer(Part):
     def state_spec(self) -> Optional[StateSpec]:
         return None
 
+    #: a mixer that sets this takes ``handoff=`` in ``forward`` and may fill it (see :class:`NormHandoff`)
+    fills_handoff = False
+
     def forward(self, h, batch, cache, state, position, residual, reads_only: bool = False) -> None:
         raise NotImplementedError
 
 
 class FeedForward(Part):
+    def accepts_handoff(self, tokens: int) -> bool:
+        """Whether ``forward`` takes a filled :class:`NormHandoff` (``handoff=``, with ``h`` None) for ``tokens`` rows."""
+        return False
+
     def forward(self, h, batch, residual) -> None:
         raise NotImplementedError
 

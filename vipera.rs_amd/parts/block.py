@@ -37,9 +37,20 @@ class PreNormBlock(Block):
 
     def forward(self, x, batch, cache, state, reads_only: bool = False) -> None:
         h = self.mixer_norm.forward(x)
-        self.mixer.forward(h, batch, cache, state, self.position, x, reads_only)
-        h = self.ffn_norm.forward(x)
-        self.ffn.forward(h, batch, x)
+        # with a few tokens the second norm may be split between the mixer's last product and the feed-forward's
+        # first, if all three can (see NormHandoff); otherwise it is a kernel of its own
+        handoff = None
+        if self.mixer.fills_handoff and self.ffn.accepts_handoff(x.shape[0]):
+            handoff = self.ffn_norm.handoff(x.shape[0])
+        if handoff is None:
+            self.mixer.forward(h, batch, cache, state, self.position, x, reads_only)
+        else:
+            self.mixer.forward(h, batch, cache, state, self.position, x, reads_only, handoff=handoff)
+        if handoff is not None and handoff.groups:
+            self.ffn.forward(None, batch, x, handoff=handoff)
+        else:
+            h = self.ffn_norm.forward(x)
+            self.ffn.forward(h, batch, x)
 
 
 register_block("prenorm", PreNormBlock)

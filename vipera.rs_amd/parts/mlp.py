@@ -13,7 +13,7 @@ import torch
 from ..config.base import PartSpec
 from ..errors import UnsupportedError
 from ..ops import kernels
-from ..ops.linear import interleave_gate_up, linear, linear_gated
+from ..ops.linear import gated_plan, interleave_gate_up, linear, linear_gated
 from ..weights.checkpoint import MATRIX, TensorSpec
 from .attention import _cat
 from .base import FeedForward, register_ffn
@@ -48,10 +48,19 @@ class GatedMLP(FeedForward):
         self.w_gate_up = interleave_gate_up(gate, up) if self.interleaved else _cat([gate, up])
         self.w_down = tensors[base + "down_proj.weight"]
 
-    def forward(self, h, batch, residual) -> None:
-        tokens = h.shape[0]
+    def accepts_handoff(self, tokens: int) -> bool:
+        # where the gate/up product is the kernel with resident activations, which can divide by the norm itself
+        return (self.interleaved and self.w_gate_up.dtype == torch.bfloat16 and self.runtime.dtype == torch.bfloat16
+                and tokens <= 16 and gated_plan(tokens, *self.w_gate_up.shape,
+                                                kernels.compute_units(self.w_gate_up.device)) == 0)
+
+    def forward(self, h, batch, residual, handoff=None) -> None:
+        tokens = residual.shape[0]
         act = self.runtime.empty((tokens, self.inter))
-        linear_gated(h, self.w_gate_up, act, self.interleaved)
+        if handoff is not None:
+            kernels.gemm_bf16_gated_scaled(handoff.scaled, self.w_gate_up, act, handoff.sumsq, handoff.groups, handoff.eps)
+        else:
+            linear_gated(h, self.w_gate_up, act, self.interleaved)
         linear(act, self.w_down, None, residual, accumulate=True)
 
 

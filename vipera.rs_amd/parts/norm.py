@@ -12,7 +12,7 @@ import torch
 from ..config.base import PartSpec
 from ..ops import kernels
 from ..weights.checkpoint import VECTOR, TensorSpec
-from .base import Norm, register_norm
+from .base import Norm, NormHandoff, register_norm
 
 
 class RMSNorm(Norm):
@@ -29,6 +29,13 @@ class RMSNorm(Norm):
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         self.weight = tensors[f"{self.prefix}{self.spec.params['name']}.weight"]
+
+    def handoff(self, tokens: int) -> Optional[NormHandoff]:
+        if self.runtime.dtype != torch.bfloat16 or self.weight is None or self.weight.dtype != torch.float32:
+            return None
+        return NormHandoff(self.weight, self.eps, self.runtime.empty((tokens, self.width)),
+                           torch.empty(kernels.follow_sumsq_floats(self.width), dtype=torch.float32,
+                                       device=self.weight.device))
 
     def forward(self, x, out=None, rows=None):
         count = x.shape[0] if rows is None else rows.numel()
