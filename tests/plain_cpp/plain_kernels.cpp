@@ -231,14 +231,34 @@ extern "C" int plain_gemm_bf16_gated(const void* A, const void* W, void* C, int 
   return 0;
 }
 
-// The fused q/k/v product: the product in bfloat16, then the rotation and the cache write on its output.
+// The fused q/k/v product: the product in bfloat16, then the rotation and the cache write on its output. With
+// `sumsq`, A is x * gain of a norm whose division is still due: the product's sums are divided by the root mean
+// square that the `norm_groups` sums of squares give, before the bias.
+extern "C" int plain_rope_kvwrite(void* qkv, int dtype, const int* positions, const float* inv_freq,
+                                  const float* angles, int rotary_dim, void* k_cache, void* v_cache,
+                                  const int* entry_of_token, const int* block_table, int table_width, int block_size,
+                                  int num_tokens, int heads, int kv_heads, int hd, void*);
 extern "C" int plain_gemm_bf16_qkv_rope(const void* A, const void* W, const float* bias, void* C, int M, int N, int K,
                                         long long lda, long long ldc, const int* positions, const float* inv_freq,
                                         void* k_cache, void* v_cache, const int* entry_of_token, const int* block_table,
-                                        int table_width, int block_size, int heads, int kv_heads, int hd, void*) {
+                                        int table_width, int block_size, int heads, int kv_heads, int hd,
+                                        const float* sumsq, int norm_groups, float eps, void*) {
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0 || lda < K || ldc != N || (long long)(heads + 2 * kv_heads) * hd != N) return BAD_ARGUMENT;
-  product(A, DT_BF16, W, DT_BF16, bias, C, DT_BF16, M, N, K, lda, ldc, false);
+  for (int m = 0; m < M; ++m) {
+    double inv = 1.0;
+    if (sumsq) {
+      double squares = 0.0;
+      for (int g = 0; g < norm_groups; ++g) squares += (double)sumsq[(size_t)g * 16 + m];
+      inv = 1.0 / std::sqrt(squares / (double)K + (double)eps);
+    }
+    for (int n = 0; n < N; ++n) {
+      double sum = 0.0;
+      for (int k = 0; k < K; ++k)
+        sum += (double)load(A, DT_BF16, (size_t)m * lda + k) * (double)load(W, DT_BF16, (size_t)n * K + k);
+      store(C, DT_BF16, (size_t)m * ldc + n, (float)(sum * inv) + (bias ? bias[n] : 0.f));
+    }
+  }
   return plain_rope_kvwrite(C, DT_BF16, positions, inv_freq, nullptr, hd, k_cache, v_cache, entry_of_token, block_table,
                             table_width, block_size, M, heads, kv_heads, hd, nullptr);
 }
@@ -262,6 +282,19 @@ extern "C" int plain_gemm_bf16_follow(const void* A, const void* W, const float*
   }
   *groups = 1;
   return 0;
+}
+
+extern "C" int plain_gemm_bf16_follow(const void* A, const void* W, const float* bias, float* C, int M, int N, int K,
+                                      long long lda, long long ldc, const float* gain, void* scaled, long long ld_scaled,
+                                      float* sumsq, long long sumsq_floats, int* groups, void*);
+// The same where the kernel splits K over workgroups (no difference for the twin).
+extern "C" int plain_gemm_bf16_mid_follow(const void* A, const void* W, const float* bias, float* C, int M, int N, int K,
+                                          long long lda, long long ldc, int, int, float*, long long, const float* gain,
+                                          void* scaled, long long ld_scaled, float* sumsq, long long sumsq_floats,
+                                          int* groups, void*) {
+  if (M > 16) return BAD_ARGUMENT;  // the twin's sums of squares hold 16 tokens, as the consumers do
+  return plain_gemm_bf16_follow(A, W, bias, C, M, N, K, lda, ldc, gain, scaled, ld_scaled, sumsq, sumsq_floats, groups,
+                                nullptr);
 }
 
 // The gated product on such a scaled input: gate and up divided by the root mean square first.

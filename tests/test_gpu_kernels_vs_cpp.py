@@ -103,7 +103,7 @@ def test_fused_qkv_product_beside_its_twin_and_the_two_kernels(m, heads, kv_head
     k_cache = torch.full((40, kv_heads, bs, hd), 9.0, dtype=torch.bfloat16) if with_cache else None
     v_cache = torch.full((40, kv_heads, hd, bs), 9.0, dtype=torch.bfloat16) if with_cache else None
     args = [a, w, bias, torch.empty(m, n, dtype=torch.bfloat16), m, n, k, k, n, i32(positions), inv, k_cache, v_cache,
-            i32(entry_of), table, 130, bs, heads, kv_heads, hd, None]
+            i32(entry_of), table, 130, bs, heads, kv_heads, hd, None, 0, 0.0, None]
     outs = both("gemm_bf16", "gemm_bf16_qkv_rope", args, [3, 11, 12] if with_cache else [3])
     for got, want in outs:
         assert rel_err(got.float().numpy(), want.double().numpy()) < 8e-3
@@ -121,6 +121,68 @@ def test_fused_qkv_product_beside_its_twin_and_the_two_kernels(m, heads, kv_head
     if with_cache:
         assert torch.equal(kc, dev[11]) and torch.equal(vc, dev[12])
         assert torch.equal(kc.cpu(), outs[1][0]) and float((kc == 9.0).float().mean()) > 0.5
+
+
+@pytest.mark.parametrize("m,width,k_in,heads,kv_heads,hd,split", [(8, 512, 2048, 6, 2, 32, True), (3, 256, 1024, 2, 1, 64, False),
+                                                                  (16, 1024, 4096, 12, 4, 16, True), (1, 384, 520, 5, 1, 48, False)])
+def test_the_first_norm_of_a_layer_split_between_the_layers(m, width, k_in, heads, kv_heads, hd, split):
+    """x += act Wd^T (K split over workgroups or not), h = rms_norm(x) * g, q/k/v = h W^T + b, rotation, cache write
+    as two kernels, each beside its twin and together against 64-bit."""
+    from vipera_rs_amd.ops import kernels
+    n = (heads + 2 * kv_heads) * hd
+    g = torch.Generator().manual_seed(m + width + k_in)
+    act = torch.randn(m, k_in, generator=g).to(torch.bfloat16)
+    w_d = (torch.randn(width, k_in, generator=g) / math.sqrt(k_in)).to(torch.bfloat16)
+    x0 = torch.randn(m, width, generator=g) * 2
+    gain = 1 + 0.2 * torch.randn(width, generator=g)
+    w = (torch.randn(n, width, generator=g) / math.sqrt(width)).to(torch.bfloat16)
+    bias = torch.randn(n, generator=g)
+    floats = kernels.follow_sumsq_floats(width)
+    groups_d, groups_h = ctypes.c_int(0), ctypes.c_int(0)
+    if split:
+        partial = torch.empty(4 * 64 * width)
+        name, args = "gemm_bf16_mid_follow", [act, w_d, None, x0, m, width, k_in, k_in, width, 4, 1, partial, partial.numel(), gain,
+                                              torch.empty(m, width, dtype=torch.bfloat16), width, torch.zeros(floats), floats]
+    else:
+        name, args = "gemm_bf16_follow", [act, w_d, None, x0, m, width, k_in, k_in, width, gain,
+                                          torch.empty(m, width, dtype=torch.bfloat16), width, torch.zeros(floats), floats]
+    x_at, scaled_at, sumsq_at = (3, 14, 16) if split else (3, 10, 12)
+    host = [a.clone() if isinstance(a, torch.Tensor) else a for a in args]
+    dev = [a.to(DEV) if isinstance(a, torch.Tensor) else a for a in args]
+    from plain_cpp import library, ptr
+    twin = getattr(library(), "plain_" + name)
+    assert twin(*[ptr(a) if isinstance(a, torch.Tensor) else a for a in host], ctypes.byref(groups_h), None) == 0
+    fn = _kernel_with_pointer(name)
+    assert fn(*[a.data_ptr() if isinstance(a, torch.Tensor) else a for a in dev], ctypes.byref(groups_d), None) == 0
+    torch.cuda.synchronize()
+    assert rel_err(dev[x_at].cpu().numpy(), host[x_at].double().numpy()) < 1e-5
+    assert rel_err(dev[scaled_at].float().cpu().numpy(), host[scaled_at].double().numpy()) < 6e-3
+    got = dev[sumsq_at][: groups_d.value * 16].view(groups_d.value, 16).double().sum(0)[:m].cpu()
+    assert rel_err(got.numpy(), host[sumsq_at][:m].double().numpy()) < 1e-5
+    # the product after the norm, on the device's own output
+    positions, entry_of = list(range(40, 40 + m)), list(range(m))
+    inv = (1.0 / torch.pow(torch.tensor(1e6), torch.arange(hd // 2).float() * 2 / hd)).float()
+    table = torch.arange(m * 4, dtype=torch.int32).view(m, 4)
+    bs = 16
+    k_cache = torch.zeros(m * 4, kv_heads, bs, hd, dtype=torch.bfloat16)
+    v_cache = torch.zeros(m * 4, kv_heads, hd, bs, dtype=torch.bfloat16)
+    args = [dev[scaled_at].cpu(), w, bias, torch.empty(m, n, dtype=torch.bfloat16), m, n, width, width, n, i32(positions), inv,
+            k_cache, v_cache, i32(entry_of), table, 4, bs, heads, kv_heads, hd, dev[sumsq_at].cpu(), groups_d.value, 1e-5, None]
+    for got, want in both("gemm_bf16", "gemm_bf16_qkv_rope", args, [3, 11, 12]):
+        assert rel_err(got.float().numpy(), want.double().numpy()) < 8e-3
+    # and against 64-bit from the start
+    x = x0.double() + act.double() @ w_d.double().T
+    h = x * torch.rsqrt((x ** 2).mean(-1, keepdim=True) + 1e-5) * gain.double()
+    want_v = (h @ w.double().T + bias.double())[:, (heads + kv_heads) * hd:]
+    (got, _), _, _ = both("gemm_bf16", "gemm_bf16_qkv_rope", args, [3, 11, 12])
+    assert rel_err(got.float().numpy()[:, (heads + kv_heads) * hd:], want_v.numpy()) < 1e-2
+
+
+def _kernel_with_pointer(name):
+    from vipera_rs_amd.ops.build import load_module
+    fn = getattr(load_module("gemm_bf16"), "vk_" + name)
+    fn.argtypes, fn.restype = SIGNATURES["plain_" + name], ctypes.c_int
+    return fn
 
 
 PRODUCTS = [(1, 48, 64), (7, 300, 96), (33, 1000, 264), (65, 130, 72), (200, 257, 136), (300, 520, 1024), (515, 384, 192)]

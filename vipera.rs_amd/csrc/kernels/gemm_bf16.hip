@@ -549,6 +549,48 @@ struct FollowNorm {
   long long ld_scaled;
 };
 
+// The consumer's side of FollowNorm in a workgroup of 256 threads. request_squares: thread t asks for the sums of
+// groups t and t + 256 (at most 512 groups), unconditionally at clamped addresses, because a load behind a branch
+// would make the compiler wait for every load in flight; call it before the kernel's other loads. add_squares: the
+// 16 tokens' sums over the wave's lanes with 17 exchanges (at each of four steps a lane keeps one half of its
+// values and adds the partner's copy of that half, the lane bit choosing which; then two full steps), left in
+// wave_sums[wave * 16 + token]; every index is a compile-time constant, so the values stay in registers.
+// inv_rms: after a barrier, 1 / sqrt(mean + eps) of a token from the four waves' sums (a fixed order throughout).
+struct Squares {
+  f32x4 first[4], second[4];
+};
+__device__ __forceinline__ Squares request_squares(const float* __restrict__ sumsq, int groups, int tid) {
+  Squares q;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    q.first[i] = *(const f32x4*)(sumsq + (size_t)min(tid, groups - 1) * 16 + i * 4);
+    q.second[i] = *(const f32x4*)(sumsq + (size_t)min(tid + 256, groups - 1) * 16 + i * 4);
+  }
+  return q;
+}
+__device__ __forceinline__ void add_squares(const Squares& q, int groups, int tid, float* wave_sums) {
+  const int lane = tid & 63, wave = tid >> 6;
+  const bool has = tid < groups, has_more = tid + 256 < groups;
+  float v[16];
+#pragma unroll
+  for (int m = 0; m < 16; ++m) v[m] = (has ? q.first[m / 4][m % 4] : 0.f) + (has_more ? q.second[m / 4][m % 4] : 0.f);
+  static_for<4>([&](auto step) {
+    constexpr int bit = 1 << step.value, n = 8 >> step.value;
+    const bool upper = (lane & bit) != 0;
+    static_for<n>([&](auto i) {
+      const float got = __shfl_xor(upper ? v[i.value] : v[i.value + n], bit);
+      v[i.value] = (upper ? v[i.value + n] : v[i.value]) + got;
+    });
+  });
+  v[0] += __shfl_xor(v[0], 16);
+  v[0] += __shfl_xor(v[0], 32);
+  if (lane < 16) wave_sums[wave * 16 + ((lane & 1) * 8 + (lane & 2) * 2 + (lane & 4) / 2 + (lane & 8) / 8)] = v[0];
+}
+__device__ __forceinline__ float inv_rms(const float* wave_sums, int token, int width, float eps) {
+  const float sum = wave_sums[token] + wave_sums[16 + token] + wave_sums[32 + token] + wave_sums[48 + token];
+  return 1.0f / sqrtf(sum / (float)width + eps);
+}
+
 template <int CB, int RT, int WAVES, typename TC, bool ACCUMULATE, int SETS = (CB == 1 ? VK_SKINNY_SETS : 2),
           bool FOLLOW = false>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const __bf16* __restrict__ A,
@@ -756,18 +798,24 @@ struct QkvRope {
   const int* entry_of_token;
   const int* block_table;
   int table_width, block_size, heads, kv_heads, hd, pairs, values;
+  const float* sumsq;  // SCALED: A is x * gain of the norm before (see FollowNorm), `groups` sums of squares, `eps`
+  int groups;
+  float eps;
 };
 
-template <int RT>
+template <int RT, bool SCALED>
 __global__ __launch_bounds__(256) void gemm_qkv_rope_kernel(const __bf16* __restrict__ A, const __bf16* __restrict__ W,
                                                             const float* __restrict__ bias, __bf16* __restrict__ C,
                                                             int M, int N, int K, long long lda, long long ldc, QkvRope r) {
   constexpr int WAVES = 4;
   constexpr unsigned NO_ROW = 0x80000000u;  // past the end of the weight's view (the launcher checks its size)
   __shared__ f32x4 partial[WAVES][RT][64];
+  __shared__ float wave_sums[64];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lr = lane & 15, lg = lane >> 4;
+  Squares squares;
+  if constexpr (SCALED) squares = request_squares(r.sumsq, r.groups, tid);
   const int hd = r.hd, half = hd / 2;
   const int all_pairs = (r.heads + r.kv_heads) * half, all_values = r.kv_heads * hd, first_value_row = (r.heads + r.kv_heads) * hd;
   // Row i of the first tile -> its output column, or -1: slots 0 .. pairs - 1 of each half of the tile hold the
@@ -820,6 +868,7 @@ __global__ __launch_bounds__(256) void gemm_qkv_rope_kernel(const __bf16* __rest
   int page = -1;
   float sn[4], cs[4];
   auto lookups = [&]() {
+    if constexpr (SCALED) add_squares(squares, r.groups, tid, wave_sums);
     if (r.k_cache) page = r.block_table[(size_t)entry * r.table_width + pos / r.block_size];
 #pragma unroll
     for (int j = 0; j < 4; ++j) sincosf((float)pos * freq[j], &sn[j], &cs[j]);
@@ -833,6 +882,7 @@ __global__ __launch_bounds__(256) void gemm_qkv_rope_kernel(const __bf16* __rest
 #pragma unroll
   for (int w = 1; w < WAVES; ++w) sum += partial[w][wave][lane];
   const int slot = pos % r.block_size;
+  if constexpr (SCALED) sum *= inv_rms(wave_sums, token, K, r.eps);  // the barrier above has published the waves' sums
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const float x = (float)(__bf16)(sum[j] + b[j]);
@@ -1123,44 +1173,16 @@ __global__ __launch_bounds__(256) void gemm_resident_gated_kernel(const __bf16* 
       for (int j = 0; j < BATCH; ++j)
         if (at[j] >= 0) *(bf16x8*)(acts + at[j]) = stage[j];
     };
-    // The sums of squares are requested first of all and used after the other requests, so that adding them
-    // waits for nothing else: two groups per thread (at most 512 groups), unconditionally at clamped addresses,
-    // because a load behind a branch would make the compiler wait for every load in flight.
-    f32x4 squares[4], more[4];
-    if constexpr (SCALED) {
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        squares[q] = *(const f32x4*)(sumsq + (size_t)min(tid, groups - 1) * 16 + q * 4);
-        more[q] = *(const f32x4*)(sumsq + (size_t)min(tid + 256, groups - 1) * 16 + q * 4);
-      }
-    }
+    // the sums of squares are requested first of all and added after the other requests, so that adding them waits
+    // for nothing else
+    Squares squares;
+    if constexpr (SCALED) squares = request_squares(sumsq, groups, tid);
     request();
     // unconditionally (a stretch shorter than the pipeline requests units past its end, which it does not use:
     // memory of the next pairs, or nothing past the weight's end): behind a branch these loads would make the
     // copy below wait for them, since the compiler could not tell how many are in flight
     static_for<SETS - 1>([&](auto j) { load_next(w[j.value]); });
-    if constexpr (SCALED) {
-      const float has = tid < groups ? 1.f : 0.f, has_more = tid + 256 < groups ? 1.f : 0.f;
-#pragma unroll
-      for (int q = 0; q < 4; ++q) squares[q] = squares[q] * has + more[q] * has_more;
-      // 16 sums over the wave's 64 lanes with 17 exchanges: at each of four steps a lane keeps one half of its
-      // values and adds the partner's copy of that half (the lane bit chooses which), then two full steps; lane
-      // l ends with the wave's sum of token 8 b0 + 4 b1 + 2 b2 + b3 (b: the bits of l)
-      float v[16];
-#pragma unroll
-      for (int m = 0; m < 16; ++m) v[m] = squares[m / 4][m % 4];
-      static_for<4>([&](auto step) {  // every index a compile-time constant: the values stay in registers
-        constexpr int bit = 1 << step.value, n = 8 >> step.value;
-        const bool upper = (lane & bit) != 0;
-        static_for<n>([&](auto i) {
-          const float got = __shfl_xor(upper ? v[i.value] : v[i.value + n], bit);
-          v[i.value] = (upper ? v[i.value + n] : v[i.value]) + got;
-        });
-      });
-      v[0] += __shfl_xor(v[0], 16);
-      v[0] += __shfl_xor(v[0], 32);
-      if (lane < 16) norm_part[wave * 16 + ((lane & 1) * 8 + (lane & 2) * 2 + (lane & 4) / 2 + (lane & 8) / 8)] = v[0];
-    }
+    if constexpr (SCALED) add_squares(squares, groups, tid, norm_part);
     copy();
     for (int base = 256 * BATCH; base < pieces; base += 256 * BATCH) {
       request();
@@ -1172,10 +1194,7 @@ __global__ __launch_bounds__(256) void gemm_resident_gated_kernel(const __bf16* 
   // a token past M gives a column of the instruction that is never stored: its lanes read the last row
   const int token = min(lr, M - 1);
   float inv = 1.f;
-  if constexpr (SCALED) {
-    const float sum = norm_part[token] + norm_part[16 + token] + norm_part[32 + token] + norm_part[48 + token];
-    inv = 1.0f / sqrtf(sum / (float)K + eps);
-  }
+  if constexpr (SCALED) inv = inv_rms(norm_part, token, K, eps);
   const __bf16* a_lane = acts + token * row_elems + lg * 8;
   f32x4 acc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
   int mul_c = first_chunk, mul_p = first_pair;
@@ -1296,10 +1315,50 @@ __global__ void gemm_reduce_kernel(const float* __restrict__ partial, const floa
   store4<TC, ACCUMULATE>(C, ldc, m, n, M, N, sum, bias, vector_ok != 0);
 }
 
+// The same sum for the residual (C float, += ) that also prepares the norm after it (see FollowNorm): grid
+// (ceil(N / 1024), M), a workgroup adds the squares of its up to 1,024 columns of one token in a fixed tree and
+// leaves them in sumsq[blockIdx.x][token].
+__global__ __launch_bounds__(256) void gemm_reduce_follow_kernel(const float* __restrict__ partial,
+                                                                 const float* __restrict__ bias, float* __restrict__ C,
+                                                                 int M, int N, long long ldc, int ranges, int vector_ok,
+                                                                 FollowNorm follow) {
+  __shared__ float wave_sum[4];
+  const int m = blockIdx.y, n = (blockIdx.x * 256 + threadIdx.x) * 4;
+  float squares = 0.f;
+  if (n < N) {
+    f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+    const bool whole = n + 3 < N && vector_ok;
+    for (int r = 0; r < ranges; ++r) {
+      const float* src = partial + ((size_t)r * M + m) * N + n;
+      if (whole) {
+        sum += *(const f32x4*)src;
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (n + j < N) sum[j] += src[j];
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (n + j < N) {
+        float* at = C + (size_t)m * ldc + n + j;
+        const float x = sum[j] + (bias ? bias[n + j] : 0.f) + *at;
+        *at = x;
+        follow.scaled[(size_t)m * follow.ld_scaled + n + j] = (__bf16)(x * follow.gain[n + j]);
+        squares += x * x;
+      }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) squares += __shfl_xor(squares, off);
+  if ((threadIdx.x & 63) == 0) wave_sum[threadIdx.x >> 6] = squares;
+  __syncthreads();
+  if (threadIdx.x == 0) follow.sumsq[(size_t)blockIdx.x * 16 + m] = wave_sum[0] + wave_sum[1] + wave_sum[2] + wave_sum[3];
+}
+
 template <int CB, int RT, typename TC, bool ACC>
 int launch_mid_as(const __bf16* A, const __bf16* W, const float* bias, TC* C, float* partial, long long partial_floats,
                   int ranges, int forced_rows, int M, int N, int K, long long lda, long long ldc, int vector_ok,
-                  hipStream_t s) {
+                  hipStream_t s, const FollowNorm* follow = nullptr) {
   constexpr int lds_bytes = 2 * CB * 16 * MID_ROW * (int)sizeof(__bf16);
   const int rows = RT == 2 ? 32 : forced_rows ? forced_rows : balanced_rows(M, N, 4, ranges < 1 ? 1 : ranges);  // per wave
   const int blocks = (N + 4 * rows - 1) / (4 * rows);
@@ -1328,6 +1387,14 @@ int launch_mid_as(const __bf16* A, const __bf16* W, const float* bias, TC* C, fl
   kernel<<<dim3(blocks, used), 256, lds_bytes, s>>>(A, W, nullptr, partial, M, N, K, lda, N, k_per_range,
                                                     (long long)M * N, (N & 3) == 0 ? 1 : 0, rows);
   VK_LAUNCH_CHECK();
+  if constexpr (ACC && sizeof(TC) == 4) {
+    if (follow) {
+      gemm_reduce_follow_kernel<<<dim3((N + 1023) / 1024, M), 256, 0, s>>>(partial, bias, (float*)C, M, N, ldc, used,
+                                                                           (N & 3) == 0 ? 1 : 0, *follow);
+      VK_LAUNCH_CHECK();
+      return 0;
+    }
+  }
   const long long threads = (long long)M * ((N + 3) / 4);
   gemm_reduce_kernel<TC, ACC><<<(int)((threads + 255) / 256), 256, 0, s>>>(partial, bias, C, M, N, ldc, used, vector_ok);
   VK_LAUNCH_CHECK();
@@ -1337,11 +1404,11 @@ int launch_mid_as(const __bf16* A, const __bf16* W, const float* bias, TC* C, fl
 template <typename TC, bool ACC>
 int launch_mid(const __bf16* A, const __bf16* W, const float* bias, TC* C, float* partial, long long partial_floats,
                int ranges, int rows_per_wave, int M, int N, int K, long long lda, long long ldc, int vector_ok,
-               hipStream_t s) {
+               hipStream_t s, const FollowNorm* follow = nullptr) {
   const int cb = (M + 15) / 16;
   // 108 to 116: one tile per wave with a forced number of rows (8 to 16), for tests and measurements
   const int forced = rows_per_wave >= 108 && rows_per_wave <= 116 ? rows_per_wave - 100 : 0;
-#define VK_MID(CBV, RTV) return launch_mid_as<CBV, RTV, TC, ACC>(A, W, bias, C, partial, partial_floats, ranges, forced, M, N, K, lda, ldc, vector_ok, s)
+#define VK_MID(CBV, RTV) return launch_mid_as<CBV, RTV, TC, ACC>(A, W, bias, C, partial, partial_floats, ranges, forced, M, N, K, lda, ldc, vector_ok, s, follow)
   if (rows_per_wave == 2) {
     switch (cb) { case 1: VK_MID(1, 2); case 2: VK_MID(2, 2); case 3: VK_MID(3, 2); case 4: VK_MID(4, 2); }
   } else {
@@ -1593,10 +1660,14 @@ extern "C" int vk_gemm_bf16_gated(const void* A, const void* W, void* C, int M, 
 // holds hd / 2 floats) and the tokens' K and V stored in their pages, as vk_gemm_bf16 followed by vk_rope_kvwrite
 // would leave them. N = (heads + 2 kv_heads) hd, hd even. k_cache null: no cache is written.
 // K pages [page, kv_head, slot, hd], V pages [page, kv_head, hd, slot]; a negative page id writes nothing.
+// `sumsq` (may be null): A is x * gain of the norm before the product as vk_gemm_bf16_follow or
+// vk_gemm_bf16_mid_follow left it, with `norm_groups` sums of squares; the sums of the product are divided by
+// the root mean square (`eps` inside the root) before the bias.
 extern "C" int vk_gemm_bf16_qkv_rope(const void* A, const void* W, const float* bias, void* C, int M, int N, int K,
                                      long long lda, long long ldc, const int* positions, const float* inv_freq,
                                      void* k_cache, void* v_cache, const int* entry_of_token, const int* block_table,
-                                     int table_width, int block_size, int heads, int kv_heads, int hd, void* stream) {
+                                     int table_width, int block_size, int heads, int kv_heads, int hd,
+                                     const float* sumsq, int norm_groups, float eps, void* stream) {
   if (M <= 0 || N <= 0) return 0;
   if (M > 16) return VK_UNSUPPORTED_SIZE;
   if (K <= 0 || (K & 7) || (lda & 7) || lda < K || ldc < N) return VK_BAD_ARGUMENT;
@@ -1609,14 +1680,19 @@ extern "C" int vk_gemm_bf16_qkv_rope(const void* A, const void* W, const float* 
   if ((long long)N * K * 2 >= (1ll << 31) || lda >= (1 << 23)) return VK_UNSUPPORTED_SIZE;
   int pairs = 8, values = 16, groups = 1;
   qkv_rope_plan(M, heads, kv_heads, hd, &pairs, &values, &groups);
+  if (sumsq && (norm_groups <= 0 || norm_groups > 512 || ((uintptr_t)sumsq & 15))) return VK_BAD_ARGUMENT;
   const QkvRope r{positions, inv_freq, (__bf16*)k_cache, (__bf16*)v_cache, entry_of_token, block_table,
-                  table_width, block_size, heads, kv_heads, hd, pairs, values};
-  if (values <= 2 * (8 - pairs))
-    gemm_qkv_rope_kernel<1><<<groups, 256, 0, (hipStream_t)stream>>>((const __bf16*)A, (const __bf16*)W, bias, (__bf16*)C,
-                                                                     M, N, K, lda, ldc, r);
-  else
-    gemm_qkv_rope_kernel<2><<<groups, 256, 0, (hipStream_t)stream>>>((const __bf16*)A, (const __bf16*)W, bias, (__bf16*)C,
-                                                                     M, N, K, lda, ldc, r);
+                  table_width, block_size, heads, kv_heads, hd, pairs, values, sumsq, norm_groups, eps};
+  const bool one_tile = values <= 2 * (8 - pairs);
+#define VK_QKV(RTV, SCALEDV)                                                                                          \
+  gemm_qkv_rope_kernel<RTV, SCALEDV><<<groups, 256, 0, (hipStream_t)stream>>>((const __bf16*)A, (const __bf16*)W, bias, \
+                                                                              (__bf16*)C, M, N, K, lda, ldc, r)
+  if (sumsq) {
+    if (one_tile) VK_QKV(1, true); else VK_QKV(2, true);
+  } else {
+    if (one_tile) VK_QKV(1, false); else VK_QKV(2, false);
+  }
+#undef VK_QKV
   VK_LAUNCH_CHECK();
   return 0;
 }
@@ -1644,6 +1720,30 @@ extern "C" int vk_gemm_bf16_follow(const void* A, const void* W, const float* bi
       FollowNorm{gain, (__bf16*)scaled, sumsq, ld_scaled});
   VK_LAUNCH_CHECK();
   return 0;
+}
+
+// vk_gemm_bf16_follow for up to 64 tokens where K is split over workgroups (vk_gemm_bf16_mid with `ranges` > 1
+// into a float C with accumulation): the kernel that adds the ranges also leaves `scaled` and the sums of squares,
+// here ceil(N / 1024) groups.
+extern "C" int vk_gemm_bf16_mid_follow(const void* A, const void* W, const float* bias, float* C, int M, int N, int K,
+                                       long long lda, long long ldc, int ranges, int rows_per_wave, float* partial,
+                                       long long partial_floats, const float* gain, void* scaled, long long ld_scaled,
+                                       float* sumsq, long long sumsq_floats, int* groups, void* stream) {
+  if (M <= 0 || N <= 0 || M > 64) return VK_UNSUPPORTED_SIZE;
+  if (K <= 0 || (K & 7) || (lda & 7) || lda < K || ldc < N || ranges < 2 || ld_scaled < N || !gain || !scaled || !sumsq ||
+      !groups || !partial)
+    return VK_BAD_ARGUMENT;
+  if (((uintptr_t)A & 15) || ((uintptr_t)W & 15) || ((uintptr_t)partial & 15)) return VK_BAD_ARGUMENT;
+  if (K >= (1 << 24) || lda >= (1 << 24)) return VK_UNSUPPORTED_SIZE;
+  const int blocks = (N + 1023) / 1024;
+  if ((long long)blocks * 16 > sumsq_floats) return VK_UNSUPPORTED_SIZE;
+  // the ranges must really be split, or the product would write C without the kernel that adds them
+  const int k_per_range = ((K + ranges - 1) / ranges + MID_CHUNK - 1) / MID_CHUNK * MID_CHUNK;
+  if ((K + k_per_range - 1) / k_per_range < 2) return VK_UNSUPPORTED_SIZE;
+  *groups = blocks;
+  const FollowNorm follow{gain, (__bf16*)scaled, sumsq, ld_scaled};
+  return launch_mid<float, true>((const __bf16*)A, (const __bf16*)W, bias, C, partial, partial_floats, ranges, rows_per_wave,
+                                 M, N, K, lda, ldc, 0, (hipStream_t)stream, &follow);
 }
 
 // vk_gemm_bf16_gated with resident activations (rows_per_wave 0) on the output of vk_gemm_bf16_follow: A = scaled,

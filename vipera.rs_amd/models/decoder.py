@@ -105,10 +105,24 @@ class DecoderModel:
             x = self.embedding.forward(batch.tokens, batch.num_tokens, batch.token_source, batch.sampled_tokens)
         else:
             x = self.embedding.forward(batch.tokens, batch.num_tokens)
+        tokens = x.shape[0]
+        incoming = None
         for index, entry in enumerate(self.schedule):
             owner = index if entry.cache_of is None else entry.cache_of
-            self.layers[entry.layer].forward(x, batch, storage.kv[owner], storage.state[owner],
-                                             reads_only=entry.cache_of is not None)
+            layer = self.layers[entry.layer]
+            if not layer.hands_off:
+                layer.forward(x, batch, storage.kv[owner], storage.state[owner], reads_only=entry.cache_of is not None)
+                incoming = None
+                continue
+            # the next layer's first norm may be prepared by this layer's last product (see parts.NormHandoff)
+            outgoing = None
+            if index + 1 < len(self.schedule) and layer.fills_outgoing():
+                following = self.layers[self.schedule[index + 1].layer]
+                if following.hands_off:
+                    outgoing = following.accepts_incoming(tokens, batch)
+            layer.forward(x, batch, storage.kv[owner], storage.state[owner], reads_only=entry.cache_of is not None,
+                          incoming=incoming, outgoing=outgoing)
+            incoming = outgoing
         if batch.num_logit_rows == 0:
             return None
         h = self.final_norm.forward(x, rows=batch.logit_rows)

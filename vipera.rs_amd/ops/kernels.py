@@ -336,11 +336,17 @@ def gemm_bf16_qkv_rope_supported(a: torch.Tensor, w: torch.Tensor, qkv: torch.Te
 def gemm_bf16_qkv_rope(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], qkv: torch.Tensor,
                        positions: torch.Tensor, inv_freq: torch.Tensor, k_cache: Optional[torch.Tensor],
                        v_cache: Optional[torch.Tensor], entry_of_token: torch.Tensor, block_table: Optional[torch.Tensor],
-                       heads: int, kv_heads: int, head_dim: int) -> None:
+                       heads: int, kv_heads: int, head_dim: int, sumsq: Optional[torch.Tensor] = None, groups: int = 0,
+                       eps: float = 0.0) -> None:
     """``qkv = a @ w.T + bias`` for up to 16 tokens with the full rotation of its q and k heads and the write of
     the tokens' K and V into their pages in the product's epilogue: what :func:`gemm_bf16` followed by
-    :func:`rope_kvwrite` (without a table of angles) leaves, in one launch."""
-    _dev(a, w, bias, qkv, positions, inv_freq, k_cache, v_cache, entry_of_token, block_table)
+    :func:`rope_kvwrite` (without a table of angles) leaves, in one launch.  With ``sumsq``, ``a`` is ``x * gain`` as
+    :func:`gemm_bf16_follow` left it and the product's sums are divided by the root mean square of ``x`` (from the
+    ``groups`` sums of squares and ``eps``) before the bias: the norm in front of the product costs no kernel."""
+    _dev(a, w, bias, qkv, positions, inv_freq, k_cache, v_cache, entry_of_token, block_table, sumsq)
+    if sumsq is not None:
+        _need(sumsq.dtype == torch.float32 and 1 <= groups <= 512 and sumsq.numel() >= groups * 16,
+              "gemm_bf16_qkv_rope: sumsq")
     m, k = a.shape
     n = w.shape[0]
     _need(w.shape[1] == k and qkv.shape == (m, n) and n == (heads + 2 * kv_heads) * head_dim, "gemm_bf16_qkv_rope: shapes")
@@ -362,10 +368,10 @@ def gemm_bf16_qkv_rope(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Te
     lda = a.stride(0) if m > 1 else max(a.stride(0), k)
     lda = lda if lda % 8 == 0 else k
     fn = _fn("gemm_bf16", "vk_gemm_bf16_qkv_rope",
-             [_p, _p, _p, _p, _i, _i, _i, _ll, _ll, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _p])
+             [_p, _p, _p, _p, _i, _i, _i, _ll, _ll, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _p, _i, _f, _p])
     _status(fn(_ptr(a), _ptr(w), _ptr(bias), _ptr(qkv), m, n, k, lda, n, _ptr(positions), _ptr(inv_freq), _ptr(k_cache),
                _ptr(v_cache), _ptr(entry_of_token), _ptr(block_table), table_width, block_size, heads, kv_heads, head_dim,
-               _stream()), "gemm_bf16_qkv_rope")
+               _ptr(sumsq), int(groups), float(eps), _stream()), "gemm_bf16_qkv_rope")
 
 
 def gemm_bf16_follow_supported(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> bool:
@@ -404,6 +410,37 @@ def gemm_bf16_follow(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tens
                                                   ctypes.POINTER(ctypes.c_int), _p])
     _status(fn(_ptr(a), _ptr(w), _ptr(bias), _ptr(out), m, n, k, lda, n, _ptr(gain), _ptr(scaled), n, _ptr(sumsq),
                sumsq.numel(), ctypes.byref(groups), _stream()), "gemm_bf16_follow")
+    return int(groups.value)
+
+
+def gemm_bf16_mid_follow(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
+                         ranges: int, rows_per_wave: int, gain: torch.Tensor, scaled: torch.Tensor,
+                         sumsq: torch.Tensor) -> int:
+    """:func:`gemm_bf16_follow` for up to 64 tokens where K is split into ``ranges`` > 1 over workgroups
+    (:func:`gemm_bf16_mid` with accumulation): the kernel that adds the ranges leaves ``scaled`` and the sums of
+    squares.  Returns the number of groups."""
+    _dev(a, w, bias, out, gain, scaled, sumsq)
+    m, k = a.shape
+    n = w.shape[0]
+    _need(m <= 64 and ranges >= 2, "gemm_bf16_mid_follow: at most 64 tokens and at least two ranges")
+    _need(w.shape[1] == k and out.shape == (m, n) and scaled.shape == (m, n), "gemm_bf16_mid_follow: shapes")
+    _need(out.dtype == torch.float32 and out.is_contiguous() and gemm_bf16_supported(a, w, out),
+          "gemm_bf16_mid_follow: bfloat16 operands and a float32 output")
+    _need(scaled.dtype == torch.bfloat16 and scaled.is_contiguous(), "gemm_bf16_mid_follow: scaled must be bfloat16 [m, n]")
+    _need(gain.dtype == torch.float32 and gain.numel() == n and gain.is_contiguous(), "gemm_bf16_mid_follow: gain")
+    _need(sumsq.dtype == torch.float32 and sumsq.is_contiguous() and sumsq.numel() >= follow_sumsq_floats(n),
+          "gemm_bf16_mid_follow: sumsq is too small")
+    if bias is not None:
+        _need(bias.dtype == torch.float32 and bias.numel() == n and bias.is_contiguous(), "gemm: bias must be float32 [n]")
+    lda = a.stride(0) if m > 1 else max(a.stride(0), k)
+    lda = lda if lda % 8 == 0 else k
+    partial = _split_k_workspace(a.device, ranges * 64 * n, "mid")
+    groups = ctypes.c_int(0)
+    fn = _fn("gemm_bf16", "vk_gemm_bf16_mid_follow", [_p, _p, _p, _p, _i, _i, _i, _ll, _ll, _i, _i, _p, _ll, _p, _p, _ll, _p,
+                                                      _ll, ctypes.POINTER(ctypes.c_int), _p])
+    _status(fn(_ptr(a), _ptr(w), _ptr(bias), _ptr(out), m, n, k, lda, n, int(ranges), int(rows_per_wave), _ptr(partial),
+               partial.numel(), _ptr(gain), _ptr(scaled), n, _ptr(sumsq), sumsq.numel(), ctypes.byref(groups), _stream()),
+            "gemm_bf16_mid_follow")
     return int(groups.value)
 
 

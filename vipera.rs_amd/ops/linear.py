@@ -54,6 +54,25 @@ def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: 
     return out
 
 
+def linear_follow(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], residual: torch.Tensor,
+                  gain: torch.Tensor, scaled: torch.Tensor, sumsq: torch.Tensor) -> int:
+    """``residual += a @ w.T + bias`` and, where the kernel that :func:`linear` would pick can do it, the first half
+    of the RMS norm that follows (``scaled = residual * gain`` in bfloat16 and the sums of squares in groups, see
+    :func:`kernels.gemm_bf16_follow`).  Returns the number of groups, or 0 where the product ran without it."""
+    m, k = a.shape
+    n = w.shape[0]
+    bf16 = a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
+    if bf16 and m <= 16 and streams_in_wave_order(m, n, k) and kernels.gemm_bf16_follow_supported(a, w, residual):
+        return kernels.gemm_bf16_follow(a, w, bias, residual, gain, scaled, sumsq)
+    if (bf16 and m <= 16 and residual.dtype == torch.float32 and residual.is_contiguous()
+            and kernels.gemm_bf16_supported(a, w, residual)):
+        ranges, rows_per_wave = mid_plan(m, n, k)
+        if ranges >= 2 and k // ranges >= 512:
+            return kernels.gemm_bf16_mid_follow(a, w, bias, residual, ranges, rows_per_wave, gain, scaled, sumsq)
+    linear(a, w, bias, residual, accumulate=True)
+    return 0
+
+
 def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     """The fused weight of a gated feed-forward with rows interleaved in groups of 16: rows ``[32 p, 32 p + 16)``
     are gate rows ``[16 p, 16 p + 16)``, rows ``[32 p + 16, 32 p + 32)`` the up rows of the same outputs."""

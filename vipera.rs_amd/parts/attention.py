@@ -14,7 +14,7 @@ from typing import Dict, List, Optional
 import torch
 
 from ..config.base import PartSpec
-from ..errors import InvalidArgumentError
+from ..errors import InvalidArgumentError, UnsupportedError
 from ..ops import kernels
 from ..ops.attention import paged_attention
 from ..ops.linear import linear, streams_in_wave_order
@@ -78,22 +78,41 @@ class Attention(Mixer):
 
     fills_handoff = True
 
-    def forward(self, h, batch, cache, state, position, residual, reads_only: bool = False, handoff=None) -> None:
-        tokens = h.shape[0]
+    def _one_kernel(self, tokens: int, position, batch) -> bool:
+        """Whether product, rotation and cache write of a step of ``tokens`` are one kernel: a few tokens, all
+        bfloat16, a full rotation computed in the kernel (no table of the step's angles)."""
+        fused = position.fused_rotary()
+        return (fused is not None and fused[1] == self.head_dim and self.runtime.dtype == torch.bfloat16
+                and self.w_qkv.dtype == torch.bfloat16 and tokens <= 16 and self.head_dim % 2 == 0
+                and streams_in_wave_order(tokens, *self.w_qkv.shape)
+                and self.w_qkv.shape[0] * self.w_qkv.shape[1] * 2 < 2 ** 31 and self.w_qkv.shape[1] % 8 == 0
+                and position.step_angles(batch) is None)
+
+    def accepts_handoff(self, tokens: int, position, batch) -> bool:
+        # the one-kernel product can divide by the norm itself
+        return self._one_kernel(tokens, position, batch)
+
+    def forward(self, h, batch, cache, state, position, residual, reads_only: bool = False, handoff=None,
+                incoming=None) -> None:
+        tokens = residual.shape[0]
+        if incoming is not None and not self._one_kernel(tokens, position, batch):
+            raise UnsupportedError("attention was handed a split norm for a step it does not run as one kernel")
+        scaled = {} if incoming is None else {"sumsq": incoming.sumsq, "groups": incoming.groups, "eps": incoming.eps}
+        if incoming is not None:
+            h = incoming.scaled
         qkv = self.runtime.empty((tokens, self.q_width + 2 * self.kv_width))
         table = batch.block_tables[cache.group]
         fused = position.fused_rotary()
         inv_freq, rotary_dim = fused if fused is not None else (None, 0)
         angles = position.step_angles(batch) if rotary_dim else None
-        if (rotary_dim == self.head_dim and angles is None and h.dtype == torch.bfloat16
-                and self.w_qkv.dtype == torch.bfloat16 and streams_in_wave_order(tokens, *self.w_qkv.shape)
-                and kernels.gemm_bf16_qkv_rope_supported(h, self.w_qkv, qkv, self.head_dim)):
-            # a few tokens with a full rotation: product, rotation and cache write are one kernel
+        if self._one_kernel(tokens, position, batch) and kernels.gemm_bf16_qkv_rope_supported(h, self.w_qkv, qkv, self.head_dim):
             kernels.gemm_bf16_qkv_rope(h, self.w_qkv, self.b_qkv, qkv, batch.positions, inv_freq,
                                        None if reads_only else cache.k, None if reads_only else cache.v,
                                        batch.entry_of_token, None if reads_only else table, self.heads, self.kv_heads,
-                                       self.head_dim)
+                                       self.head_dim, **scaled)
         else:
+            if incoming is not None:
+                raise UnsupportedError("attention was handed a split norm for operands its one-kernel product does not take")
             linear(h, self.w_qkv, self.b_qkv, qkv)
             if fused is None:
                 position.apply(qkv, batch, self.heads, self.kv_heads, self.head_dim)

@@ -113,11 +113,19 @@ class Mixer(Part):
     #: a mixer that sets this takes ``handoff=`` in ``forward`` and may fill it (see :class:`NormHandoff`)
     fills_handoff = False
 
+    def accepts_handoff(self, tokens: int, position, batch) -> bool:
+        """Whether ``forward`` takes a filled :class:`NormHandoff` of the norm before it (``incoming=``, with ``h``
+        None) for a step of ``tokens`` rows."""
+        return False
+
     def forward(self, h, batch, cache, state, position, residual, reads_only: bool = False) -> None:
         raise NotImplementedError
 
 
 class FeedForward(Part):
+    #: a feed-forward that sets this takes ``outgoing=`` in ``forward`` and may fill it for the next layer's first norm
+    fills_handoff = False
+
     def accepts_handoff(self, tokens: int) -> bool:
         """Whether ``forward`` takes a filled :class:`NormHandoff` (``handoff=``, with ``h`` None) for ``tokens`` rows."""
         return False
@@ -141,6 +149,11 @@ class Block:
 
     def load(self, tensors) -> None:
         raise NotImplementedError
+
+    #: a block that sets this takes ``incoming=`` and ``outgoing=`` in ``forward`` and has ``accepts_incoming`` and
+    #: ``fills_outgoing`` (see :class:`NormHandoff`: its first norm prepared by the layer before, the next layer's
+    #: first norm prepared by this one)
+    hands_off = False
 
     def forward(self, x, batch, cache, state, reads_only: bool = False) -> None:
         raise NotImplementedError

@@ -35,22 +35,40 @@ class PreNormBlock(Block):
         for part in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn, self.position):
             part.load(tensors)
 
-    def forward(self, x, batch, cache, state, reads_only: bool = False) -> None:
-        h = self.mixer_norm.forward(x)
-        # with a few tokens the second norm may be split between the mixer's last product and the feed-forward's
-        # first, if all three can (see NormHandoff); otherwise it is a kernel of its own
-        handoff = None
-        if self.mixer.fills_handoff and self.ffn.accepts_handoff(x.shape[0]):
-            handoff = self.ffn_norm.handoff(x.shape[0])
-        if handoff is None:
-            self.mixer.forward(h, batch, cache, state, self.position, x, reads_only)
+    hands_off = True
+
+    def accepts_incoming(self, tokens: int, batch):
+        """A :class:`NormHandoff` of this block's first norm for the layer before to fill, or None."""
+        if not self.mixer.accepts_handoff(tokens, self.position, batch):
+            return None
+        return self.mixer_norm.handoff(tokens)
+
+    def fills_outgoing(self) -> bool:
+        return self.ffn.fills_handoff
+
+    def forward(self, x, batch, cache, state, reads_only: bool = False, incoming=None, outgoing=None) -> None:
+        """With a few tokens a norm may be split between the product before it and the product after it, if all
+        three can (see NormHandoff); otherwise it is a kernel of its own. ``incoming``: this block's first norm,
+        filled by the layer before (``groups`` > 0) or not; ``outgoing``: the next layer's first norm, for this
+        block's feed-forward to fill."""
+        if incoming is not None and incoming.groups:
+            h = None
+            mixer_kwargs = {"incoming": incoming}
         else:
-            self.mixer.forward(h, batch, cache, state, self.position, x, reads_only, handoff=handoff)
-        if handoff is not None and handoff.groups:
-            self.ffn.forward(None, batch, x, handoff=handoff)
+            h = self.mixer_norm.forward(x)
+            mixer_kwargs = {}
+        between = None
+        if self.mixer.fills_handoff and self.ffn.accepts_handoff(x.shape[0]):
+            between = self.ffn_norm.handoff(x.shape[0])
+            if between is not None:
+                mixer_kwargs["handoff"] = between
+        self.mixer.forward(h, batch, cache, state, self.position, x, reads_only, **mixer_kwargs)
+        ffn_kwargs = {"outgoing": outgoing} if outgoing is not None and self.ffn.fills_handoff else {}
+        if between is not None and between.groups:
+            self.ffn.forward(None, batch, x, handoff=between, **ffn_kwargs)
         else:
             h = self.ffn_norm.forward(x)
-            self.ffn.forward(h, batch, x)
+            self.ffn.forward(h, batch, x, **ffn_kwargs)
 
 
 register_block("prenorm", PreNormBlock)

@@ -13,7 +13,7 @@ import torch
 from ..config.base import PartSpec
 from ..errors import UnsupportedError
 from ..ops import kernels
-from ..ops.linear import gated_plan, interleave_gate_up, linear, linear_gated
+from ..ops.linear import gated_plan, interleave_gate_up, linear, linear_follow, linear_gated
 from ..weights.checkpoint import MATRIX, TensorSpec
 from .attention import _cat
 from .base import FeedForward, register_ffn
@@ -54,14 +54,20 @@ class GatedMLP(FeedForward):
                 and tokens <= 16 and gated_plan(tokens, *self.w_gate_up.shape,
                                                 kernels.compute_units(self.w_gate_up.device)) == 0)
 
-    def forward(self, h, batch, residual, handoff=None) -> None:
+    fills_handoff = True
+
+    def forward(self, h, batch, residual, handoff=None, outgoing=None) -> None:
         tokens = residual.shape[0]
         act = self.runtime.empty((tokens, self.inter))
         if handoff is not None:
             kernels.gemm_bf16_gated_scaled(handoff.scaled, self.w_gate_up, act, handoff.sumsq, handoff.groups, handoff.eps)
         else:
             linear_gated(h, self.w_gate_up, act, self.interleaved)
-        linear(act, self.w_down, None, residual, accumulate=True)
+        if outgoing is not None:
+            # the down product also prepares the next layer's first norm where its kernel can
+            outgoing.groups = linear_follow(act, self.w_down, None, residual, outgoing.gain, outgoing.scaled, outgoing.sumsq)
+        else:
+            linear(act, self.w_down, None, residual, accumulate=True)
 
 
 register_ffn("gated_mlp", GatedMLP)
