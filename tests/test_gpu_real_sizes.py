@@ -63,6 +63,41 @@ def test_real_layer_sizes_under_every_cut(real, dtype, tol):
     assert runner.cache.check() == ""
 
 
+CONFIG_SPLIT_NORMS = {
+    "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2",
+    "num_hidden_layers": 3, "hidden_size": 512, "num_attention_heads": 4, "num_key_value_heads": 2, "head_dim": 128,
+    "intermediate_size": 4096, "vocab_size": 300, "rope_theta": 10000.0, "rms_norm_eps": 1e-5,
+    "tie_word_embeddings": True, "max_position_embeddings": 4096, "hidden_act": "silu",
+}
+
+
+def test_norms_split_between_the_products_around_them(tmp_path, monkeypatch):
+    """Sizes at which a step of up to 16 tokens runs its norms inside the neighbouring products (the second norm of
+    a layer between output and gate/up product, the first between the layer before's down product, with K split
+    over workgroups or not, and the fused q/k/v product): single tokens, steps of 2 to 16 tokens and whole prompts
+    against the plain implementation, and the norm kernel runs only where no product precedes it."""
+    from vipera_rs_amd.engine.batch import StepEntry
+    from vipera_rs_amd.engine.runner import ModelRunner
+    from vipera_rs_amd.ops import kernels
+    folder = make_folder(tmp_path / "split", CONFIG_SPLIT_NORMS, 5, torch.bfloat16)
+    cfg, w = P.load_folder(folder)
+    tokens = random_tokens(300, 70, 31)
+    want = P.forward(cfg, w, tokens)
+    runner = ModelRunner.from_folder(folder, dtype="bfloat16", block_size=16, num_blocks=24, num_slots=4)
+    calls = []
+    real_rmsnorm = kernels.rmsnorm
+    monkeypatch.setattr(kernels, "rmsnorm", lambda *a, **k: (calls.append(1), real_rmsnorm(*a, **k))[1])
+    rows, at = [], 0
+    for size in [20, 16, 9, 5, 4, 2] + [1] * 14:                 # the first portion is too long for the split
+        runner.cache.reserve(0, at, at + size)
+        calls.clear()
+        rows.append(runner.step([StepEntry(0, at, tokens[at:at + size], list(range(size)))]).cpu().numpy())
+        assert len(calls) == (2 * 3 + 1 if size > 16 else 2), (size, len(calls))
+        at += size
+    assert at == len(tokens)
+    assert rel_err(np.concatenate(rows), want) < 3e-2
+
+
 def test_the_full_vocabulary_head_and_greedy_choice():
     """152064 columns are no power of two: the output projection and the argmax at that width."""
     from vipera_rs_amd.ops import kernels
