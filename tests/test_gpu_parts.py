@@ -524,6 +524,87 @@ def test_a_routed_feed_forward_and_another_position_encoding(tmp_path):
         unregister("position", "tilt")
 
 
+def test_a_toy_feed_forward_takes_a_norm_handed_to_it(tmp_path):
+    """A feed-forward defined here accepts a handed-off norm (`parts.NormHandoff`): for steps of up to 16 tokens
+    the attention before it leaves `x * gain` and its workgroups' sums of squares instead of the norm running
+    as a kernel, and the toy divides by the root mean square itself.  Longer steps reach it with `h` as ever.
+    Both ways give the plain implementation's logits."""
+    from vipera_rs_amd.config import (LayerSpec, PartSpec, Qwen2Config, register_architecture, unregister_architecture)
+    from vipera_rs_amd.engine.batch import StepEntry
+    from vipera_rs_amd.engine.runner import ModelRunner
+    from vipera_rs_amd.models.decoder import DecoderModel
+    from vipera_rs_amd.parts import FeedForward, register_ffn, unregister
+    from vipera_rs_amd.weights import MATRIX, TensorSpec
+    INNER = 48
+    seen = {"handed": 0, "plain": 0}
+
+    class Handed(FeedForward):
+        @classmethod
+        def declare(cls, spec, prefix):
+            hidden = spec.params["hidden"]
+            return [TensorSpec(f"{prefix}toy.up.weight", (INNER, hidden), MATRIX, std=0.2),
+                    TensorSpec(f"{prefix}toy.down.weight", (hidden, INNER), MATRIX, std=0.2)]
+
+        def load(self, tensors):
+            self.up = tensors[f"{self.prefix}toy.up.weight"].float()
+            self.down = tensors[f"{self.prefix}toy.down.weight"].float()
+
+        def accepts_handoff(self, tokens):
+            return tokens <= 16
+
+        def forward(self, h, batch, residual, handoff=None):
+            if handoff is not None:
+                seen["handed"] += 1
+                tokens, width = handoff.scaled.shape
+                squares = handoff.sumsq[: handoff.groups * 16].view(handoff.groups, 16).sum(0)[:tokens]
+                h = handoff.scaled.float() * torch.rsqrt(squares / width + handoff.eps)[:, None]
+            else:
+                seen["plain"] += 1
+            residual += torch.relu(h.float() @ self.up.T) @ self.down.T
+
+    class ToyConfig(Qwen2Config):
+        architecture = "ToyHandedForCausalLM"
+
+        def layer_specs(self) -> List[LayerSpec]:
+            specs = super().layer_specs()
+            first = specs[0]
+            specs[0] = LayerSpec(first.block, first.mixer, PartSpec("handed", {"hidden": self.hidden_size}),
+                                 first.mixer_norm, first.ffn_norm, first.position, first.prefix)
+            return specs
+
+    def plain(cfg, w, tokens):
+        cfg = P.normalize_config(cfg)
+        x = w["model.embed_tokens.weight"][np.asarray(tokens)]
+        h = P.rms_norm(x, w["model.layers.0.input_layernorm.weight"], cfg["rms_norm_eps"])
+        x = x + P.attention_block(h, w, "model.layers.0.self_attn.", cfg, 0)
+        h = P.rms_norm(x, w["model.layers.0.post_attention_layernorm.weight"], cfg["rms_norm_eps"])
+        x = x + np.maximum(h @ w["model.layers.0.toy.up.weight"].T, 0.0) @ w["model.layers.0.toy.down.weight"].T
+        h = P.rms_norm(x, w["model.layers.1.input_layernorm.weight"], cfg["rms_norm_eps"])
+        x = x + P.attention_block(h, w, "model.layers.1.self_attn.", cfg, 0)
+        h = P.rms_norm(x, w["model.layers.1.post_attention_layernorm.weight"], cfg["rms_norm_eps"])
+        x = x + P.swiglu_mlp(h, *(w[f"model.layers.1.mlp.{n}_proj.weight"] for n in ("gate", "up", "down")))
+        return P.linear(P.rms_norm(x, w["model.norm.weight"], cfg["rms_norm_eps"]), w["model.embed_tokens.weight"])
+
+    register_ffn("handed", Handed)
+    register_architecture("ToyHandedForCausalLM", ToyConfig, lambda config, runtime: DecoderModel(config, runtime))
+    try:
+        folder = make_folder(tmp_path / "handed", dict(CONFIG_A, architectures=["ToyHandedForCausalLM"]), 9, torch.bfloat16)
+        cfg, w = P.load_folder(folder)
+        tokens = random_tokens(256, 45, 6)
+        want = plain(cfg, w, tokens)
+        runner = ModelRunner.from_folder(folder, dtype="bfloat16", block_size=8, num_blocks=16, num_slots=2)
+        rows, at = [], 0
+        for size in (20, 1, 1, 16, 2, 5):
+            runner.cache.reserve(0, at, at + size)
+            rows.append(runner.step([StepEntry(0, at, tokens[at:at + size], list(range(size)))]).cpu().numpy())
+            at += size
+        assert rel_err(np.concatenate(rows), want) < 3e-2
+        assert seen == {"handed": 5, "plain": 1}
+    finally:
+        unregister_architecture("ToyHandedForCausalLM")
+        unregister("ffn", "handed")
+
+
 # --- the first tokens of a sequence --------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_first_tokens_of_a_sequence(tmp_path, dtype):
