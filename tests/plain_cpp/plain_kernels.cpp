@@ -381,7 +381,8 @@ extern "C" int plain_attn_bf16_decode(const void* q, long long q_stride, const v
 // logit; min_p against the best weight) and, as the kernel documents for itself, the draw walks the kept tokens in
 // id order: the first whose running mass exceeds u * kept mass. A row without a finite logit gives -1.
 extern "C" int plain_sample(const float* logits, int num_rows, int vocab, const float* temperature, const int* top_k,
-                            const float* top_p, const float* min_p, const double* uniform, int* out, void*) {
+                            const float* top_p, const float* min_p, const double* uniform, int* out, float*, int*, int,
+                            void*) {
   if (num_rows <= 0) return 0;
   if (vocab <= 0) return BAD_ARGUMENT;
   for (int r = 0; r < num_rows; ++r) {

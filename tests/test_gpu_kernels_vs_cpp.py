@@ -283,12 +283,14 @@ def test_sampling_kernels_beside_their_twins():
     top_p = torch.where(torch.arange(rows) % 2 == 0, torch.full((rows,), 0.9), torch.ones(rows))
     min_p = torch.where(torch.arange(rows) % 5 == 0, torch.full((rows,), 0.02), torch.zeros(rows))
     uniform = torch.rand(rows, generator=g, dtype=torch.float64)
-    (got, want), = both("sampling", "sample", [logits, rows, vocab, temperature, top_k, top_p, min_p, uniform,
-                                               torch.empty(rows, dtype=torch.int32), None], [8])
-    assert torch.equal(got[:8], want[:8]) and got[4] == -1 and got[5] == 100
-    # a sampled row could differ where u * mass falls within rounding of a boundary between two kept tokens, or where a
-    # cut's edge rounds the other way; none of these seeded rows does
-    assert torch.equal(got, want)
+    for slices in (0, 7, 32):     # the rows' best logits searched by one workgroup a row, or by `slices` of them first
+        scratch = [torch.empty(rows * slices), torch.empty(rows * slices, dtype=torch.int32)] if slices else [None, None]
+        (got, want), = both("sampling", "sample", [logits, rows, vocab, temperature, top_k, top_p, min_p, uniform,
+                                                   torch.empty(rows, dtype=torch.int32), *scratch, slices, None], [8])
+        assert torch.equal(got[:8], want[:8]) and got[4] == -1 and got[5] == 100
+        # a sampled row could differ where u * mass falls within rounding of a boundary between two kept tokens, or where
+        # a cut's edge rounds the other way; none of these seeded rows does
+        assert torch.equal(got, want)
     pen = torch.randn(3, 500, generator=g)
     args = [pen, 500, i32([0, 0, 2]), i32([3, 499, 3]), i32([2, 1, 4]), torch.tensor([1.3, 1.0, 0.7]), torch.tensor([0.2, 0.0, 0.1]),
             torch.tensor([0.1, 0.5, 0.0]), 3, None]

@@ -56,13 +56,72 @@ struct Cut {
   int ties;         // of the tokens with exactly this key, the first `ties` by id are kept
 };
 
-// One row. Returns the chosen token in *out (or -1 when no logit is finite).
+// The best finite logit of a slice of a row (ties to the lowest id; id 0x7fffffff when none is finite): grid
+// (slices, rows). One workgroup per row reads a 152,064-column row at what one CU can pull (25 us); thirty-two
+// slices a row spread it over the GPU, and sample_kernel then compares the slices' winners.
+__global__ __launch_bounds__(256) void argmax_slices_kernel(const float* __restrict__ logits, int vocab, int slice_len,
+                                                            float* __restrict__ slice_best, int* __restrict__ slice_id) {
+  __shared__ float red_f[4];
+  __shared__ int red_i[4];
+  const int row = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const float* x = logits + (size_t)row * vocab;
+  const int begin = blockIdx.x * slice_len, end = min(vocab, begin + slice_len);
+  float b4[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+  int i4[4] = {0x7fffffff, 0x7fffffff, 0x7fffffff, 0x7fffffff};
+  for (int base = begin + tid; base < end; base += 4 * 256) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int i = base + u * 256;
+      const float v = i < end ? x[i] : NAN;
+      if (finite_f(v) && v > b4[u]) {  // within one candidate the indices ascend, so ties keep the lower one
+        b4[u] = v;
+        i4[u] = i;
+      }
+    }
+  }
+  float best = -INFINITY;
+  int best_id = 0x7fffffff;
+#pragma unroll
+  for (int u = 0; u < 4; ++u)
+    if (b4[u] > best || (b4[u] == best && i4[u] < best_id)) {
+      best = b4[u];
+      best_id = i4[u];
+    }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(best, off, 64);
+    const int oi = __shfl_xor(best_id, off, 64);
+    if (ov > best || (ov == best && oi < best_id)) {
+      best = ov;
+      best_id = oi;
+    }
+  }
+  if (lane == 0) {
+    red_f[wave] = best;
+    red_i[wave] = best_id;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    for (int w = 1; w < 4; ++w)
+      if (red_f[w] > best || (red_f[w] == best && red_i[w] < best_id)) {
+        best = red_f[w];
+        best_id = red_i[w];
+      }
+    slice_best[(size_t)row * gridDim.x + blockIdx.x] = best;
+    slice_id[(size_t)row * gridDim.x + blockIdx.x] = best_id;
+  }
+}
+
+// One row. Returns the chosen token in *out (or -1 when no logit is finite). `slices` > 0: the row's best logit
+// comes from the winners that argmax_slices_kernel left.
 __global__ __launch_bounds__(THREADS) void sample_kernel(const float* __restrict__ logits, int vocab,
                                                          const float* __restrict__ temperature,
                                                          const int* __restrict__ top_k,
                                                          const float* __restrict__ top_p,
                                                          const float* __restrict__ min_p,
-                                                         const double* __restrict__ uniform, int* __restrict__ out) {
+                                                         const double* __restrict__ uniform, int* __restrict__ out,
+                                                         const float* __restrict__ slice_best,
+                                                         const int* __restrict__ slice_id, int slices) {
   __shared__ float red_f[16];
   __shared__ int red_i[WAVES];
   __shared__ unsigned long long red_u[WAVES];
@@ -77,7 +136,16 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(const float* __restrict
   // --- best finite logit, ties to the lowest id ----------------------------------------------
   float best = -INFINITY;
   int best_id = 0x7fffffff;
-  {
+  if (slices > 0) {
+    for (int s = tid; s < slices; s += THREADS) {
+      const float v = slice_best[(size_t)row * slices + s];
+      const int i = slice_id[(size_t)row * slices + s];
+      if (i != 0x7fffffff && (v > best || (v == best && i < best_id))) {
+        best = v;
+        best_id = i;
+      }
+    }
+  } else {
     // four independent candidates per thread keep four loads in flight; they are merged in index order
     float b4[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
     int i4[4] = {0x7fffffff, 0x7fffffff, 0x7fffffff, 0x7fffffff};
@@ -364,12 +432,22 @@ __global__ void bias_kernel(float* __restrict__ logits, int vocab, const int* __
 }
 }  // namespace
 
+// `slices` > 0 with room for num_rows * slices values in `slice_best` and `slice_id`: the rows' best logits are
+// found by slices * num_rows workgroups first (worth it for a wide vocabulary); the result is the same.
 extern "C" int vk_sample(const float* logits, int num_rows, int vocab, const float* temperature, const int* top_k,
-                         const float* top_p, const float* min_p, const double* uniform, int* out, void* stream) {
+                         const float* top_p, const float* min_p, const double* uniform, int* out, float* slice_best,
+                         int* slice_id, int slices, void* stream) {
   if (num_rows <= 0) return 0;
-  if (vocab <= 0) return VK_BAD_ARGUMENT;
+  if (vocab <= 0 || slices < 0 || slices > 65535 || num_rows > 65535) return VK_BAD_ARGUMENT;
+  if (slices > 0) {
+    if (!slice_best || !slice_id) return VK_BAD_ARGUMENT;
+    const int slice_len = (vocab + slices - 1) / slices;
+    argmax_slices_kernel<<<dim3(slices, num_rows), 256, 0, (hipStream_t)stream>>>(logits, vocab, slice_len, slice_best,
+                                                                                 slice_id);
+    VK_LAUNCH_CHECK();
+  }
   sample_kernel<<<num_rows, THREADS, 0, (hipStream_t)stream>>>(logits, vocab, temperature, top_k, top_p, min_p,
-                                                                uniform, out);
+                                                                uniform, out, slice_best, slice_id, slices);
   VK_LAUNCH_CHECK();
   return 0;
 }

@@ -240,6 +240,10 @@ def attn_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, 
 
 
 # ----------------------------------------------------------------------------------------------
+SAMPLE_SLICES = 32
+SAMPLE_SLICES_FROM = 32_768   # columns from which a row's best logit is searched in slices
+
+
 def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
            min_p: torch.Tensor, uniform: torch.Tensor, out: torch.Tensor) -> None:
     """One token per row: greedy where ``temperature`` is 0, else a draw after the top-k/top-p/min-p cuts.
@@ -254,9 +258,13 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
                                 ("uniform", uniform, torch.float64), ("out", out, torch.int32)):
         _need(tensor.dtype == dtype and tensor.numel() == rows and tensor.is_contiguous(),
               f"sample: {name} must hold one {dtype} per row")
-    fn = _fn("sampling", "vk_sample", [_p, _i, _i, _p, _p, _p, _p, _p, _p, _p])
+    # a wide vocabulary: the rows' best logits are found by 32 workgroups a row before the one that draws
+    slices = SAMPLE_SLICES if vocab >= SAMPLE_SLICES_FROM else 0
+    best = torch.empty(rows * slices, dtype=torch.float32, device=logits.device) if slices else None
+    best_id = torch.empty(rows * slices, dtype=torch.int32, device=logits.device) if slices else None
+    fn = _fn("sampling", "vk_sample", [_p, _i, _i, _p, _p, _p, _p, _p, _p, _p, _p, _i, _p])
     _status(fn(_ptr(logits), rows, vocab, _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(min_p), _ptr(uniform),
-               _ptr(out), _stream()), "sample")
+               _ptr(out), _ptr(best), _ptr(best_id), slices, _stream()), "sample")
 
 
 def penalize(logits: torch.Tensor, rows: torch.Tensor, tokens: torch.Tensor, counts: torch.Tensor,
