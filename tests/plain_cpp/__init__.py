@@ -30,7 +30,8 @@ SIGNATURES = {
     "plain_gemm_bf16_follow": [P, P, P, P, I, I, I, LL, LL, P, P, LL, P, LL, P, P],
     "plain_gemm_bf16_gated_scaled": [P, P, P, I, I, I, LL, LL, P, I, F, P],
     "plain_gemm_bf16_qkv_rope": [P, P, P, P, I, I, I, LL, LL, P, P, P, P, P, P, I, I, I, I, I, P, I, F, P],
-    "plain_gemm_bf16_mid_follow": [P, P, P, P, I, I, I, LL, LL, I, I, P, LL, P, P, LL, P, LL, P, P],
+    "plain_gemm_bf16_mid_follow": [P, P, P, P, I, I, I, LL, LL, I, I, P, LL, P, P, LL, P, LL, I, P, P],
+    "plain_gemm_bf16_mid_qkv_rope": [P, P, P, P, I, I, I, LL, LL, I, I, P, LL, P, P, P, P, P, P, I, I, I, I, I, P, I, I, F, P],
     "plain_attn_generic": [P, LL, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, P],
     "plain_attn_bf16_prefill": [P, LL, P, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P],
     "plain_attn_bf16_decode": [P, LL, P, P, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, I, P],

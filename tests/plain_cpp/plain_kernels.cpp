@@ -238,18 +238,39 @@ extern "C" int plain_rope_kvwrite(void* qkv, int dtype, const int* positions, co
                                   const float* angles, int rotary_dim, void* k_cache, void* v_cache,
                                   const int* entry_of_token, const int* block_table, int table_width, int block_size,
                                   int num_tokens, int heads, int kv_heads, int hd, void*);
+static int qkv_rope(const void* A, const void* W, const float* bias, void* C, int M, int N, int K, long long lda,
+                    long long ldc, const int* positions, const float* inv_freq, void* k_cache, void* v_cache,
+                    const int* entry_of_token, const int* block_table, int table_width, int block_size, int heads,
+                    int kv_heads, int hd, const float* sumsq, int norm_groups, int sumsq_stride, float eps);
 extern "C" int plain_gemm_bf16_qkv_rope(const void* A, const void* W, const float* bias, void* C, int M, int N, int K,
                                         long long lda, long long ldc, const int* positions, const float* inv_freq,
                                         void* k_cache, void* v_cache, const int* entry_of_token, const int* block_table,
                                         int table_width, int block_size, int heads, int kv_heads, int hd,
                                         const float* sumsq, int norm_groups, float eps, void*) {
+  return qkv_rope(A, W, bias, C, M, N, K, lda, ldc, positions, inv_freq, k_cache, v_cache, entry_of_token, block_table,
+                  table_width, block_size, heads, kv_heads, hd, sumsq, norm_groups, 16, eps);
+}
+// The same where the kernel splits K over workgroups and takes up to 64 tokens (no difference for the twin).
+extern "C" int plain_gemm_bf16_mid_qkv_rope(const void* A, const void* W, const float* bias, void* C, int M, int N, int K,
+                                            long long lda, long long ldc, int, int, float*, long long,
+                                            const int* positions, const float* inv_freq, void* k_cache, void* v_cache,
+                                            const int* entry_of_token, const int* block_table, int table_width,
+                                            int block_size, int heads, int kv_heads, int hd, const float* sumsq,
+                                            int norm_groups, int sumsq_stride, float eps, void*) {
+  return qkv_rope(A, W, bias, C, M, N, K, lda, ldc, positions, inv_freq, k_cache, v_cache, entry_of_token, block_table,
+                  table_width, block_size, heads, kv_heads, hd, sumsq, norm_groups, sumsq_stride, eps);
+}
+static int qkv_rope(const void* A, const void* W, const float* bias, void* C, int M, int N, int K, long long lda,
+                    long long ldc, const int* positions, const float* inv_freq, void* k_cache, void* v_cache,
+                    const int* entry_of_token, const int* block_table, int table_width, int block_size, int heads,
+                    int kv_heads, int hd, const float* sumsq, int norm_groups, int sumsq_stride, float eps) {
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0 || lda < K || ldc != N || (long long)(heads + 2 * kv_heads) * hd != N) return BAD_ARGUMENT;
   for (int m = 0; m < M; ++m) {
     double inv = 1.0;
     if (sumsq) {
       double squares = 0.0;
-      for (int g = 0; g < norm_groups; ++g) squares += (double)sumsq[(size_t)g * 16 + m];
+      for (int g = 0; g < norm_groups; ++g) squares += (double)sumsq[(size_t)g * sumsq_stride + m];
       inv = 1.0 / std::sqrt(squares / (double)K + (double)eps);
     }
     for (int n = 0; n < N; ++n) {
@@ -291,10 +312,22 @@ extern "C" int plain_gemm_bf16_follow(const void* A, const void* W, const float*
 extern "C" int plain_gemm_bf16_mid_follow(const void* A, const void* W, const float* bias, float* C, int M, int N, int K,
                                           long long lda, long long ldc, int, int, float*, long long, const float* gain,
                                           void* scaled, long long ld_scaled, float* sumsq, long long sumsq_floats,
-                                          int* groups, void*) {
-  if (M > 16) return BAD_ARGUMENT;  // the twin's sums of squares hold 16 tokens, as the consumers do
-  return plain_gemm_bf16_follow(A, W, bias, C, M, N, K, lda, ldc, gain, scaled, ld_scaled, sumsq, sumsq_floats, groups,
-                                nullptr);
+                                          int sumsq_stride, int* groups, void*) {
+  if (M <= 0 || N <= 0 || M > sumsq_stride || K <= 0 || lda < K || ldc < N || ld_scaled < N || sumsq_floats < sumsq_stride)
+    return BAD_ARGUMENT;
+  product(A, DT_BF16, W, DT_BF16, bias, C, DT_F32, M, N, K, lda, ldc, true);
+  for (int m = 0; m < sumsq_stride; ++m) sumsq[m] = 0.f;
+  for (int m = 0; m < M; ++m) {
+    double sum = 0.0;
+    for (int n = 0; n < N; ++n) {
+      const float x = C[(size_t)m * ldc + n];
+      sum += (double)x * (double)x;
+      ((uint16_t*)scaled)[(size_t)m * ld_scaled + n] = float_to_bf16(x * gain[n]);
+    }
+    sumsq[m] = (float)sum;
+  }
+  *groups = 1;
+  return 0;
 }
 
 // The gated product on such a scaled input: gate and up divided by the root mean square first.

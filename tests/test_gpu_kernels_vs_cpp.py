@@ -142,7 +142,7 @@ def test_the_first_norm_of_a_layer_split_between_the_layers(m, width, k_in, head
     if split:
         partial = torch.empty(4 * 64 * width)
         name, args = "gemm_bf16_mid_follow", [act, w_d, None, x0, m, width, k_in, k_in, width, 4, 1, partial, partial.numel(), gain,
-                                              torch.empty(m, width, dtype=torch.bfloat16), width, torch.zeros(floats), floats]
+                                              torch.empty(m, width, dtype=torch.bfloat16), width, torch.zeros(floats), floats, 16]
     else:
         name, args = "gemm_bf16_follow", [act, w_d, None, x0, m, width, k_in, k_in, width, gain,
                                           torch.empty(m, width, dtype=torch.bfloat16), width, torch.zeros(floats), floats]
@@ -176,6 +176,46 @@ def test_the_first_norm_of_a_layer_split_between_the_layers(m, width, k_in, head
     want_v = (h @ w.double().T + bias.double())[:, (heads + kv_heads) * hd:]
     (got, _), _, _ = both("gemm_bf16", "gemm_bf16_qkv_rope", args, [3, 11, 12])
     assert rel_err(got.float().numpy()[:, (heads + kv_heads) * hd:], want_v.numpy()) < 1e-2
+
+
+@pytest.mark.parametrize("m,heads,kv_heads,hd,k,scaled", [(17, 5, 2, 48, 1024, False), (64, 4, 4, 128, 2048, True),
+                                                          (33, 7, 1, 64, 1536, True), (40, 3, 1, 16, 1024, False)])
+def test_split_qkv_product_that_rotates_while_it_adds_its_ranges(m, heads, kv_heads, hd, k, scaled):
+    """17 to 64 tokens: K split over workgroups, and the kernel that adds the ranges divides by the norm (if scaled),
+    adds the bias, rotates and writes the cache. Beside its twin; and without the norm bit for bit what the split
+    product, its sum and the rotation kernel leave."""
+    from vipera_rs_amd.ops import kernels
+    bs, n = 8, (heads + 2 * kv_heads) * hd
+    g = torch.Generator().manual_seed(m + n + k)
+    a = torch.randn(m, k, generator=g).to(torch.bfloat16)
+    w = (torch.randn(n, k, generator=g) / math.sqrt(k)).to(torch.bfloat16)
+    bias = torch.randn(n, generator=g)
+    positions = [(7 * i) % 61 + (i // 9) * 64 for i in range(m)]
+    entry_of = [i // 9 for i in range(m)]
+    inv = (1.0 / torch.pow(torch.tensor(1e6), torch.arange(hd // 2).float() * 2 / hd)).float()
+    entries = max(entry_of) + 1
+    table = torch.arange(entries * 70, dtype=torch.int32).view(entries, 70)
+    k_cache = torch.full((entries * 70, kv_heads, bs, hd), 9.0, dtype=torch.bfloat16)
+    v_cache = torch.full((entries * 70, kv_heads, hd, bs), 9.0, dtype=torch.bfloat16)
+    stride = 64
+    sumsq = (torch.rand(3 * stride, generator=g) * k).float() if scaled else None
+    partial = torch.empty(2 * 64 * n)
+    args = [a, w, bias, torch.empty(m, n, dtype=torch.bfloat16), m, n, k, k, n, 2, 1, partial, partial.numel(), i32(positions), inv,
+            k_cache, v_cache, i32(entry_of), table, 70, bs, heads, kv_heads, hd, sumsq, 3 if scaled else 0, stride, 1e-5, None]
+    for got, want in both("gemm_bf16", "gemm_bf16_mid_qkv_rope", args, [3, 15, 16]):
+        assert rel_err(got.float().numpy(), want.double().numpy()) < 8e-3
+    if scaled:
+        return
+    dev = [x.to(DEV) if isinstance(x, torch.Tensor) else x for x in args]
+    qkv = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
+    kernels.gemm_bf16_mid(dev[0], dev[1], dev[2], qkv, ranges=2, rows_per_wave=1)
+    kc, vc = torch.full_like(dev[15], 9.0), torch.full_like(dev[16], 9.0)
+    kernels.rope_kvwrite(qkv, dev[13], dev[14], hd, kc, vc, dev[17], dev[18], heads, kv_heads, hd)
+    fused = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
+    kc2, vc2 = torch.full_like(dev[15], 9.0), torch.full_like(dev[16], 9.0)
+    kernels.gemm_bf16_mid_qkv_rope(dev[0], dev[1], dev[2], fused, 2, 1, dev[13], dev[14], kc2, vc2, dev[17], dev[18], heads,
+                                   kv_heads, hd)
+    assert torch.equal(fused, qkv) and torch.equal(kc2, kc) and torch.equal(vc2, vc)
 
 
 def _kernel_with_pointer(name):

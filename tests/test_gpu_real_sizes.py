@@ -65,7 +65,7 @@ def test_real_layer_sizes_under_every_cut(real, dtype, tol):
 
 CONFIG_SPLIT_NORMS = {
     "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2",
-    "num_hidden_layers": 3, "hidden_size": 512, "num_attention_heads": 4, "num_key_value_heads": 2, "head_dim": 128,
+    "num_hidden_layers": 3, "hidden_size": 1024, "num_attention_heads": 4, "num_key_value_heads": 2, "head_dim": 128,
     "intermediate_size": 4096, "vocab_size": 300, "rope_theta": 10000.0, "rms_norm_eps": 1e-5,
     "tie_word_embeddings": True, "max_position_embeddings": 4096, "hidden_act": "silu",
 }
@@ -81,18 +81,20 @@ def test_norms_split_between_the_products_around_them(tmp_path, monkeypatch):
     from vipera_rs_amd.ops import kernels
     folder = make_folder(tmp_path / "split", CONFIG_SPLIT_NORMS, 5, torch.bfloat16)
     cfg, w = P.load_folder(folder)
-    tokens = random_tokens(300, 70, 31)
+    tokens = random_tokens(300, 170, 31)
     want = P.forward(cfg, w, tokens)
     runner = ModelRunner.from_folder(folder, dtype="bfloat16", block_size=16, num_blocks=24, num_slots=4)
     calls = []
     real_rmsnorm = kernels.rmsnorm
     monkeypatch.setattr(kernels, "rmsnorm", lambda *a, **k: (calls.append(1), real_rmsnorm(*a, **k))[1])
     rows, at = [], 0
-    for size in [20, 16, 9, 5, 4, 2] + [1] * 14:                 # the first portion is too long for the split
+    # up to 16 tokens both norms of a layer run inside products; from 17 to 64 the first one does (the kernel that
+    # adds the K ranges of the q/k/v product divides by it), beyond that none
+    for size in [70, 40, 17, 16, 9, 5, 4, 2] + [1] * 7:
         runner.cache.reserve(0, at, at + size)
         calls.clear()
         rows.append(runner.step([StepEntry(0, at, tokens[at:at + size], list(range(size)))]).cpu().numpy())
-        assert len(calls) == (2 * 3 + 1 if size > 16 else 2), (size, len(calls))
+        assert len(calls) == (2 * 3 + 1 if size > 64 else 3 + 2 if size > 16 else 2), (size, len(calls))
         at += size
     assert at == len(tokens)
     assert rel_err(np.concatenate(rows), want) < 3e-2

@@ -547,6 +547,7 @@ struct FollowNorm {
   __bf16* scaled;
   float* sumsq;
   long long ld_scaled;
+  int sumsq_stride = 16;  // floats per workgroup: 16 tokens for the consumers of up to 16 tokens, 64 beyond
 };
 
 // The consumer's side of FollowNorm in a workgroup of 256 threads. request_squares: thread t asks for the sums of
@@ -1352,13 +1353,86 @@ __global__ __launch_bounds__(256) void gemm_reduce_follow_kernel(const float* __
   for (int off = 32; off > 0; off >>= 1) squares += __shfl_xor(squares, off);
   if ((threadIdx.x & 63) == 0) wave_sum[threadIdx.x >> 6] = squares;
   __syncthreads();
-  if (threadIdx.x == 0) follow.sumsq[(size_t)blockIdx.x * 16 + m] = wave_sum[0] + wave_sum[1] + wave_sum[2] + wave_sum[3];
+  if (threadIdx.x == 0)
+    follow.sumsq[(size_t)blockIdx.x * follow.sumsq_stride + m] = wave_sum[0] + wave_sum[1] + wave_sum[2] + wave_sum[3];
+}
+
+// The sum of a split q/k/v product's K ranges with what gemm_qkv_rope_kernel does in its epilogue: (division by
+// the root mean square of the norm before, if `sumsq`,) bias, rounding to bfloat16, rotation, cache write. Grid
+// (ceil(units / 256), M): a thread owns four consecutive dims below half the width of a q or k head together with
+// their partners, or four dims of a v head. Without `sumsq` bit for bit what gemm_reduce_kernel followed by
+// rope_kvwrite_kernel leaves. Needs a head width that is a multiple of 8 and N a multiple of 4.
+struct ReduceRope {
+  QkvRope r;
+  int sumsq_stride;
+};
+__global__ __launch_bounds__(256) void gemm_reduce_rope_kernel(const float* __restrict__ partial,
+                                                               const float* __restrict__ bias, __bf16* __restrict__ C,
+                                                               int M, int N, int K, long long ldc, int ranges,
+                                                               ReduceRope rr) {
+  const QkvRope& r = rr.r;
+  const int hd = r.hd, half = hd / 2, quads = half / 4;
+  const int rotated_units = (r.heads + r.kv_heads) * quads, units = rotated_units + r.kv_heads * (hd / 4);
+  const int u = blockIdx.x * 256 + threadIdx.x, m = blockIdx.y;
+  if (u >= units) return;
+  const bool rotated = u < rotated_units;
+  const int head = rotated ? u / quads : r.heads + r.kv_heads + (u - rotated_units) / (hd / 4);
+  const int d0 = rotated ? (u % quads) * 4 : ((u - rotated_units) % (hd / 4)) * 4;
+  const int lo_col = head * hd + d0, hi_col = lo_col + half;
+  f32x4 lo = {0.f, 0.f, 0.f, 0.f}, hi = {0.f, 0.f, 0.f, 0.f};
+  for (int range = 0; range < ranges; ++range) {
+    const float* src = partial + ((size_t)range * M + m) * N;
+    lo += *(const f32x4*)(src + lo_col);
+    if (rotated) hi += *(const f32x4*)(src + hi_col);
+  }
+  if (r.sumsq) {
+    float squares = 0.f;
+    for (int g = 0; g < r.groups; ++g) squares += r.sumsq[(size_t)g * rr.sumsq_stride + m];
+    const float inv = 1.0f / sqrtf(squares / (float)K + r.eps);
+    lo *= inv;
+    hi *= inv;
+  }
+  if (bias) {
+    lo += *(const f32x4*)(bias + lo_col);
+    if (rotated) hi += *(const f32x4*)(bias + hi_col);
+  }
+  const int pos = r.positions[m];
+  int page = -1;
+  if (r.k_cache && head >= r.heads) page = r.block_table[(size_t)r.entry_of_token[m] * r.table_width + pos / r.block_size];
+  const int slot = pos % r.block_size;
+  bf16x4 a, b;
+  if (rotated) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float sn, cs;
+      sincosf((float)pos * r.inv_freq[d0 + j], &sn, &cs);
+      const float l = (float)(__bf16)lo[j], h = (float)(__bf16)hi[j];
+      a[j] = (__bf16)(l * cs - h * sn);
+      b[j] = (__bf16)(l * sn + h * cs);
+    }
+    *(bf16x4*)(C + (size_t)m * ldc + lo_col) = a;
+    *(bf16x4*)(C + (size_t)m * ldc + hi_col) = b;
+    if (page >= 0) {
+      __bf16* at = r.k_cache + (((size_t)page * r.kv_heads + (head - r.heads)) * r.block_size + slot) * hd + d0;
+      *(bf16x4*)at = a;
+      *(bf16x4*)(at + half) = b;
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) a[j] = (__bf16)lo[j];
+    *(bf16x4*)(C + (size_t)m * ldc + lo_col) = a;
+    if (page >= 0) {
+      __bf16* at = r.v_cache + (((size_t)page * r.kv_heads + (head - r.heads - r.kv_heads)) * hd + d0) * r.block_size + slot;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) at[(size_t)j * r.block_size] = a[j];
+    }
+  }
 }
 
 template <int CB, int RT, typename TC, bool ACC>
 int launch_mid_as(const __bf16* A, const __bf16* W, const float* bias, TC* C, float* partial, long long partial_floats,
                   int ranges, int forced_rows, int M, int N, int K, long long lda, long long ldc, int vector_ok,
-                  hipStream_t s, const FollowNorm* follow = nullptr) {
+                  hipStream_t s, const FollowNorm* follow = nullptr, const ReduceRope* rope = nullptr) {
   constexpr int lds_bytes = 2 * CB * 16 * MID_ROW * (int)sizeof(__bf16);
   const int rows = RT == 2 ? 32 : forced_rows ? forced_rows : balanced_rows(M, N, 4, ranges < 1 ? 1 : ranges);  // per wave
   const int blocks = (N + 4 * rows - 1) / (4 * rows);
@@ -1395,6 +1469,14 @@ int launch_mid_as(const __bf16* A, const __bf16* W, const float* bias, TC* C, fl
       return 0;
     }
   }
+  if constexpr (!ACC && sizeof(TC) == 2) {
+    if (rope) {
+      const int units = (rope->r.heads + rope->r.kv_heads) * (rope->r.hd / 8) + rope->r.kv_heads * (rope->r.hd / 4);
+      gemm_reduce_rope_kernel<<<dim3((units + 255) / 256, M), 256, 0, s>>>(partial, bias, (__bf16*)C, M, N, K, ldc, used, *rope);
+      VK_LAUNCH_CHECK();
+      return 0;
+    }
+  }
   const long long threads = (long long)M * ((N + 3) / 4);
   gemm_reduce_kernel<TC, ACC><<<(int)((threads + 255) / 256), 256, 0, s>>>(partial, bias, C, M, N, ldc, used, vector_ok);
   VK_LAUNCH_CHECK();
@@ -1404,11 +1486,11 @@ int launch_mid_as(const __bf16* A, const __bf16* W, const float* bias, TC* C, fl
 template <typename TC, bool ACC>
 int launch_mid(const __bf16* A, const __bf16* W, const float* bias, TC* C, float* partial, long long partial_floats,
                int ranges, int rows_per_wave, int M, int N, int K, long long lda, long long ldc, int vector_ok,
-               hipStream_t s, const FollowNorm* follow = nullptr) {
+               hipStream_t s, const FollowNorm* follow = nullptr, const ReduceRope* rope = nullptr) {
   const int cb = (M + 15) / 16;
   // 108 to 116: one tile per wave with a forced number of rows (8 to 16), for tests and measurements
   const int forced = rows_per_wave >= 108 && rows_per_wave <= 116 ? rows_per_wave - 100 : 0;
-#define VK_MID(CBV, RTV) return launch_mid_as<CBV, RTV, TC, ACC>(A, W, bias, C, partial, partial_floats, ranges, forced, M, N, K, lda, ldc, vector_ok, s, follow)
+#define VK_MID(CBV, RTV) return launch_mid_as<CBV, RTV, TC, ACC>(A, W, bias, C, partial, partial_floats, ranges, forced, M, N, K, lda, ldc, vector_ok, s, follow, rope)
   if (rows_per_wave == 2) {
     switch (cb) { case 1: VK_MID(1, 2); case 2: VK_MID(2, 2); case 3: VK_MID(3, 2); case 4: VK_MID(4, 2); }
   } else {
@@ -1724,26 +1806,56 @@ extern "C" int vk_gemm_bf16_follow(const void* A, const void* W, const float* bi
 
 // vk_gemm_bf16_follow for up to 64 tokens where K is split over workgroups (vk_gemm_bf16_mid with `ranges` > 1
 // into a float C with accumulation): the kernel that adds the ranges also leaves `scaled` and the sums of squares,
-// here ceil(N / 1024) groups.
+// here ceil(N / 1024) groups of `sumsq_stride` floats (16, or 64 for more than 16 tokens).
 extern "C" int vk_gemm_bf16_mid_follow(const void* A, const void* W, const float* bias, float* C, int M, int N, int K,
                                        long long lda, long long ldc, int ranges, int rows_per_wave, float* partial,
                                        long long partial_floats, const float* gain, void* scaled, long long ld_scaled,
-                                       float* sumsq, long long sumsq_floats, int* groups, void* stream) {
+                                       float* sumsq, long long sumsq_floats, int sumsq_stride, int* groups, void* stream) {
   if (M <= 0 || N <= 0 || M > 64) return VK_UNSUPPORTED_SIZE;
   if (K <= 0 || (K & 7) || (lda & 7) || lda < K || ldc < N || ranges < 2 || ld_scaled < N || !gain || !scaled || !sumsq ||
       !groups || !partial)
     return VK_BAD_ARGUMENT;
   if (((uintptr_t)A & 15) || ((uintptr_t)W & 15) || ((uintptr_t)partial & 15)) return VK_BAD_ARGUMENT;
   if (K >= (1 << 24) || lda >= (1 << 24)) return VK_UNSUPPORTED_SIZE;
+  if ((sumsq_stride != 16 && sumsq_stride != 64) || M > sumsq_stride) return VK_BAD_ARGUMENT;
   const int blocks = (N + 1023) / 1024;
-  if ((long long)blocks * 16 > sumsq_floats) return VK_UNSUPPORTED_SIZE;
+  if ((long long)blocks * sumsq_stride > sumsq_floats) return VK_UNSUPPORTED_SIZE;
   // the ranges must really be split, or the product would write C without the kernel that adds them
   const int k_per_range = ((K + ranges - 1) / ranges + MID_CHUNK - 1) / MID_CHUNK * MID_CHUNK;
   if ((K + k_per_range - 1) / k_per_range < 2) return VK_UNSUPPORTED_SIZE;
   *groups = blocks;
-  const FollowNorm follow{gain, (__bf16*)scaled, sumsq, ld_scaled};
+  const FollowNorm follow{gain, (__bf16*)scaled, sumsq, ld_scaled, sumsq_stride};
   return launch_mid<float, true>((const __bf16*)A, (const __bf16*)W, bias, C, partial, partial_floats, ranges, rows_per_wave,
                                  M, N, K, lda, ldc, 0, (hipStream_t)stream, &follow);
+}
+
+// vk_gemm_bf16_qkv_rope for up to 64 tokens where K is split over workgroups (vk_gemm_bf16_mid with `ranges` > 1):
+// the kernel that adds the ranges also divides by the norm's root mean square (if `sumsq`: `norm_groups` groups of
+// `sumsq_stride` floats), adds the bias, rotates and writes the cache. hd a multiple of 8.
+extern "C" int vk_gemm_bf16_mid_qkv_rope(const void* A, const void* W, const float* bias, void* C, int M, int N, int K,
+                                         long long lda, long long ldc, int ranges, int rows_per_wave, float* partial,
+                                         long long partial_floats, const int* positions, const float* inv_freq,
+                                         void* k_cache, void* v_cache, const int* entry_of_token, const int* block_table,
+                                         int table_width, int block_size, int heads, int kv_heads, int hd,
+                                         const float* sumsq, int norm_groups, int sumsq_stride, float eps, void* stream) {
+  if (M <= 0 || N <= 0 || M > 64) return VK_UNSUPPORTED_SIZE;
+  if (K <= 0 || (K & 7) || (lda & 7) || lda < K || ldc < N || (ldc & 3) || ranges < 2 || !partial) return VK_BAD_ARGUMENT;
+  if (((uintptr_t)A & 15) || ((uintptr_t)W & 15) || ((uintptr_t)partial & 15) || ((uintptr_t)C & 7) ||
+      ((uintptr_t)bias & 15) || ((uintptr_t)k_cache & 7))
+    return VK_BAD_ARGUMENT;
+  if (heads <= 0 || kv_heads <= 0 || hd <= 0 || (hd & 7) || (long long)(heads + 2 * kv_heads) * hd != N || !positions ||
+      !inv_freq)
+    return VK_BAD_ARGUMENT;
+  if (k_cache && (!v_cache || !entry_of_token || !block_table || table_width <= 0 || block_size <= 0)) return VK_BAD_ARGUMENT;
+  if (sumsq && (norm_groups <= 0 || (sumsq_stride != 16 && sumsq_stride != 64) || M > sumsq_stride)) return VK_BAD_ARGUMENT;
+  if (K >= (1 << 24) || lda >= (1 << 24)) return VK_UNSUPPORTED_SIZE;
+  const int k_per_range = ((K + ranges - 1) / ranges + MID_CHUNK - 1) / MID_CHUNK * MID_CHUNK;
+  if ((K + k_per_range - 1) / k_per_range < 2) return VK_UNSUPPORTED_SIZE;
+  const ReduceRope rope{QkvRope{positions, inv_freq, (__bf16*)k_cache, (__bf16*)v_cache, entry_of_token, block_table,
+                                table_width, block_size, heads, kv_heads, hd, 0, 0, sumsq, norm_groups, eps},
+                        sumsq_stride};
+  return launch_mid<__bf16, false>((const __bf16*)A, (const __bf16*)W, bias, (__bf16*)C, partial, partial_floats, ranges,
+                                   rows_per_wave, M, N, K, lda, ldc, 0, (hipStream_t)stream, nullptr, &rope);
 }
 
 // vk_gemm_bf16_gated with resident activations (rows_per_wave 0) on the output of vk_gemm_bf16_follow: A = scaled,

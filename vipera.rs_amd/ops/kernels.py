@@ -421,12 +421,17 @@ def gemm_bf16_follow(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tens
     return int(groups.value)
 
 
+def follow_stride(tokens: int) -> int:
+    """Floats per group of the sums of squares that :func:`gemm_bf16_mid_follow` leaves for ``tokens`` rows."""
+    return 16 if tokens <= 16 else 64
+
+
 def gemm_bf16_mid_follow(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
                          ranges: int, rows_per_wave: int, gain: torch.Tensor, scaled: torch.Tensor,
                          sumsq: torch.Tensor) -> int:
     """:func:`gemm_bf16_follow` for up to 64 tokens where K is split into ``ranges`` > 1 over workgroups
     (:func:`gemm_bf16_mid` with accumulation): the kernel that adds the ranges leaves ``scaled`` and the sums of
-    squares.  Returns the number of groups."""
+    squares, :func:`follow_stride` floats per group.  Returns the number of groups."""
     _dev(a, w, bias, out, gain, scaled, sumsq)
     m, k = a.shape
     n = w.shape[0]
@@ -445,11 +450,54 @@ def gemm_bf16_mid_follow(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.
     partial = _split_k_workspace(a.device, ranges * 64 * n, "mid")
     groups = ctypes.c_int(0)
     fn = _fn("gemm_bf16", "vk_gemm_bf16_mid_follow", [_p, _p, _p, _p, _i, _i, _i, _ll, _ll, _i, _i, _p, _ll, _p, _p, _ll, _p,
-                                                      _ll, ctypes.POINTER(ctypes.c_int), _p])
+                                                      _ll, _i, ctypes.POINTER(ctypes.c_int), _p])
     _status(fn(_ptr(a), _ptr(w), _ptr(bias), _ptr(out), m, n, k, lda, n, int(ranges), int(rows_per_wave), _ptr(partial),
-               partial.numel(), _ptr(gain), _ptr(scaled), n, _ptr(sumsq), sumsq.numel(), ctypes.byref(groups), _stream()),
-            "gemm_bf16_mid_follow")
+               partial.numel(), _ptr(gain), _ptr(scaled), n, _ptr(sumsq), sumsq.numel(), follow_stride(m),
+               ctypes.byref(groups), _stream()), "gemm_bf16_mid_follow")
     return int(groups.value)
+
+
+def gemm_bf16_mid_qkv_rope(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], qkv: torch.Tensor,
+                           ranges: int, rows_per_wave: int, positions: torch.Tensor, inv_freq: torch.Tensor,
+                           k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor], entry_of_token: torch.Tensor,
+                           block_table: Optional[torch.Tensor], heads: int, kv_heads: int, head_dim: int,
+                           sumsq: Optional[torch.Tensor] = None, groups: int = 0, eps: float = 0.0) -> None:
+    """:func:`gemm_bf16_qkv_rope` for up to 64 tokens where K is split into ``ranges`` > 1 over workgroups: the
+    kernel that adds the ranges also divides by the norm (``sumsq``: ``groups`` groups of :func:`follow_stride`
+    floats), adds the bias, rotates and writes the cache."""
+    _dev(a, w, bias, qkv, positions, inv_freq, k_cache, v_cache, entry_of_token, block_table, sumsq)
+    m, k = a.shape
+    n = w.shape[0]
+    _need(m <= 64 and ranges >= 2 and head_dim % 8 == 0, "gemm_bf16_mid_qkv_rope: at most 64 tokens, two ranges or more, "
+          "a head width that is a multiple of 8")
+    _need(w.shape[1] == k and qkv.shape == (m, n) and n == (heads + 2 * kv_heads) * head_dim, "gemm_bf16_mid_qkv_rope: shapes")
+    _need(qkv.dtype == torch.bfloat16 and qkv.is_contiguous() and gemm_bf16_supported(a, w, qkv),
+          "gemm_bf16_mid_qkv_rope: bfloat16 operands and a contiguous output")
+    if bias is not None:
+        _need(bias.dtype == torch.float32 and bias.numel() == n and bias.is_contiguous(), "gemm: bias must be float32 [n]")
+    _need(positions.dtype == torch.int32 and positions.numel() >= m, "gemm_bf16_mid_qkv_rope: positions")
+    _need(inv_freq.dtype == torch.float32 and inv_freq.numel() == head_dim // 2 and inv_freq.is_contiguous(),
+          "gemm_bf16_mid_qkv_rope: inv_freq must hold head_dim / 2 floats")
+    table_width = block_size = 0
+    if k_cache is not None:
+        _need(v_cache is not None and block_table is not None, "gemm_bf16_mid_qkv_rope: cache without table")
+        _need(_cache_ok(k_cache, v_cache, kv_heads, head_dim, qkv.dtype), "gemm_bf16_mid_qkv_rope: cache shape or dtype")
+        _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(),
+              "gemm_bf16_mid_qkv_rope: block table")
+        _need(entry_of_token.dtype == torch.int32 and entry_of_token.numel() >= m, "gemm_bf16_mid_qkv_rope: entries")
+        table_width, block_size = block_table.shape[1], k_cache.shape[2]
+    if sumsq is not None:
+        _need(sumsq.dtype == torch.float32 and groups >= 1 and sumsq.numel() >= groups * follow_stride(m),
+              "gemm_bf16_mid_qkv_rope: sumsq")
+    lda = a.stride(0) if m > 1 else max(a.stride(0), k)
+    lda = lda if lda % 8 == 0 else k
+    partial = _split_k_workspace(a.device, ranges * 64 * n, "mid")
+    fn = _fn("gemm_bf16", "vk_gemm_bf16_mid_qkv_rope",
+             [_p, _p, _p, _p, _i, _i, _i, _ll, _ll, _i, _i, _p, _ll, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _p, _i, _i, _f, _p])
+    _status(fn(_ptr(a), _ptr(w), _ptr(bias), _ptr(qkv), m, n, k, lda, n, int(ranges), int(rows_per_wave), _ptr(partial),
+               partial.numel(), _ptr(positions), _ptr(inv_freq), _ptr(k_cache), _ptr(v_cache), _ptr(entry_of_token),
+               _ptr(block_table), table_width, block_size, heads, kv_heads, head_dim, _ptr(sumsq), int(groups),
+               follow_stride(m), float(eps), _stream()), "gemm_bf16_mid_qkv_rope")
 
 
 def gemm_bf16_gated_scaled(scaled: torch.Tensor, w: torch.Tensor, out: torch.Tensor, sumsq: torch.Tensor, groups: int,

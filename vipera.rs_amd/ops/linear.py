@@ -64,13 +64,22 @@ def linear_follow(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor]
     bf16 = a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
     if bf16 and m <= 16 and streams_in_wave_order(m, n, k) and kernels.gemm_bf16_follow_supported(a, w, residual):
         return kernels.gemm_bf16_follow(a, w, bias, residual, gain, scaled, sumsq)
-    if (bf16 and m <= 16 and residual.dtype == torch.float32 and residual.is_contiguous()
+    if (bf16 and m <= 64 and residual.dtype == torch.float32 and residual.is_contiguous()
             and kernels.gemm_bf16_supported(a, w, residual)):
         ranges, rows_per_wave = mid_plan(m, n, k)
         if ranges >= 2 and k // ranges >= 512:
             return kernels.gemm_bf16_mid_follow(a, w, bias, residual, ranges, rows_per_wave, gain, scaled, sumsq)
     linear(a, w, bias, residual, accumulate=True)
     return 0
+
+
+def split_qkv_plan(m: int, n: int, k: int) -> Optional[Tuple[int, int]]:
+    """``(ranges, tiles per wave)`` if a q/k/v product of ``m`` tokens runs with K split over workgroups, so that the
+    kernel that adds the ranges can also rotate and write the cache (17 to 64 tokens), else None."""
+    if m <= 16 or m > 64 or streams_in_wave_order(m, n, k):
+        return None
+    ranges, rows_per_wave = mid_plan(m, n, k)
+    return (ranges, rows_per_wave) if ranges >= 2 and k // ranges >= 512 else None
 
 
 def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:

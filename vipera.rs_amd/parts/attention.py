@@ -17,7 +17,7 @@ from ..config.base import PartSpec
 from ..errors import InvalidArgumentError, UnsupportedError
 from ..ops import kernels
 from ..ops.attention import paged_attention
-from ..ops.linear import linear, streams_in_wave_order
+from ..ops.linear import linear, split_qkv_plan, streams_in_wave_order
 from ..weights.checkpoint import MATRIX, VECTOR, TensorSpec
 from .base import KVCacheSpec, Mixer, register_mixer
 
@@ -78,25 +78,33 @@ class Attention(Mixer):
 
     fills_handoff = True
 
-    def _one_kernel(self, tokens: int, position, batch) -> bool:
-        """Whether product, rotation and cache write of a step of ``tokens`` are one kernel: a few tokens, all
-        bfloat16, a full rotation computed in the kernel (no table of the step's angles)."""
+    def _fused(self, tokens: int, position, batch) -> Optional[str]:
+        """How product, rotation and cache write of a step of ``tokens`` run as one launch sequence without a
+        rotation kernel, if they do: "stream" (up to 16 tokens, one kernel) or "split" (17 to 64 tokens, K split
+        over workgroups and the kernel that adds the ranges rotates).  All bfloat16, a full rotation computed in the
+        kernel (no table of the step's angles)."""
         fused = position.fused_rotary()
-        return (fused is not None and fused[1] == self.head_dim and self.runtime.dtype == torch.bfloat16
-                and self.w_qkv.dtype == torch.bfloat16 and tokens <= 16 and self.head_dim % 2 == 0
-                and streams_in_wave_order(tokens, *self.w_qkv.shape)
-                and self.w_qkv.shape[0] * self.w_qkv.shape[1] * 2 < 2 ** 31 and self.w_qkv.shape[1] % 8 == 0
-                and position.step_angles(batch) is None)
+        n, k = self.w_qkv.shape
+        if not (fused is not None and fused[1] == self.head_dim and self.runtime.dtype == torch.bfloat16
+                and self.w_qkv.dtype == torch.bfloat16 and self.head_dim % 2 == 0 and k % 8 == 0
+                and position.step_angles(batch) is None):
+            return None
+        if tokens <= 16 and streams_in_wave_order(tokens, n, k) and n * k * 2 < 2 ** 31:
+            return "stream"
+        if self.head_dim % 8 == 0 and split_qkv_plan(tokens, n, k) is not None:
+            return "split"
+        return None
 
     def accepts_handoff(self, tokens: int, position, batch) -> bool:
-        # the one-kernel product can divide by the norm itself
-        return self._one_kernel(tokens, position, batch)
+        # the fused products can divide by the norm themselves
+        return self._fused(tokens, position, batch) is not None
 
     def forward(self, h, batch, cache, state, position, residual, reads_only: bool = False, handoff=None,
                 incoming=None) -> None:
         tokens = residual.shape[0]
-        if incoming is not None and not self._one_kernel(tokens, position, batch):
-            raise UnsupportedError("attention was handed a split norm for a step it does not run as one kernel")
+        how = self._fused(tokens, position, batch)
+        if incoming is not None and how is None:
+            raise UnsupportedError("attention was handed a split norm for a step whose product cannot divide by it")
         scaled = {} if incoming is None else {"sumsq": incoming.sumsq, "groups": incoming.groups, "eps": incoming.eps}
         if incoming is not None:
             h = incoming.scaled
@@ -105,14 +113,17 @@ class Attention(Mixer):
         fused = position.fused_rotary()
         inv_freq, rotary_dim = fused if fused is not None else (None, 0)
         angles = position.step_angles(batch) if rotary_dim else None
-        if self._one_kernel(tokens, position, batch) and kernels.gemm_bf16_qkv_rope_supported(h, self.w_qkv, qkv, self.head_dim):
-            kernels.gemm_bf16_qkv_rope(h, self.w_qkv, self.b_qkv, qkv, batch.positions, inv_freq,
-                                       None if reads_only else cache.k, None if reads_only else cache.v,
-                                       batch.entry_of_token, None if reads_only else table, self.heads, self.kv_heads,
-                                       self.head_dim, **scaled)
+        caches = (None, None, batch.entry_of_token, None) if reads_only else (cache.k, cache.v, batch.entry_of_token, table)
+        if how == "stream" and kernels.gemm_bf16_qkv_rope_supported(h, self.w_qkv, qkv, self.head_dim):
+            kernels.gemm_bf16_qkv_rope(h, self.w_qkv, self.b_qkv, qkv, batch.positions, inv_freq, *caches, self.heads,
+                                       self.kv_heads, self.head_dim, **scaled)
+        elif how == "split" and kernels.gemm_bf16_supported(h, self.w_qkv, qkv):
+            ranges, rows_per_wave = split_qkv_plan(tokens, *self.w_qkv.shape)
+            kernels.gemm_bf16_mid_qkv_rope(h, self.w_qkv, self.b_qkv, qkv, ranges, rows_per_wave, batch.positions, inv_freq,
+                                           *caches, self.heads, self.kv_heads, self.head_dim, **scaled)
         else:
             if incoming is not None:
-                raise UnsupportedError("attention was handed a split norm for operands its one-kernel product does not take")
+                raise UnsupportedError("attention was handed a split norm for operands its fused product does not take")
             linear(h, self.w_qkv, self.b_qkv, qkv)
             if fused is None:
                 position.apply(qkv, batch, self.heads, self.kv_heads, self.head_dim)
