@@ -390,9 +390,9 @@ def gemm_bf16_follow_supported(a: torch.Tensor, w: torch.Tensor, out: torch.Tens
 
 
 def follow_sumsq_floats(n: int) -> int:
-    """Floats that the sums of squares of :func:`gemm_bf16_follow` may take for an output of ``n`` columns
-    (16 per workgroup, a workgroup owns at least 8 columns)."""
-    return ((n + 7) // 8) * 16
+    """Floats that the sums of squares of :func:`gemm_bf16_follow` and :func:`gemm_bf16_mid_follow` may take for an
+    output of ``n`` columns (16 per workgroup that owns at least 8 columns, or 64 per 1,024 columns)."""
+    return max(((n + 7) // 8) * 16, ((n + 1023) // 1024) * 64)
 
 
 def gemm_bf16_follow(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
