@@ -1,0 +1,62 @@
+"""Which kernel a product or an attention step is given: the decisions of ``ops/linear.py`` and ``ops/attention.py``
+at the layer sizes of the 1.5B, 7B and 32B shapes.  Pure functions of the sizes: no GPU is touched."""
+from vipera_rs_amd.ops.attention import decode_chunking
+from vipera_rs_amd.ops.kernels import follow_stride, follow_sumsq_floats
+from vipera_rs_amd.ops.linear import (gated_plan, gated_resident_fits, mid_plan, split_qkv_plan, streams_in_wave_order)
+
+QKV_7B, O_7B, GATE_UP_7B, DOWN_7B, HEAD_7B = (4608, 3584), (3584, 3584), (37888, 3584), (3584, 18944), (152064, 3584)
+
+
+def test_few_tokens_stream_the_weights_with_k_split_inside_a_workgroup():
+    for n, k in (QKV_7B, O_7B, DOWN_7B, HEAD_7B):
+        assert streams_in_wave_order(1, n, k) and streams_in_wave_order(4, n, k)
+    assert streams_in_wave_order(16, *QKV_7B) and streams_in_wave_order(16, *O_7B)
+    assert not streams_in_wave_order(8, *DOWN_7B)          # a long K: activations are shared through LDS instead
+    assert not streams_in_wave_order(8, *HEAD_7B)          # many rows: likewise
+    assert not streams_in_wave_order(17, *QKV_7B)
+
+
+def test_the_lds_shared_product_splits_k_where_rows_are_few():
+    assert mid_plan(8, *DOWN_7B) == (4, 1)                 # 56 row blocks x 4 ranges fill 256 CUs
+    assert mid_plan(64, *DOWN_7B) == (9, 2)                # many tokens and a long K: two tiles per wave, 28 row blocks x 9
+    assert mid_plan(8, *HEAD_7B) == (1, 1) and mid_plan(64, *HEAD_7B) == (1, 2)
+    assert mid_plan(64, *QKV_7B) == (3, 1) and mid_plan(64, *O_7B) == (4, 1)
+    ranges, _ = mid_plan(64, 2048, 1536)                   # 1.5B q/k/v: no range shorter than 512
+    assert 1536 // ranges >= 512
+
+
+def test_the_gated_product_goes_resident_tiled_or_lds_shared():
+    assert gated_resident_fits(16, *GATE_UP_7B) and not gated_resident_fits(17, *GATE_UP_7B)
+    assert not gated_resident_fits(16, 55296, 5120)        # 32B: 16 tokens x 5120 do not fit a CU's LDS
+    assert gated_resident_fits(8, 55296, 5120)
+    assert not gated_resident_fits(8, 37888, 3584 + 64)    # K in whole chunks of 256 only
+    for m in (1, 8, 16):
+        assert gated_plan(m, *GATE_UP_7B) == 0             # 1184 pairs over 256 CUs: 4 or 5 each
+    assert gated_plan(8, 17920, 1536) in (1, 2)            # 1.5B: 560 pairs would be 2 or 3 each, too uneven
+    assert gated_plan(8, 55296, 5120) == 0
+    assert gated_plan(32, *GATE_UP_7B) in (1, 2) and gated_plan(64, *GATE_UP_7B) == 3
+    assert gated_plan(24, 55296, 5120) == 3 and gated_plan(64, 17920, 1536) in (1, 2)
+    assert gated_plan(8, *GATE_UP_7B, cus=304) == 0        # 1184 pairs over 304 CUs: 3 or 4 each, 3 % above the mean
+    assert gated_plan(8, *GATE_UP_7B, cus=500) != 0        # over 500: 2 or 3 each, 27 % above the mean
+
+
+def test_q_k_v_of_17_to_64_tokens_rotates_in_the_kernel_that_adds_its_ranges():
+    assert split_qkv_plan(64, *QKV_7B) == (3, 1) and split_qkv_plan(17, *QKV_7B) == (3, 1)
+    assert split_qkv_plan(16, *QKV_7B) is None and split_qkv_plan(65, *QKV_7B) is None
+    assert split_qkv_plan(32, 1024, 512) is None           # K too short to split
+
+
+def test_room_for_the_sums_of_squares():
+    assert follow_stride(16) == 16 and follow_stride(17) == 64
+    for n in (16, 64, 1000, 3584, 8192):
+        assert follow_sumsq_floats(n) >= ((n + 7) // 8) * 16           # a workgroup per 8 columns, 16 tokens
+        assert follow_sumsq_floats(n) >= ((n + 1023) // 1024) * 64     # a workgroup per 1,024 columns, 64 tokens
+
+
+def test_decode_attention_chunks():
+    assert decode_chunking(4096, 8, 4, 1) == (256, 16)     # 8 requests x 4 key heads x 16 chunks = 512 waves
+    assert decode_chunking(4096, 64, 4, 1) == (1024, 4)
+    assert decode_chunking(4096, 1, 4, 1) == (128, 32)     # never below 128 positions a chunk
+    assert decode_chunking(100, 1, 4, 1) == (128, 1)
+    chunk, chunks = decode_chunking(1 << 20, 1, 1, 1)      # never more than 128 chunks
+    assert chunks <= 128 and chunk * chunks >= 1 << 20 and chunk % 32 == 0
