@@ -28,12 +28,13 @@ def solo(prompt, max_new, eos=None):
 
 
 class Harness:
-    def __init__(self, blocks=64, block_size=4, seqs=4, budget=32, chunk=8, max_len=256, window_blocks=None):
+    def __init__(self, blocks=64, block_size=4, seqs=4, budget=32, chunk=8, max_len=256, window_blocks=None,
+                 eager=False):
         groups = [CacheGroupSpec(block_size, blocks)]
         if window_blocks:
             groups.append(CacheGroupSpec(block_size, window_blocks, window=10))
         self.cache = CacheManager(groups, seqs)
-        self.sched = Scheduler(self.cache, seqs, budget, chunk, max_len)
+        self.sched = Scheduler(self.cache, seqs, budget, chunk, max_len, eager_admission=eager)
         self.budget, self.chunk, self.seqs = budget, chunk, seqs
         self.fed = {}        # request -> tokens fed so far in its current run
         self.out = {}        # request -> generated tokens
@@ -82,7 +83,8 @@ class Harness:
     def drain(self, limit=10_000):
         steps = 0
         while self.sched.has_work():
-            self.step()
+            plan = self.step()
+            assert plan.entries, "a plan is empty although requests wait or run"
             steps += 1
             assert steps < limit, "the scheduler makes no progress"
         return steps
@@ -251,3 +253,103 @@ def test_random_arrivals_on_a_small_cache_with_a_windowed_group(seed):
     assert h.out == expected
     assert h.cache.live_requests() == 0 and h.cache.check() == ""
     assert all(h.cache.used_blocks(g) == 0 for g in range(2))
+
+
+def test_two_long_prompts_on_a_pool_that_holds_one_both_finish():
+    # 10 pages of 16 positions; each 120-token prompt needs 8. Started side by side they would both stall
+    # at 5 pages with nothing free: the second is admitted only once the first one's pages leave room.
+    h = Harness(blocks=10, block_size=16, seqs=4, budget=32, chunk=16, max_len=256)
+    prompts = {0: prompt_of(120, 0), 1: prompt_of(120, 1)}
+    for r, p in prompts.items():
+        h.add(r, p, 5)
+    first = h.step()
+    assert [(e.request, len(e.tokens)) for e in first.entries] == [(0, 16)]     # no room for request 1 beside it
+    h.drain()
+    assert all(h.out[r] == solo(p, 5) for r, p in prompts.items())
+    assert h.sched.preemptions == 0
+    assert h.cache.free_blocks(0) == 10 and h.cache.live_requests() == 0
+
+
+def test_started_side_by_side_the_newer_of_two_stalled_prompts_gives_way():
+    # the same pool and prompts with eager admission: both are started, both stall at 5 pages of 8 with nothing
+    # free and no decoding request to push anyone out; the newer one gives way, the older one always moves
+    h = Harness(blocks=10, block_size=16, seqs=4, budget=32, chunk=16, max_len=256, eager=True)
+    prompts = {0: prompt_of(120, 0), 1: prompt_of(120, 1)}
+    for r, p in prompts.items():
+        h.add(r, p, 5)
+    preempted = []
+    while h.sched.has_work():
+        plan = h.step()
+        assert plan.entries, "a plan is empty although requests wait or run"
+        assert not h.cache.knows(0) or plan.entries[0].request == 0      # the oldest moves in every step
+        preempted += plan.preempted
+        assert len(h.history) < 500
+    assert preempted and set(preempted) == {1}
+    assert all(h.out[r] == solo(p, 5) for r, p in prompts.items())
+    assert h.cache.free_blocks(0) == 10 and h.cache.live_requests() == 0
+
+
+def test_when_every_running_prompt_waits_for_a_page_the_newest_gives_way():
+    # both requests run (their prompts fitted side by side when they were admitted) and have grown by decoding;
+    # after a preemption both recompute, meet in the middle of their tokens with no page left, and the newer one
+    # gives way instead of both waiting for ever
+    h = Harness(blocks=6, block_size=4, seqs=3, budget=32, chunk=4, max_len=64)
+    h.add(0, prompt_of(4, 0), 14)
+    h.add(1, prompt_of(4, 1), 14)
+    h.add(2, prompt_of(4, 2), 14)
+    preempted = []
+    while h.sched.has_work():
+        plan = h.step()
+        assert plan.entries
+        preempted += plan.preempted
+        assert len(h.history) < 2000
+    assert preempted and 0 not in preempted
+    assert all(h.out[r] == solo(prompt_of(4, r), 14) for r in range(3))
+    assert h.cache.free_blocks(0) == 6 and h.cache.live_requests() == 0
+
+
+def test_a_stall_of_running_prompts_is_broken_from_the_back():
+    # admission is by the tokens known at the time; here two requests are put into the running list by hand
+    # in a state that admission would not have produced (both mid-prompt, no page free)
+    h = Harness(blocks=4, block_size=4, seqs=2, budget=8, chunk=4, max_len=64)
+    h.add(0, prompt_of(12, 0), 2)
+    plan = h.step()                       # request 0 holds one page
+    assert [(e.request, len(e.tokens)) for e in plan.entries] == [(0, 4)]
+    h.add(1, prompt_of(4, 1), 9)          # fits beside what request 0 still needs (two more pages) exactly
+    plan = h.step()
+    assert [(e.request, len(e.tokens)) for e in plan.entries] == [(0, 4), (1, 4)]
+    plan = h.step()                       # request 1 decodes on the last free page, request 0's portion waits
+    assert [(e.request, len(e.tokens)) for e in plan.entries] == [(1, 1)] and plan.preempted == []
+    for _ in range(3):                    # request 1 decodes within its page
+        plan = h.step()
+        assert [(e.request, len(e.tokens)) for e in plan.entries] == [(1, 1)]
+    plan = h.step()                       # request 1 needs a page too: it is the newest, so it gives way itself,
+    assert plan.preempted == [1]          # and request 0 goes on in the same step
+    assert [(e.request, e.start, len(e.tokens)) for e in plan.entries] == [(0, 8, 4)]
+    h.drain()
+    assert h.out[0] == solo(prompt_of(12, 0), 2) and h.out[1] == solo(prompt_of(4, 1), 9)
+
+
+@pytest.mark.parametrize("eager", (False, True))
+@pytest.mark.parametrize("seed", range(8))
+def test_random_arrivals_of_long_prompts_on_pools_that_hold_one_or_two(seed, eager):
+    rng = random.Random(1000 + seed)
+    block_size = rng.choice((4, 8, 16))
+    blocks = rng.randrange(6, 12)
+    capacity = blocks * block_size
+    h = Harness(blocks=blocks, block_size=block_size, seqs=4, budget=rng.randrange(8, 40), chunk=rng.randrange(3, 20),
+                max_len=capacity + 8, eager=eager)
+    expected, next_id = {}, 0
+    for step in range(600):
+        if rng.random() < 0.2 and next_id < 14:
+            n = rng.randrange(1, 12)
+            length = rng.randrange(capacity // 3, capacity - n)      # most pairs do not fit side by side
+            p = prompt_of(length, 7000 * seed + next_id)
+            h.add(next_id, p, n)
+            expected[next_id] = solo(p, n)
+            next_id += 1
+        if h.sched.has_work():
+            assert h.step().entries, "a plan is empty although requests wait or run"
+    h.drain()
+    assert h.out == expected
+    assert h.cache.live_requests() == 0 and h.cache.check() == "" and h.cache.used_blocks(0) == 0

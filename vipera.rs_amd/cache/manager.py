@@ -48,7 +48,7 @@ def _host():
         "vk_cache_live_requests": ([p], i),
         "vk_cache_blocks_needed": ([p, i, i, i], i),
         "vk_cache_check": ([p, c.c_char_p, i], i),
-        "vk_sched_create": ([p, i, i, i, i], p),
+        "vk_sched_create": ([p, i, i, i, i, i], p),
         "vk_sched_destroy": ([p], None),
         "vk_sched_add": ([p, u64, ip, i, i], i),
         "vk_sched_plan": ([p, ip, ip], i),

@@ -94,10 +94,11 @@ int vk_cache_check(void* handle, char* out, int capacity) {
   return (int)text.size();
 }
 
-void* vk_sched_create(void* cache, int max_num_seqs, int max_batched_tokens, int chunk_size, int max_model_len) {
+void* vk_sched_create(void* cache, int max_num_seqs, int max_batched_tokens, int chunk_size, int max_model_len,
+                      int eager_admission) {
   if (!cache) return nullptr;
-  return new (std::nothrow)
-      SchedulerHandle(static_cast<CacheManager*>(cache), {max_num_seqs, max_batched_tokens, chunk_size, max_model_len});
+  return new (std::nothrow) SchedulerHandle(
+      static_cast<CacheManager*>(cache), {max_num_seqs, max_batched_tokens, chunk_size, max_model_len, eager_admission});
 }
 
 void vk_sched_destroy(void* handle) { delete static_cast<SchedulerHandle*>(handle); }

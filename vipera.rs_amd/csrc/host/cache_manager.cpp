@@ -128,6 +128,12 @@ int CacheManager::slot(uint64_t id) const {
   return found == requests_.end() ? -1 : found->second.slot;
 }
 
+int CacheManager::held_blocks(uint64_t id, int g) const {
+  int held = 0;
+  for (int page : table(id, g)) held += page >= 0;
+  return held;
+}
+
 std::string CacheManager::check() const {
   std::ostringstream problem;
   if (bad_frees_) problem << bad_frees_ << " pages were freed while not held; ";

@@ -64,6 +64,8 @@ class CacheManager {
   // Block table of a request in a group: page per logical block, -1 where no page is held.
   const std::vector<int>& table(uint64_t id, int group) const;
   int slot(uint64_t id) const;
+  // Pages the request holds in group g now.
+  int held_blocks(uint64_t id, int g) const;
   int num_groups() const { return (int)groups_.size(); }
   const GroupConfig& group(int g) const { return groups_[g]; }
   int free_blocks(int g) const { return pools_[g].free_count(); }

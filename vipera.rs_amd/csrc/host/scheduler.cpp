@@ -44,6 +44,20 @@ void Scheduler::preempt(uint64_t id, Plan* plan) {
   plan->preempted.push_back(id);
 }
 
+bool Scheduler::room_beside_running(int tokens) const {
+  const int portion = std::min(config_.chunk_size, config_.max_batched_tokens);
+  for (int g = 0; g < cache_->num_groups(); ++g) {
+    long spoken_for = 0;
+    for (uint64_t id : running_) {
+      const Request& request = requests_.at(id);
+      const int need = cache_->blocks_needed(g, (int)request.tokens.size(), portion);
+      spoken_for += std::max(0, need - cache_->held_blocks(id, g));
+    }
+    if (cache_->free_blocks(g) - spoken_for < cache_->blocks_needed(g, tokens, portion)) return false;
+  }
+  return true;
+}
+
 Plan Scheduler::plan() {
   Plan plan;
   int budget = config_.max_batched_tokens;
@@ -73,7 +87,8 @@ Plan Scheduler::plan() {
     }
   }
 
-  // 2. running requests in the middle of a prompt (or recomputing after a preemption)
+  // 2. running requests in the middle of a prompt (or recomputing after a preemption); a portion that
+  //    finds no page waits as long as anything else moves in this step
   for (uint64_t id : running_) {
     if (budget < 1) break;
     Request& request = requests_[id];
@@ -88,12 +103,14 @@ Plan Scheduler::plan() {
     budget -= count;
   }
 
-  // 3. admit waiting requests, oldest first, while their first portion fits
+  // 3. admit waiting requests, oldest first, while all they hold so far fits beside what the running
+  //    requests still need for theirs
   while (!waiting_.empty() && budget >= 1 && (int)running_.size() < config_.max_num_seqs) {
     const uint64_t id = waiting_.front();
     // a request that was preempted while this plan was made waits for the next step
     if (std::find(plan.preempted.begin(), plan.preempted.end(), id) != plan.preempted.end()) break;
     Request& request = requests_[id];
+    if (!config_.eager_admission && !room_beside_running((int)request.tokens.size())) break;
     const int count = std::min({(int)request.tokens.size(), config_.chunk_size, budget});
     if (cache_->reserve(id, 0, count) != RESERVE_OK) break;
     waiting_.pop_front();
@@ -103,6 +120,28 @@ Plan Scheduler::plan() {
     plan.entries.push_back({id, 0, count, count == (int)request.tokens.size() ? 1 : 0});
     request.planned_end = count;
     budget -= count;
+  }
+
+  // 4. nothing moves although requests are running: every one of them waits for a page that only
+  //    another one can give back. The most recently admitted ones give way until the oldest can go on.
+  //    It cannot end up giving way itself: alone it fits, or it would have been refused when added.
+  if (plan.entries.empty() && !running_.empty() && budget >= 1) {
+    const uint64_t id = running_.front();
+    Request& request = requests_[id];
+    const int remaining = (int)request.tokens.size() - request.processed;
+    const int count = std::min({remaining, config_.chunk_size, budget});
+    while (count >= 1) {
+      if (cache_->reserve(id, request.processed, request.processed + count) == RESERVE_OK) {
+        const int end = request.processed + count;
+        plan.entries.push_back({id, request.processed, count, end == (int)request.tokens.size() ? 1 : 0});
+        request.planned_end = end;
+        budget -= count;
+        break;
+      }
+      const uint64_t victim = running_.back();
+      if (victim == id) break;
+      preempt(victim, &plan);
+    }
   }
 
   for (const PlanEntry& entry : plan.entries) {

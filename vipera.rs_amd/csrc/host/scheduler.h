@@ -7,9 +7,24 @@
 // at its token budget, or when the context is full (1062-1110). It builds batches of one kind and
 // alternates (683-730), and when a reservation fails it fails every request of the batch (731-741).
 // Here a step mixes decode tokens and prompt portions under one token budget, and a failed
-// reservation for a decode token preempts the most recently admitted running request instead: its
-// pages are given back, it keeps its tokens, goes to the front of the waiting queue and is
-// recomputed later.
+// reservation preempts instead: the most recently admitted running request gives its pages back,
+// keeps its tokens, goes to the front of the waiting queue and is recomputed later.
+//
+// When pages run out:
+//  * a decode token that finds no page preempts from the back of the running list (admission order)
+//    until it has its page, or until it is the one that gives way;
+//  * a prompt portion that finds no page waits while anything else moves in the step; when nothing
+//    moves at all, the requests at the back give way until the oldest running request has its portion;
+//  * a waiting request is admitted only while the pages of all its known tokens fit into the free
+//    pages that the running requests do not still need for their known tokens, so that two long
+//    prompts are not started into a pool that holds only one of them.
+// Every plan moves at least one token while there is work. The request at the front of the running
+// list is only ever asked to give way by itself, and then it is alone, every page is free, and its
+// reservation succeeds, because `add` refuses a request that does not fit an empty pool. So the
+// front request gets a token in every step unless the budget went to decode tokens, which is
+// progress as well; with nothing running, every page is free and the front of the waiting queue
+// passes the admission rule for the same reason. Requests end after finitely many tokens, hence
+// no stall and no livelock.
 #pragma once
 #include <cstdint>
 #include <deque>
@@ -25,6 +40,9 @@ struct SchedulerConfig {
   int max_batched_tokens;  // tokens of one step
   int chunk_size;          // longest portion of one prompt in one step
   int max_model_len;       // longest sequence (prompt + generated)
+  // 1: admit a waiting request as soon as its first portion finds pages, without leaving room for what the
+  // running requests still need (more requests side by side, more recomputation when pages run out)
+  int eager_admission = 0;
 };
 
 enum AddResult : int {
@@ -83,6 +101,8 @@ class Scheduler {
     uint64_t admitted_at = 0;
   };
   void preempt(uint64_t id, Plan* plan);
+  // Whether a request of `tokens` known tokens fits beside what the running requests still need.
+  bool room_beside_running(int tokens) const;
   CacheManager* cache_;
   SchedulerConfig config_;
   std::map<uint64_t, Request> requests_;

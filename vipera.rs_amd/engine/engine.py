@@ -97,13 +97,16 @@ class Engine:
     is the same.  A request that ends on an end-of-sequence token has one token more computed, which is
     dropped.  While a live request uses penalties (they look at the last tokens on the host), steps run
     one after the other as without the option.
+
+    ``eager_admission``: start a waiting request as soon as its first portion finds pages, instead of only
+    when all its tokens fit beside what the running requests still need (see ``csrc/host/scheduler.h``).
     """
 
     def __init__(self, model: str, dtype: str = "bfloat16", device: str = "cuda:0", block_size: int = 16,
                  num_blocks: Optional[int] = None, max_num_seqs: int = 8, max_num_batched_tokens: int = 2048,
                  chunk_size: int = 512, max_model_len: Optional[int] = None,
                  eos_token_ids: Optional[Sequence[int]] = None, runner: Optional[ModelRunner] = None,
-                 use_graphs: Optional[bool] = None, pipelined: bool = False):
+                 use_graphs: Optional[bool] = None, pipelined: bool = False, eager_admission: bool = False):
         if runner is None:
             runtime = Runtime(device, dtype)
             from ..config.registry import load_config
@@ -123,7 +126,8 @@ class Engine:
         self.runner = runner
         self.config = config
         self.max_model_len = limit
-        self.scheduler = Scheduler(runner.cache, max_num_seqs, max_num_batched_tokens, chunk_size, limit)
+        self.scheduler = Scheduler(runner.cache, max_num_seqs, max_num_batched_tokens, chunk_size, limit,
+                                   eager_admission)
         self.sampler = BatchSampler(runner.runtime.device, out=runner.sampled_tokens)
         self.pipelined = bool(pipelined) and runner.sampled_tokens is not None
         self._inflight: Optional[_InFlight] = None   # the launched step whose tokens have not been collected

@@ -2,7 +2,8 @@
 
 It admits requests, cuts prompts into portions under a token budget, hands every decoding
 request its one token, ends requests and gives back what they hold, and preempts the most
-recently admitted running request when a decode token finds no page.  See
+recently admitted running request when a decode token finds no page, or when every running prompt
+waits for one.  See
 ``csrc/host/scheduler.h`` for the policy and what it takes from the reference's
 ``Engine`` (crates/vipera-runtime/src/engine.rs).
 """
@@ -39,7 +40,7 @@ class StepPlan:
 
 class Scheduler:
     def __init__(self, cache: CacheManager, max_num_seqs: int, max_num_batched_tokens: int, chunk_size: int,
-                 max_model_len: int):
+                 max_model_len: int, eager_admission: bool = False):
         if max_num_seqs < 1 or max_num_batched_tokens < 1 or chunk_size < 1 or max_model_len < 2:
             raise InvalidArgumentError(
                 "scheduler limits must be positive: "
@@ -52,7 +53,7 @@ class Scheduler:
         self.max_model_len = max_model_len
         self._lib = _host()
         self._handle = self._lib.vk_sched_create(cache._handle, max_num_seqs, max_num_batched_tokens, chunk_size,
-                                                 max_model_len)
+                                                 max_model_len, 1 if eager_admission else 0)
         if not self._handle:
             raise InternalError("the native scheduler could not be created")
 
