@@ -8,8 +8,9 @@ from typing import Dict, List, Sequence
 import numpy as np
 import torch
 
-# Two tiny configurations that differ in every size and option, and a third whose head width is not
-# hidden / heads.
+# Two tiny configurations that differ in every size and option (A and B), a third whose head width is not
+# hidden / heads (C), and B with windowed layers (D).  B's `max_position_embeddings` of 256 is above every
+# trace length the tests use on it (at most 246 positions).
 CONFIG_A = {
     "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2",
     "num_hidden_layers": 2, "hidden_size": 64, "num_attention_heads": 4, "num_key_value_heads": 2,
@@ -21,8 +22,8 @@ CONFIG_B = {
     "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2",
     "num_hidden_layers": 3, "hidden_size": 96, "num_attention_heads": 3, "num_key_value_heads": 1,
     "head_dim": 32, "intermediate_size": 200, "vocab_size": 300, "rope_theta": 1000000.0,
-    "rms_norm_eps": 1e-5, "tie_word_embeddings": False, "max_position_embeddings": 1024,
-    "hidden_act": "silu", "use_sliding_window": True, "sliding_window": 21, "max_window_layers": 1,
+    "rms_norm_eps": 1e-5, "tie_word_embeddings": False, "max_position_embeddings": 256,
+    "hidden_act": "silu", "use_sliding_window": False, "sliding_window": 21, "max_window_layers": 1,
 }
 CONFIG_C = {
     "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2",
@@ -31,7 +32,13 @@ CONFIG_C = {
     "rms_norm_eps": 1e-6, "tie_word_embeddings": False, "max_position_embeddings": 512,
     "hidden_act": "silu",
 }
-CONFIGS = {"A": (CONFIG_A, 0), "B": (CONFIG_B, 1), "C": (CONFIG_C, 2)}
+# Layers from `max_window_layers` on see the last `sliding_window` positions.  The reference has no such layer
+# rule (its window is a run-time option over all layers, crates/vipera-core/src/window.rs:38-55) and pins only
+# the visible range [p + 1 - w, p] (crates/vipera-backend-cpu/src/model.rs:2509): which layers are windowed is
+# this engine's reading of the config keys, parity unpinned, and D is reported apart from A, B and C.
+CONFIG_D = dict(CONFIG_B, use_sliding_window=True, sliding_window=21, max_window_layers=1,
+                max_position_embeddings=1024)
+CONFIGS = {"A": (CONFIG_A, 0), "B": (CONFIG_B, 1), "C": (CONFIG_C, 2), "D": (CONFIG_D, 3)}
 
 
 def make_folder(path: str, config: dict, seed: int, dtype=torch.float32) -> str:
@@ -53,6 +60,21 @@ def random_tokens(vocab: int, count: int, seed: int) -> List[int]:
 def rel_err(got: np.ndarray, want: np.ndarray) -> float:
     """Largest difference relative to the largest wanted magnitude."""
     return float(np.max(np.abs(got.astype(np.float64) - want)) / max(np.max(np.abs(want)), 1e-30))
+
+
+def assert_tokens_follow_plain(logits: np.ndarray, prompt_len: int, tokens: Sequence[int], tol: float,
+                               label: str = "") -> int:
+    """``tokens`` were generated greedily after a prompt of ``prompt_len``; ``logits`` are the plain
+    implementation's over prompt + tokens[:-1].  Every token must be the plain implementation's best one
+    wherever its lead over the runner-up is clear of ``tol``; returns how many were clear."""
+    checked = 0
+    for k, token in enumerate(tokens):
+        row = logits[prompt_len - 1 + k]
+        order = np.argsort(row)
+        if row[order[-1]] - row[order[-2]] > 4 * tol * np.max(np.abs(row)):
+            assert int(token) == int(order[-1]), f"{label}: generated token {k} is not the plain implementation's"
+            checked += 1
+    return checked
 
 
 # --- traces ---------------------------------------------------------------------------------------

@@ -3,7 +3,7 @@ import json
 
 import pytest
 
-from helpers import CONFIG_A, CONFIG_B, CONFIG_C
+from helpers import CONFIG_A, CONFIG_B, CONFIG_C, CONFIG_D
 
 import vipera_rs_amd  # noqa: F401
 from vipera_rs_amd import models  # noqa: F401  (registers architectures)
@@ -18,7 +18,7 @@ def test_reads_every_size_from_the_file():
     assert (cfg.num_hidden_layers, cfg.hidden_size, cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim,
             cfg.intermediate_size, cfg.vocab_size) == (3, 96, 3, 1, 32, 200, 300)
     assert cfg.rope_theta == 1e6 and cfg.rms_norm_eps == 1e-5 and not cfg.tie_word_embeddings
-    assert cfg.context_limit == 1024
+    assert cfg.context_limit == 256 and not cfg.use_sliding_window
 
 
 def test_defaults_follow_the_reference():
@@ -87,13 +87,14 @@ def test_registry_is_open():
 
 
 def test_layers_are_described_one_by_one_with_their_windows():
-    cfg = config_from_dict(CONFIG_B)
+    cfg = config_from_dict(CONFIG_D)
     specs = cfg.layer_specs()
     assert [s.mixer.params["window"] for s in specs] == [0, 21, 21]   # the first max_window_layers see everything
     assert all(s.mixer.kind == "attention" and s.ffn.kind == "gated_mlp" and s.block == "prenorm" for s in specs)
     assert specs[2].prefix == "model.layers.2." and specs[0].position.params["base"] == 1e6
     assert [e.layer for e in cfg.schedule()] == [0, 1, 2] and all(e.cache_of is None for e in cfg.schedule())
     assert [s.mixer.params["window"] for s in config_from_dict(CONFIG_A).layer_specs()] == [0, 0]
+    assert [s.mixer.params["window"] for s in config_from_dict(CONFIG_B).layer_specs()] == [0, 0, 0]   # switched off
 
 
 def test_round_trip_through_a_folder(tmp_path):

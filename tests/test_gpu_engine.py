@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import CONFIG_A, CONFIG_B, make_folder, random_tokens
+from helpers import CONFIG_A, CONFIG_B, CONFIG_D, assert_tokens_follow_plain, make_folder, random_tokens
 from plain import qwen2_plain
 
 pytestmark = pytest.mark.gpu
@@ -15,6 +15,8 @@ def folders(tmp_path_factory):
     return {
         "A": make_folder(tmp_path_factory.mktemp("engine_A"), CONFIG_A, 0, torch.float32),
         "B": make_folder(tmp_path_factory.mktemp("engine_B"), CONFIG_B, 1, torch.float32),
+        "D": make_folder(tmp_path_factory.mktemp("engine_D"), CONFIG_D, 3, torch.float32),
+        "B16": make_folder(tmp_path_factory.mktemp("engine_B16"), CONFIG_B, 1, torch.bfloat16),
     }
 
 
@@ -38,22 +40,34 @@ def test_greedy_generation_equals_the_plain_implementation(folders):
     assert [g.processed_tokens for g in got] == [len(p) + 7 for p in prompts]
 
 
-def test_greedy_generation_with_an_untied_head_and_windowed_layers(folders):
-    # tied embeddings make a random model repeat its last token; the second configuration does not
-    cfg, weights = qwen2_plain.load_folder(folders["B"])
+@pytest.mark.parametrize("name", ["B", "D"])
+def test_greedy_generation_with_an_untied_head(folders, name):
+    # tied embeddings make a random model repeat its last token; the second configuration does not (D: the same
+    # with windowed layers, prompts and continuations past the window of 21)
+    cfg, weights = qwen2_plain.load_folder(folders[name])
     prompts = [random_tokens(CONFIG_B["vocab_size"], n, 60 + n) for n in (3, 30, 11)]
-    want = [qwen2_plain.greedy_generate(cfg, weights, p, 12) for p in prompts]
-    assert any(len(set(w)) > 3 for w in want), "the continuation should not be one repeated token"
-    engine = _engine(folders["B"], block_size=8, num_blocks=24, max_num_seqs=3, chunk_size=7)
-    assert [g.tokens for g in engine.generate(prompts, max_new_tokens=12)] == want
+    want = [qwen2_plain.greedy_generate(cfg, weights, p, 24) for p in prompts]
+    assert all(len(set(w)) > 3 for w in want), "the continuation should not be one repeated token"
+    engine = _engine(folders[name], block_size=8, num_blocks=24, max_num_seqs=3, chunk_size=7)
+    assert [g.tokens for g in engine.generate(prompts, max_new_tokens=24)] == want
 
 
-def test_bfloat16_generation_runs_and_mostly_agrees(folders):
-    prompts = [random_tokens(CONFIG_A["vocab_size"], n, 40 + n) for n in (5, 8, 13)]
-    ref = _engine(folders["A"], num_blocks=12, max_num_seqs=4).generate(prompts, max_new_tokens=8)
-    got = _engine(folders["A"], dtype="bfloat16", num_blocks=12, max_num_seqs=4).generate(prompts, max_new_tokens=8)
-    assert all(len(g.tokens) == 8 for g in got)
-    assert sum(a.tokens[0] == b.tokens[0] for a, b in zip(ref, got)) >= 2
+@pytest.mark.parametrize("graphs", [False, True])
+def test_bfloat16_generation_follows_the_plain_implementation(folders, graphs):
+    """bfloat16 through the entry point, prompts in portions beside decoding requests: every generated token is
+    the plain implementation's best one (on the same bfloat16 weights) wherever that one's lead is clear."""
+    cfg, weights = qwen2_plain.load_folder(folders["B16"])
+    prompts = [random_tokens(CONFIG_B["vocab_size"], n, 80 + n) for n in (2, 37, 9, 21, 50)]
+    engine = _engine(folders["B16"], dtype="bfloat16", block_size=8, num_blocks=48, max_num_seqs=3, chunk_size=6,
+                     max_num_batched_tokens=11, use_graphs=graphs)
+    got = engine.generate(prompts, max_new_tokens=40)
+    checked = 0
+    for p, g in zip(prompts, got):
+        assert len(g.tokens) == 40 and len(set(g.tokens)) > 3
+        logits = qwen2_plain.forward(cfg, weights, p + g.tokens[:-1])
+        checked += assert_tokens_follow_plain(logits, len(p), g.tokens, 3e-2, f"prompt of {len(p)}")
+    assert checked > 100, "too few tokens had a clear lead to say anything"
+    assert engine.runner.cache.check() == "" and engine.runner.cache.live_requests() == 0
 
 
 def test_end_of_sequence_stops_and_is_kept_in_the_tokens(folders):
@@ -146,14 +160,7 @@ def test_long_decoding_follows_the_plain_implementation(folders):
     tokens = engine.generate([prompt], 240)[0].tokens
     assert len(tokens) == 240
     logits = qwen2_plain.forward(cfg, weights, prompt + tokens[:-1])
-    checked = 0
-    for k, token in enumerate(tokens):
-        row = logits[len(prompt) - 1 + k]
-        order = np.argsort(row)
-        if row[order[-1]] - row[order[-2]] > 1e-4 * np.max(np.abs(row)):
-            assert token == int(order[-1]), f"token {k} differs from the plain implementation"
-            checked += 1
-    assert checked > 200
+    assert assert_tokens_follow_plain(logits, len(prompt), tokens, 2.5e-5, "long decoding") > 200
 
 
 def test_captured_decode_steps_equal_eager_steps_on_every_replay(folders):
@@ -196,6 +203,37 @@ def test_captured_decode_steps_equal_eager_steps_on_every_replay(folders):
                 runner.step([StepEntry(3, 0, prompts[3], [20])])
             lengths[3] = 21
     assert runners[1].graphs.replays == 24 and len(runners[1].graphs.graphs) >= 2
+
+
+def test_a_captured_step_of_many_requests_rotates_by_the_positions_of_each_replay(folders):
+    """From 128 tokens on a step computes its sines and cosines once into a table: a captured step has to
+    compute it in every replay, from that replay's positions."""
+    from vipera_rs_amd.engine.batch import StepEntry
+    from vipera_rs_amd.engine.graphs import DecodeGraphs
+    from vipera_rs_amd.engine.runner import ModelRunner
+    vocab, live = CONFIG_B["vocab_size"], 130
+    runners = [ModelRunner.from_folder(folders["B16"], dtype="bfloat16", block_size=8, num_blocks=live * 4,
+                                       num_slots=live) for _ in range(2)]
+    runners[1].graphs = DecodeGraphs(runners[1], 256)
+    prompts = {r: random_tokens(vocab, 3 + r % 11, 900 + r) for r in range(live)}
+    for runner in runners:
+        for r, tokens in prompts.items():
+            runner.cache.reserve(r, 0, len(tokens))
+        runner.step([StepEntry(r, 0, tokens, []) for r, tokens in prompts.items()])
+    lengths = {r: len(tokens) for r, tokens in prompts.items()}
+    for step in range(6):
+        outs = []
+        for runner in runners:
+            entries = []
+            for r in prompts:
+                runner.cache.reserve(r, lengths[r], lengths[r] + 1)
+                entries.append(StepEntry(r, lengths[r], [(7 * r + 13 * step) % vocab], [0]))
+            outs.append(runner.step(entries).float().cpu())
+            torch.cuda.synchronize()
+        assert torch.equal(outs[0], outs[1]), f"replay {step} differs from the eager step"
+        for r in prompts:
+            lengths[r] += 1
+    assert runners[1].graphs.replays == 6 and list(runners[1].graphs.graphs) == [(192, 256)]
 
 
 # --- steps launched ahead of their tokens ---------------------------------------------------------------------------

@@ -1,6 +1,7 @@
 """The small kernels alone, each part of a layer alone, a run order that repeats a layer and shares a
 cache, and a toy mixer with state of its own that is registered, built and stepped from this file
 without any change to the package."""
+import contextlib
 import math
 from dataclasses import dataclass
 from typing import List
@@ -9,7 +10,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import CONFIG_A, CONFIG_B, make_folder, random_tokens, rel_err
+from helpers import CONFIG_A, CONFIG_B, assert_tokens_follow_plain, make_folder, random_tokens, rel_err
 from plain import qwen2_plain as P
 
 pytestmark = pytest.mark.gpu
@@ -307,17 +308,18 @@ def test_the_run_order_is_data(tmp_path):
 
 
 # --- a toy mixer with state of its own, defined here ----------------------------------------------------------------
-def test_a_stateful_toy_mixer_is_registered_built_and_stepped(tmp_path):
-    """``s_t = decay * s_{t-1} + W_in h_t``, ``y_t = W_out s_t``: one vector of state per request, no pages.
-    Layer 0 uses it, layer 1 is ordinary attention: different mixers in different layers of one model."""
+STATE_DECAY, STATE_WIDTH = 0.9, 24
+
+
+@contextlib.contextmanager
+def _stateful_toy():
+    """Registers ``s_t = decay * s_{t-1} + W_in h_t``, ``y_t = W_out s_t`` (one vector of state per request, no
+    pages) as the mixer of layer 0 of a toy architecture whose layer 1 is ordinary attention: different mixers
+    in different layers of one model.  Yields the plain implementation of that model."""
     from vipera_rs_amd.config import (LayerSpec, PartSpec, Qwen2Config, register_architecture, unregister_architecture)
-    from vipera_rs_amd.engine.batch import StepEntry
-    from vipera_rs_amd.engine.runner import ModelRunner
     from vipera_rs_amd.models.decoder import DecoderModel
     from vipera_rs_amd.parts import Mixer, StateSpec, register_mixer, unregister
     from vipera_rs_amd.weights import MATRIX, TensorSpec
-
-    DECAY, WIDTH = 0.9, 24
 
     class RunningState(Mixer):
         def __init__(self, spec, prefix, runtime):
@@ -328,23 +330,32 @@ def test_a_stateful_toy_mixer_is_registered_built_and_stepped(tmp_path):
         @classmethod
         def declare(cls, spec, prefix):
             base = f"{prefix}{spec.params['name']}."
-            return [TensorSpec(base + "in.weight", (WIDTH, spec.params["hidden"]), MATRIX, std=0.3),
-                    TensorSpec(base + "out.weight", (spec.params["hidden"], WIDTH), MATRIX, std=0.3)]
+            return [TensorSpec(base + "in.weight", (STATE_WIDTH, spec.params["hidden"]), MATRIX, std=0.3),
+                    TensorSpec(base + "out.weight", (spec.params["hidden"], STATE_WIDTH), MATRIX, std=0.3)]
 
         def load(self, tensors):
             base = f"{self.prefix}{self.spec.params['name']}."
             self.w_in, self.w_out = tensors[base + "in.weight"].float(), tensors[base + "out.weight"].float()
 
-        def state_spec(self):
-            return StateSpec((WIDTH,), torch.float32)
+        @classmethod
+        def declare_cache(cls, spec):
+            return None, StateSpec((STATE_WIDTH,), torch.float32)
 
         def forward(self, h, batch, cache, state, position, residual, reads_only=False):
             u = h.float() @ self.w_in.T
+            if batch.all_single:
+                # one token per entry: only what lies on the device is looked at, so the step can be captured
+                slots = batch.slots.long()
+                fresh = (batch.entry_first_pos == 0).unsqueeze(1)                      # zero on first use
+                s = STATE_DECAY * torch.where(fresh, torch.zeros_like(u), state.index_select(0, slots)) + u
+                residual += s @ self.w_out.T
+                state.index_copy_(0, slots, s)
+                return
             at = 0
             for count, first, slot in zip(batch.host_counts, batch.host_first_pos, batch.host_slots):
-                s = torch.zeros(WIDTH, device=h.device) if first == 0 else state[slot].clone()   # zero on first use
+                s = torch.zeros(STATE_WIDTH, device=h.device) if first == 0 else state[slot].clone()
                 for t in range(at, at + count):
-                    s = DECAY * s + u[t]
+                    s = STATE_DECAY * s + u[t]
                     residual[t] += s @ self.w_out.T
                 state[slot] = s
                 at += count
@@ -363,9 +374,9 @@ def test_a_stateful_toy_mixer_is_registered_built_and_stepped(tmp_path):
         cfg = P.normalize_config(cfg)
         x = w["model.embed_tokens.weight"][np.asarray(tokens)]
         h = P.rms_norm(x, w["model.layers.0.input_layernorm.weight"], cfg["rms_norm_eps"])
-        s, ys = np.zeros(WIDTH), []
+        s, ys = np.zeros(STATE_WIDTH), []
         for t in range(len(tokens)):
-            s = DECAY * s + w["model.layers.0.state.in.weight"] @ h[t]
+            s = STATE_DECAY * s + w["model.layers.0.state.in.weight"] @ h[t]
             ys.append(w["model.layers.0.state.out.weight"] @ s)
         x = x + np.stack(ys)
         h = P.rms_norm(x, w["model.layers.0.post_attention_layernorm.weight"], cfg["rms_norm_eps"])
@@ -374,16 +385,29 @@ def test_a_stateful_toy_mixer_is_registered_built_and_stepped(tmp_path):
         x = x + P.attention_block(h, w, "model.layers.1.self_attn.", cfg, 0)
         h = P.rms_norm(x, w["model.layers.1.post_attention_layernorm.weight"], cfg["rms_norm_eps"])
         x = x + P.swiglu_mlp(h, *(w[f"model.layers.1.mlp.{n}_proj.weight"] for n in ("gate", "up", "down")))
-        return P.linear(P.rms_norm(x, w["model.norm.weight"], cfg["rms_norm_eps"]), w["model.embed_tokens.weight"])
+        head = w["lm_head.weight"] if "lm_head.weight" in w else w["model.embed_tokens.weight"]
+        return P.linear(P.rms_norm(x, w["model.norm.weight"], cfg["rms_norm_eps"]), head)
 
     register_mixer("running_state", RunningState)
     register_architecture("ToyStateForCausalLM", ToyConfig, lambda config, runtime: DecoderModel(config, runtime))
     try:
+        yield plain
+    finally:
+        unregister_architecture("ToyStateForCausalLM")
+        unregister("mixer", "running_state")
+
+
+def test_a_stateful_toy_mixer_is_registered_built_and_stepped(tmp_path):
+    from vipera_rs_amd.engine.batch import StepEntry
+    from vipera_rs_amd.engine.runner import ModelRunner
+
+    with _stateful_toy() as plain:
         folder = make_folder(tmp_path / "toy", dict(CONFIG_A, architectures=["ToyStateForCausalLM"]), 6)
         cfg, w = P.load_folder(folder)
         assert "model.layers.0.state.in.weight" in w and "model.layers.0.self_attn.q_proj.weight" not in w
         runner = ModelRunner.from_folder(folder, dtype="float32", block_size=8, num_blocks=24, num_slots=3)
-        assert runner.storage.state[0].shape == (3, WIDTH) and runner.storage.kv[0] is None
+        # a row per slot and the scratch row of a captured step's padding entries
+        assert runner.storage.state[0].shape == (3 + 1, STATE_WIDTH) and runner.storage.kv[0] is None
         assert runner.storage.kv[1] is not None and runner.storage.state[1] is None
         requests = {0: random_tokens(256, 23, 1), 1: random_tokens(256, 17, 2), 2: random_tokens(256, 9, 3)}
         want = {r: plain(cfg, w, toks) for r, toks in requests.items()}
@@ -405,9 +429,35 @@ def test_a_stateful_toy_mixer_is_registered_built_and_stepped(tmp_path):
                 if at[r] == len(requests[r]):
                     runner.cache.release(r)
         assert at == {r: len(t) for r, t in requests.items()} and runner.cache.check() == ""
-    finally:
-        unregister_architecture("ToyStateForCausalLM")
-        unregister("mixer", "running_state")
+
+
+def test_a_stateful_toy_mixer_generates_through_captured_steps_with_padding(tmp_path):
+    """Three live requests decode in a captured step of four entries.  The padding entry writes the scratch
+    state row and not slot 0, which a live request holds, and the first use of a graph runs a step once: either
+    fault would change a request's state and, from there on, its tokens."""
+    from vipera_rs_amd import Engine
+    from vipera_rs_amd.cli import plan_model
+
+    with _stateful_toy() as plain:
+        config = dict(CONFIG_A, architectures=["ToyStateForCausalLM"], tie_word_embeddings=False)
+        folder = make_folder(tmp_path / "toy", config, 8)
+        cfg, w = P.load_folder(folder)
+        prompts = [random_tokens(256, n, 50 + n) for n in (7, 12, 3)]
+        engine = Engine(folder, dtype="float32", block_size=8, num_blocks=24, max_num_seqs=3, use_graphs=True)
+        got = engine.generate(prompts, max_new_tokens=20)
+        graphs = engine.runner.graphs
+        assert graphs.replays >= 19 and any(bucket == 4 for bucket, _ in graphs.graphs), "no padded captured step ran"
+        assert engine.runner.storage.scratch_slot == 3
+        checked = 0
+        for p, g in zip(prompts, got):
+            assert len(g.tokens) == 20
+            logits = plain(cfg, w, p + g.tokens[:-1])
+            checked += assert_tokens_follow_plain(logits, len(p), g.tokens, 2.5e-5, f"prompt of {len(p)}")
+        assert checked > 40
+        # the state's bytes are part of the memory plan: one row per request and the scratch row
+        planned = plan_model(folder, 64, 3, "float32", 8)
+        assert planned["state_bytes"] == (3 + 1) * STATE_WIDTH * 4
+        assert engine.stats()["kv_bytes"] == engine.runner.storage.bytes >= planned["state_bytes"]
 
 
 # --- a feed-forward with routing and another position encoding, defined here --------------------------------------

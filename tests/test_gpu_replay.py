@@ -20,7 +20,7 @@ TOL = {"float32": 1e-4, "bfloat16": 3e-2}
 LENGTHS = [70, 33, 5, 49, 91, 18, 64]
 
 
-@pytest.fixture(scope="module", params=["A", "B", "C"])
+@pytest.fixture(scope="module", params=["A", "B", "C", "D"])
 def case(request, tmp_path_factory):
     name = request.param
     config, seed = CONFIGS[name]

@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import CONFIG_A, CONFIG_B, make_folder
+from helpers import CONFIG_A, CONFIG_B, CONFIG_D, make_folder
 from plain import qwen2_plain as P
 from plain import sampler_plain as S
 
@@ -160,10 +160,12 @@ def test_a_prefix_never_depends_on_what_follows(model_b):
     tokens = [4, 8, 15, 16, 23, 42, 108, 299, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16, 17, 18, 19, 20]
     whole = P.forward(c, w, tokens)
     np.testing.assert_allclose(P.forward(c, w, tokens[:10]), whole[:10], rtol=1e-9, atol=1e-12)
-    # the windowed layers (21 positions) matter: beyond the window the logits differ from full attention
-    full = P.forward(dict(c, use_sliding_window=False), w, tokens)
-    np.testing.assert_allclose(full[:21], whole[:21], rtol=1e-9, atol=1e-12)
-    assert np.max(np.abs(full[27] - whole[27])) > 1e-6
+    # with windowed layers (21 positions, the fourth configuration's option) the logits beyond the window differ
+    # from full attention, and not before
+    windowed = P.forward(dict(c, **{k: CONFIG_D[k] for k in ("use_sliding_window", "sliding_window",
+                                                             "max_window_layers")}), w, tokens)
+    np.testing.assert_allclose(windowed[:21], whole[:21], rtol=1e-9, atol=1e-12)
+    assert np.max(np.abs(windowed[27] - whole[27])) > 1e-6
 
 
 def test_float32_arithmetic_stays_close_to_float64(model_b):

@@ -233,7 +233,7 @@ def _forward_through_twins(cfg, w, tokens, bs=8):
     return logits.numpy()
 
 
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_a_whole_model_through_the_twins_equals_the_python_plain_implementation(name, tmp_path):
     config, seed = CONFIGS[name]
     cfg, w = P.load_folder(make_folder(tmp_path / name, config, seed))

@@ -4,7 +4,9 @@ Layout of the paged tensors: keys ``[pages + 1, kv_heads, block_size, head_dim]`
 ``[pages + 1, kv_heads, head_dim, block_size]`` (the attention kernels read consecutive positions of
 one output dim); the last page is a scratch page that is never handed out, which padding tokens of
 a captured step write to.  A state
-tensor is ``[slots, *shape]``.
+tensor is ``[slots + 1, *shape]``: the last row is the scratch row of those padding entries
+(``CacheStorage.scratch_slot``), so that a mixer that keeps state never sees a padding entry in a live
+request's row.
 """
 from __future__ import annotations
 
@@ -40,6 +42,7 @@ class CacheStorage:
         self.state: List[Optional[torch.Tensor]] = [None] * len(needs)
         self.groups = list(groups)
         self.bytes = 0
+        self.scratch_slot = num_slots
         for index, need in enumerate(needs):
             if need.owner != index:
                 continue
@@ -49,11 +52,11 @@ class CacheStorage:
                     raise InvalidArgumentError(f"no cache group keeps a window of {need.kv.window}")
                 spec = self.groups[group]
                 k = runtime.zeros((spec.num_blocks + 1, need.kv.kv_heads, spec.block_size, need.kv.head_dim))
-                v = runtime.zeros((spec.num_blocks + 1, need.kv.kv_heads, need.kv.head_dim, spec.block_size))
+                v = runtime.zeros((spec.num_blocks + 1, need.kv.kv_heads, need.kv.value_width, spec.block_size))
                 self.kv[index] = PagedKV(k, v, group, spec.block_size)
-                self.bytes += 2 * k.numel() * k.element_size()
+                self.bytes += (k.numel() + v.numel()) * k.element_size()
             if need.state is not None:
-                tensor = torch.zeros((num_slots,) + tuple(need.state.shape), dtype=need.state.dtype,
+                tensor = torch.zeros((num_slots + 1,) + tuple(need.state.shape), dtype=need.state.dtype,
                                      device=runtime.device)
                 self.state[index] = tensor
                 self.bytes += tensor.numel() * tensor.element_size()
@@ -68,5 +71,19 @@ class CacheStorage:
         for entry in self.kv:
             if entry is not None and id(entry) not in seen:
                 seen.add(id(entry))
-                total += 2 * entry.k.shape[1] * entry.k.shape[3] * entry.k.element_size()
+                total += entry.k.shape[1] * (entry.k.shape[3] + entry.v.shape[2]) * entry.k.element_size()
         return total
+
+
+def cache_bytes(needs, element: int):
+    """``(bytes per cached position, bytes per state slot)`` over the entries of ``needs`` that own their
+    storage; ``element`` is the size of a cached key or value."""
+    per_position = per_slot = 0
+    for index, need in enumerate(needs):
+        if need.owner != index:
+            continue
+        if need.kv is not None:
+            per_position += need.kv.bytes_per_position(element)
+        if need.state is not None:
+            per_slot += need.state.bytes_per_slot()
+    return per_position, per_slot

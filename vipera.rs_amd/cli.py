@@ -181,8 +181,9 @@ def plan_model(folder: str, ctx: Optional[int], batch: int, dtype: str, block_si
     The cache costs ``2 * kv_heads * head_dim * bytes`` per position and attention layer, the
     reference's arithmetic (crates/vipera-core/src/planner.rs:191-206).
     """
+    from .cache import cache_bytes
     from .config.registry import load_config
-    from .models import declare_model
+    from .models import declare_cache_needs, declare_model
     from .weights.checkpoint import MATRIX
 
     config = load_config(folder)
@@ -208,24 +209,21 @@ def plan_model(folder: str, ctx: Optional[int], batch: int, dtype: str, block_si
     embedding_elements = int(emb["vocab"]) * int(emb["width"])
     tied = bool(config.head_spec().params.get("tied_to"))
     head_elements = embedding_elements
-    kv_per_token = 0
-    for layer in config.layer_specs():
-        p = layer.mixer.params
-        if "kv_heads" in p:
-            kv_per_token += 2 * int(p["kv_heads"]) * int(p["head_dim"]) * element
+    kv_per_token, state_per_slot = cache_bytes(declare_cache_needs(config), element)
     blocks = batch * ((ctx + block_size - 1) // block_size)
     kv_bytes = blocks * block_size * kv_per_token
+    state_bytes = (batch + 1) * state_per_slot      # one row per request and the scratch row of padding entries
     workspace = 2048 * (int(emb["width"]) * 4 + int(emb["vocab"]) * 4) + 256 * 1024 * 1024
-    total = weight_bytes + kv_bytes + workspace + DEVICE_RESERVE
+    total = weight_bytes + kv_bytes + state_bytes + workspace + DEVICE_RESERVE
     # a decode step reads every matrix once (the embedding table only when it is also the head)
     step_weights = (matrix_elements - (0 if tied else embedding_elements)) * element
     linear_elements = matrix_elements - embedding_elements - (0 if tied else head_elements)
     plan = {
         "dtype": dtype, "context": ctx, "batch": batch, "block_size": block_size,
         "weight_bytes": weight_bytes, "kv_bytes_per_token": kv_per_token, "kv_blocks": blocks,
-        "kv_bytes": kv_bytes, "workspace_bytes": workspace, "reserve_bytes": DEVICE_RESERVE,
+        "kv_bytes": kv_bytes, "state_bytes": state_bytes, "workspace_bytes": workspace, "reserve_bytes": DEVICE_RESERVE,
         "required_bytes": total, "available_bytes": HBM_BYTES,
-        "decode_step_read_bytes": step_weights + batch * ctx * kv_per_token,
+        "decode_step_read_bytes": step_weights + batch * (ctx * kv_per_token + state_per_slot),
         "prefill_flops_per_token_linear": 2 * linear_elements,
         "feasible": total <= HBM_BYTES, "violations": [],
     }

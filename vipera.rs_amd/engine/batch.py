@@ -86,17 +86,19 @@ class PackedStep:
 
 
 def pack_entries(entries: Sequence[StepEntry], cache, vocab_size: int, min_table_width: int = 1,
-                 pad_entries: int = 0, pad_page: int = -1) -> PackedStep:
+                 pad_entries: int = 0, pad_page: int = -1, pad_slot: int = 0) -> PackedStep:
     """Check ``entries`` and lay them out for the device.
 
     The pages of every token must already be reserved in ``cache``.  ``pad_entries`` appends
-    single-token dummy entries (token 0 at position 0, every table entry ``pad_page``), which a
-    captured graph of a fixed batch size needs; their logits are computed and ignored.
+    single-token dummy entries (token 0 at position 0, every table entry ``pad_page``, state slot
+    ``pad_slot``), which a captured graph of a fixed batch size needs; their logits are computed and
+    ignored, and what they write goes to the scratch page and the scratch state row, which belong to
+    no request.  A step of padding only (no ``entries``) is what a graph is warmed up and captured on.
     """
-    if not entries:
+    if not entries and pad_entries < 1:
         raise InvalidArgumentError("a step needs at least one entry")
     counts = [len(e.tokens) for e in entries]
-    if min(counts) < 1:
+    if counts and min(counts) < 1:
         raise InvalidArgumentError("every entry of a step needs at least one token")
     seen = set()
     for e in entries:
@@ -106,14 +108,14 @@ def pack_entries(entries: Sequence[StepEntry], cache, vocab_size: int, min_table
     real = len(entries)
     T_real = sum(counts)
     flat = np.fromiter((t for e in entries for t in e.tokens), dtype=np.int64, count=T_real)
-    if flat.min() < 0 or flat.max() >= vocab_size:
+    if T_real and (flat.min() < 0 or flat.max() >= vocab_size):
         bad = int(flat[(flat < 0) | (flat >= vocab_size)][0])
         raise InvalidArgumentError(f"token {bad} is outside the vocabulary of {vocab_size}")
     first_real = [int(e.start) for e in entries]
-    if min(first_real) < 0:
+    if first_real and min(first_real) < 0:
         raise InvalidArgumentError("an entry starts at a negative position")
     slots_real = [cache.slot(e.request) for e in entries]
-    if min(slots_real) < 0:
+    if slots_real and min(slots_real) < 0:
         missing = entries[int(np.argmin(slots_real))].request
         raise InternalError(f"request {missing} has no slot: nothing was reserved for it")
 
@@ -128,7 +130,7 @@ def pack_entries(entries: Sequence[StepEntry], cache, vocab_size: int, min_table
     kv_len = first + np.array(counts_all, dtype=np.int32)
     entry_of = np.repeat(np.arange(E, dtype=np.int32), counts_all)
     positions = np.arange(T, dtype=np.int32) - starts[entry_of] + first[entry_of]
-    slots = np.array(slots_real + [0] * pad_entries, dtype=np.int32)
+    slots = np.array(slots_real + [pad_slot] * pad_entries, dtype=np.int32)
     rows: List[int] = []
     for k, e in enumerate(entries):
         for w in e.want:
@@ -165,7 +167,7 @@ def pack_entries(entries: Sequence[StepEntry], cache, vocab_size: int, min_table
             need_from = [max(0, e.start + 1 - spec.window) // spec.block_size for e in entries]
         else:
             need_from = [0] * real
-        failed = cache.fill_tables(requests, g, table, need_from, need_to)
+        failed = cache.fill_tables(requests, g, table, need_from, need_to) if real else -1
         if failed >= 0:
             e = entries[failed]
             lo = max(0, e.start + 1 - spec.window) if spec.window > 0 else 0

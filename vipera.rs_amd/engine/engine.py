@@ -142,28 +142,24 @@ class Engine:
 
     @staticmethod
     def _load(folder, config, runtime, block_size, num_blocks, num_slots, use_graphs, max_context) -> ModelRunner:
-        from ..models import build_model
-        from ..weights import Checkpoint, load_tensors
+        from ..cache import cache_bytes
 
-        model = build_model(config, runtime)
-        checkpoint = Checkpoint(folder)
-        try:
-            tensors = load_tensors(checkpoint, model.tensor_specs(), runtime.dtype, runtime.device)
-        finally:
-            checkpoint.close()
-        model.load(tensors)
+        model = ModelRunner.load_model(folder, config, runtime)
         free, _ = torch.cuda.mem_get_info(runtime.device)
-        needs = model.cache_needs()
-        element = 4 if runtime.dtype == torch.float32 else 2
-        per_page = sum(2 * n.kv.kv_heads * n.kv.head_dim * block_size * element
-                       for i, n in enumerate(needs) if n.kv is not None and n.owner == i)
-        if per_page and num_blocks * per_page > 0.9 * free:
-            fit = int(0.9 * free // per_page)
+        num_slots = max(num_slots, 1)
+        per_position, per_slot = cache_bytes(model.cache_needs(), 4 if runtime.dtype == torch.float32 else 2)
+        per_page = per_position * block_size
+        room = 0.9 * free - per_slot * (num_slots + 1)       # fixed-size state first: one row per slot and a scratch row
+        if room < 0:
+            raise InfeasibleError(
+                f"no room for {num_slots} state slots of {per_slot} bytes in {free} free bytes of device memory")
+        if per_page and num_blocks * per_page > room:
+            fit = int(room // per_page)
             if fit < 1:
                 raise InfeasibleError(
                     f"no room for a single cache page of {per_page} bytes in {free} free bytes of device memory")
             num_blocks = fit
-        return ModelRunner(model, runtime, block_size, num_blocks, max(num_slots, 1), use_graphs, max_context)
+        return ModelRunner(model, runtime, block_size, num_blocks, num_slots, use_graphs, max_context)
 
     # --- requests ---------------------------------------------------------------------------------
     def add_request(self, prompt: Sequence[int], max_new_tokens: int = 32,

@@ -4,6 +4,10 @@ A decode step launches a few hundred small kernels; launched one by one from Pyt
 slower than the GPU.  A graph of the step is captured once per (padded batch size, context bucket)
 and replayed with new metadata copied into its standing buffers.  The kernels, their order and their
 arithmetic are those of the eager step.  Nothing that clears memory is recorded into a graph.
+
+A graph is warmed up and captured on a step of padding entries only (token 0 at position 0 on the scratch
+page and the scratch state row), so that a real step runs exactly once, as the graph's first replay: a
+mixer that keeps state advances it once.
 """
 from __future__ import annotations
 
@@ -54,7 +58,8 @@ class DecodeGraphs:
         cache = self.runner.cache
         width = max((context_bucket + g.block_size - 1) // g.block_size for g in cache.groups) if cache.groups else 1
         packed = pack_entries(entries, cache, self.runner.vocab_size, min_table_width=width,
-                              pad_entries=batch_bucket - len(entries), pad_page=self.runner.num_blocks)
+                              pad_entries=batch_bucket - len(entries), pad_page=self.runner.num_blocks,
+                              pad_slot=self.runner.storage.scratch_slot)
         # every row's logits are computed; the caller picks the wanted ones
         packed.sections[7] = np.arange(batch_bucket, dtype=np.int32)
         packed.num_logit_rows = batch_bucket
@@ -78,9 +83,10 @@ class DecodeGraphs:
             # the step before may still be waiting in the stream when the next step is packed
             staging = [torch.empty(flat.size, dtype=torch.int32).pin_memory() for _ in range(2)]
             buffer = torch.empty(flat.size, dtype=torch.int32, device=device)
-            staging[0].numpy()[:] = flat
+            padding = self._pack([], batch_bucket, context_bucket)
+            staging[0].numpy()[:] = padding.flat()
             buffer.copy_(staging[0], non_blocking=True)
-            batch = batch_from_buffer(packed, buffer)
+            batch = batch_from_buffer(padding, buffer)
             batch.sampled_tokens = runner.sampled_tokens
             # an eager run first: it loads every kernel module the step needs, outside of the capture
             runner.model.forward(batch, runner.storage)
@@ -103,11 +109,10 @@ class DecodeGraphs:
                 self.pool = graph.pool()
             captured = _Captured(graph, buffer, staging, batch, logits)
             self.graphs[key] = captured
-        else:
-            captured.turn ^= 1
-            staging = captured.staging[captured.turn]
-            staging.numpy()[:] = flat
-            captured.buffer.copy_(staging, non_blocking=True)
+        captured.turn ^= 1
+        staging = captured.staging[captured.turn]
+        staging.numpy()[:] = flat
+        captured.buffer.copy_(staging, non_blocking=True)
         captured.graph.replay()
         self.replays += 1
         rows = [k for k, e in enumerate(entries) if len(e.want)]

@@ -52,11 +52,9 @@ class ModelRunner:
             self.graphs = DecodeGraphs(self, max_context or block_size * num_blocks)
 
     # --- construction helpers -----------------------------------------------------------------
-    @classmethod
-    def from_folder(cls, folder: str, dtype="bfloat16", device="cuda:0", block_size: int = 16,
-                    num_blocks: int = 256, num_slots: int = 8, progress=None) -> "ModelRunner":
-        runtime = Runtime(device, dtype)
-        config = load_config(folder)
+    @staticmethod
+    def load_model(folder: str, config: ModelConfig, runtime: Runtime, progress=None):
+        """The model of ``config`` with the weights of ``folder`` on the runtime's device."""
         model = build_model(config, runtime)
         checkpoint = Checkpoint(folder)
         try:
@@ -64,7 +62,15 @@ class ModelRunner:
         finally:
             checkpoint.close()
         model.load(tensors)
-        return cls(model, runtime, block_size, num_blocks, num_slots)
+        return model
+
+    @classmethod
+    def from_folder(cls, folder: str, dtype="bfloat16", device="cuda:0", block_size: int = 16,
+                    num_blocks: int = 256, num_slots: int = 8, progress=None, use_graphs: bool = False,
+                    max_context: int = 0) -> "ModelRunner":
+        runtime = Runtime(device, dtype)
+        model = cls.load_model(folder, load_config(folder), runtime, progress)
+        return cls(model, runtime, block_size, num_blocks, num_slots, use_graphs, max_context)
 
     # --- the step ---------------------------------------------------------------------------------
     def prepare(self, entries: Sequence[StepEntry]) -> StepBatch:

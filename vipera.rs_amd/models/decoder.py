@@ -62,6 +62,19 @@ def declare_model(config: ModelConfig) -> List[TensorSpec]:
     return specs
 
 
+def declare_cache_needs(config: ModelConfig) -> List[CacheNeed]:
+    """What every entry of ``config``'s run order keeps per request, from the configuration alone. Touches no GPU."""
+    layers = config.layer_specs()
+    schedule = list(config.schedule())
+    check_schedule(schedule, len(layers))
+    needs = []
+    for index, entry in enumerate(schedule):
+        mixer = layers[entry.layer].mixer
+        kv, state = part_class("mixer", mixer.kind).declare_cache(mixer)
+        needs.append(CacheNeed(index if entry.cache_of is None else entry.cache_of, kv, state))
+    return needs
+
+
 class DecoderModel:
     def __init__(self, config: ModelConfig, runtime):
         self.config = config
@@ -101,6 +114,9 @@ class DecoderModel:
 
     def forward(self, batch, storage) -> Optional[torch.Tensor]:
         """Run the step's tokens through the run order; returns ``[wanted rows, vocab]`` 32-bit logits."""
+        # what parts share within a step is computed anew in every run: a run that is being captured into a graph
+        # must launch it too, or the graph would replay with what an earlier run left
+        batch.shared.clear()
         if batch.sampled_tokens is not None and batch.token_source is not None:  # ids the sampler left on the device
             x = self.embedding.forward(batch.tokens, batch.num_tokens, batch.token_source, batch.sampled_tokens)
         else:

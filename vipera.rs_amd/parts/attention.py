@@ -73,8 +73,10 @@ class Attention(Mixer):
         if self.out_bias:
             self.b_o = tensors[base + "o_proj.bias"]
 
-    def cache_spec(self) -> Optional[KVCacheSpec]:
-        return KVCacheSpec(self.kv_heads, self.head_dim, self.window)
+    @classmethod
+    def declare_cache(cls, spec: PartSpec):
+        p = spec.params
+        return KVCacheSpec(int(p["kv_heads"]), int(p["head_dim"]), int(p.get("window") or 0)), None
 
     fills_handoff = True
 

@@ -14,7 +14,7 @@ Kinds of parts and what each must provide:
 ``PositionEncoding``  ``apply(qkv, batch, heads, kv_heads, head_dim)`` rotates (or otherwise marks)
                       the q and k heads of the fused buffer in place; ``fused_rotary()`` may return
                       ``(inv_freq, rotary_dim)`` to let a mixer fold the rotation into its cache write.
-``Mixer``             ``cache_spec()`` / ``state_spec()`` say what it keeps per request;
+``Mixer``             ``declare_cache(spec)`` says what it keeps per request (pages, state);
                       ``forward(h, batch, cache, state, position, residual, reads_only)`` adds its
                       output to ``residual`` (32-bit, in place).
 ``FeedForward``       ``forward(h, batch, residual)`` adds its output to ``residual``.
@@ -34,11 +34,20 @@ from ..weights.checkpoint import TensorSpec
 
 @dataclass(frozen=True)
 class KVCacheSpec:
-    """Keys and values in pages: per position ``kv_heads * head_dim`` of each; ``window`` 0 keeps all."""
+    """Keys and values in pages: per position ``kv_heads * head_dim`` keys and ``kv_heads * value_dim``
+    values (``value_dim`` 0: as wide as the keys); ``window`` 0 keeps all."""
 
     kv_heads: int
     head_dim: int
     window: int = 0
+    value_dim: int = 0
+
+    @property
+    def value_width(self) -> int:
+        return self.value_dim or self.head_dim
+
+    def bytes_per_position(self, element: int) -> int:
+        return self.kv_heads * (self.head_dim + self.value_width) * element
 
 
 @dataclass(frozen=True)
@@ -47,6 +56,12 @@ class StateSpec:
 
     shape: Tuple[int, ...]
     dtype: torch.dtype = torch.float32
+
+    def bytes_per_slot(self) -> int:
+        count = 1
+        for dim in self.shape:
+            count *= int(dim)
+        return count * torch.empty(0, dtype=self.dtype).element_size()
 
 
 class Part:
@@ -104,11 +119,17 @@ class PositionEncoding(Part):
 
 
 class Mixer(Part):
+    @classmethod
+    def declare_cache(cls, spec: PartSpec) -> Tuple[Optional[KVCacheSpec], Optional[StateSpec]]:
+        """What a mixer of ``spec`` keeps per request: pages of keys and values, state of fixed size, both or
+        neither.  From the spec alone, so that memory can be planned before anything is built."""
+        return None, None
+
     def cache_spec(self) -> Optional[KVCacheSpec]:
-        return None
+        return type(self).declare_cache(self.spec)[0]
 
     def state_spec(self) -> Optional[StateSpec]:
-        return None
+        return type(self).declare_cache(self.spec)[1]
 
     #: a mixer that sets this takes ``handoff=`` in ``forward`` and may fill it (see :class:`NormHandoff`)
     fills_handoff = False
