@@ -32,7 +32,10 @@
 // Reference for what is computed: crates/vipera-backend-cpu/src/model.rs:1005-1031 (batched products,
 // bias after the product); the idea of reading a weight row once for many tokens is that of the
 // reference's batched matvec (crates/vipera-backend-gpu/src/q4k_matvec_q8_batch.cu:40-116).
+#include <mutex>
+
 #include "common.h"
+#include "no_alloc.h"
 #include "pipeline.h"
 
 // Depth of the load pipelines of the weight-streaming kernels: register sets of operands, one being
@@ -1671,9 +1674,9 @@ extern "C" int vk_gemm_bf16(const void* A, const void* W, const float* bias, voi
 // workgroups: partial sums go to `partial` (at least ranges * M * N floats) and a second kernel adds them.
 // rows_per_wave: 1 or 2 tiles of 16 weight rows per wave; with 1 the launcher may give a wave fewer than 16 rows
 // (balanced_rows), and 108 to 116 force one tile with 8 to 16 rows.
-extern "C" int vk_gemm_bf16_mid(const void* A, const void* W, const float* bias, void* C, int c_dtype, int M, int N,
-                                int K, long long lda, long long ldc, int accumulate, int ranges, int rows_per_wave,
-                                float* partial, long long partial_floats, void* stream) {
+static int gemm_mid_checked(const void* A, const void* W, const float* bias, void* C, int c_dtype, int M, int N, int K,
+                            long long lda, long long ldc, int accumulate, int ranges, int rows_per_wave,
+                            float* partial, long long partial_floats, void* stream) {
   if (M <= 0 || N <= 0) return 0;
   if (M > 64) return VK_UNSUPPORTED_SIZE;
   if (K <= 0 || (K & 7) || (lda & 7) || lda < K || ldc < N || ranges < 1) return VK_BAD_ARGUMENT;
@@ -1694,6 +1697,57 @@ extern "C" int vk_gemm_bf16_mid(const void* A, const void* W, const float* bias,
   if (c_dtype == DT_BF16)
     return launch_mid<__bf16, false>(a, w, bias, (__bf16*)C, partial, partial_floats, ranges, rows_per_wave, M, N, K, lda, ldc, vector_ok, s);
   return VK_BAD_ARGUMENT;
+}
+
+extern "C" int vk_gemm_bf16_mid(const void* A, const void* W, const float* bias, void* C, int c_dtype, int M, int N,
+                                int K, long long lda, long long ldc, int accumulate, int ranges, int rows_per_wave,
+                                float* partial, long long partial_floats, void* stream) {
+  return gemm_mid_checked(A, W, bias, C, c_dtype, M, N, K, lda, ldc, accumulate, ranges, rows_per_wave, partial,
+                          partial_floats, stream);
+}
+
+// --- the split-K product without a workspace argument (declared in no_alloc.h) ---------------------------------
+// The partial sums of the K ranges live in this array, which every GPU that loads the library holds at an
+// address of its own until the process ends. In host code the array's name stands for the symbol, not for device
+// memory: its address on the current device is asked for once per device and only that pointer is ever used.
+static __device__ __align__(256) float scratch[VK_NO_ALLOC_SCRATCH_FLOATS];
+
+namespace {
+constexpr int NO_ALLOC_MAX_DEVICES = 64;
+float* g_scratch_of_device[NO_ALLOC_MAX_DEVICES] = {};
+std::mutex g_scratch_lock;
+
+// The array's address on the current device; nullptr and `*status` set when it cannot be had.
+float* scratch_of_current_device(int* status) {
+  int device = -1;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) { *status = (int)e; return nullptr; }
+  if (device < 0 || device >= NO_ALLOC_MAX_DEVICES) { *status = VK_UNSUPPORTED_SIZE; return nullptr; }
+  std::lock_guard<std::mutex> hold(g_scratch_lock);
+  if (!g_scratch_of_device[device]) {
+    float* address = nullptr;
+    e = hipGetSymbolAddress((void**)&address, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !address) { *status = e != hipSuccess ? (int)e : VK_BAD_ARGUMENT; return nullptr; }
+    g_scratch_of_device[device] = address;
+  }
+  return g_scratch_of_device[device];
+}
+}  // namespace
+
+extern "C" long long vk_gemm_bf16_mid_no_alloc_capacity() { return VK_NO_ALLOC_SCRATCH_FLOATS; }
+
+extern "C" int vk_gemm_bf16_mid_no_alloc(const void* A, const void* W, const float* bias, void* C, int c_dtype, int M,
+                                         int N, int K, long long lda, long long ldc, int accumulate, int ranges,
+                                         int rows_per_wave, void* stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (ranges < 1) return VK_BAD_ARGUMENT;
+  // every range writes all of its M x N sums before the second kernel reads them, so nothing has to be cleared
+  if (ranges > 1 && (long long)ranges * M * N > VK_NO_ALLOC_SCRATCH_FLOATS) return VK_UNSUPPORTED_SIZE;
+  int status = 0;
+  float* partial = scratch_of_current_device(&status);
+  if (!partial) return status;
+  return gemm_mid_checked(A, W, bias, C, c_dtype, M, N, K, lda, ldc, accumulate, ranges, rows_per_wave, partial,
+                          VK_NO_ALLOC_SCRATCH_FLOATS, stream);
 }
 
 // out[M, N / 2] = up * silu(gate) of the product with a fused gate/up weight W[N, K] whose rows are

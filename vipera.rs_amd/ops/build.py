@@ -33,7 +33,7 @@ MODULES: Dict[str, tuple] = {
     "elementwise": ("hip", ["kernels/elementwise.hip"], ["kernels/common.h"]),
     "gemm_generic": ("hip", ["kernels/gemm_generic.hip"], ["kernels/common.h"]),
     "attn_generic": ("hip", ["kernels/attn_generic.hip"], ["kernels/common.h"]),
-    "gemm_bf16": ("hip", ["kernels/gemm_bf16.hip"], ["kernels/common.h", "kernels/pipeline.h"]),
+    "gemm_bf16": ("hip", ["kernels/gemm_bf16.hip"], ["kernels/common.h", "kernels/pipeline.h", "kernels/no_alloc.h"]),
     "sampling": ("hip", ["kernels/sampling.hip"], ["kernels/common.h"]),
     "host": ("host", ["host/cache_manager.cpp", "host/scheduler.cpp", "host/c_api.cpp"],
              ["host/cache_manager.h", "host/scheduler.h"]),
