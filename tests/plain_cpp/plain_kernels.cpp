@@ -413,13 +413,30 @@ extern "C" int plain_attn_bf16_decode(const void* q, long long q_stride, const v
 // reference's cuts (candidates by logit descending then id ascending; top_k; top_p against the mass of every finite
 // logit; min_p against the best weight) and, as the kernel documents for itself, the draw walks the kept tokens in
 // id order: the first whose running mass exceeds u * kept mass. A row without a finite logit gives -1.
+// The uniform of a row is uniform[r], or with a slot table the next output of the xorshift64* generator whose state
+// sits in the row's slot (crates/vipera-sampler/src/rng.rs:13-57), seeded first where `reseed` says so; a greedy row
+// does not draw; the row's position is recorded beside the state.
 extern "C" int plain_sample(const float* logits, int num_rows, int vocab, const float* temperature, const int* top_k,
                             const float* top_p, const float* min_p, const double* uniform, int* out, float*, int*, int,
-                            void*) {
+                            const int* slot, const int* position, const int* reseed,
+                            const unsigned long long* seed_state, unsigned long long* slot_table, int num_slots, void*) {
   if (num_rows <= 0) return 0;
   if (vocab <= 0) return BAD_ARGUMENT;
+  if (!slot_table && !uniform) return BAD_ARGUMENT;
   for (int r = 0; r < num_rows; ++r) {
     const float* row = logits + (size_t)r * vocab;
+    double u = uniform ? uniform[r] : 0.0;
+    if (slot_table && slot[r] >= 0 && slot[r] < num_slots) {
+      unsigned long long state = reseed[r] ? seed_state[r] : slot_table[2 * slot[r]];
+      if (temperature[r] > 0.f) {
+        state ^= state >> 12;
+        state ^= state << 25;
+        state ^= state >> 27;
+        u = (double)((state * 0x2545F4914F6CDD1Dull) >> 11) / 9007199254740992.0;
+      }
+      slot_table[2 * slot[r]] = state;
+      slot_table[2 * slot[r] + 1] = (unsigned long long)(long long)position[r];
+    }
     std::vector<int> order;
     for (int i = 0; i < vocab; ++i)
       if (finite(row[i])) order.push_back(i);
@@ -454,7 +471,7 @@ extern "C" int plain_sample(const float* logits, int num_rows, int vocab, const 
     std::sort(kept.begin(), kept.end());   // by id
     double mass = 0.0;
     for (auto& kv : kept) mass += kv.second;
-    const double target = uniform[r] * mass;
+    const double target = u * mass;
     running = 0.0;
     out[r] = kept.back().first;
     for (auto& kv : kept) {

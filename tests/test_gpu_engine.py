@@ -125,6 +125,22 @@ def test_preemption_when_pages_run_out_keeps_every_request_right(folders):
     assert engine.runner.cache.free_blocks(0) == 10
 
 
+@pytest.mark.parametrize("pipelined", [False, True])
+def test_a_preempted_request_goes_on_with_its_own_stream_of_draws(folders, pipelined):
+    """A request's generator lives in its state slot; a preempted request loses the slot and, when it comes back,
+    its new slot is seeded with the generator wound forward by the draws it has made."""
+    from vipera_rs_amd import SamplingParams
+    prompts = [random_tokens(CONFIG_B["vocab_size"], n, 90 + n) for n in (30, 28, 25, 31)]
+    params = [SamplingParams(temperature=0.9, seed=21 + k) for k in range(4)]
+    solo = [_engine(folders["B"], block_size=16, num_blocks=8, max_num_seqs=1).generate([p], 40, s)[0].tokens
+            for p, s in zip(prompts, params)]
+    engine = _engine(folders["B"], block_size=16, num_blocks=10, max_num_seqs=4, chunk_size=16, pipelined=pipelined)
+    got = engine.generate(prompts, 40, params)
+    assert engine.stats()["preemptions"] > 0
+    assert [g.tokens for g in got] == solo
+    assert engine.runner.cache.check() == "" and engine.runner.cache.live_requests() == 0
+
+
 def test_a_request_that_can_never_fit_is_refused_at_admission(folders):
     from vipera_rs_amd.errors import InfeasibleError, InvalidArgumentError
     engine = _engine(folders["A"], block_size=16, num_blocks=2, max_num_seqs=2)

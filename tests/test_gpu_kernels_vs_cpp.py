@@ -3,8 +3,12 @@
 import ctypes
 import math
 
+import numpy as np
+
 import pytest
 import torch
+
+from plain import sampler_plain
 
 from helpers import rel_err
 from plain_cpp import DT, SIGNATURES, call
@@ -326,11 +330,45 @@ def test_sampling_kernels_beside_their_twins():
     for slices in (0, 7, 32):     # the rows' best logits searched by one workgroup a row, or by `slices` of them first
         scratch = [torch.empty(rows * slices), torch.empty(rows * slices, dtype=torch.int32)] if slices else [None, None]
         (got, want), = both("sampling", "sample", [logits, rows, vocab, temperature, top_k, top_p, min_p, uniform,
-                                                   torch.empty(rows, dtype=torch.int32), *scratch, slices, None], [8])
+                                                   torch.empty(rows, dtype=torch.int32), *scratch, slices,
+                                                   None, None, None, None, None, 0, None], [8])
         assert torch.equal(got[:8], want[:8]) and got[4] == -1 and got[5] == 100
         # a sampled row could differ where u * mass falls within rounding of a boundary between two kept tokens, or where
         # a cut's edge rounds the other way; none of these seeded rows does
         assert torch.equal(got, want)
+    # uniforms from the generators in the rows' state slots: two launches, the first seeds every second slot, the
+    # others go on from what the table held; greedy rows record their position and leave the state alone
+    slots = 64
+    table = torch.randint(1, 2 ** 62, (slots, 2), generator=g, dtype=torch.int64)
+    slot = torch.randperm(slots, generator=g)[:rows].to(torch.int32)
+    for launch in range(2):
+        position = torch.randint(0, 4096, (rows,), generator=g, dtype=torch.int32)
+        reseed = ((torch.arange(rows) % 2 == 0) & (launch == 0)).to(torch.int32)
+        seeds = torch.randint(1, 2 ** 62, (rows,), generator=g, dtype=torch.int64)
+        (got, want), (got_table, want_table) = both(
+            "sampling", "sample", [logits, rows, vocab, temperature, top_k, top_p, min_p, None,
+                                   torch.empty(rows, dtype=torch.int32), None, None, 0,
+                                   slot, position, reseed, seeds, table, slots, None], [8, 16])
+        assert torch.equal(got_table, want_table), (got_table - want_table).nonzero()
+        # the kernel's masses are 2^-40 fixed point, the twin's doubles: where u * mass falls within that rounding of
+        # the boundary between two kept tokens they may pick either side, and nowhere else
+        for r in (got != want).nonzero().flatten().tolist():
+            state = (seeds[r] if reseed[r] else table[slot[r], 0]).item()
+            state ^= state >> 12
+            state ^= (state << 25) % 2 ** 64
+            state ^= state >> 27
+            u = ((state * 0x2545F4914F6CDD1D) % 2 ** 64 >> 11) / 2.0 ** 53
+            kept = sorted(sampler_plain.kept_set(logits[r].numpy(), temperature[r].item(), top_k[r].item(),
+                                                 top_p[r].item(), min_p[r].item()))
+            ids = [i for i, _ in kept]
+            shares = np.cumsum([float(w) for _, w in kept])
+            shares /= shares[-1]
+            a, b = sorted((ids.index(got[r].item()), ids.index(want[r].item())))
+            assert b == a + 1 and abs(shares[a] - u) < 1e-6, (r, u, shares[a])
+        assert torch.equal(got_table[slot.long(), 1], position.long())
+        assert torch.equal(got_table[slot.long()[:8], 0], torch.where(reseed[:8].bool(), seeds[:8], table[slot.long()[:8], 0]))
+        assert not torch.equal(got_table[slot.long()[8:], 0], table[slot.long()[8:], 0])
+        table = got_table
     pen = torch.randn(3, 500, generator=g)
     args = [pen, 500, i32([0, 0, 2]), i32([3, 499, 3]), i32([2, 1, 4]), torch.tensor([1.3, 1.0, 0.7]), torch.tensor([0.2, 0.0, 0.1]),
             torch.tensor([0.1, 0.5, 0.0]), 3, None]

@@ -110,7 +110,7 @@ def test_kept_set_and_distribution(vocab, temperature, top_k, top_p, min_p):
 
 
 def test_penalties_match_the_plain_formula():
-    from vipera_rs_amd.sampling import BatchSampler, Rng, RowRequest, SamplingParams
+    from vipera_rs_amd.sampling import BatchSampler, RowRequest, SamplingParams
     rng = np.random.default_rng(11)
     vocab = 400
     base = rng.normal(size=(3, vocab)).astype(np.float32)
@@ -126,7 +126,7 @@ def test_penalties_match_the_plain_formula():
             base[r, token] = abs(base[r, token]) + 3.0
     logits = torch.tensor(base, device="cuda:0").contiguous()
     sampler = BatchSampler("cuda:0")
-    got = sampler.sample(logits, [RowRequest(p, Rng(0), rec) for p, rec in zip(params, recent)])
+    got = sampler.sample(logits, [RowRequest(p, slot, 0, rec, 1) for slot, (p, rec) in enumerate(zip(params, recent))])
     after = logits.cpu().numpy()
     for r in range(3):
         want = sampler_plain.penalize(base[r], recent[r], params[r].repetition_penalty, params[r].presence_penalty,
@@ -136,23 +136,54 @@ def test_penalties_match_the_plain_formula():
 
 
 def test_the_stream_of_a_request_does_not_depend_on_its_company():
-    from vipera_rs_amd.sampling import BatchSampler, Rng, RowRequest, SamplingParams
+    """A request's generator lives in its state slot on the device and the kernel advances it; the host's
+    generator (the reference's xorshift64* behind SplitMix64) is only the oracle here."""
+    from vipera_rs_amd.sampling import BatchSampler, RowRequest, SamplingParams, seeded_state
     rng = np.random.default_rng(5)
     vocab = 300
     rows = rng.normal(size=(4, vocab)).astype(np.float32) * 2
     params = [SamplingParams(temperature=0.8, seed=s) for s in (1, 2, 3, 4)]
-    sampler = BatchSampler("cuda:0")
+    # the oracle: the plain sampler's kept set walked in id order with the plain generator's uniforms
+    want = []
+    for r in range(4):
+        gen = sampler_plain.Rng(params[r].seed)
+        kept = sorted(sampler_plain.kept_set(rows[r], 0.8, params[r].top_k, params[r].top_p, params[r].min_p))
+        tokens = []
+        for _ in range(6):
+            u = gen.next_f64()
+            ids = [i for i, _ in kept]
+            shares = np.cumsum([float(w) for _, w in kept])
+            tokens.append((u, ids, shares / shares[-1]))
+        want.append(tokens)
+    sampler = BatchSampler("cuda:0", slots=8)
     alone = []
     for r in range(4):
-        gen = Rng(params[r].seed)
-        alone.append([sampler.sample(torch.tensor(rows[r:r + 1], device="cuda:0"), [RowRequest(params[r], gen)])[0]
-                      for _ in range(6)])
-    gens = [Rng(p.seed) for p in params]
+        alone.append([sampler.sample(torch.tensor(rows[r:r + 1], device="cuda:0"),
+                                     [RowRequest(params[r], 5, k, (), seeded_state(params[r].seed) if k == 0 else None)])[0]
+                      for k in range(6)])
+        assert sampler.slot_table[5, 1].item() == 5                                   # the position is recorded
+        assert sampler.slot_table[5, 0].item() % 2 ** 64 == seeded_state(params[r].seed, 6)   # the host's, wound on
+    for r in range(4):     # each draw falls where the plain generator's uniform points, up to rounding of the shares
+        for token, (u, ids, cumulative) in zip(alone[r], want[r]):
+            at = ids.index(token)
+            lo = cumulative[at - 1] if at else 0.0
+            assert lo - 1e-4 <= u <= cumulative[at] + 1e-4, (r, token, u)
     together = [[] for _ in range(4)]
-    for _ in range(6):
-        order = [2, 0, 3, 1]
+    slot_of = {0: 3, 1: 0, 2: 7, 3: 1}
+    for k in range(6):
+        order = [2, 0, 3, 1] if k % 2 else [1, 3, 0, 2]
         out = sampler.sample(torch.tensor(rows[order], device="cuda:0").contiguous(),
-                             [RowRequest(params[r], gens[r]) for r in order])
+                             [RowRequest(params[r], slot_of[r], k, (), seeded_state(params[r].seed) if k == 0 else None)
+                              for r in order])
         for r, token in zip(order, out):
             together[r].append(token)
     assert together == alone
+    # a request that comes back into another slot after 3 draws goes on where it was
+    again = [sampler.sample(torch.tensor(rows[2:3], device="cuda:0"),
+                            [RowRequest(params[2], 6, k, (), seeded_state(params[2].seed, 3) if k == 3 else None)])[0]
+             for k in range(3, 6)]
+    assert again == alone[2][3:]
+    # a greedy row leaves its generator alone
+    before = sampler.slot_table[6, 0].item()
+    sampler.sample(torch.tensor(rows[0:1], device="cuda:0"), [RowRequest(SamplingParams(), 6, 9)])
+    assert sampler.slot_table[6, 0].item() == before and sampler.slot_table[6, 1].item() == 9

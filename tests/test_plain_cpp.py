@@ -168,7 +168,8 @@ def test_sampling_twins():
     min_p = torch.tensor([0.0, 0.05, 0.0, 0.0, 0.0, 0.0])
     uniform = torch.tensor([0.3, 0.41, 0.5, 0.5, 0.5, 0.77], dtype=torch.float64)
     out = torch.empty(6, dtype=torch.int32)
-    call("plain_sample", logits, 6, 50, temperature, top_k, top_p, min_p, uniform, out, None, None, 0, None)
+    call("plain_sample", logits, 6, 50, temperature, top_k, top_p, min_p, uniform, out, None, None, 0,
+         None, None, None, None, None, 0, None)
     assert out[0] == S.greedy(logits[0].numpy()) and out[2] == S.greedy(logits[2].numpy())
     assert out[3] == -1 and out[4] == 10
     for row in (1, 5):   # the kept set is the reference's; the draw walks it in id order

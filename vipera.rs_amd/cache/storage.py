@@ -6,7 +6,9 @@ one output dim); the last page is a scratch page that is never handed out, which
 a captured step write to.  A state
 tensor is ``[slots + 1, *shape]``: the last row is the scratch row of those padding entries
 (``CacheStorage.scratch_slot``), so that a mixer that keeps state never sees a padding entry in a live
-request's row.
+request's row.  ``slot_table`` (int64 ``[slots + 1, 2]``) holds what every request keeps whatever the model: the
+state of its sampling generator and the position of its next token (the reference keeps both per turn,
+crates/vipera-runtime/src/engine.rs:130-159, crates/vipera-sampler/src/rng.rs:13-38).
 """
 from __future__ import annotations
 
@@ -43,6 +45,10 @@ class CacheStorage:
         self.groups = list(groups)
         self.bytes = 0
         self.scratch_slot = num_slots
+        # what every request keeps whatever the model: the state of its sampling generator and the position of
+        # its next token, two 64-bit words per slot, written by the sampling kernel
+        self.slot_table = torch.zeros((num_slots + 1, 2), dtype=torch.int64, device=runtime.device)
+        self.bytes += self.slot_table.numel() * 8
         for index, need in enumerate(needs):
             if need.owner != index:
                 continue

@@ -285,15 +285,15 @@ def sample_command(argv: List[str]) -> int:
     import torch
 
     from .runtime import Runtime
-    from .sampling import BatchSampler, Rng, RowRequest
+    from .sampling import BatchSampler, RowRequest, seeded_state
 
     runtime = Runtime("cuda:0", "float32")
     sampler = BatchSampler(runtime.device)
-    rng = Rng(params.seed)
     tokens = []
-    for _ in range(count):
+    for draw in range(count):
         logits = torch.tensor([values], dtype=torch.float32, device=runtime.device)
-        token = sampler.sample(logits, [RowRequest(params, rng, recent)])[0]
+        row = RowRequest(params, 0, draw, recent, seeded_state(params.seed) if draw == 0 else None)
+        token = sampler.sample(logits, [row])[0]
         if token < 0:
             raise InvalidArgumentError("the logits hold no finite value")
         tokens.append(token)

@@ -112,6 +112,20 @@ __global__ __launch_bounds__(256) void argmax_slices_kernel(const float* __restr
   }
 }
 
+// Where a row's uniform comes from when it is not handed in: the request's record in the table of state slots,
+// two 64-bit words per slot: the state of its xorshift64* generator (crates/vipera-sampler/src/rng.rs:13-57:
+// x ^= x >> 12, x ^= x << 25, x ^= x >> 27, output x * 0x2545F4914F6CDD1D, top 53 bits as a double in [0, 1))
+// and the position of the request's next token. A row that draws advances its generator by one step; a
+// greedy row leaves it alone; `reseed` puts `seed_state` into the slot first (a request's first row in a slot).
+struct SlotRows {
+  const int* slot;                         // per row
+  const int* position;                     // per row: where the token drawn now will sit
+  const int* reseed;                       // per row: 0 or 1
+  const unsigned long long* seed_state;    // per row
+  unsigned long long* table;               // [num_slots, 2], or nullptr: the uniforms are handed in
+  int num_slots;
+};
+
 // One row. Returns the chosen token in *out (or -1 when no logit is finite). `slices` > 0: the row's best logit
 // comes from the winners that argmax_slices_kernel left.
 __global__ __launch_bounds__(THREADS) void sample_kernel(const float* __restrict__ logits, int vocab,
@@ -121,7 +135,7 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(const float* __restrict
                                                          const float* __restrict__ min_p,
                                                          const double* __restrict__ uniform, int* __restrict__ out,
                                                          const float* __restrict__ slice_best,
-                                                         const int* __restrict__ slice_id, int slices) {
+                                                         const int* __restrict__ slice_id, int slices, SlotRows slots) {
   __shared__ float red_f[16];
   __shared__ int red_i[WAVES];
   __shared__ unsigned long long red_u[WAVES];
@@ -130,8 +144,27 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(const float* __restrict
   __shared__ long long sh_remaining;
   __shared__ unsigned long long sh_below;
 
+  __shared__ double sh_uniform;
+
   const int row = blockIdx.x, tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
   const float* x = logits + (size_t)row * vocab;
+  if (tid == 0) {
+    double u = uniform ? uniform[row] : 0.0;
+    const int slot = slots.table ? slots.slot[row] : -1;
+    if (slot >= 0 && slot < slots.num_slots) {
+      unsigned long long* record = slots.table + 2 * (size_t)slot;
+      unsigned long long state = slots.reseed[row] ? slots.seed_state[row] : record[0];
+      if (temperature[row] > 0.f) {
+        state ^= state >> 12;
+        state ^= state << 25;
+        state ^= state >> 27;
+        u = (double)((state * 0x2545F4914F6CDD1Dull) >> 11) * (1.0 / 9007199254740992.0);
+      }
+      record[0] = state;
+      record[1] = (unsigned long long)(long long)slots.position[row];
+    }
+    sh_uniform = u;   // read after the barriers below
+  }
 
   // --- best finite logit, ties to the lowest id ----------------------------------------------
   float best = -INFINITY;
@@ -368,7 +401,7 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(const float* __restrict
     if (tid == 0) out[row] = best_id;
     return;
   }
-  unsigned long long target = (unsigned long long)(uniform[row] * (double)mass);
+  unsigned long long target = (unsigned long long)(sh_uniform * (double)mass);
   if (target >= mass) target = mass - 1;
   // the wave whose share holds the target walks its range once more
   if (target >= before && target < before + red_u[wave]) {
@@ -434,11 +467,19 @@ __global__ void bias_kernel(float* __restrict__ logits, int vocab, const int* __
 
 // `slices` > 0 with room for num_rows * slices values in `slice_best` and `slice_id`: the rows' best logits are
 // found by slices * num_rows workgroups first (worth it for a wide vocabulary); the result is the same.
+//
+// The uniform of a row that draws is `uniform[row]`, or with a `slot_table` ([num_slots, 2] 64-bit words; then
+// `uniform` may be null) the next output of the generator in the row's slot, see SlotRows.
 extern "C" int vk_sample(const float* logits, int num_rows, int vocab, const float* temperature, const int* top_k,
                          const float* top_p, const float* min_p, const double* uniform, int* out, float* slice_best,
-                         int* slice_id, int slices, void* stream) {
+                         int* slice_id, int slices, const int* slot, const int* position, const int* reseed,
+                         const unsigned long long* seed_state, unsigned long long* slot_table, int num_slots,
+                         void* stream) {
   if (num_rows <= 0) return 0;
   if (vocab <= 0 || slices < 0 || slices > 65535 || num_rows > 65535) return VK_BAD_ARGUMENT;
+  if (!slot_table && !uniform) return VK_BAD_ARGUMENT;
+  if (slot_table && (!slot || !position || !reseed || !seed_state || num_slots < 1)) return VK_BAD_ARGUMENT;
+  const SlotRows slots{slot, position, reseed, seed_state, slot_table, num_slots};
   if (slices > 0) {
     if (!slice_best || !slice_id) return VK_BAD_ARGUMENT;
     const int slice_len = (vocab + slices - 1) / slices;
@@ -447,7 +488,7 @@ extern "C" int vk_sample(const float* logits, int num_rows, int vocab, const flo
     VK_LAUNCH_CHECK();
   }
   sample_kernel<<<num_rows, THREADS, 0, (hipStream_t)stream>>>(logits, vocab, temperature, top_k, top_p, min_p,
-                                                                uniform, out, slice_best, slice_id, slices);
+                                                                uniform, out, slice_best, slice_id, slices, slots);
   VK_LAUNCH_CHECK();
   return 0;
 }

@@ -16,7 +16,7 @@ import torch
 
 from ..errors import InfeasibleError, InvalidArgumentError, ViperaError
 from ..runtime import Runtime
-from ..sampling import RECENT_WINDOW, BatchSampler, Rng, RowRequest, SamplingParams
+from ..sampling import RECENT_WINDOW, BatchSampler, RowRequest, SamplingParams, seeded_state
 from .batch import StepEntry
 from .runner import ModelRunner
 from .scheduler import FINISH_NAMES, FINISH_STOP, NOT_FINISHED, Scheduler
@@ -57,8 +57,9 @@ class _Live:
     prompt: List[int]
     generated: List[int]
     params: SamplingParams
-    rng: Rng
     eos: frozenset
+    draws: int = 0            # uniforms its generator has given out
+    seeded: bool = False      # whether the slot it holds now has its generator's state
     processed: int = 0
     preemptions: int = 0
     on_token: Optional[Callable[[int], None]] = None
@@ -128,7 +129,8 @@ class Engine:
         self.max_model_len = limit
         self.scheduler = Scheduler(runner.cache, max_num_seqs, max_num_batched_tokens, chunk_size, limit,
                                    eager_admission)
-        self.sampler = BatchSampler(runner.runtime.device, out=runner.sampled_tokens)
+        self.sampler = BatchSampler(runner.runtime.device, out=runner.sampled_tokens,
+                                    slot_table=runner.storage.slot_table)
         self.pipelined = bool(pipelined) and runner.sampled_tokens is not None
         self._inflight: Optional[_InFlight] = None   # the launched step whose tokens have not been collected
         default_eos = getattr(config, "eos_token_ids", ()) or ()
@@ -176,7 +178,7 @@ class Engine:
         self.scheduler.add(request, prompt, int(max_new_tokens))
         self._next_id += 1
         eos = frozenset(eos_token_ids) if eos_token_ids is not None else self.eos_token_ids
-        self._live[request] = _Live(prompt, [], params, Rng(params.seed), eos, on_token=on_token)
+        self._live[request] = _Live(prompt, [], params, eos, on_token=on_token)
         return request
 
     def cancel(self, request: int) -> Optional[Generation]:
@@ -186,6 +188,27 @@ class Engine:
             return None
         self.scheduler.cancel(request)
         return Generation(request, len(live.prompt), live.generated, "cancelled", live.processed, live.preemptions)
+
+    def _row(self, entry, recent=()) -> RowRequest:
+        """How the last token of ``entry`` is sampled: from the generator in the request's slot, which is seeded
+        when the request draws for the first time in that slot (at its start, or wound forward by the draws it
+        had made when it comes back after a preemption)."""
+        live = self._live[entry.request]
+        seed_state = None
+        if not live.seeded:
+            seed_state = seeded_state(live.params.seed, live.draws)
+            live.seeded = True
+        if not live.params.greedy:
+            live.draws += 1
+        return RowRequest(live.params, self.runner.cache.slot(entry.request), entry.start + len(entry.tokens), recent,
+                          seed_state)
+
+    def _note_preempted(self, plan, report: StepReport) -> None:
+        for request in plan.preempted:
+            if request in self._live:
+                self._live[request].preemptions += 1
+                self._live[request].seeded = False      # its slot is given back; the next one starts unseeded
+        report.preempted = list(plan.preempted)
 
     def has_work(self) -> bool:
         return self.scheduler.has_work() or self._inflight is not None
@@ -204,10 +227,7 @@ class Engine:
         report = StepReport()
         started = time.perf_counter()
         plan = self.scheduler.plan()
-        for request in plan.preempted:
-            if request in self._live:
-                self._live[request].preemptions += 1
-        report.preempted = list(plan.preempted)
+        self._note_preempted(plan, report)
         scheduled = time.perf_counter()
         self.micros["schedule"] += int((scheduled - started) * 1e6)
         previous, launched = self._inflight, None
@@ -237,7 +257,7 @@ class Engine:
                 self._live[e.request].processed += len(e.tokens)
             wanting = [e for e in plan.entries if e.wants_logits]
             if wanting:
-                rows = [RowRequest(self._live[e.request].params, self._live[e.request].rng, ()) for e in wanting]
+                rows = [self._row(e) for e in wanting]
                 pending = self.sampler.launch(logits, rows)
                 # the scheduler goes on as if the token were known: a placeholder stands for it until it arrives
                 reasons = [self.scheduler.append(e.request, 0, False) for e in wanting]
@@ -285,10 +305,7 @@ class Engine:
     def _step_in_turn(self, report: StepReport) -> StepReport:
         started = time.perf_counter()
         plan = self.scheduler.plan()
-        for request in plan.preempted:
-            if request in self._live:
-                self._live[request].preemptions += 1
-        report.preempted = list(plan.preempted)
+        self._note_preempted(plan, report)
         scheduled = time.perf_counter()
         self.micros["schedule"] += int((scheduled - started) * 1e6)
         if not plan.entries:
@@ -312,7 +329,7 @@ class Engine:
             rows = []
             for e in wanting:
                 live = self._live[e.request]
-                rows.append(RowRequest(live.params, live.rng, _recent_tokens(live) if live.params.penalizes else ()))
+                rows.append(self._row(e, _recent_tokens(live) if live.params.penalizes else ()))
             tokens = self.sampler.sample(logits, rows)
             for e, token in zip(wanting, tokens):
                 if token < 0:

@@ -245,26 +245,42 @@ SAMPLE_SLICES_FROM = 32_768   # columns from which a row's best logit is searche
 
 
 def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
-           min_p: torch.Tensor, uniform: torch.Tensor, out: torch.Tensor) -> None:
+           min_p: torch.Tensor, uniform: Optional[torch.Tensor], out: torch.Tensor,
+           slot: Optional[torch.Tensor] = None, position: Optional[torch.Tensor] = None,
+           reseed: Optional[torch.Tensor] = None, seed_state: Optional[torch.Tensor] = None,
+           slot_table: Optional[torch.Tensor] = None) -> None:
     """One token per row: greedy where ``temperature`` is 0, else a draw after the top-k/top-p/min-p cuts.
 
-    ``out[r]`` is -1 when row ``r`` has no finite logit.
+    ``out[r]`` is -1 when row ``r`` has no finite logit.  The uniform of a row that draws is ``uniform[r]``, or
+    with a ``slot_table`` (int64 ``[slots, 2]``: generator state and next position per state slot) the next
+    output of the xorshift64* generator in slot ``slot[r]``, which the kernel advances; ``reseed[r]`` puts
+    ``seed_state[r]`` there first, and ``position[r]`` is recorded beside it.
     """
-    _dev(logits, temperature, top_k, top_p, min_p, uniform, out)
+    _dev(logits, temperature, top_k, top_p, min_p, uniform, out, slot, position, reseed, seed_state, slot_table)
     rows, vocab = logits.shape
     _need(logits.dtype == torch.float32 and logits.is_contiguous(), "sample: logits must be contiguous float32")
-    for name, tensor, dtype in (("temperature", temperature, torch.float32), ("top_k", top_k, torch.int32),
-                                ("top_p", top_p, torch.float32), ("min_p", min_p, torch.float32),
-                                ("uniform", uniform, torch.float64), ("out", out, torch.int32)):
-        _need(tensor.dtype == dtype and tensor.numel() == rows and tensor.is_contiguous(),
+    columns = [("temperature", temperature, torch.float32), ("top_k", top_k, torch.int32),
+               ("top_p", top_p, torch.float32), ("min_p", min_p, torch.float32), ("out", out, torch.int32)]
+    if slot_table is None:
+        _need(uniform is not None, "sample: either uniforms or a table of state slots")
+        columns.append(("uniform", uniform, torch.float64))
+    else:
+        _need(slot_table.dtype == torch.int64 and slot_table.dim() == 2 and slot_table.shape[1] == 2
+              and slot_table.is_contiguous(), "sample: the slot table must be contiguous int64 [slots, 2]")
+        columns += [("slot", slot, torch.int32), ("position", position, torch.int32), ("reseed", reseed, torch.int32),
+                    ("seed_state", seed_state, torch.int64)]
+    for name, tensor, dtype in columns:
+        _need(tensor is not None and tensor.dtype == dtype and tensor.numel() == rows and tensor.is_contiguous(),
               f"sample: {name} must hold one {dtype} per row")
     # a wide vocabulary: the rows' best logits are found by 32 workgroups a row before the one that draws
     slices = SAMPLE_SLICES if vocab >= SAMPLE_SLICES_FROM else 0
     best = torch.empty(rows * slices, dtype=torch.float32, device=logits.device) if slices else None
     best_id = torch.empty(rows * slices, dtype=torch.int32, device=logits.device) if slices else None
-    fn = _fn("sampling", "vk_sample", [_p, _i, _i, _p, _p, _p, _p, _p, _p, _p, _p, _i, _p])
+    fn = _fn("sampling", "vk_sample", [_p, _i, _i, _p, _p, _p, _p, _p, _p, _p, _p, _i, _p, _p, _p, _p, _p, _i, _p])
     _status(fn(_ptr(logits), rows, vocab, _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(min_p), _ptr(uniform),
-               _ptr(out), _ptr(best), _ptr(best_id), slices, _stream()), "sample")
+               _ptr(out), _ptr(best), _ptr(best_id), slices, _ptr(slot), _ptr(position), _ptr(reseed),
+               _ptr(seed_state), _ptr(slot_table), slot_table.shape[0] if slot_table is not None else 0, _stream()),
+            "sample")
 
 
 def penalize(logits: torch.Tensor, rows: torch.Tensor, tokens: torch.Tensor, counts: torch.Tensor,

@@ -1,4 +1,4 @@
 from .rng import Rng
-from .sampler import MAX_LOGIT_BIAS, RECENT_WINDOW, BatchSampler, RowRequest, SamplingParams
+from .sampler import MAX_LOGIT_BIAS, RECENT_WINDOW, BatchSampler, RowRequest, SamplingParams, seeded_state
 
-__all__ = ["Rng", "MAX_LOGIT_BIAS", "RECENT_WINDOW", "BatchSampler", "RowRequest", "SamplingParams"]
+__all__ = ["Rng", "MAX_LOGIT_BIAS", "RECENT_WINDOW", "BatchSampler", "RowRequest", "SamplingParams", "seeded_state"]

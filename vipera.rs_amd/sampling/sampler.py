@@ -70,11 +70,20 @@ class SamplingParams:
 
 @dataclass
 class RowRequest:
-    """What one row of logits is sampled with: options, the request's generator, its recent tokens."""
+    """What one row of logits is sampled with: options, the request's state slot (where its generator lives),
+    the position the drawn token will take, its recent tokens, and ``seed_state``: the generator state to put
+    into the slot first (the request's first row in this slot), or None to go on from what the slot holds."""
 
     params: SamplingParams
-    rng: Rng
+    slot: int = 0
+    position: int = 0
     recent: Sequence[int] = ()
+    seed_state: Optional[int] = None
+
+
+def seeded_state(seed: int, draws: int = 0) -> int:
+    """The generator state of a request with ``seed`` that has drawn ``draws`` times."""
+    return Rng(seed).skip(draws).state
 
 
 class PendingSample:
@@ -87,18 +96,24 @@ class PendingSample:
 class BatchSampler:
     """Samples one token per row of ``[rows, vocab]`` logits on the device.
 
-    Per-row options go up in one small copy; the drawn ids come back in one.  Each random row
-    consumes exactly one uniform of its request's generator per token, so a request's stream does
-    not depend on its company in the batch or on the order of arrival (the invariant of
-    crates/vipera-runtime/src/engine.rs:665-670).
+    Per-row options go up in one small copy; the drawn ids come back in one.  A request's generator lives in
+    its row of ``slot_table`` (int64 ``[slots, 2]`` on the device: generator state, position of the next token)
+    and the kernel advances it: each random row consumes exactly one uniform of its request's generator per
+    token, so a request's stream does not depend on its company in the batch or on the order of arrival (the
+    invariant of crates/vipera-runtime/src/engine.rs:665-670), and a step that is launched before the tokens
+    of the step before have reached the host needs nothing from the host to draw.
 
     ``launch`` enqueues the work and returns at once, ``collect`` waits for the ids; ``out`` (optional,
-    int32 on the device) is where the ids are left for a next step that reads them there.
+    int32 on the device) is where the ids are left for a next step that reads them there.  Without a
+    ``slot_table`` the sampler keeps one of ``slots`` rows of its own.
     """
 
-    def __init__(self, device, out: Optional[torch.Tensor] = None):
+    def __init__(self, device, out: Optional[torch.Tensor] = None, slot_table: Optional[torch.Tensor] = None,
+                 slots: int = 64):
         self.device = torch.device(device)
         self.out = out
+        self.slot_table = slot_table if slot_table is not None else torch.zeros((slots, 2), dtype=torch.int64,
+                                                                                 device=self.device)
         # pinned host words of the per-row options and of the ids, two of each used in turn (a launch may
         # follow before the copies of the one before have run), and the options' place on the device
         self._options = [None, None]
@@ -118,19 +133,28 @@ class BatchSampler:
         self._penalize(logits, rows, vocab)
         self._turn ^= 1
         turn = self._turn
-        # one pinned staging buffer, one copy: 4-byte columns first, then the 8-byte uniforms
-        words = 6 * count
+        slots = self.slot_table.shape[0]
+        for r in rows:
+            if not 0 <= r.slot < slots:
+                raise InvalidArgumentError(f"state slot {r.slot} is outside the table of {slots}")
+        # one pinned staging buffer, one copy: seven 4-byte columns (of an even length, so that the 8-byte
+        # column behind them is aligned), then the generator states for rows that seed their slot
+        n = count + (count & 1)
+        words = 10 * n
         if self._options[turn] is None or self._options[turn].numel() < words:
-            self._options[turn] = torch.empty(max(words, 6 * 64), dtype=torch.int32).pin_memory()
+            self._options[turn] = torch.empty(max(words, 10 * 64), dtype=torch.int32).pin_memory()
             self._ids[turn] = torch.empty(max(count, 64), dtype=torch.int32).pin_memory()
         if self._device_words is None or self._device_words.numel() < words:
-            self._device_words = torch.empty(max(words, 6 * 64), dtype=torch.int32, device=self.device)
+            self._device_words = torch.empty(max(words, 10 * 64), dtype=torch.int32, device=self.device)
         host = self._options[turn].numpy()
         host[0:count].view(np.float32)[:] = [r.params.temperature for r in rows]
-        host[count:2 * count] = [r.params.top_k for r in rows]
-        host[2 * count:3 * count].view(np.float32)[:] = [r.params.top_p for r in rows]
-        host[3 * count:4 * count].view(np.float32)[:] = [r.params.min_p for r in rows]
-        host[4 * count:6 * count].view(np.float64)[:] = [0.0 if r.params.greedy else r.rng.next_f64() for r in rows]
+        host[n:n + count] = [r.params.top_k for r in rows]
+        host[2 * n:2 * n + count].view(np.float32)[:] = [r.params.top_p for r in rows]
+        host[3 * n:3 * n + count].view(np.float32)[:] = [r.params.min_p for r in rows]
+        host[4 * n:4 * n + count] = [r.slot for r in rows]
+        host[5 * n:5 * n + count] = [r.position for r in rows]
+        host[6 * n:6 * n + count] = [0 if r.seed_state is None else 1 for r in rows]
+        host[8 * n:8 * n + 2 * count].view(np.uint64)[:] = [r.seed_state or 0 for r in rows]
         dev = self._device_words
         dev[:words].copy_(self._options[turn][:words], non_blocking=True)
         if self.out is not None:
@@ -139,9 +163,11 @@ class BatchSampler:
             out = self.out[:count]
         else:
             out = torch.empty(count, dtype=torch.int32, device=self.device)
-        kernels.sample(logits, dev[0:count].view(torch.float32), dev[count:2 * count],
-                       dev[2 * count:3 * count].view(torch.float32), dev[3 * count:4 * count].view(torch.float32),
-                       dev[4 * count:6 * count].view(torch.float64), out)
+        kernels.sample(logits, dev[0:count].view(torch.float32), dev[n:n + count],
+                       dev[2 * n:2 * n + count].view(torch.float32), dev[3 * n:3 * n + count].view(torch.float32),
+                       None, out, slot=dev[4 * n:4 * n + count], position=dev[5 * n:5 * n + count],
+                       reseed=dev[6 * n:6 * n + count], seed_state=dev[8 * n:8 * n + 2 * count].view(torch.int64),
+                       slot_table=self.slot_table)
         ids = self._ids[turn]
         ids[:count].copy_(out, non_blocking=True)
         event = torch.cuda.Event()
