@@ -77,6 +77,26 @@ def attention(q: np.ndarray, k: np.ndarray, v: np.ndarray, scale: Optional[float
     return out
 
 
+def attention_by_head(q: np.ndarray, k: np.ndarray, v: np.ndarray, scale: Optional[float] = None,
+                      window: int = 0) -> np.ndarray:
+    """The same function as :func:`attention` with one matrix of scores per head instead of one dot product per
+    pair of positions, for sequences of thousands of tokens; ``tests/test_plain.py`` holds it to ``attention``."""
+    T, heads, hd = q.shape
+    group = heads // k.shape[1]
+    if scale is None:
+        scale = 1.0 / math.sqrt(hd)
+    position = np.arange(T)
+    visible = position[None, :] <= position[:, None]
+    if window > 0:
+        visible &= position[None, :] > position[:, None] - window
+    out = np.zeros_like(q)
+    for h in range(heads):
+        scores = np.where(visible, (q[:, h] @ k[:, h // group].T) * scale, -np.inf)
+        e = np.exp(scores - scores.max(axis=1, keepdims=True))
+        out[:, h] = (e / e.sum(axis=1, keepdims=True)) @ v[:, h // group]
+    return out
+
+
 def silu(z: np.ndarray) -> np.ndarray:
     """model.rs:4368-4370: ``z / (1 + exp(-z))``."""
     return z / (1.0 + np.exp(-z))
@@ -95,7 +115,8 @@ def swiglu_mlp(h: np.ndarray, w_gate: np.ndarray, w_up: np.ndarray, w_down: np.n
     return linear(linear(h, w_up) * silu(linear(h, w_gate)), w_down)
 
 
-def attention_block(h: np.ndarray, w: Dict[str, np.ndarray], prefix: str, cfg: dict, window: int) -> np.ndarray:
+def attention_block(h: np.ndarray, w: Dict[str, np.ndarray], prefix: str, cfg: dict, window: int,
+                    attend=attention) -> np.ndarray:
     """model.rs:1005-1126: project with bias, rotate q and k (after the bias, 649-656), attend, project out."""
     T = h.shape[0]
     heads, kv_heads, hd = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
@@ -105,7 +126,7 @@ def attention_block(h: np.ndarray, w: Dict[str, np.ndarray], prefix: str, cfg: d
     for t in range(T):
         q[t] = rope_neox(q[t], t, cfg["rope_theta"])
         k[t] = rope_neox(k[t], t, cfg["rope_theta"])
-    a = attention(q, k, v, window=window).reshape(T, heads * hd)
+    a = attend(q, k, v, window=window).reshape(T, heads * hd)
     return linear(a, w[prefix + "o_proj.weight"])
 
 
@@ -126,7 +147,7 @@ def normalize_config(cfg: dict) -> dict:
     return cfg
 
 
-def forward(cfg: dict, w: Dict[str, np.ndarray], tokens, dtype=np.float64) -> np.ndarray:
+def forward(cfg: dict, w: Dict[str, np.ndarray], tokens, dtype=np.float64, attend=attention) -> np.ndarray:
     """Logits ``[T, vocab]`` of a whole sequence (model.rs:956-1237): embedding (no scaling, 607-616),
     pre-norm blocks, final norm, output projection; the embedding table is the output matrix when the
     file has none (425)."""
@@ -137,7 +158,7 @@ def forward(cfg: dict, w: Dict[str, np.ndarray], tokens, dtype=np.float64) -> np
     for i in range(cfg["num_hidden_layers"]):
         p = f"model.layers.{i}."
         h = rms_norm(x, w[p + "input_layernorm.weight"], eps)
-        x = x + attention_block(h, w, p + "self_attn.", cfg, layer_window(cfg, i))
+        x = x + attention_block(h, w, p + "self_attn.", cfg, layer_window(cfg, i), attend)
         h = rms_norm(x, w[p + "post_attention_layernorm.weight"], eps)
         x = x + swiglu_mlp(h, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
     h = rms_norm(x, w["model.norm.weight"], eps)

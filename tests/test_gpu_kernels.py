@@ -196,10 +196,14 @@ class _Paged:
             table = [order.pop() for _ in range(blocks)]
             keys = torch.randn(n, kv_heads, hd, generator=g).to(dtype)
             values = torch.randn(n, kv_heads, hd, generator=g).to(dtype)
-            for p in range(n):
-                page, slot = table[p // block_size], p % block_size
-                self.k[page, :, slot, :] = keys[p]
-                self.v[page, :, :, slot] = values[p]
+            whole, rest = n // block_size, n % block_size       # position p sits in slot p % size of page table[p // size]
+            if whole:
+                pages_of = torch.tensor(table[:whole])
+                self.k[pages_of] = keys[:whole * block_size].view(whole, block_size, kv_heads, hd).permute(0, 2, 1, 3)
+                self.v[pages_of] = values[:whole * block_size].view(whole, block_size, kv_heads, hd).permute(0, 2, 3, 1)
+            if rest:
+                self.k[table[whole], :, :rest, :] = keys[whole * block_size:].permute(1, 0, 2)
+                self.v[table[whole], :, :, :rest] = values[whole * block_size:].permute(1, 2, 0)
             self.tables.append(table)
             self.keys.append(keys)
             self.values.append(values)
@@ -305,6 +309,128 @@ def test_decode_attention_over_thousands_of_positions(window):
         kernels.attn_bf16_decode(qkv_d, k_d, v_d, out, partial, singles, es, fp, table_d, heads, kv_heads, hd, scale,
                                  window, chunk, chunks)
         assert _rel(out.cpu(), want) < 1.2e-2, f"chunk {chunk}"
+
+
+def _plain_attention_by_head(q, k, v, first_pos, window, scale):
+    """The same as ``_plain_attention`` with one matrix of scores per head, for thousands of positions."""
+    T, heads, hd = q.shape
+    group = heads // k.shape[1]
+    pos = first_pos + torch.arange(T)[:, None]
+    key = torch.arange(k.shape[0])[None, :]
+    visible = key <= pos
+    if window > 0:
+        visible &= key > pos - window
+    out = torch.zeros(T, heads, hd, dtype=torch.float64)
+    for h in range(heads):
+        scores = (q[:, h] @ k[:, h // group].T) * scale
+        out[:, h] = torch.softmax(scores.masked_fill(~visible, float("-inf")), dim=1) @ v[:, h // group]
+    return out
+
+
+def test_the_two_plain_attentions_agree():
+    g = torch.Generator().manual_seed(0)
+    q, k, v = (torch.randn(n, h, 16, generator=g, dtype=torch.float64) for n, h in ((5, 6), (40, 2), (40, 2)))
+    for window in (0, 7):
+        a = _plain_attention(q, k, v, 35, window, 0.25)
+        b = _plain_attention_by_head(q, k, v, 35, window, 0.25)
+        assert float((a - b).abs().max()) < 1e-12
+
+
+BENCH_HEADS = [(28, 4, 128), (40, 8, 128), (12, 2, 128)]   # the 7B, 32B and 1.5B head shapes
+
+
+def _context_bucket(kv_len):
+    bucket = 256
+    while bucket < kv_len:
+        bucket *= 2
+    return bucket
+
+
+@pytest.mark.parametrize("heads,kv_heads,hd", BENCH_HEADS, ids=[f"h{h}kv{k}" for h, k, _ in BENCH_HEADS])
+@pytest.mark.parametrize("batch", [8, 64])
+def test_decode_attention_at_the_benchmark_head_shapes(heads, kv_heads, hd, batch):
+    """Single-token entries at 4,096 and 3,000 positions (and a few short ones) in batches of 8 and 64, with the
+    chunking the engine picks for the longest entry and for the context bucket a captured step is built for.
+    In every entry one far key is made to stand out for the first head of each group, so that a chunk or a page
+    that is dropped shows."""
+    from vipera_rs_amd.ops import kernels
+    from vipera_rs_amd.ops.attention import decode_chunking
+    if batch == 64 and heads != 28:
+        pytest.skip("the batch of 64 runs at the 7B head shape")
+    bs, scale, dtype = 16, 1.0 / math.sqrt(hd), torch.bfloat16
+    lengths = [(4096, 3000, 2049, 4095, 1, 3001, 130, 4096)[e % 8] for e in range(batch)]
+    cache = _Paged(lengths, kv_heads, hd, bs, dtype, seed=heads)
+    g = torch.Generator().manual_seed(batch)
+    qkv = torch.randn(batch, (heads + 2 * kv_heads) * hd, generator=g).to(dtype)
+    group = heads // kv_heads
+    for e, n in enumerate(lengths):
+        far = (17 * (e + 1)) % n
+        page, slot = cache.tables[e][far // bs], far % bs
+        for kv in range(kv_heads):
+            q = qkv[e, kv * group * hd:(kv * group + 1) * hd].float()
+            key = (q / q.norm() * (9.0 / scale / q.norm())).to(dtype)      # a score of about 9 for that head
+            cache.keys[e][far, kv] = key
+            cache.k[page, kv, slot, :] = key
+    first = [n - 1 for n in lengths]
+    want = torch.zeros(batch, heads, hd, dtype=torch.float64)
+    for e in range(batch):
+        q = qkv[e:e + 1, :heads * hd].double().view(1, heads, hd)
+        want[e] = _plain_attention_by_head(q, cache.keys[e].double(), cache.values[e].double(), first[e], 0, scale)[0]
+    want = want.view(batch, heads * hd)
+    dev = lambda t: t.to(DEV)  # noqa: E731
+    qkv_d, k_d, v_d = dev(qkv), dev(cache.k), dev(cache.v)
+    es = dev(torch.arange(batch + 1, dtype=torch.int32))
+    fp = dev(torch.tensor(first, dtype=torch.int32))
+    singles = dev(torch.arange(batch, dtype=torch.int32))
+    longest = max(lengths)
+    for visible in (longest, _context_bucket(longest), 2 * _context_bucket(longest)):
+        # a captured step is built for a context bucket: its table is that wide and its chunks cover all of it
+        width = (visible + bs - 1) // bs
+        table = torch.full((batch, width), -1, dtype=torch.int32)
+        table[:, :cache.table.shape[1]] = cache.table
+        chunk, chunks = decode_chunking(visible, batch, kv_heads, (group + 15) // 16)
+        out = torch.zeros(batch, heads * hd, dtype=dtype, device=DEV)
+        partial = torch.full((batch * heads * chunks * (hd + 2),), float("nan"), device=DEV)
+        kernels.attn_bf16_decode(qkv_d, k_d, v_d, out, partial, singles, es, fp, dev(table), heads, kv_heads, hd, scale, 0,
+                                 chunk, chunks)
+        assert _rel(out.cpu(), want) < 1.2e-2, f"visible {visible}: chunk {chunk} x {chunks}"
+    out = torch.zeros(batch, heads * hd, dtype=dtype, device=DEV)
+    kernels.attn_generic(qkv_d, k_d, v_d, out, fp, singles, dev(cache.table), heads, kv_heads, hd, scale, 0)
+    assert _rel(out.cpu(), want) < 1.2e-2, "32-bit-arithmetic kernel on the bfloat16 cache"
+
+
+@pytest.mark.parametrize("heads,kv_heads,hd", BENCH_HEADS, ids=[f"h{h}kv{k}" for h, k, _ in BENCH_HEADS])
+def test_prompt_attention_at_the_benchmark_head_shapes(heads, kv_heads, hd):
+    """One prompt of 2,048 tokens from position 0 and one portion of 512 tokens from position 3,584 in one step."""
+    from vipera_rs_amd.engine.batch import TILE_TOKENS
+    from vipera_rs_amd.ops import kernels
+    bs, scale, dtype = 16, 1.0 / math.sqrt(hd), torch.bfloat16
+    entries = [(2048, 2048), (4096, 512)]       # (positions in the cache after the step, tokens of the step)
+    cache = _Paged([kv for kv, _ in entries], kv_heads, hd, bs, dtype, seed=hd + heads)
+    g = torch.Generator().manual_seed(heads)
+    counts = [n for _, n in entries]
+    T = sum(counts)
+    qkv = torch.randn(T, (heads + 2 * kv_heads) * hd, generator=g).to(dtype)
+    starts, first = [0, counts[0], T], [kv - n for kv, n in entries]
+    want = torch.zeros(T, heads, hd, dtype=torch.float64)
+    for e, (kv, n) in enumerate(entries):
+        q = qkv[starts[e]:starts[e + 1], :heads * hd].double().view(n, heads, hd)
+        want[starts[e]:starts[e + 1]] = _plain_attention_by_head(q, cache.keys[e].double(), cache.values[e].double(),
+                                                                 first[e], 0, scale)
+    want = want.view(T, heads * hd)
+    dev = lambda t: t.to(DEV)  # noqa: E731
+    tiles = [(first[e] + off, e, off) for e, n in enumerate(counts) for off in range(0, n, TILE_TOKENS)]
+    tiles = [x for _, e, off in sorted(tiles) for x in (e, off)]                # as the engine orders them
+    out = torch.zeros(T, heads * hd, dtype=dtype, device=DEV)
+    kernels.attn_bf16_prefill(dev(qkv), dev(cache.k), dev(cache.v), out, dev(torch.tensor(tiles, dtype=torch.int32)),
+                              dev(torch.tensor(starts, dtype=torch.int32)), dev(torch.tensor(first, dtype=torch.int32)),
+                              dev(cache.table), heads, kv_heads, hd, scale, 0)
+    got = out.cpu()
+    assert _rel(got, want) < 1.2e-2
+    # row by row too: the first tokens of a prompt see few keys, their outputs are large and would hide a fault
+    # in a late row of small outputs
+    rows = (got.double() - want).abs().amax(dim=1) / want.abs().amax(dim=1)
+    assert float(rows.max()) < 3e-2, int(rows.argmax())
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

@@ -63,6 +63,82 @@ def test_real_layer_sizes_under_every_cut(real, dtype, tol):
     assert runner.cache.check() == ""
 
 
+def test_two_layers_at_the_7b_widths_in_32_bit_over_a_thousand_positions(tmp_path):
+    """Two layers of the benchmark's widths in true 32-bit arithmetic against the plain implementation's
+    float64: a prompt of 1,024 tokens in one step, then portions, then single tokens, 1,100 positions in all."""
+    from vipera_rs_amd.engine.batch import StepEntry
+    from vipera_rs_amd.engine.runner import ModelRunner
+    folder = make_folder(tmp_path / "two", dict(CONFIG_7B_LAYER, num_hidden_layers=2), 4, torch.float32)
+    cfg, w = P.load_folder(folder)
+    tokens = random_tokens(1000, 1100, 23)
+    want = P.forward(cfg, w, tokens, attend=P.attention_by_head)
+    del w
+    runner = ModelRunner.from_folder(folder, dtype="float32", block_size=16, num_blocks=72, num_slots=2)
+    rows, at = [], 0
+    for size in [1024, 40, 2, 17] + [1] * 17:
+        runner.cache.reserve(0, at, at + size)
+        rows.append(runner.step([StepEntry(0, at, tokens[at:at + size], list(range(size)))]).cpu().numpy())
+        at += size
+    assert at == len(tokens)
+    got = np.concatenate(rows)
+    assert rel_err(got, want) < 1e-4
+    worst = max(rel_err(got[t], want[t]) for t in range(len(tokens)))       # row by row as well
+    assert worst < 1e-4, worst
+
+
+CONFIG_BENCH_HEADS = {
+    "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2",
+    "num_hidden_layers": 2, "hidden_size": 256, "num_attention_heads": 28, "num_key_value_heads": 4, "head_dim": 128,
+    "intermediate_size": 512, "vocab_size": 300, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6,
+    "tie_word_embeddings": False, "max_position_embeddings": 8192, "hidden_act": "silu",
+}
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 1e-4), ("bfloat16", 3e-2)])
+def test_thousands_of_positions_at_the_benchmark_head_shape(tmp_path, dtype, tol):
+    """28 query heads over 4 key heads of width 128 (a narrow model otherwise, so that the plain implementation
+    stays affordable): a prompt of 2,030 tokens whole, then captured decode steps that cross 2,048 positions,
+    where the context bucket of the captured step and the number of chunks of the decode attention change,
+    beside a second, short request; then the same tokens as a second request in portions of 512."""
+    from vipera_rs_amd.engine.batch import StepEntry
+    from vipera_rs_amd.engine.runner import ModelRunner
+    stored = torch.float32 if dtype == "float32" else torch.bfloat16
+    folder = make_folder(tmp_path / "heads", CONFIG_BENCH_HEADS, 9, stored)
+    cfg, w = P.load_folder(folder)
+    tokens = random_tokens(300, 2075, 41)
+    short = random_tokens(300, 80, 42)
+    want = P.forward(cfg, w, tokens, attend=P.attention_by_head)
+    want_short = P.forward(cfg, w, short, attend=P.attention_by_head)
+    runner = ModelRunner.from_folder(folder, dtype=dtype, block_size=16, num_blocks=2 * 131 + 8, num_slots=4,
+                                     use_graphs=True, max_context=8192)
+    head = 2030
+    wanted = list(range(0, head, 97)) + list(range(head - 5, head))
+    runner.cache.reserve(0, 0, head)
+    runner.cache.reserve(1, 0, 35)
+    logits = runner.step([StepEntry(0, 0, tokens[:head], wanted), StepEntry(1, 0, short[:35], [34])]).cpu().numpy()
+    assert rel_err(logits[:-1], want[wanted]) < tol and rel_err(logits[-1], want_short[34]) < tol
+    for k in range(len(tokens) - head):           # single tokens of both requests, replayed as captured steps
+        at, at_short = head + k, 35 + k
+        runner.cache.reserve(0, at, at + 1)
+        runner.cache.reserve(1, at_short, at_short + 1)
+        logits = runner.step([StepEntry(1, at_short, [short[at_short]], [0]), StepEntry(0, at, [tokens[at]], [0])])
+        logits = logits.cpu().numpy()
+        assert rel_err(logits[1], want[at]) < tol, f"position {at}"
+        assert rel_err(logits[0], want_short[at_short]) < tol, f"position {at_short} of the short request"
+    assert {bucket for _, bucket in runner.graphs.graphs} == {2048, 4096}
+    runner.cache.release(0)
+    runner.cache.release(1)
+    at = 0
+    while at < len(tokens):                       # pages that the first request gave back
+        size = min(512, len(tokens) - at)
+        runner.cache.reserve(2, at, at + size)
+        rows = list(range(0, size, 61)) + [size - 1]
+        logits = runner.step([StepEntry(2, at, tokens[at:at + size], rows)]).cpu().numpy()
+        assert rel_err(logits, want[[at + r for r in rows]]) < tol, f"portion from {at}"
+        at += size
+    assert runner.cache.check() == ""
+
+
 CONFIG_SPLIT_NORMS = {
     "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2",
     "num_hidden_layers": 3, "hidden_size": 1024, "num_attention_heads": 4, "num_key_value_heads": 2, "head_dim": 128,

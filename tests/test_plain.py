@@ -128,6 +128,15 @@ def test_softmax_is_shift_invariant_and_causal():
     assert not np.allclose(P.attention(q, k, v, window=3)[5], out[5])
 
 
+def test_attention_by_head_is_the_same_function():
+    rng = np.random.default_rng(8)
+    q, k, v = rng.normal(size=(23, 6, 8)), rng.normal(size=(23, 2, 8)), rng.normal(size=(23, 2, 8))
+    for window in (0, 1, 5, 23, 40):
+        np.testing.assert_allclose(P.attention_by_head(q, k, v, window=window), P.attention(q, k, v, window=window),
+                                   rtol=1e-12, atol=1e-14)
+    np.testing.assert_allclose(P.attention_by_head(q, k, v, scale=0.3), P.attention(q, k, v, scale=0.3), rtol=1e-12)
+
+
 # --- the whole model ------------------------------------------------------------------------------------------
 @pytest.fixture(scope="module")
 def model_b(tmp_path_factory):
