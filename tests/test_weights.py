@@ -80,7 +80,7 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
     tensors = load_file(os.path.join(folder, "model.safetensors"))
     del tensors["model.layers.1.mlp.up_proj.weight"]
     del tensors["model.norm.weight"]
-    tensors["lm_head.weight"] = torch.zeros(256, 64)           # the configuration ties the embeddings
+    tensors["model.embed_positions.weight"] = torch.zeros(256, 64)   # nobody asked for it
     tensors["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(8)
     tensors["model.layers.0.self_attn.k_proj.weight"] = torch.zeros(64, 64)
     tensors["model.layers.0.self_attn.q_proj.bias"] = torch.zeros(32)
@@ -89,7 +89,7 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
         Checkpoint(folder).check(specs)
     e = err.value
     assert sorted(e.missing) == ["model.layers.1.mlp.up_proj.weight", "model.norm.weight"]
-    assert sorted(e.unexpected) == ["lm_head.weight", "model.layers.0.self_attn.rotary_emb.inv_freq"]
+    assert sorted(e.unexpected) == ["model.embed_positions.weight", "model.layers.0.self_attn.rotary_emb.inv_freq"]
     assert sorted(n for n, _, _ in e.wrong_shapes) == ["model.layers.0.self_attn.k_proj.weight",
                                                        "model.layers.0.self_attn.q_proj.bias"]
     text = str(e)
@@ -147,3 +147,41 @@ def test_a_bfloat16_folder(tmp_path):
     ck = Checkpoint(folder)
     assert {ck.info(n).dtype for n in ck.names()} == {"BF16"}
     ck.check(declare_model(config_from_dict(CONFIG_A)))
+
+
+def test_a_tied_model_may_hold_an_output_matrix_that_is_not_read(tmp_path):
+    cfg = config_from_dict(CONFIG_A)                        # tied embeddings
+    folder = make_folder(tmp_path / "m", CONFIG_A, 0)
+    specs = declare_model(cfg)
+    assert [s.name for s in specs if s.unused] == ["lm_head.weight"]
+    ck = Checkpoint(folder)
+    assert "lm_head.weight" not in ck.names()               # random weights do not write it
+    ck.check(specs)
+    tensors = {name: ck.read(name) for name in ck.names()}
+    ck.close()
+    tensors["lm_head.weight"] = tensors["model.embed_tokens.weight"].clone()
+    write_safetensors(os.path.join(folder, "model.safetensors"), tensors.items())
+    ck = Checkpoint(folder)
+    ck.check(specs)                                         # present: tolerated
+    ck.close()
+    tensors["lm_head.weight"] = torch.zeros(3, 64)
+    write_safetensors(os.path.join(folder, "model.safetensors"), tensors.items())
+    with pytest.raises(WeightsError) as err:
+        Checkpoint(folder).check(specs)                     # but it has to be the output matrix's shape
+    assert err.value.wrong_shapes == [("lm_head.weight", (3, 64), (256, 64))] and not err.value.unexpected
+
+
+def test_a_shard_index_may_only_name_files_of_its_folder(tmp_path):
+    folder = make_folder(tmp_path / "m", CONFIG_A, 0)
+    outside = tmp_path / "elsewhere.safetensors"
+    os.rename(os.path.join(folder, "model.safetensors"), outside)
+    index = os.path.join(folder, "model.safetensors.index.json")
+    for name in ("../elsewhere.safetensors", str(outside), "sub/../../elsewhere.safetensors", 7):
+        with open(index, "w") as handle:
+            json.dump({"weight_map": {"model.norm.weight": name}}, handle)
+        with pytest.raises(ParseError, match="does not name a file of this folder"):
+            Checkpoint(folder)
+    os.rename(outside, os.path.join(folder, "part-1.safetensors"))
+    with open(index, "w") as handle:
+        json.dump({"weight_map": {"model.norm.weight": "part-1.safetensors"}}, handle)
+    assert "model.norm.weight" in Checkpoint(folder).names()

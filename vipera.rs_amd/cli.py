@@ -199,6 +199,8 @@ def plan_model(folder: str, ctx: Optional[int], batch: int, dtype: str, block_si
     matrix_elements = 0
     head_elements = 0
     for spec in declare_model(config):
+        if spec.unused:
+            continue
         count = 1
         for dim in spec.shape:
             count *= dim

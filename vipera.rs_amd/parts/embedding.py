@@ -53,10 +53,10 @@ class LMHead(Part):
 
     @classmethod
     def declare(cls, spec: PartSpec, prefix: str) -> List[TensorSpec]:
-        if spec.params.get("tied_to"):
-            return []
+        # with tied embeddings a folder may still hold an output matrix (a copy of the table): it is not read
         return [TensorSpec(f"{prefix}{spec.params['name']}.weight",
-                           (int(spec.params["vocab"]), int(spec.params["width"])), MATRIX)]
+                           (int(spec.params["vocab"]), int(spec.params["width"])), MATRIX,
+                           unused=bool(spec.params.get("tied_to")))]
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         name = self.tied_to if self.tied_to else f"{self.prefix}{self.spec.params['name']}"

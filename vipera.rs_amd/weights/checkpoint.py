@@ -32,6 +32,7 @@ class TensorSpec:
     role: str = MATRIX
     init: str = "normal"      # "normal" N(0, std) | "one_plus_normal" 1 + N(0, std) | "zeros" | "ones"
     std: float = 0.02
+    unused: bool = False      # a folder may hold it, the model does not read it: its shape is checked, nothing is loaded
 
 
 class WeightsError(InvalidArgumentError):
@@ -73,7 +74,14 @@ class Checkpoint:
                 shard_names = sorted(set(index["weight_map"].values()))
             except (OSError, ValueError, KeyError, AttributeError, TypeError) as err:
                 raise ParseError(f"{index_path}: cannot read the shard index: {err}") from None
-            paths = [os.path.join(folder, name) for name in shard_names]
+            paths = []
+            root = os.path.realpath(folder)
+            for name in shard_names:
+                # a shard is a file of this folder: an index is not let to point anywhere else
+                path = os.path.realpath(os.path.join(root, name)) if isinstance(name, str) else ""
+                if not isinstance(name, str) or os.path.isabs(name) or os.path.dirname(path) != root:
+                    raise ParseError(f"{index_path}: shard name {name!r} does not name a file of this folder")
+                paths.append(path)
         else:
             raise IoError(f"{folder} holds neither model.safetensors nor model.safetensors.index.json")
         for path in paths:
@@ -98,7 +106,7 @@ class Checkpoint:
     def check(self, specs: Iterable[TensorSpec]) -> None:
         """Raise one :class:`WeightsError` that lists everything wrong, or return."""
         wanted = {spec.name: spec for spec in specs}
-        missing = [name for name in wanted if name not in self.tensors]
+        missing = [name for name, spec in wanted.items() if name not in self.tensors and not spec.unused]
         unexpected = [name for name in self.tensors if name not in wanted]
         wrong = []
         for name, spec in wanted.items():
@@ -136,6 +144,8 @@ def load_tensors(checkpoint: Checkpoint, specs: Sequence[TensorSpec], run_dtype:
     checkpoint.check(specs)
     out: Dict[str, torch.Tensor] = {}
     for spec in specs:
+        if spec.unused:
+            continue
         stored = checkpoint.read(spec.name)
         dtype = kept_dtype(spec, stored.dtype, run_dtype)
         if not (stored.dtype.is_floating_point or spec.role == INT_TABLE):

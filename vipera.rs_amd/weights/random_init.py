@@ -73,7 +73,8 @@ def random_tensor(spec: TensorSpec, seed: int, dtype: torch.dtype) -> torch.Tens
 
 def random_tensors(specs: Iterable[TensorSpec], seed: int, dtype: torch.dtype):
     for spec in specs:
-        yield spec.name, random_tensor(spec, seed, dtype)
+        if not spec.unused:
+            yield spec.name, random_tensor(spec, seed, dtype)
 
 
 def write_random_model(folder: str, config: ModelConfig, specs: Sequence[TensorSpec], seed: int,
@@ -100,6 +101,8 @@ def random_device_tensors(specs: Sequence[TensorSpec], seed: int, run_dtype: tor
 
     out: Dict[str, torch.Tensor] = {}
     for spec in specs:
+        if spec.unused:
+            continue
         dtype = kept_dtype(spec, run_dtype, run_dtype)
         tensor = torch.empty(spec.shape, dtype=dtype, device=device)
         if spec.role == INT_TABLE or spec.init == "zeros":
