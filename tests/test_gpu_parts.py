@@ -131,6 +131,8 @@ def _random_part_tensors(cls, spec, prefix, seed, runtime):
     from vipera_rs_amd.weights import kept_dtype, random_tensor
     host, device = {}, {}
     for t in cls.declare(spec, prefix):
+        if t.unused:      # a tensor a folder may hold but the part does not read
+            continue
         value = random_tensor(t, seed, torch.float32)
         kept = kept_dtype(t, torch.float32 if runtime.dtype == torch.float32 else torch.bfloat16, runtime.dtype)
         device[t.name] = value.to(kept).to(runtime.device)
@@ -458,6 +460,122 @@ def test_a_stateful_toy_mixer_generates_through_captured_steps_with_padding(tmp_
         planned = plan_model(folder, 64, 3, "float32", 8)
         assert planned["state_bytes"] == (3 + 1) * STATE_WIDTH * 4
         assert engine.stats()["kv_bytes"] == engine.runner.storage.bytes >= planned["state_bytes"]
+
+
+# --- an arrangement with four norms and an embedding that adds a learned position, defined here -------------------
+def test_a_block_with_four_norms_and_an_embedding_that_adds_positions(tmp_path):
+    """``x += norm_b(mixer(norm_a(x))); x += norm_d(ffn(norm_c(x)))`` with the two extra norms named in
+    ``LayerSpec.extras``, and ``x_0 = table[token] + places[position]``: another arrangement and another embedding
+    are registered from this file; the framework's blocks, models and step function are not touched."""
+    from vipera_rs_amd.config import (LayerSpec, PartSpec, Qwen2Config, register_architecture, unregister_architecture)
+    from vipera_rs_amd.engine.batch import StepEntry
+    from vipera_rs_amd.engine.runner import ModelRunner
+    from vipera_rs_amd.models.decoder import DecoderModel
+    from vipera_rs_amd.parts import Block, Part, part_class, register_block, register_embedding, unregister
+    from vipera_rs_amd.weights import MATRIX, TensorSpec
+
+    ROLES = ("mixer_norm", "after_mixer", "ffn_norm", "after_ffn")
+
+    class Sandwich(Block):
+        def __init__(self, spec, runtime):
+            super().__init__(spec, runtime)
+            norms = {"mixer_norm": spec.mixer_norm, "ffn_norm": spec.ffn_norm, **spec.extras}
+            self.norms = {role: part_class("norm", norms[role].kind)(norms[role], spec.prefix, runtime) for role in ROLES}
+            self.mixer = part_class("mixer", spec.mixer.kind)(spec.mixer, spec.prefix, runtime)
+            self.ffn = part_class("ffn", spec.ffn.kind)(spec.ffn, spec.prefix, runtime)
+            self.position = part_class("position", spec.position.kind)(spec.position, spec.prefix, runtime)
+
+        @classmethod
+        def declare(cls, spec):
+            norms = {"mixer_norm": spec.mixer_norm, "ffn_norm": spec.ffn_norm, **spec.extras}
+            out = []
+            for role in ROLES:
+                out += part_class("norm", norms[role].kind).declare(norms[role], spec.prefix)
+            out += part_class("mixer", spec.mixer.kind).declare(spec.mixer, spec.prefix)
+            out += part_class("ffn", spec.ffn.kind).declare(spec.ffn, spec.prefix)
+            return out
+
+        def load(self, tensors):
+            for part in (*self.norms.values(), self.mixer, self.ffn, self.position):
+                part.load(tensors)
+
+        def forward(self, x, batch, cache, state, reads_only=False):
+            # a part adds its output into the 32-bit buffer it is given: an empty one collects the output alone
+            branch = torch.zeros_like(x)
+            self.mixer.forward(self.norms["mixer_norm"].forward(x), batch, cache, state, self.position, branch, reads_only)
+            x += self.norms["after_mixer"].forward(branch).float()
+            branch.zero_()
+            self.ffn.forward(self.norms["ffn_norm"].forward(x), batch, branch)
+            x += self.norms["after_ffn"].forward(branch).float()
+
+    class PlacedEmbedding(Part):
+        reads_device_tokens = False
+
+        @classmethod
+        def declare(cls, spec, prefix):
+            p = spec.params
+            return [TensorSpec("model.embed_tokens.weight", (p["vocab"], p["width"]), MATRIX),
+                    TensorSpec("model.embed_places.weight", (p["places"], p["width"]), MATRIX, std=0.05)]
+
+        def load(self, tensors):
+            self.table = tensors["model.embed_tokens.weight"]
+            self.places = tensors["model.embed_places.weight"]
+
+        def embed(self, batch):
+            return (self.table[batch.tokens[:batch.num_tokens].long()].float()
+                    + self.places[batch.positions[:batch.num_tokens].long()].float())
+
+    class SandwichConfig(Qwen2Config):
+        architecture = "ToySandwichForCausalLM"
+
+        def layer_specs(self) -> List[LayerSpec]:
+            out = []
+            for spec in super().layer_specs():
+                norm = spec.mixer_norm.params
+                extras = {"after_mixer": PartSpec("rmsnorm", dict(norm, name="post_mixer_norm")),
+                          "after_ffn": PartSpec("rmsnorm", dict(norm, name="post_ffn_norm"))}
+                out.append(LayerSpec("sandwich", spec.mixer, spec.ffn, spec.mixer_norm, spec.ffn_norm, spec.position,
+                                     spec.prefix, extras))
+            return out
+
+        def embedding_spec(self):
+            return PartSpec("placed", {"vocab": self.vocab_size, "width": self.hidden_size, "places": 96})
+
+    def plain(cfg, w, tokens):
+        cfg = P.normalize_config(cfg)
+        eps = cfg["rms_norm_eps"]
+        x = w["model.embed_tokens.weight"][np.asarray(tokens)] + w["model.embed_places.weight"][:len(tokens)]
+        for i in range(cfg["num_hidden_layers"]):
+            p = f"model.layers.{i}."
+            h = P.rms_norm(x, w[p + "input_layernorm.weight"], eps)
+            x = x + P.rms_norm(P.attention_block(h, w, p + "self_attn.", cfg, 0), w[p + "post_mixer_norm.weight"], eps)
+            h = P.rms_norm(x, w[p + "post_attention_layernorm.weight"], eps)
+            y = P.swiglu_mlp(h, *(w[f"{p}mlp.{n}_proj.weight"] for n in ("gate", "up", "down")))
+            x = x + P.rms_norm(y, w[p + "post_ffn_norm.weight"], eps)
+        return P.linear(P.rms_norm(x, w["model.norm.weight"], eps), w["lm_head.weight"])
+
+    register_block("sandwich", Sandwich)
+    register_embedding("placed", PlacedEmbedding)
+    register_architecture("ToySandwichForCausalLM", SandwichConfig, lambda config, runtime: DecoderModel(config, runtime))
+    try:
+        config = dict(CONFIG_B, architectures=["ToySandwichForCausalLM"])
+        for dtype, stored, tol in (("float32", torch.float32, 1e-4), ("bfloat16", torch.bfloat16, 3e-2)):
+            folder = make_folder(tmp_path / f"sandwich_{dtype}", config, 12, stored)
+            cfg, w = P.load_folder(folder)
+            assert "model.layers.2.post_ffn_norm.weight" in w and "model.embed_places.weight" in w
+            tokens = random_tokens(300, 60, 77)
+            want = plain(cfg, w, tokens)
+            runner = ModelRunner.from_folder(folder, dtype=dtype, block_size=8, num_blocks=12, num_slots=2)
+            rows, at = [], 0
+            for size in (23, 2, 1, 17, 1, 1, 15):
+                runner.cache.reserve(0, at, at + size)
+                rows.append(runner.step([StepEntry(0, at, tokens[at:at + size], list(range(size)))]).cpu().numpy())
+                at += size
+            assert at == len(tokens) and rel_err(np.concatenate(rows), want) < tol, dtype
+    finally:
+        unregister_architecture("ToySandwichForCausalLM")
+        unregister("block", "sandwich")
+        unregister("embedding", "placed")
 
 
 # --- a feed-forward with routing and another position encoding, defined here --------------------------------------

@@ -38,7 +38,10 @@ class LayerSpec:
 
     ``block`` names the arrangement of the parts (for example ``"prenorm"``:
     ``x += mixer(norm(x)); x += ffn(norm(x))``).  ``prefix`` is the tensor-name
-    prefix under which the layer's weights are stored.
+    prefix under which the layer's weights are stored.  ``extras`` holds further
+    parts by a role name for arrangements that have more than these five (norms
+    after the mixer and the feed-forward, say); a block kind defines which roles
+    it reads and of which family (norm, mixer, ...) each is.
     """
 
     block: str
@@ -48,6 +51,7 @@ class LayerSpec:
     ffn_norm: PartSpec
     position: PartSpec
     prefix: str
+    extras: Dict[str, PartSpec] = field(default_factory=dict)
 
 
 @dataclass(frozen=True)

@@ -117,10 +117,7 @@ class DecoderModel:
         # what parts share within a step is computed anew in every run: a run that is being captured into a graph
         # must launch it too, or the graph would replay with what an earlier run left
         batch.shared.clear()
-        if batch.sampled_tokens is not None and batch.token_source is not None:  # ids the sampler left on the device
-            x = self.embedding.forward(batch.tokens, batch.num_tokens, batch.token_source, batch.sampled_tokens)
-        else:
-            x = self.embedding.forward(batch.tokens, batch.num_tokens)
+        x = self.embedding.embed(batch)
         tokens = x.shape[0]
         incoming = None
         for index, entry in enumerate(self.schedule):

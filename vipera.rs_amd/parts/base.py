@@ -18,7 +18,13 @@ Kinds of parts and what each must provide:
                       ``forward(h, batch, cache, state, position, residual, reads_only)`` adds its
                       output to ``residual`` (32-bit, in place).
 ``FeedForward``       ``forward(h, batch, residual)`` adds its output to ``residual``.
-``Block``             ``forward(x, batch, cache, state, reads_only)`` runs its parts on the residual ``x``.
+``Block``             ``forward(x, batch, cache, state, reads_only)`` runs its parts on the residual ``x``;
+                      it has a ``mixer`` attribute (the part whose cache the model provides) and may
+                      read further parts from ``LayerSpec.extras``.
+embedding             ``embed(batch) -> x``: the 32-bit residual ``[tokens, width]`` a step starts from
+                      (the batch brings tokens and positions); ``reads_device_tokens`` says whether it
+                      takes token ids that the sampler left on the device (``batch.token_source``).
+head                  ``forward(h) -> logits`` (32-bit) and ``vocab``.
 """
 from __future__ import annotations
 

@@ -34,6 +34,13 @@ class Embedding(Part):
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         self.table = tensors[f"{self.prefix}{self.spec.params['name']}.weight"]
 
+    def embed(self, batch) -> torch.Tensor:
+        """The 32-bit residual ``[tokens, width]`` a step starts from.  An embedding sees the whole batch, so one
+        that adds something by position (``batch.positions``) needs nothing else."""
+        if batch.sampled_tokens is not None and batch.token_source is not None:  # ids the sampler left on the device
+            return self.forward(batch.tokens, batch.num_tokens, batch.token_source, batch.sampled_tokens)
+        return self.forward(batch.tokens, batch.num_tokens)
+
     def forward(self, tokens: torch.Tensor, count: int, source: Optional[torch.Tensor] = None,
                 sampled: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Rows of the table for ``tokens``; where ``source`` is not negative the id is read from
