@@ -396,10 +396,11 @@ extern "C" int plain_attn_bf16_decode(const void* q, long long q_stride, const v
                                       void* out, float*, const int* entries, int num_entries, const int* entry_start,
                                       const int* entry_first_pos, const int* block_table, int table_width,
                                       int block_size, int heads, int kv_heads, int hd, float scale, int window, int,
-                                      int, void*) {
+                                      int, int dense, void*) {
   if (hd <= 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads || block_size <= 0 || window < 0) return BAD_ARGUMENT;
   for (int e = 0; e < num_entries; ++e) {
-    const int entry = entries[e], t = entry_start[entry];
+    // dense: entry e is the e-th single-token entry and holds token e
+    const int entry = dense ? e : entries[e], t = dense ? e : entry_start[entry];
     for (int h = 0; h < heads; ++h)
       attend((const uint16_t*)q + (size_t)t * q_stride + (size_t)h * hd, k_cache, v_cache, DT_BF16,
              block_table + (size_t)entry * table_width, block_size, kv_heads, h / (heads / kv_heads), hd, scale,

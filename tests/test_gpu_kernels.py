@@ -306,9 +306,11 @@ def test_decode_attention_over_thousands_of_positions(window):
         chunks = (longest + chunk - 1) // chunk
         out = torch.zeros(len(lengths), heads * hd, dtype=dtype, device=DEV)
         partial = torch.empty(len(lengths) * heads * chunks * (hd + 2), device=DEV)
-        kernels.attn_bf16_decode(qkv_d, k_d, v_d, out, partial, singles, es, fp, table_d, heads, kv_heads, hd, scale,
-                                 window, chunk, chunks)
-        assert _rel(out.cpu(), want) < 1.2e-2, f"chunk {chunk}"
+        for dense in (False, True):
+            out = torch.zeros(len(lengths), heads * hd, dtype=dtype, device=DEV)
+            kernels.attn_bf16_decode(qkv_d, k_d, v_d, out, partial, singles, es, fp, table_d, heads, kv_heads, hd, scale,
+                                     window, chunk, chunks, dense=dense)
+            assert _rel(out.cpu(), want) < 1.2e-2, f"chunk {chunk}, dense {dense}"
 
 
 def _plain_attention_by_head(q, k, v, first_pos, window, scale):
@@ -394,6 +396,11 @@ def test_decode_attention_at_the_benchmark_head_shapes(heads, kv_heads, hd, batc
         kernels.attn_bf16_decode(qkv_d, k_d, v_d, out, partial, singles, es, fp, dev(table), heads, kv_heads, hd, scale, 0,
                                  chunk, chunks)
         assert _rel(out.cpu(), want) < 1.2e-2, f"visible {visible}: chunk {chunk} x {chunks}"
+        # a step of single tokens only: the kernel is told that entry i is slot i and token i and looks neither up
+        dense = torch.zeros(batch, heads * hd, dtype=dtype, device=DEV)
+        kernels.attn_bf16_decode(qkv_d, k_d, v_d, dense, partial, singles, es, fp, dev(table), heads, kv_heads, hd, scale, 0,
+                                 chunk, chunks, dense=True)
+        assert torch.equal(dense, out)
     out = torch.zeros(batch, heads * hd, dtype=dtype, device=DEV)
     kernels.attn_generic(qkv_d, k_d, v_d, out, fp, singles, dev(cache.table), heads, kv_heads, hd, scale, 0)
     assert _rel(out.cpu(), want) < 1.2e-2, "32-bit-arithmetic kernel on the bfloat16 cache"

@@ -14,10 +14,13 @@
 // of v_mfma_f32_16x16x32_bf16 (a lane holds 8 consecutive k of one row) is how K lies in the cache,
 // [page, kv_head, slot, head_dim], and V is cached transposed, [page, kv_head, head_dim, slot], so
 // that a lane reads consecutive positions of one output dim.
-//     S^T = K Q^T : lane (c = l % 16, g = l / 16), register j  <->  S[position 4g + j of a 16-tile][column c]
-//     O^T = V^T P : the 32 positions of a step feed the instruction in the order the scores arrive in
-//                   (slot 8g + i <-> position 4g + i for i < 4, 16 + 4g + i - 4 for i >= 4); V is read in
-//                   that same order, and a sum does not care how its terms are numbered.
+//     S^T = K Q^T : lane (c = l % 16, g = l / 16), register j  <->  S[row 4g + j of a 16-row tile][column c]
+//     O^T = V^T P : the 32 positions of a step feed the instruction in the order the scores arrive in, and a
+//                   sum does not care how its terms are numbered. Prompts: row r of tile t is position 16t + r
+//                   (slot 8g + i <-> position 4g + i for i < 4, 16 + 4g + i - 4 for i >= 4), and the V^T tile
+//                   is laid out in LDS in that order. Decoding: which position a K row holds is free, since every
+//                   lane fetches its own row: row 4g + j of tile t is position 8g + 4t + j, so that a lane's eight
+//                   weights are the eight consecutive positions 8g .. 8g + 7 and its V^T operand one 16-byte read.
 // The softmax is online over steps of 32 positions that start at multiples of 32, so a token's
 // arithmetic depends on its position and the cache only.
 #include "common.h"
@@ -75,8 +78,8 @@ __device__ __forceinline__ int page_of(const CacheView& cv, int p) {
 
 // The K and V^T operands of one step of 32 positions.
 struct StepOperands {
-  bf16x8 kf[2][KS];  // two 16-position tiles of K
-  bf16x8 vf[DT];     // V^T: positions kb + 4g .. +3 and kb + 16 + 4g .. +3 of output dim 16 dt + lr
+  bf16x8 kf[2][KS];  // two 16-row tiles of K: row r of tile t is position kb + 8 (r / 4) + 4 t + r % 4
+  bf16x8 vf[DT];     // V^T: positions kb + 8g .. +7 of output dim 16 dt + lr
 };
 
 // Issue the loads of the step that starts at kb. No load sits behind a branch (the compiler can then
@@ -92,7 +95,7 @@ __device__ __forceinline__ void load_step(int kb, int begin, int end, const Cach
   const int bs = cv.ps.size, hd = cv.hd;
 #pragma unroll
   for (int sub = 0; sub < 2; ++sub) {
-    const int p = min(max(kb + sub * 16 + lr, begin), end - 1);
+    const int p = min(max(kb + (lr >> 2) * 8 + sub * 4 + (lr & 3), begin), end - 1);
     const int page = max(page_of<REGS>(cv, p), 0);
     const __bf16* row = cv.k + (((size_t)page * cv.kv_heads + cv.kvh) * bs + cv.ps.slot(p)) * hd;
 #pragma unroll
@@ -101,26 +104,14 @@ __device__ __forceinline__ void load_step(int kb, int begin, int end, const Cach
       r.kf[sub][ks] = *(const bf16x8*)(row + (dim < hd ? dim : 0));
     }
   }
-  const __bf16* vrow[2];
-#pragma unroll
-  for (int half = 0; half < 2; ++half) {
-    // groups of four positions start at multiples of 4 and lie in one page (4 divides the page size)
-    const int p = min(max(kb + half * 16 + lg * 4, begin & ~3), (end - 1) & ~3);
-    const int page = max(page_of<REGS>(cv, p), 0);
-    vrow[half] = cv.v + (((size_t)page * cv.kv_heads + cv.kvh) * hd) * bs + cv.ps.slot(p);
-  }
+  // groups of eight positions start at multiples of 8 and lie in one page (8 divides the page size)
+  const int pv = min(max(kb + lg * 8, begin & ~7), (end - 1) & ~7);
+  const int vpage = max(page_of<REGS>(cv, pv), 0);
+  const __bf16* vrow = cv.v + (((size_t)vpage * cv.kv_heads + cv.kvh) * hd) * bs + cv.ps.slot(pv);
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) {
     const int d = dt * 16 + lr;
-    const size_t offset = (size_t)(d < hd ? d : 0) * bs;
-    const bf16x4 x0 = *(const bf16x4*)(vrow[0] + offset), x1 = *(const bf16x4*)(vrow[1] + offset);
-    bf16x8 f;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      f[i] = x0[i];
-      f[4 + i] = x1[i];
-    }
-    r.vf[dt] = f;
+    r.vf[dt] = *(const bf16x8*)(vrow + (size_t)(d < hd ? d : 0) * bs);
   }
 }
 
@@ -157,7 +148,7 @@ __device__ __forceinline__ void attend_range(const bf16x8 (&qf)[KS], int col_lo,
     for (int sub = 0; sub < 2; ++sub)
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const int p = kb + sub * 16 + lg * 4 + j;
+        const int p = kb + lg * 8 + sub * 4 + j;
         const bool visible = p >= col_lo && p <= col_pos && p >= begin && p < end;
         const float x = visible ? s[sub][j] * scale : -INFINITY;
         sv[sub * 4 + j] = x;
@@ -473,12 +464,19 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void at
     const __bf16* __restrict__ v_cache, float* __restrict__ partial, const int* __restrict__ entries,
     const int* __restrict__ entry_start, const int* __restrict__ entry_first_pos,
     const int* __restrict__ block_table, int table_width, int block_size, int heads, int kv_heads, int hd,
-    float scale, int window, int chunk, int head_blocks) {
+    float scale, int window, int chunk, int head_blocks, int dense) {
   const int lane = threadIdx.x & 63, lr = lane & 15, lg = lane >> 4;
-  const int slot = blockIdx.x, entry = entries[slot];
+  // dense: entry i is slot i and holds token i (a step of single tokens only), which saves two reads that the
+  // position, and with it every other read, would wait for
+  const int slot = blockIdx.x, entry = dense ? slot : entries[slot];
   const int kvh = blockIdx.y / head_blocks, hb = blockIdx.y % head_blocks;
   const int group = heads / kv_heads;
-  const int token = entry_start[entry];
+  const int token = dense ? slot : entry_start[entry];
+  const PageSize ps(block_size);
+  // without a window a chunk's first page does not depend on the position: its page ids are asked for beside it
+  int early_pages = -1;
+  if (REGS && window == 0)
+    early_pages = block_table[(size_t)entry * table_width + min(ps.page(blockIdx.z * chunk) + lane, table_width - 1)];
   const int pos = entry_first_pos[entry];
   const int lo = (window > 0 && pos + 1 > window) ? pos + 1 - window : 0;
   const int begin = max(lo, blockIdx.z * chunk), end = min(pos + 1, (blockIdx.z + 1) * chunk);
@@ -495,10 +493,9 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void at
   }
   bf16x8 qf[KS];
   load_q(col_ok ? q + (size_t)token * q_stride + (size_t)h * hd : nullptr, hd, qf);
-  const PageSize ps(block_size);
   CacheView cv{k_cache, v_cache, block_table + (size_t)entry * table_width, table_width, ps,
-               kv_heads, hd, kvh, ps.page(begin), -1};
-  if (REGS) {
+               kv_heads, hd, kvh, ps.page(begin), early_pages};
+  if (REGS && window != 0) {
     const int index = cv.page0 + lane;
     if (index <= ps.page(end - 1) && index < table_width) cv.pages = cv.table[index];
   }
@@ -661,7 +658,7 @@ extern "C" int vk_attn_bf16_decode(const void* q, long long q_stride, const void
                                    void* out, float* partial, const int* entries, int num_entries,
                                    const int* entry_start, const int* entry_first_pos, const int* block_table,
                                    int table_width, int block_size, int heads, int kv_heads, int hd, float scale,
-                                   int window, int chunk, int chunks, void* stream) {
+                                   int window, int chunk, int chunks, int dense, void* stream) {
   if (num_entries <= 0) return 0;
   if (hd <= 0 || hd > HDP || (hd & 7) || block_size <= 0 || (block_size & 7) || heads <= 0 || kv_heads <= 0 ||
       heads % kv_heads || (q_stride & 7) || window < 0 || chunk < 32 || (chunk & 31) || chunks <= 0 ||
@@ -676,7 +673,7 @@ extern "C" int vk_attn_bf16_decode(const void* q, long long q_stride, const void
   auto kernel = chunk_pages <= 64 ? attn_decode_kernel<true> : attn_decode_kernel<false>;
   kernel<<<grid, 64, 0, s>>>((const __bf16*)q, q_stride, (const __bf16*)k_cache, (const __bf16*)v_cache, partial,
                              entries, entry_start, entry_first_pos, block_table, table_width, block_size, heads,
-                             kv_heads, hd, scale, window, chunk, head_blocks);
+                             kv_heads, hd, scale, window, chunk, head_blocks, dense);
   VK_LAUNCH_CHECK();
   dim3 cgrid(num_entries, heads);
   attn_combine_kernel<<<cgrid, 64, 0, s>>>(partial, (__bf16*)out, entries, entry_start, heads, hd, chunks);

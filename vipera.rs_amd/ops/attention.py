@@ -44,7 +44,7 @@ def paged_attention(qkv, k_cache, v_cache, out, batch, table, heads, kv_heads, h
                                   device=qkv.device)
             kernels.attn_bf16_decode(qkv, k_cache, v_cache, out, partial, batch.decode_entries, batch.entry_start,
                                      batch.entry_first_pos, table, heads, kv_heads, head_dim, scale, window, chunk,
-                                     chunks)
+                                     chunks, dense=batch.all_single)
         return
     kernels.attn_generic(qkv, k_cache, v_cache, out, batch.positions, batch.entry_of_token, table, heads, kv_heads,
                          head_dim, scale, window)

@@ -586,8 +586,10 @@ def attn_bf16_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
 def attn_bf16_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
                      partial: torch.Tensor, entries: torch.Tensor, entry_start: torch.Tensor,
                      entry_first_pos: torch.Tensor, block_table: torch.Tensor, heads: int, kv_heads: int,
-                     head_dim: int, scale: float, window: int, chunk: int, chunks: int) -> None:
-    """Attention of the single-token entries listed in ``entries``, positions split into ``chunks`` of ``chunk``."""
+                     head_dim: int, scale: float, window: int, chunk: int, chunks: int, dense: bool = False) -> None:
+    """Attention of the single-token entries listed in ``entries``, positions split into ``chunks`` of ``chunk``.
+    ``dense``: the step holds single-token entries only, so entry i is the i-th of them and holds token i; the
+    kernel then need not look either up."""
     _dev(q, k_cache, v_cache, out, partial, entries, entry_start, entry_first_pos, block_table)
     _need(attn_bf16_supported(q, k_cache, head_dim), "attn_bf16: operands must be bfloat16 with 16-byte rows")
     _need(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= heads * head_dim, "attention: q")
@@ -601,10 +603,11 @@ def attn_bf16_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(), "attention: table")
     module = f"attn_bf16_hd{attn_bf16_padded_width(head_dim)}"
     fn = _fn(module, "vk_attn_bf16_decode",
-             [_p, _ll, _p, _p, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _f, _i, _i, _i, _p], key=module + ".decode")
+             [_p, _ll, _p, _p, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _f, _i, _i, _i, _i, _p], key=module + ".decode")
     _status(fn(_ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(partial), _ptr(entries), count,
                _ptr(entry_start), _ptr(entry_first_pos), _ptr(block_table), block_table.shape[1], k_cache.shape[2],
-               heads, kv_heads, head_dim, float(scale), int(window), int(chunk), int(chunks), _stream()),
+               heads, kv_heads, head_dim, float(scale), int(window), int(chunk), int(chunks), 1 if dense else 0,
+               _stream()),
             "attn_bf16_decode")
 
 
