@@ -67,7 +67,7 @@ def test_gemm_bf16_every_tiling_of_the_tiled_kernel(tiling, ranges):
         kernels.gemm_bf16_force_tiling(-1)
 
 
-@pytest.mark.parametrize("tiling", [0, 2, 3, 4, 9, 7, 8, 5])
+@pytest.mark.parametrize("tiling", [0, 2, 3, 4, 9, 7, 8, 5, 10, 11, 12])   # the last three: 128 tokens x 96, 160, 224 rows
 def test_gated_product_with_every_tiling(tiling):
     from vipera_rs_amd.ops import kernels
     from vipera_rs_amd.ops.linear import interleave_gate_up

@@ -1553,7 +1553,8 @@ int launch_tile_as(const __bf16* A, const __bf16* W, const float* bias, TC* C, i
   return 0;
 }
 
-int g_tile_config = -1;  // -1: chosen by shape; else 10 * ranges + tiling (see launch_tile) forces a plan, for measurements
+int g_tile_config = -1;  // -1: chosen by shape; else a tiling (see launch_tile) and g_tile_ranges force a plan, for measurements
+int g_tile_ranges = 1;
 
 // Which tiling, and into how many ranges K is split: the pair with the shortest estimated time. A full GPU
 // of 256x256 tiles runs at about 1.15 PFLOP/s with the kernel that loads straight into LDS and at 1.0
@@ -1567,7 +1568,7 @@ int g_tile_config = -1;  // -1: chosen by shape; else 10 * ranges + tiling (see 
 // Ties go to the larger tile and to fewer ranges.
 struct TilePlan { int config, ranges; };
 int g_compute_units = 0;
-TilePlan choose_tile_plan(int M, int N, int K, long long partial_floats, bool direct) {
+TilePlan choose_tile_plan(int M, int N, int K, long long partial_floats, bool direct, bool gated = false) {
   if (g_compute_units == 0) {
     int device = 0, count = 0;
     if (hipGetDevice(&device) != hipSuccess ||
@@ -1577,13 +1578,17 @@ TilePlan choose_tile_plan(int M, int N, int K, long long partial_floats, bool di
   }
   struct Tiling { int config, tokens, rows, resident; double speed; };
   static const Tiling staged[] = {{4, 256, 256, 1, 1.0}, {2, 256, 128, 1, 0.8}, {3, 128, 256, 1, 0.8}, {0, 128, 128, 2, 0.75}};
+  // the last three (the gated product of up to 128 tokens only): the weight of a feed-forward has so many rows
+  // that with 128 of them a tile the tiles come in more than one round and less than two (7B width at 64 tokens:
+  // 296 tiles of 128 rows, two to a CU on 40 CUs, one on the others); a width of 96, 160 or 224 rows can come
+  // close to one tile per CU (237 tiles of 160 rows)
   static const Tiling straight[] = {{5, 256, 256, 1, 1.15}, {7, 256, 128, 1, 0.92}, {8, 128, 256, 1, 0.88}, {9, 128, 128, 2, 0.9},
-                                    {6, 256, 192, 1, 1.05}};
+                                    {6, 256, 192, 1, 1.05}, {10, 128, 96, 2, 0.85}, {11, 128, 160, 2, 0.88}, {12, 128, 224, 1, 0.88}};
   const Tiling* tilings = direct ? straight : staged;
   TilePlan best{tilings[3].config, 1};
   double best_time = 1e30;
   const double flops = 2.0 * M * N * (double)K, output_bytes = 4.0 * M * N;
-  for (int i = 0; i < (direct ? 5 : 4); ++i) {
+  for (int i = 0; i < (direct ? (gated && M <= 128 ? 8 : 5) : 4); ++i) {
     const Tiling& t = tilings[i];
     if (M <= 128 && t.tokens > 128) continue;
     if (M > 128 && t.tokens == 128 && t.rows == 256) continue;  // with many tokens the wide side goes to the tokens
@@ -1612,15 +1617,26 @@ template <typename TC, bool ACC, bool GATED = false>
 int launch_tile(const __bf16* A, const __bf16* W, const float* bias, TC* C, int M, int N, int K, long long lda,
                 long long ldc, int vector_ok, float* partial, long long partial_floats, hipStream_t s) {
   const bool direct = (K & 63) == 0;
-  TilePlan plan = choose_tile_plan(M, N, K, (GATED || !partial) ? 0 : partial_floats, direct);
-  if (g_tile_config >= 0) plan = TilePlan{g_tile_config % 10, g_tile_config >= 10 && !GATED && partial ? g_tile_config / 10 : 1};
+  TilePlan plan = choose_tile_plan(M, N, K, (GATED || !partial) ? 0 : partial_floats, direct, GATED);
+  if (g_tile_config >= 0) plan = TilePlan{g_tile_config, g_tile_ranges > 1 && !GATED && partial ? g_tile_ranges : 1};
   if (plan.ranges > 1 && (long long)plan.ranges * M * N > partial_floats) plan.ranges = 1;
+  if (plan.config >= 10 && !GATED) plan.config = 9;   // the narrow tiles exist for the gated product only
   if (!direct) {
-    switch (plan.config) { case 5: case 6: plan.config = 4; break; case 7: plan.config = 2; break; case 8: plan.config = 3; break; case 9: plan.config = 0; break; }
+    switch (plan.config) { case 5: case 6: plan.config = 4; break; case 7: plan.config = 2; break; case 8: plan.config = 3; break;
+                           case 9: case 10: case 11: case 12: plan.config = 0; break; }
   }
   const int r = plan.ranges;
 #define VK_TILE(BMV, BNV, WMV, WNV, DIRECTV) \
   return launch_tile_as<BMV, BNV, WMV, WNV, TC, ACC, GATED, DIRECTV>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, r, partial, s)
+  if constexpr (GATED) {
+    switch (plan.config) {
+      // four waves side by side along the tokens: a wave owns all rows of the tile, an even number of 16-row
+      // tiles, so gate and up rows of the same outputs meet in one wave
+      case 10: VK_TILE(128, 96, 4, 1, true);
+      case 11: VK_TILE(128, 160, 4, 1, true);
+      case 12: VK_TILE(128, 224, 4, 1, true);
+    }
+  }
   switch (plan.config) {
     case 5: VK_TILE(256, 256, 4, 2, true);
     case 6: VK_TILE(256, 192, 4, 2, true);
@@ -1925,7 +1941,8 @@ extern "C" int vk_gemm_bf16_gated_scaled(const void* A, const void* W, void* C, 
                                      (hipStream_t)stream);
 }
 
-extern "C" int vk_gemm_bf16_tile_config(int config) {
-  g_tile_config = config;
+extern "C" int vk_gemm_bf16_tile_config(int tiling, int ranges) {
+  g_tile_config = tiling;
+  g_tile_ranges = ranges;
   return 0;
 }

@@ -536,7 +536,8 @@ def gemm_bf16_gated_scaled(scaled: torch.Tensor, w: torch.Tensor, out: torch.Ten
 
 
 TILE_TILINGS = {0: "128x128 staged", 2: "256x128 staged", 3: "128x256 staged", 4: "256x256 staged",
-                9: "128x128 direct", 7: "256x128 direct", 8: "128x256 direct", 5: "256x256 direct", 6: "256x192 direct"}
+                9: "128x128 direct", 7: "256x128 direct", 8: "128x256 direct", 5: "256x256 direct", 6: "256x192 direct",
+                10: "128x96 direct, gated only", 11: "128x160 direct, gated only", 12: "128x224 direct, gated only"}
 
 
 def gemm_bf16_force_tiling(tiling: int = -1, ranges: int = 1) -> None:
@@ -545,8 +546,8 @@ def gemm_bf16_force_tiling(tiling: int = -1, ranges: int = 1) -> None:
     to the launcher.  A "direct" tiling falls back to its staged twin when K is no multiple of 64."""
     if tiling >= 0:
         _need(tiling in TILE_TILINGS and 1 <= ranges <= 8, "gemm_bf16_force_tiling: unknown tiling or ranges")
-    fn = _fn("gemm_bf16", "vk_gemm_bf16_tile_config", [_i])
-    _status(fn(-1 if tiling < 0 else (10 * ranges if ranges > 1 else 0) + tiling), "gemm_bf16_force_tiling")
+    fn = _fn("gemm_bf16", "vk_gemm_bf16_tile_config", [_i, _i])
+    _status(fn(-1 if tiling < 0 else tiling, int(ranges)), "gemm_bf16_force_tiling")
 
 
 # ----------------------------------------------------------------------------------------------
