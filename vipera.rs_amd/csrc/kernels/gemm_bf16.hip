@@ -1432,6 +1432,33 @@ __global__ __launch_bounds__(256) void gemm_reduce_rope_kernel(const float* __re
   }
 }
 
+// The kernel that adds the `used` K ranges of a split product of up to 64 tokens: the plain sum, or the sum that also
+// prepares the norm after the residual (`follow`), or the one that rotates q and k and writes the cache (`rope`).
+template <typename TC, bool ACC>
+int reduce_ranges(const float* partial, const float* bias, TC* C, int M, int N, int K, long long ldc, int used,
+                  int vector_ok, hipStream_t s, const FollowNorm* follow, const ReduceRope* rope) {
+  if constexpr (ACC && sizeof(TC) == 4) {
+    if (follow) {
+      gemm_reduce_follow_kernel<<<dim3((N + 1023) / 1024, M), 256, 0, s>>>(partial, bias, (float*)C, M, N, ldc, used,
+                                                                           (N & 3) == 0 ? 1 : 0, *follow);
+      VK_LAUNCH_CHECK();
+      return 0;
+    }
+  }
+  if constexpr (!ACC && sizeof(TC) == 2) {
+    if (rope) {
+      const int units = (rope->r.heads + rope->r.kv_heads) * (rope->r.hd / 8) + rope->r.kv_heads * (rope->r.hd / 4);
+      gemm_reduce_rope_kernel<<<dim3((units + 255) / 256, M), 256, 0, s>>>(partial, bias, (__bf16*)C, M, N, K, ldc, used, *rope);
+      VK_LAUNCH_CHECK();
+      return 0;
+    }
+  }
+  const long long threads = (long long)M * ((N + 3) / 4);
+  gemm_reduce_kernel<TC, ACC><<<(int)((threads + 255) / 256), 256, 0, s>>>(partial, bias, C, M, N, ldc, used, vector_ok);
+  VK_LAUNCH_CHECK();
+  return 0;
+}
+
 template <int CB, int RT, typename TC, bool ACC>
 int launch_mid_as(const __bf16* A, const __bf16* W, const float* bias, TC* C, float* partial, long long partial_floats,
                   int ranges, int forced_rows, int M, int N, int K, long long lda, long long ldc, int vector_ok,
@@ -1464,26 +1491,7 @@ int launch_mid_as(const __bf16* A, const __bf16* W, const float* bias, TC* C, fl
   kernel<<<dim3(blocks, used), 256, lds_bytes, s>>>(A, W, nullptr, partial, M, N, K, lda, N, k_per_range,
                                                     (long long)M * N, (N & 3) == 0 ? 1 : 0, rows);
   VK_LAUNCH_CHECK();
-  if constexpr (ACC && sizeof(TC) == 4) {
-    if (follow) {
-      gemm_reduce_follow_kernel<<<dim3((N + 1023) / 1024, M), 256, 0, s>>>(partial, bias, (float*)C, M, N, ldc, used,
-                                                                           (N & 3) == 0 ? 1 : 0, *follow);
-      VK_LAUNCH_CHECK();
-      return 0;
-    }
-  }
-  if constexpr (!ACC && sizeof(TC) == 2) {
-    if (rope) {
-      const int units = (rope->r.heads + rope->r.kv_heads) * (rope->r.hd / 8) + rope->r.kv_heads * (rope->r.hd / 4);
-      gemm_reduce_rope_kernel<<<dim3((units + 255) / 256, M), 256, 0, s>>>(partial, bias, (__bf16*)C, M, N, K, ldc, used, *rope);
-      VK_LAUNCH_CHECK();
-      return 0;
-    }
-  }
-  const long long threads = (long long)M * ((N + 3) / 4);
-  gemm_reduce_kernel<TC, ACC><<<(int)((threads + 255) / 256), 256, 0, s>>>(partial, bias, C, M, N, ldc, used, vector_ok);
-  VK_LAUNCH_CHECK();
-  return 0;
+  return reduce_ranges<TC, ACC>(partial, bias, C, M, N, K, ldc, used, vector_ok, s, follow, rope);
 }
 
 template <typename TC, bool ACC>
