@@ -221,6 +221,11 @@ ATTN_CASES = [
     (28, 4, 128, 16, 0, [(300, 1), (257, 130), (31, 1)]),
     (20, 1, 80, 32, 50, [(200, 1), (97, 96)]),
     (2, 2, 256, 64, 0, [(129, 1), (70, 70)]),
+    # widths that fill their padded width with pages that divide 64: prompts go through the kernel that loads into LDS directly
+    (8, 2, 64, 8, 40, [(200, 150), (64, 64), (300, 1), (391, 130)]),
+    (4, 4, 128, 32, 100, [(333, 300), (128, 128), (2, 2)]),
+    (5, 5, 64, 64, 0, [(190, 190), (321, 129)]),
+    (2, 1, 256, 16, 70, [(260, 200)]),
 ]
 
 

@@ -35,6 +35,10 @@ typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 namespace {
+// Until none of the wave's vector memory loads is in flight (s_waitcnt vmcnt(0), the other counters left alone).
+// A barrier alone does not wait for loads that write LDS.
+__device__ __forceinline__ void wait_own_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
 constexpr int KS = HDP / 32;  // instruction steps over the head width
 constexpr int DT = HDP / 16;  // 16-wide tiles of the output width
 
@@ -454,6 +458,234 @@ __global__ __launch_bounds__(PT_THREADS) void attn_prefill_kernel(
 }
 
 // ---------------------------------------------------------------------------------------------
+// The prompt kernel for head widths of 64, 128 and 256 that fill their padded width, and page sizes that are
+// powers of two dividing 64: K and V^T tiles go from the cache straight into LDS (loads with the lds modifier:
+// no staging registers, no LDS stores) into one of two stages, so that a tile costs one barrier and the next
+// tile's loads run under this tile's arithmetic. A load instruction fills 1 KB of LDS, lane L the 16 bytes at
+// 16 L, so rows cannot be padded against bank conflicts; instead the 16-byte chunk c of row r sits in slot
+// c ^ f(r), the loading lane fetching the chunk that belongs in its slot, with f chosen so that the 16 rows
+// which the lanes of an operand read touch different banks. Which position an instruction's K row holds is free
+// (every lane reads its own row), and as in the decode kernel row 4g + j of tile t of a 32-position step is
+// position 8g + 4t + j: a lane's eight weights are then eight consecutive positions and its V^T operand one
+// 16-byte chunk of a V^T row that is stored as it lies in the cache.
+#if HDP == 64 || HDP == 128 || HDP == 256
+#define VK_PREFILL_DIRECT 1
+constexpr int PD_ROWB = HDP * 2;                        // bytes of a K row in LDS
+constexpr int PD_C = HDP / 8;                           // 16-byte chunks of a K row
+constexpr int PD_KBYTES = PT_KV * PD_ROWB;              // K tile: 64 rows
+constexpr int PD_VBYTES = HDP * 128;                    // V^T tile: HDP rows of 64 positions
+constexpr int PD_STAGE = PD_KBYTES + PD_VBYTES;
+constexpr int PD_KLOADS = PD_KBYTES / 1024 / PT_WAVES;  // load instructions per wave and tile
+constexpr int PD_VLOADS = PD_VBYTES / 1024 / PT_WAVES;
+constexpr int PD_ROWS_PER_LOAD = 1024 / PD_ROWB;
+
+// slot = chunk ^ k_swizzle(row). The lanes lr = 0..15 of an operand read rows 8 (lr / 4) + lr % 4 (+ a constant):
+// with rows of 256 or 512 bytes every row starts at bank 0 and lr itself separates them; rows of 128 bytes
+// alternate between the two halves of the banks with lr % 2 and lr % 8 does.
+__device__ __forceinline__ int k_swizzle(int r) {
+  return PD_C == 8 ? ((((r >> 3) & 1) << 2) | (r & 3)) : ((((r >> 3) & 3) << 2) | (r & 3));
+}
+
+__global__ __launch_bounds__(PT_THREADS) void attn_prefill_direct_kernel(
+    const __bf16* __restrict__ q, long long q_stride, const __bf16* __restrict__ k_cache,
+    const __bf16* __restrict__ v_cache, __bf16* __restrict__ out, const int* __restrict__ tiles,
+    const int* __restrict__ entry_start, const int* __restrict__ entry_first_pos,
+    const int* __restrict__ block_table, int table_width, int block_size, int heads, int kv_heads, float scale,
+    int window, int cus) {
+  typedef __attribute__((address_space(3))) void* lds_ptr;
+  typedef __attribute__((address_space(1))) const void* global_ptr;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];  // [2][K tile | V^T tile]
+  constexpr int hd = HDP;
+  const int tid = threadIdx.x, lane = tid & 63, lr = lane & 15, lg = lane >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  // work items as in attn_prefill_kernel: long ones first, paired with short ones on a CU
+  const int total = (int)gridDim.x, round = blockIdx.x / cus;
+  const int taken = (round >> 1) * cus + blockIdx.x % cus;
+  const int item = (round & 1) ? taken : total - 1 - taken;
+  const int tile = item / heads;
+  const int entry = tiles[2 * tile], tile_off = tiles[2 * tile + 1];
+  const int h = item % heads, kvh = h / (heads / kv_heads);
+  const int tok0 = entry_start[entry], count = entry_start[entry + 1] - tok0;
+  const int first_pos = entry_first_pos[entry];
+  const int* table = block_table + (size_t)entry * table_width;
+  const int bs = block_size;
+  const PageSize ps(block_size);
+
+  const int tile_cols = min(PT_TOKENS, count - tile_off);
+  const int tile_first_pos = first_pos + tile_off;
+  const int begin = (window > 0 && tile_first_pos + 1 > window) ? tile_first_pos + 1 - window : 0;
+  const int end = tile_first_pos + tile_cols;
+
+  const int q_off = tile_off + wave * 16;
+  const int c = q_off + lr;
+  const bool col_ok = c < count;
+  const int col_pos = col_ok ? first_pos + c : -1;
+  const int col_lo = (window > 0 && col_pos + 1 > window) ? col_pos + 1 - window : 0;
+  bf16x8 qf[KS];
+  load_q(col_ok ? q + (size_t)(tok0 + c) * q_stride + (size_t)h * hd : nullptr, hd, qf);
+  const int wave_cols = max(0, min(16, count - q_off));
+  const int wave_end = wave_cols > 0 ? first_pos + q_off + wave_cols : 0;
+  const int wave_first = first_pos + q_off;
+  const int wave_begin = (window > 0 && wave_first + 1 > window) ? wave_first + 1 - window : 0;
+  const int wave_last = wave_end - 1;
+  const int wave_lo_max = (window > 0 && wave_last + 1 > window) ? wave_last + 1 - window : 0;
+
+  f32x4 o[DT];
+  float m = -INFINITY, l = 0.f;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // Per lane and load instruction: which page of a tile its chunk lies in and where in that page; both are the
+  // same for every tile, since tiles start at multiples of 64 and the page size divides 64. Nothing is loaded
+  // conditionally: a chunk outside [begin, end) reads a page of the same request inside that range (finite
+  // numbers: the pool starts zeroed), and its positions are masked, or weigh zero, for every column.
+  int k_tab[PD_KLOADS], v_tab[PD_VLOADS];
+  unsigned k_in[PD_KLOADS], v_in[PD_VLOADS];
+  const unsigned page_bytes = (unsigned)(kv_heads * bs * hd * 2);
+  const int page_lo = ps.page(begin), page_hi = ps.page(end - 1);
+#pragma unroll
+  for (int i = 0; i < PD_KLOADS; ++i) {
+    const int r = (wave * PD_KLOADS + i) * PD_ROWS_PER_LOAD + lane / PD_C;
+    const int chunk = (lane % PD_C) ^ k_swizzle(r);
+    k_tab[i] = r >> ps.shift;
+    k_in[i] = (unsigned)(((kvh * bs + (r & (bs - 1))) * hd + chunk * 8) * 2);
+  }
+#pragma unroll
+  for (int i = 0; i < PD_VLOADS; ++i) {
+    const int d = (wave * PD_VLOADS + i) * 8 + (lane >> 3);
+    const int p8 = ((lane & 7) ^ (d & 7)) * 8;  // first of the chunk's eight positions within the tile
+    v_tab[i] = p8 >> ps.shift;
+    v_in[i] = (unsigned)(((kvh * hd + d) * bs + (p8 & (bs - 1))) * 2);
+  }
+  int k_page[PD_KLOADS], v_page[PD_VLOADS];
+  auto lookup = [&](int p0) {
+    const int tp = p0 >> ps.shift;
+#pragma unroll
+    for (int i = 0; i < PD_KLOADS; ++i) k_page[i] = table[min(max(tp + k_tab[i], page_lo), page_hi)];
+#pragma unroll
+    for (int i = 0; i < PD_VLOADS; ++i) v_page[i] = table[min(max(tp + v_tab[i], page_lo), page_hi)];
+  };
+  auto issue = [&](int stage) {
+    unsigned char* to_k = lds_raw + stage * PD_STAGE + wave * PD_KLOADS * 1024;
+    unsigned char* to_v = lds_raw + stage * PD_STAGE + PD_KBYTES + wave * PD_VLOADS * 1024;
+#pragma unroll
+    for (int i = 0; i < PD_KLOADS; ++i)
+      __builtin_amdgcn_global_load_lds(
+          (global_ptr)((const char*)k_cache + ((size_t)(unsigned)k_page[i] * page_bytes + k_in[i])),
+          (lds_ptr)(to_k + i * 1024), 16, 0, 0);
+#pragma unroll
+    for (int i = 0; i < PD_VLOADS; ++i)
+      __builtin_amdgcn_global_load_lds(
+          (global_ptr)((const char*)v_cache + ((size_t)(unsigned)v_page[i] * page_bytes + v_in[i])),
+          (lds_ptr)(to_v + i * 1024), 16, 0, 0);
+  };
+
+  // a lane's operand addresses within a stage
+  const int fk = PD_C == 8 ? (lr & 7) : lr;
+  unsigned k_at[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks)
+    k_at[ks] = (unsigned)((8 * (lr >> 2) + (lr & 3)) * PD_ROWB + (((ks * 4 + lg) ^ fk) * 16));
+  unsigned v_at[2];
+#pragma unroll
+  for (int st = 0; st < 2; ++st)
+    v_at[st] = (unsigned)(PD_KBYTES + lr * 128 + (((st * 4 + lg) ^ (lr & 7)) * 16));
+
+  const float c2 = scale * 1.44269504088896341f;
+  auto tile_body = [&](bool masked, int p0, const unsigned char* base) {
+    // ---- scores: tile sub = 2 st + t holds positions p0 + 32 st + 8 g + 4 t + j in register j of lane group g
+    f32x4 s[4];
+#pragma unroll
+    for (int sub = 0; sub < 4; ++sub) {
+      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const bf16x8 kf = *(const bf16x8*)(base + k_at[ks] + ((sub >> 1) * 32 + (sub & 1) * 4) * PD_ROWB);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[ks], acc, 0, 0, 0);
+      }
+      s[sub] = acc;
+    }
+    if (masked) {
+#pragma unroll
+      for (int sub = 0; sub < 4; ++sub)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int p = p0 + (sub >> 1) * 32 + lg * 8 + (sub & 1) * 4 + j;
+          if (!(p >= col_lo && p <= col_pos)) s[sub][j] = -INFINITY;
+        }
+    }
+    float tile_max = -INFINITY;
+#pragma unroll
+    for (int sub = 0; sub < 4; ++sub)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) tile_max = fmaxf(tile_max, s[sub][j]);
+    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, 64));
+    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
+    const float m_new = fmaxf(m, tile_max);
+    bf16x8 pf[2] = {zero8(), zero8()};
+    if (__builtin_amdgcn_ballot_w64(m_new > m) != 0) {
+      const float alpha = (m_new > m && m > -INFINITY) ? __builtin_amdgcn_exp2f((m - m_new) * c2) : 1.f;
+      l *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) o[dt] *= alpha;
+      m = m_new;
+    }
+    if (m_new > -INFINITY) {
+      const float mc = m_new * c2;
+      float sum = 0.f;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const float w = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i >> 2][i & 3], c2, -mc));
+        sum += w;
+        pf[i >> 3][i & 7] = (__bf16)w;  // step st: tiles 2 st and 2 st + 1, eight consecutive positions
+      }
+      l += sum;
+    }
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+#pragma unroll
+      for (int st = 0; st < 2; ++st) {
+        const bf16x8 vf = *(const bf16x8*)(base + v_at[st] + dt * 16 * 128);
+        o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[st], o[dt], 0, 0, 0);
+      }
+    }
+  };
+
+  const int first_tile = begin & ~(PT_KV - 1);
+  lookup(first_tile);
+  issue(0);
+  lookup(first_tile + PT_KV);
+  wait_own_loads();
+  __syncthreads();
+  int stage = 0;
+  for (int p0 = first_tile; p0 < end; p0 += PT_KV) {
+    const bool more = p0 + PT_KV < end;
+    if (more) {
+      issue(stage ^ 1);            // nobody reads that stage any more: the barrier that ended the last tile
+      lookup(p0 + 2 * PT_KV);
+    }
+    if (p0 < wave_end && p0 + PT_KV > wave_begin)
+      tile_body(!(p0 + PT_KV - 1 <= wave_first && p0 >= wave_lo_max), p0, lds_raw + stage * PD_STAGE);
+    wait_own_loads();   // a barrier alone does not wait for loads that write LDS
+    __syncthreads();
+    stage ^= 1;
+  }
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+  if (!col_ok) return;
+  const float inv = 1.f / l;
+  __bf16* dst = out + (size_t)(tok0 + c) * heads * hd + (size_t)h * hd;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) {
+    bf16x4 r;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) r[j] = (__bf16)(o[dt][j] * inv);
+    *(bf16x4*)(dst + dt * 16 + lg * 4) = r;
+  }
+}
+#endif
+
+// ---------------------------------------------------------------------------------------------
 // Decoding: grid (entries, kv_heads * head_blocks, chunks), one wave. Columns are the query heads of
 // one key head. Chunk c covers positions [c * chunk, (c + 1) * chunk) of the visible range and leaves
 // (max, sum, weighted sum) in `partial`: [entry, head, chunk, hd + 2] floats. REGS: a chunk spans at most
@@ -644,6 +876,22 @@ extern "C" int vk_attn_bf16_prefill(const void* q, long long q_stride, const voi
     cus = count > 0 ? count : 1;
   }
   if ((long long)num_tiles * heads > 0x7fffffffLL) return VK_UNSUPPORTED_SIZE;
+#ifdef VK_PREFILL_DIRECT
+  if (fast && hd == HDP && block_size >= 8) {  // the kernel that loads straight into LDS
+    static bool direct_configured = false;
+    if (!direct_configured) {
+      hipError_t e = hipFuncSetAttribute((const void*)attn_prefill_direct_kernel,
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, 2 * PD_STAGE);
+      if (e != hipSuccess) return (int)e;
+      direct_configured = true;
+    }
+    attn_prefill_direct_kernel<<<num_tiles * heads, PT_THREADS, 2 * PD_STAGE, (hipStream_t)stream>>>(
+        (const __bf16*)q, q_stride, (const __bf16*)k_cache, (const __bf16*)v_cache, (__bf16*)out, tiles, entry_start,
+        entry_first_pos, block_table, table_width, block_size, heads, kv_heads, scale, window, cus);
+    VK_LAUNCH_CHECK();
+    return 0;
+  }
+#endif
   kernel<<<num_tiles * heads, PT_THREADS, lds_bytes, (hipStream_t)stream>>>(
       (const __bf16*)q, q_stride, (const __bf16*)k_cache, (const __bf16*)v_cache, (__bf16*)out, tiles, entry_start,
       entry_first_pos, block_table, table_width, block_size, heads, kv_heads, hd, scale, window, cus);
