@@ -477,7 +477,9 @@ def test_attention_finds_one_far_key_among_hundreds(dtype):
 
 
 @pytest.mark.parametrize("m,n,k", [(1, 48, 64), (7, 300, 96), (8, 3584, 512), (16, 200, 1544), (17, 331, 520), (33, 1000, 264),
-                                   (64, 520, 1024), (48, 130, 72), (64, 4608, 3584)])
+                                   (64, 520, 1024), (48, 130, 72), (64, 4608, 3584),
+                                   # past 64 tokens K is walked in chunks of 128: K with a rest, K shorter than a chunk
+                                   (65, 331, 520), (80, 1000, 264), (97, 200, 1544), (128, 3584, 1024), (113, 130, 72)])
 @pytest.mark.parametrize("ranges,rows_per_wave", [(1, 1), (1, 2), (3, 1), (8, 2), (2, 110), (1, 114), (3, 109)])
 def test_gemm_mid_against_float64(m, n, k, ranges, rows_per_wave):
     from vipera_rs_amd.ops import kernels

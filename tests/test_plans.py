@@ -2,7 +2,8 @@
 at the layer sizes of the 1.5B, 7B and 32B shapes.  Pure functions of the sizes: no GPU is touched."""
 from vipera_rs_amd.ops.attention import decode_chunking
 from vipera_rs_amd.ops.kernels import follow_stride, follow_sumsq_floats
-from vipera_rs_amd.ops.linear import (gated_plan, gated_resident_fits, mid_plan, split_qkv_plan, streams_in_wave_order)
+from vipera_rs_amd.ops.linear import (gated_plan, gated_resident_fits, mid_plan, split_qkv_plan, streams_in_wave_order,
+                                      streams_weights)
 
 QKV_7B, O_7B, GATE_UP_7B, DOWN_7B, HEAD_7B = (4608, 3584), (3584, 3584), (37888, 3584), (3584, 18944), (152064, 3584)
 
@@ -23,6 +24,18 @@ def test_the_lds_shared_product_splits_k_where_rows_are_few():
     assert mid_plan(64, *QKV_7B) == (3, 1) and mid_plan(64, *O_7B) == (4, 1)
     ranges, _ = mid_plan(64, 2048, 1536)                   # 1.5B q/k/v: no range shorter than 512
     assert 1536 // ranges >= 512
+
+
+def test_past_64_tokens_the_weights_are_streamed_where_tiles_would_be_few():
+    for n, k in (QKV_7B, O_7B, DOWN_7B, HEAD_7B):
+        assert streams_weights(64, n, k) and not streams_weights(129, n, k)
+    for n, k in (QKV_7B, O_7B, DOWN_7B, (5120, 27648), (2048, 1536)):
+        assert streams_weights(65, n, k) and streams_weights(80, n, k)
+    assert not streams_weights(65, *HEAD_7B)               # 152,064 rows fill the tiled kernel at any token count
+    assert streams_weights(128, *O_7B) and streams_weights(128, 2048, 1536) and streams_weights(128, 1536, 8960)
+    assert not streams_weights(128, *DOWN_7B) and not streams_weights(81, *QKV_7B) and not streams_weights(96, 5120, 27648)
+    assert mid_plan(65, *DOWN_7B) == (8, 1) and mid_plan(96, *O_7B) == (4, 1) and mid_plan(128, 2048, 1536) == (4, 1)
+    assert mid_plan(100, 1024, 320) == (1, 1)              # no range shorter than 256
 
 
 def test_the_gated_product_goes_resident_tiled_or_lds_shared():

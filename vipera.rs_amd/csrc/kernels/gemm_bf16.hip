@@ -933,7 +933,7 @@ void qkv_rope_plan(int M, int heads, int kv_heads, int hd, int* pairs, int* valu
 }
 
 // ---------------------------------------------------------------------------------------------
-// M <= 64, activations shared through LDS. A workgroup owns 64 * RT weight rows (16 * RT per wave; with
+// M <= 128, activations shared through LDS. A workgroup owns 64 * RT weight rows (16 * RT per wave; with
 // RT 1 the launcher may give a wave fewer rows, see balanced_rows) and a range of K; all four waves walk that range together in chunks of 256. A chunk's activations
 // (16 * CB tokens x 256) are fetched once per workgroup into LDS, double-buffered, one barrier per
 // chunk; the weights go from HBM straight into the instruction's operand layout, the next chunk's
@@ -942,16 +942,20 @@ void qkv_rope_plan(int M, int heads, int kv_heads, int hd, int* pairs, int* valu
 // ascending order afterwards (a second launch: kernel boundaries are what keeps the XCDs' caches coherent).
 constexpr int MID_CHUNK = 256;
 constexpr int MID_ROW = MID_CHUNK + 8;  // elements per LDS row: 528 bytes, so 16 rows hit 16 different 16-byte slots
+// More than four blocks of 16 tokens walk K in chunks of 128, so that two workgroups' buffers still share a CU's LDS.
+constexpr int mid_chunk(int cb) { return cb > 4 ? 128 : MID_CHUNK; }
 
 template <int CB, int RT, typename TC, bool ACCUMULATE, bool GATED = false,
-          int SETS = (RT == 1 && CB <= 2 ? VK_MID_SETS : 2)>
+          int SETS = (RT == 1 && CB <= 2 ? VK_MID_SETS : 2), int CHUNK = mid_chunk(CB)>
 __global__ __launch_bounds__(256) void gemm_mid_kernel(const __bf16* __restrict__ A, const __bf16* __restrict__ W,
                                                        const float* __restrict__ bias, TC* __restrict__ C, int M,
                                                        int N, int K, long long lda, long long ldc, int k_per_range,
                                                        long long range_stride, int vector_ok, int rows) {
-  extern __shared__ __attribute__((aligned(16))) __bf16 lds[];  // [2][CB * 16][MID_ROW]
-  constexpr int BUF = CB * 16 * MID_ROW;
-  constexpr int A_LOADS = CB * 2;  // 16-byte pieces of a chunk per thread
+  extern __shared__ __attribute__((aligned(16))) __bf16 lds[];  // [2][CB * 16][ROW]
+  constexpr int ROW = CHUNK + 8, PIECES = CHUNK / 8, KSTEPS = CHUNK / 32;
+  constexpr int BUF = CB * 16 * ROW;
+  constexpr int A_LOADS = CB * 16 * PIECES / 256;  // 16-byte pieces of a chunk per thread
+  static_assert(CB * 16 * PIECES % 256 == 0, "a chunk's pieces must divide among the threads");
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lr = lane & 15, lg = lane >> 4;
@@ -972,7 +976,7 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const __bf16* __restrict_
 #pragma unroll
   for (int i = 0; i < A_LOADS; ++i) {
     const int id = tid + 256 * i;
-    a_off[i] = (unsigned)(((id >> 5) * lda + (id & 31) * 8) * 2);
+    a_off[i] = (unsigned)(((id / PIECES) * lda + (id % PIECES) * 8) * 2);
   }
   f32x4 acc[RT][CB];
 #pragma unroll
@@ -980,7 +984,7 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const __bf16* __restrict_
 #pragma unroll
     for (int cb = 0; cb < CB; ++cb) acc[rt][cb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  bf16x8 a_stage[A_LOADS], w[SETS][RT][8];
+  bf16x8 a_stage[A_LOADS], w[SETS][RT][KSTEPS];
   auto load_acts = [&](int k0) {
 #pragma unroll
     for (int i = 0; i < A_LOADS; ++i) a_stage[i] = a_view.load(a_off[i] + (unsigned)k0 * 2);
@@ -989,22 +993,22 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const __bf16* __restrict_
 #pragma unroll
     for (int i = 0; i < A_LOADS; ++i) {
       const int id = tid + 256 * i;
-      *(bf16x8*)(lds + buf * BUF + (id >> 5) * MID_ROW + (id & 31) * 8) = a_stage[i];
+      *(bf16x8*)(lds + buf * BUF + (id / PIECES) * ROW + (id % PIECES) * 8) = a_stage[i];
     }
   };
-  auto load_weights = [&](int k0, bf16x8 (&dst)[RT][8]) {
+  auto load_weights = [&](int k0, bf16x8 (&dst)[RT][KSTEPS]) {
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-      for (int i = 0; i < 8; ++i) dst[rt][i] = w_view.load(w_off[rt] + (unsigned)(k0 + i * 32) * 2);
+      for (int i = 0; i < KSTEPS; ++i) dst[rt][i] = w_view.load(w_off[rt] + (unsigned)(k0 + i * 32) * 2);
   };
-  auto multiply = [&](const bf16x8 (&wf)[RT][8], int buf) {
-    const __bf16* tile = lds + buf * BUF + lr * MID_ROW + lg * 8;
+  auto multiply = [&](const bf16x8 (&wf)[RT][KSTEPS], int buf) {
+    const __bf16* tile = lds + buf * BUF + lr * ROW + lg * 8;
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
+    for (int i = 0; i < KSTEPS; ++i)
 #pragma unroll
       for (int cb = 0; cb < CB; ++cb) {
-        const bf16x8 a = *(const bf16x8*)(tile + cb * 16 * MID_ROW + i * 32);
+        const bf16x8 a = *(const bf16x8*)(tile + cb * 16 * ROW + i * 32);
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt)
           acc[rt][cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[rt][i], a, acc[rt][cb], 0, 0, 0);
@@ -1015,40 +1019,40 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const __bf16* __restrict_
   // is multiplied (SETS register sets: three while registers allow three waves a SIMD, else two), the activations
   // of chunk c + 1 wait in registers until the barrier frees their LDS buffer, those of chunk c + 2 are
   // requested right after it.
-  const int whole = (k_end - k_begin) / MID_CHUNK;
+  const int whole = (k_end - k_begin) / CHUNK;
   int buf = 0;
   constexpr int NEED = SETS - 1 > 2 ? SETS - 1 : 2;
   auto chunk = [&](auto set_, auto rem_, int c) {
     constexpr int SET = decltype(set_)::value, REM = decltype(rem_)::value;  // REM chunks follow (capped)
-    const int k0 = k_begin + c * MID_CHUNK;
-    if constexpr (REM >= SETS - 1) load_weights(k0 + (SETS - 1) * MID_CHUNK, w[(SET + SETS - 1) % SETS]);
+    const int k0 = k_begin + c * CHUNK;
+    if constexpr (REM >= SETS - 1) load_weights(k0 + (SETS - 1) * CHUNK, w[(SET + SETS - 1) % SETS]);
     multiply(w[SET], buf);
     if constexpr (REM >= 1) store_acts(buf ^ 1);
     __syncthreads();
-    if constexpr (REM >= 2) load_acts(k0 + 2 * MID_CHUNK);
+    if constexpr (REM >= 2) load_acts(k0 + 2 * CHUNK);
     buf ^= 1;
   };
   if (whole > 0) {
     // requests past the range (fewer chunks than the pipeline is deep) read weights that are not used
     load_acts(k_begin);
-    static_for<SETS - 1>([&](auto j) { load_weights(k_begin + j.value * MID_CHUNK, w[j.value]); });
+    static_for<SETS - 1>([&](auto j) { load_weights(k_begin + j.value * CHUNK, w[j.value]); });
     store_acts(0);
-    load_acts(k_begin + MID_CHUNK);
+    load_acts(k_begin + CHUNK);
     __syncthreads();
     run_pipeline<SETS, NEED>(chunk, whole);
   }
   // the rest of the range (less than a chunk): operands past k_end are zeroed
-  const int k_rest = k_begin + whole * MID_CHUNK;
+  const int k_rest = k_begin + whole * CHUNK;
   if (k_rest < k_end) {
     load_acts(k_rest);
     load_weights(k_rest, w[0]);
 #pragma unroll
     for (int i = 0; i < A_LOADS; ++i)
-      if (k_rest + ((tid + 256 * i) & 31) * 8 >= k_end) a_stage[i] = zero8();
+      if (k_rest + ((tid + 256 * i) % PIECES) * 8 >= k_end) a_stage[i] = zero8();
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-      for (int i = 0; i < 8; ++i)
+      for (int i = 0; i < KSTEPS; ++i)
         if (k_rest + i * 32 + lg * 8 >= k_end) w[0][rt][i] = zero8();
     store_acts(0);
     __syncthreads();
@@ -1463,7 +1467,8 @@ template <int CB, int RT, typename TC, bool ACC>
 int launch_mid_as(const __bf16* A, const __bf16* W, const float* bias, TC* C, float* partial, long long partial_floats,
                   int ranges, int forced_rows, int M, int N, int K, long long lda, long long ldc, int vector_ok,
                   hipStream_t s, const FollowNorm* follow = nullptr, const ReduceRope* rope = nullptr) {
-  constexpr int lds_bytes = 2 * CB * 16 * MID_ROW * (int)sizeof(__bf16);
+  constexpr int CHUNK = mid_chunk(CB);
+  constexpr int lds_bytes = 2 * CB * 16 * (CHUNK + 8) * (int)sizeof(__bf16);
   const int rows = RT == 2 ? 32 : forced_rows ? forced_rows : balanced_rows(M, N, 4, ranges < 1 ? 1 : ranges);  // per wave
   const int blocks = (N + 4 * rows - 1) / (4 * rows);
   if (ranges <= 1) {
@@ -1486,7 +1491,7 @@ int launch_mid_as(const __bf16* A, const __bf16* W, const float* bias, TC* C, fl
     if (e != hipSuccess) return (int)e;
     configured_partial = true;
   }
-  const int k_per_range = ((K + ranges - 1) / ranges + MID_CHUNK - 1) / MID_CHUNK * MID_CHUNK;
+  const int k_per_range = ((K + ranges - 1) / ranges + CHUNK - 1) / CHUNK * CHUNK;
   const int used = (K + k_per_range - 1) / k_per_range;
   kernel<<<dim3(blocks, used), 256, lds_bytes, s>>>(A, W, nullptr, partial, M, N, K, lda, N, k_per_range,
                                                     (long long)M * N, (N & 3) == 0 ? 1 : 0, rows);
@@ -1502,10 +1507,13 @@ int launch_mid(const __bf16* A, const __bf16* W, const float* bias, TC* C, float
   // 108 to 116: one tile per wave with a forced number of rows (8 to 16), for tests and measurements
   const int forced = rows_per_wave >= 108 && rows_per_wave <= 116 ? rows_per_wave - 100 : 0;
 #define VK_MID(CBV, RTV) return launch_mid_as<CBV, RTV, TC, ACC>(A, W, bias, C, partial, partial_floats, ranges, forced, M, N, K, lda, ldc, vector_ok, s, follow, rope)
+  if (cb > 4 && (follow || rope)) return VK_UNSUPPORTED_SIZE;  // the kernels that add their ranges take 64 tokens
   if (rows_per_wave == 2) {
-    switch (cb) { case 1: VK_MID(1, 2); case 2: VK_MID(2, 2); case 3: VK_MID(3, 2); case 4: VK_MID(4, 2); }
+    switch (cb) { case 1: VK_MID(1, 2); case 2: VK_MID(2, 2); case 3: VK_MID(3, 2); case 4: VK_MID(4, 2);
+                  case 5: VK_MID(5, 2); case 6: VK_MID(6, 2); case 7: VK_MID(7, 2); case 8: VK_MID(8, 2); }
   } else {
-    switch (cb) { case 1: VK_MID(1, 1); case 2: VK_MID(2, 1); case 3: VK_MID(3, 1); case 4: VK_MID(4, 1); }
+    switch (cb) { case 1: VK_MID(1, 1); case 2: VK_MID(2, 1); case 3: VK_MID(3, 1); case 4: VK_MID(4, 1);
+                  case 5: VK_MID(5, 1); case 6: VK_MID(6, 1); case 7: VK_MID(7, 1); case 8: VK_MID(8, 1); }
   }
 #undef VK_MID
   return VK_UNSUPPORTED_SIZE;
@@ -1694,7 +1702,7 @@ extern "C" int vk_gemm_bf16(const void* A, const void* W, const float* bias, voi
   return VK_BAD_ARGUMENT;
 }
 
-// The same product for M <= 64 with the activations shared through LDS. `ranges` > 1 splits K over
+// The same product for M <= 128 with the activations shared through LDS. `ranges` > 1 splits K over
 // workgroups: partial sums go to `partial` (at least ranges * M * N floats) and a second kernel adds them.
 // rows_per_wave: 1 or 2 tiles of 16 weight rows per wave; with 1 the launcher may give a wave fewer than 16 rows
 // (balanced_rows), and 108 to 116 force one tile with 8 to 16 rows.
@@ -1702,7 +1710,7 @@ static int gemm_mid_checked(const void* A, const void* W, const float* bias, voi
                             long long lda, long long ldc, int accumulate, int ranges, int rows_per_wave,
                             float* partial, long long partial_floats, void* stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (M > 64) return VK_UNSUPPORTED_SIZE;
+  if (M > 128) return VK_UNSUPPORTED_SIZE;
   if (K <= 0 || (K & 7) || (lda & 7) || lda < K || ldc < N || ranges < 1) return VK_BAD_ARGUMENT;
   if (((uintptr_t)A & 15) || ((uintptr_t)W & 15) || ((uintptr_t)partial & 15)) return VK_BAD_ARGUMENT;
   if (K >= (1 << 24) || lda >= (1 << 24)) return VK_UNSUPPORTED_SIZE;  // byte offsets inside a tile of rows are 32-bit

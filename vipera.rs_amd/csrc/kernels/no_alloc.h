@@ -4,7 +4,7 @@
 // capture, tight serving loops, harnesses that forbid allocation. The engine itself goes through
 // vk_gemm_bf16_mid and brings its own workspace.
 //
-// vk_gemm_bf16_mid_no_alloc is vk_gemm_bf16_mid (C[M,N] (+)= A[M,K] * W[N,K]^T (+ bias) for M <= 64, bfloat16
+// vk_gemm_bf16_mid_no_alloc is vk_gemm_bf16_mid (C[M,N] (+)= A[M,K] * W[N,K]^T (+ bias) for M <= 128, bfloat16
 // operands, K optionally split into `ranges` ranges over workgroups) without the workspace arguments: the
 // partial sums of the K ranges go to a file-scope device array of VK_NO_ALLOC_SCRATCH_FLOATS floats (16 MiB)
 // that each GPU which runs the library holds until the process ends. The caller still passes inputs and the

@@ -634,13 +634,13 @@ def _split_k_workspace(device: torch.device, floats: int, kind: str) -> torch.Te
 
 def gemm_bf16_mid(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
                   accumulate: bool = False, ranges: int = 1, rows_per_wave: int = 2) -> None:
-    """``out (+)= a @ w.T + bias`` for at most 64 rows of ``a``: activations shared through LDS, weights
+    """``out (+)= a @ w.T + bias`` for at most 128 rows of ``a``: activations shared through LDS, weights
     streamed; ``ranges`` > 1 splits K over workgroups and adds the ranges' partial sums in a second kernel."""
     _dev(a, w, bias, out)
     _need(a.dim() == 2 and w.dim() == 2 and out.dim() == 2, "gemm: operands must be matrices")
     m, k = a.shape
     n = w.shape[0]
-    _need(m <= 64, "gemm_bf16_mid takes at most 64 rows")
+    _need(m <= 128, "gemm_bf16_mid takes at most 128 rows")
     _need(w.shape[1] == k and out.shape == (m, n), f"gemm: shapes {tuple(a.shape)} x {tuple(w.shape)}^T -> {tuple(out.shape)}")
     _need(gemm_bf16_supported(a, w, out), "gemm_bf16: operands must be bfloat16, K a multiple of 8, rows 16-byte aligned")
     _need((rows_per_wave in (1, 2) or 108 <= rows_per_wave <= 116) and ranges >= 1,
@@ -655,7 +655,7 @@ def gemm_bf16_mid(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor]
     _need(ldc >= n, "gemm: out's row stride")
     partial = None
     if ranges > 1:
-        partial = _split_k_workspace(a.device, ranges * 64 * n, "mid")
+        partial = _split_k_workspace(a.device, ranges * (64 if m <= 64 else 128) * n, "mid")
     fn = _fn("gemm_bf16", "vk_gemm_bf16_mid", [_p, _p, _p, _p, _i, _i, _i, _i, _ll, _ll, _i, _i, _i, _p, _ll, _p])
     _status(fn(_ptr(a), _ptr(w), _ptr(bias), _ptr(out), _dt(out, "out"), m, n, k, lda, ldc, 1 if accumulate else 0,
                int(ranges), int(rows_per_wave), _ptr(partial), partial.numel() if partial is not None else 0, _stream()),

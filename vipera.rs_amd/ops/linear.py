@@ -4,11 +4,12 @@ All-bfloat16 operands whose rows are 16-byte aligned go to the matrix-core kerne
 combination (the 32-bit run, or a matrix kept in 32-bit inside a bfloat16 run) goes to the
 32-bit FMA kernel.  Among the matrix-core kernels the number of rows of ``a`` (tokens) decides:
 
-* more than 64: the LDS-tiled kernel (prompts);
-* up to 64 (decoding): the product is a stream of the weights.  Up to four tokens, or a small weight
+* many (prompts): the LDS-tiled kernel;
+* up to 64 (decoding), and up to 80 or 128 where that was measured faster (:func:`streams_weights`): the
+  product is a stream of the weights.  Up to four tokens, or a small weight
   at up to 16 tokens, use the kernel whose waves split K inside a workgroup; otherwise the kernel that
   shares the activations through LDS, with K split over workgroups where the weight has too few rows
-  to fill the GPU otherwise.  The thresholds were measured on the 7B shapes on an MI355X.  The gated
+  to fill the GPU otherwise.  The thresholds were measured on the 1.5B, 7B and 32B shapes on an MI355X.  The gated
   product of up to 16 tokens keeps all activations in LDS and gives every CU the same share of rows.
 """
 from __future__ import annotations
@@ -20,8 +21,23 @@ import torch
 from . import kernels
 
 
+def streams_weights(m: int, n: int, k: int) -> bool:
+    """Whether a bfloat16 product of ``m`` tokens runs on a weight-streaming kernel rather than the tiled one:
+    always up to 64 tokens; up to 80 for every weight but an output matrix (whose many rows fill the tiled
+    kernel as well), and up to 128 for a small weight, where 128-token tiles are too few to fill the GPU
+    (7B widths at 65 tokens: output projection 13.5 against 16.4 us, down projection 40.7 against 43.7; the 32B
+    down projection 78 against 103; 1.5B q/k/v 9.1 against 17.5; from 96 tokens on only the small weights gain)."""
+    if m <= 64:
+        return True
+    if n >= 100_000:
+        return False
+    return m <= 80 or (m <= 128 and n * k <= 16_000_000)
+
+
 def mid_plan(m: int, n: int, k: int) -> Tuple[int, int]:
     """``(ranges of K, 16-row tiles per wave)`` for the LDS-shared kernel."""
+    if m > 64:  # measured at 65, 96 and 128 tokens: one tile per wave; eight ranges of a long K, else four
+        return max(1, min(8 if k >= 8_192 else 4, k // 256)), 1
     if n >= 100_000:
         return (1, 2) if m > 16 else (1, 1)
     if n >= 16_384:
@@ -44,7 +60,7 @@ def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: 
     if a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and kernels.gemm_bf16_supported(a, w, out):
         m, k = a.shape
         n = w.shape[0]
-        if m > 64 or streams_in_wave_order(m, n, k):
+        if not streams_weights(m, n, k) or streams_in_wave_order(m, n, k):
             kernels.gemm_bf16(a, w, bias, out, accumulate)
         else:
             ranges, rows_per_wave = mid_plan(m, n, k)
