@@ -377,7 +377,7 @@ extern "C" int plain_attn_bf16_prefill(const void* q, long long q_stride, const 
                                        void* out, const int* tiles, int num_tiles, const int* entry_start,
                                        const int* entry_first_pos, const int* block_table, int table_width,
                                        int block_size, int heads, int kv_heads, int hd, float scale, int window,
-                                       void*) {
+                                       int, void*) {
   if (hd <= 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads || block_size <= 0 || window < 0) return BAD_ARGUMENT;
   for (int tile = 0; tile < num_tiles; ++tile) {
     const int entry = tiles[2 * tile], off = tiles[2 * tile + 1];

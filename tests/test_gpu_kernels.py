@@ -269,6 +269,11 @@ def test_attention_kernels_against_plain_softmax(case, dtype):
         out2 = torch.zeros(T, heads * hd, dtype=dtype, device=DEV)
         es, fp = dev(torch.tensor(starts, dtype=torch.int32)), dev(torch.tensor(first, dtype=torch.int32))
         if tiles:
+            halved = torch.zeros(T, heads * hd, dtype=dtype, device=DEV)   # a tile's positions halved between sixteen waves
+            kernels.attn_bf16_prefill(qkv_d, k_d, v_d, halved, dev(torch.tensor(tiles, dtype=torch.int32)), es, fp,
+                                      table_d, heads, kv_heads, hd, scale, window, split=True)
+            rows = [t for e, n in enumerate(counts) if n > 1 for t in range(starts[e], starts[e + 1])]
+            assert _rel(halved.cpu()[rows], want[rows]) < tol, "matrix-core prompt kernel, halved"
             kernels.attn_bf16_prefill(qkv_d, k_d, v_d, out2, dev(torch.tensor(tiles, dtype=torch.int32)), es, fp,
                                       table_d, heads, kv_heads, hd, scale, window)
         if singles:
@@ -433,16 +438,17 @@ def test_prompt_attention_at_the_benchmark_head_shapes(heads, kv_heads, hd):
     dev = lambda t: t.to(DEV)  # noqa: E731
     tiles = [(first[e] + off, e, off) for e, n in enumerate(counts) for off in range(0, n, TILE_TOKENS)]
     tiles = [x for _, e, off in sorted(tiles) for x in (e, off)]                # as the engine orders them
-    out = torch.zeros(T, heads * hd, dtype=dtype, device=DEV)
-    kernels.attn_bf16_prefill(dev(qkv), dev(cache.k), dev(cache.v), out, dev(torch.tensor(tiles, dtype=torch.int32)),
-                              dev(torch.tensor(starts, dtype=torch.int32)), dev(torch.tensor(first, dtype=torch.int32)),
-                              dev(cache.table), heads, kv_heads, hd, scale, 0)
-    got = out.cpu()
-    assert _rel(got, want) < 1.2e-2
-    # row by row too: the first tokens of a prompt see few keys, their outputs are large and would hide a fault
-    # in a late row of small outputs
-    rows = (got.double() - want).abs().amax(dim=1) / want.abs().amax(dim=1)
-    assert float(rows.max()) < 3e-2, int(rows.argmax())
+    for split in (False, True):
+        out = torch.zeros(T, heads * hd, dtype=dtype, device=DEV)
+        kernels.attn_bf16_prefill(dev(qkv), dev(cache.k), dev(cache.v), out, dev(torch.tensor(tiles, dtype=torch.int32)),
+                                  dev(torch.tensor(starts, dtype=torch.int32)), dev(torch.tensor(first, dtype=torch.int32)),
+                                  dev(cache.table), heads, kv_heads, hd, scale, 0, split=split)
+        got = out.cpu()
+        assert _rel(got, want) < 1.2e-2
+        # row by row too: the first tokens of a prompt see few keys, their outputs are large and would hide a fault
+        # in a late row of small outputs
+        rows = (got.double() - want).abs().amax(dim=1) / want.abs().amax(dim=1)
+        assert float(rows.max()) < 3e-2, (split, int(rows.argmax()))
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

@@ -302,10 +302,11 @@ def test_matrix_core_attention_beside_its_twins(hd, window):
     qkv = torch.randn(T, (heads + 2 * kv_heads) * hd, generator=g).to(torch.bfloat16)
     entry_start, first_pos = i32([0, count, count + 1]), i32([first, 499])
     tiles = i32([0, 256, 0, 0, 0, 128])           # any order of the tiles
-    (got, want), = both(module, "attn_bf16_prefill",
-                        [qkv, qkv.shape[1], k, v, torch.zeros(T, heads * hd, dtype=torch.bfloat16), tiles, 3, entry_start, first_pos,
-                         table, table.shape[1], bs, heads, kv_heads, hd, 1 / math.sqrt(hd), window, None], [4])
-    assert rel_err(got[:count].float().numpy(), want[:count].double().numpy()) < 8e-3
+    for split in (0, 1):                          # one workgroup per tile, or its positions halved between sixteen waves
+        (got, want), = both(module, "attn_bf16_prefill",
+                            [qkv, qkv.shape[1], k, v, torch.zeros(T, heads * hd, dtype=torch.bfloat16), tiles, 3, entry_start,
+                             first_pos, table, table.shape[1], bs, heads, kv_heads, hd, 1 / math.sqrt(hd), window, split, None], [4])
+        assert rel_err(got[:count].float().numpy(), want[:count].double().numpy()) < 8e-3
     chunk, chunks = 128, 4
     partial = torch.empty(1 * heads * chunks * (hd + 2))
     (got, want), = both(module, "attn_bf16_decode",

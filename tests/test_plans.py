@@ -73,3 +73,15 @@ def test_decode_attention_chunks():
     assert decode_chunking(100, 1, 4, 1) == (128, 1)
     chunk, chunks = decode_chunking(1 << 20, 1, 1, 1)      # never more than 128 chunks
     assert chunks <= 128 and chunk * chunks >= 1 << 20 and chunk % 32 == 0
+
+
+def test_prompt_tiles_are_halved_between_sixteen_waves_only_where_a_cu_would_be_left_with_one_workgroup():
+    from vipera_rs_amd.ops.attention import halves_prompt_tiles
+    reach = [128 * (t + 1) for t in range(16)]                       # one prompt of 2,048 tokens
+    assert halves_prompt_tiles(16, 28, max(reach), sum(reach), 256)  # 448 items, the longest 1.9 times the mean
+    even = [1536 + 128 * (t + 1) for t in range(4)] * 4              # four portions of 512 tokens at position 1,536
+    assert not halves_prompt_tiles(16, 28, max(even), sum(even), 256)
+    assert halves_prompt_tiles(4, 28, 512, 1280, 256)                # fewer items than CUs
+    long = [128 * (t + 1) for t in range(64)]                        # 8,192 tokens: several rounds of workgroups
+    assert not halves_prompt_tiles(64, 28, max(long), sum(long), 256)
+    assert not halves_prompt_tiles(0, 28, 0, 0, 256)

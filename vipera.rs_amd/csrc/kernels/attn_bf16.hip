@@ -468,6 +468,12 @@ __global__ __launch_bounds__(PT_THREADS) void attn_prefill_kernel(
 // (every lane reads its own row), and as in the decode kernel row 4g + j of tile t of a 32-position step is
 // position 8g + 4t + j: a lane's eight weights are then eight consecutive positions and its V^T operand one
 // 16-byte chunk of a V^T row that is stored as it lies in the cache.
+//
+// SPLIT: a workgroup of sixteen waves, one per CU; waves 0-7 walk the first half of the tile's positions and
+// waves 8-15 the second half for the same 128 columns, each half with LDS stages of its own, and the halves'
+// (max, sum, weighted sum) are merged through LDS at the end. For a step with few work items of very different
+// lengths (one long prompt): a CU then works on its longest item with all sixteen waves instead of being left
+// with one workgroup of eight once the short neighbour has finished.
 #if HDP == 64 || HDP == 128 || HDP == 256
 #define VK_PREFILL_DIRECT 1
 constexpr int PD_ROWB = HDP * 2;                        // bytes of a K row in LDS
@@ -478,6 +484,7 @@ constexpr int PD_STAGE = PD_KBYTES + PD_VBYTES;
 constexpr int PD_KLOADS = PD_KBYTES / 1024 / PT_WAVES;  // load instructions per wave and tile
 constexpr int PD_VLOADS = PD_VBYTES / 1024 / PT_WAVES;
 constexpr int PD_ROWS_PER_LOAD = 1024 / PD_ROWB;
+constexpr bool PD_CAN_SPLIT = 4 * PD_STAGE <= 128 * 1024;  // two halves with two stages each
 
 // slot = chunk ^ k_swizzle(row). The lanes lr = 0..15 of an operand read rows 8 (lr / 4) + lr % 4 (+ a constant):
 // with rows of 256 or 512 bytes every row starts at bank 0 and lr itself separates them; rows of 128 bytes
@@ -486,7 +493,8 @@ __device__ __forceinline__ int k_swizzle(int r) {
   return PD_C == 8 ? ((((r >> 3) & 1) << 2) | (r & 3)) : ((((r >> 3) & 3) << 2) | (r & 3));
 }
 
-__global__ __launch_bounds__(PT_THREADS) void attn_prefill_direct_kernel(
+template <bool SPLIT>
+__global__ __launch_bounds__(SPLIT ? 2 * PT_THREADS : PT_THREADS) void attn_prefill_direct_kernel(
     const __bf16* __restrict__ q, long long q_stride, const __bf16* __restrict__ k_cache,
     const __bf16* __restrict__ v_cache, __bf16* __restrict__ out, const int* __restrict__ tiles,
     const int* __restrict__ entry_start, const int* __restrict__ entry_first_pos,
@@ -497,11 +505,14 @@ __global__ __launch_bounds__(PT_THREADS) void attn_prefill_direct_kernel(
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];  // [2][K tile | V^T tile]
   constexpr int hd = HDP;
   const int tid = threadIdx.x, lane = tid & 63, lr = lane & 15, lg = lane >> 4;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  // work items as in attn_prefill_kernel: long ones first, paired with short ones on a CU
+  const int wave_of_group = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int half = SPLIT ? wave_of_group >> 3 : 0, wave = SPLIT ? wave_of_group & 7 : wave_of_group;
+  unsigned char* lds_half = lds_raw + half * 2 * PD_STAGE;
+  // work items as in attn_prefill_kernel: long ones first, paired with short ones on a CU (SPLIT: one
+  // workgroup per CU, longest first)
   const int total = (int)gridDim.x, round = blockIdx.x / cus;
   const int taken = (round >> 1) * cus + blockIdx.x % cus;
-  const int item = (round & 1) ? taken : total - 1 - taken;
+  const int item = SPLIT ? total - 1 - (int)blockIdx.x : (round & 1) ? taken : total - 1 - taken;
   const int tile = item / heads;
   const int entry = tiles[2 * tile], tile_off = tiles[2 * tile + 1];
   const int h = item % heads, kvh = h / (heads / kv_heads);
@@ -566,8 +577,8 @@ __global__ __launch_bounds__(PT_THREADS) void attn_prefill_direct_kernel(
     for (int i = 0; i < PD_VLOADS; ++i) v_page[i] = table[min(max(tp + v_tab[i], page_lo), page_hi)];
   };
   auto issue = [&](int stage) {
-    unsigned char* to_k = lds_raw + stage * PD_STAGE + wave * PD_KLOADS * 1024;
-    unsigned char* to_v = lds_raw + stage * PD_STAGE + PD_KBYTES + wave * PD_VLOADS * 1024;
+    unsigned char* to_k = lds_half + stage * PD_STAGE + wave * PD_KLOADS * 1024;
+    unsigned char* to_v = lds_half + stage * PD_STAGE + PD_KBYTES + wave * PD_VLOADS * 1024;
 #pragma unroll
     for (int i = 0; i < PD_KLOADS; ++i)
       __builtin_amdgcn_global_load_lds(
@@ -651,24 +662,50 @@ __global__ __launch_bounds__(PT_THREADS) void attn_prefill_direct_kernel(
     }
   };
 
+  // this half's tiles: all of them, or with SPLIT the first or the second half of them (both halves pass the
+  // same number of barriers)
   const int first_tile = begin & ~(PT_KV - 1);
-  lookup(first_tile);
-  issue(0);
-  lookup(first_tile + PT_KV);
+  const int all_tiles = (end - first_tile + PT_KV - 1) / PT_KV;
+  const int steps = SPLIT ? (all_tiles + 1) / 2 : all_tiles;
+  const int my_tiles = half ? all_tiles - steps : steps;
+  const int my_first = first_tile + (half ? steps * PT_KV : 0);
+  lookup(my_first);
+  if (my_tiles > 0) issue(0);
+  lookup(my_first + PT_KV);
   wait_own_loads();
   __syncthreads();
   int stage = 0;
-  for (int p0 = first_tile; p0 < end; p0 += PT_KV) {
-    const bool more = p0 + PT_KV < end;
-    if (more) {
+  for (int i = 0; i < steps; ++i) {
+    const int p0 = my_first + i * PT_KV;
+    if (i + 1 < my_tiles) {
       issue(stage ^ 1);            // nobody reads that stage any more: the barrier that ended the last tile
       lookup(p0 + 2 * PT_KV);
     }
-    if (p0 < wave_end && p0 + PT_KV > wave_begin)
-      tile_body(!(p0 + PT_KV - 1 <= wave_first && p0 >= wave_lo_max), p0, lds_raw + stage * PD_STAGE);
+    if (i < my_tiles && p0 < wave_end && p0 + PT_KV > wave_begin)
+      tile_body(!(p0 + PT_KV - 1 <= wave_first && p0 >= wave_lo_max), p0, lds_half + stage * PD_STAGE);
     wait_own_loads();   // a barrier alone does not wait for loads that write LDS
     __syncthreads();
     stage ^= 1;
+  }
+  if constexpr (SPLIT) {
+    // the second half hands its state over in LDS (every tile has been read: the loop's last barrier)
+    f32x4* hand_o = (f32x4*)lds_raw;                                        // [8 waves][DT][64 lanes]
+    float* hand_ml = (float*)(lds_raw + PT_WAVES * DT * 64 * sizeof(f32x4));  // [8 waves][64 lanes][m, l]
+    if (half) {
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) hand_o[(wave * DT + dt) * 64 + lane] = o[dt];
+      hand_ml[(wave * 64 + lane) * 2] = m;
+      hand_ml[(wave * 64 + lane) * 2 + 1] = l;
+    }
+    __syncthreads();
+    if (half) return;
+    const float m1 = hand_ml[(wave * 64 + lane) * 2], l1 = hand_ml[(wave * 64 + lane) * 2 + 1];
+    const float m_both = fmaxf(m, m1);
+    const float a0 = m > -INFINITY ? __builtin_amdgcn_exp2f((m - m_both) * c2) : 0.f;
+    const float a1 = m1 > -INFINITY ? __builtin_amdgcn_exp2f((m1 - m_both) * c2) : 0.f;
+    l = l * a0 + l1 * a1;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) o[dt] = o[dt] * a0 + hand_o[(wave * DT + dt) * 64 + lane] * a1;
   }
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
@@ -846,12 +883,14 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(const float* __restric
 extern "C" int vk_attn_bf16_hdp() { return HDP; }
 
 // tiles: pairs (entry, first token of the tile within the entry), 128 tokens per tile; best sorted by the
-// number of positions a tile sees, rising (any order gives the same result).
+// number of positions a tile sees, rising (any order gives the same result). split: nonzero asks for workgroups
+// of sixteen waves that halve a tile's positions between them, where the kernel in use has that form (few tiles
+// of very different lengths); the result is the same up to rounding.
 extern "C" int vk_attn_bf16_prefill(const void* q, long long q_stride, const void* k_cache, const void* v_cache,
                                     void* out, const int* tiles, int num_tiles, const int* entry_start,
                                     const int* entry_first_pos, const int* block_table, int table_width,
                                     int block_size, int heads, int kv_heads, int hd, float scale, int window,
-                                    void* stream) {
+                                    int split, void* stream) {
   if (num_tiles <= 0) return 0;
   if (hd <= 0 || hd > HDP || (hd & 7) || block_size <= 0 || (block_size & 7) || heads <= 0 || kv_heads <= 0 ||
       heads % kv_heads || (q_stride & 7) || window < 0)
@@ -878,14 +917,19 @@ extern "C" int vk_attn_bf16_prefill(const void* q, long long q_stride, const voi
   if ((long long)num_tiles * heads > 0x7fffffffLL) return VK_UNSUPPORTED_SIZE;
 #ifdef VK_PREFILL_DIRECT
   if (fast && hd == HDP && block_size >= 8) {  // the kernel that loads straight into LDS
-    static bool direct_configured = false;
-    if (!direct_configured) {
-      hipError_t e = hipFuncSetAttribute((const void*)attn_prefill_direct_kernel,
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, 2 * PD_STAGE);
-      if (e != hipSuccess) return (int)e;
-      direct_configured = true;
+    const bool halves = split != 0 && PD_CAN_SPLIT;
+    auto direct = attn_prefill_direct_kernel<false>;
+    if constexpr (PD_CAN_SPLIT) {
+      if (halves) direct = attn_prefill_direct_kernel<true>;
     }
-    attn_prefill_direct_kernel<<<num_tiles * heads, PT_THREADS, 2 * PD_STAGE, (hipStream_t)stream>>>(
+    const int direct_lds = (halves ? 4 : 2) * PD_STAGE;
+    static bool direct_configured[2] = {false, false};
+    if (!direct_configured[halves]) {
+      hipError_t e = hipFuncSetAttribute((const void*)direct, hipFuncAttributeMaxDynamicSharedMemorySize, direct_lds);
+      if (e != hipSuccess) return (int)e;
+      direct_configured[halves] = true;
+    }
+    direct<<<num_tiles * heads, halves ? 2 * PT_THREADS : PT_THREADS, direct_lds, (hipStream_t)stream>>>(
         (const __bf16*)q, q_stride, (const __bf16*)k_cache, (const __bf16*)v_cache, (__bf16*)out, tiles, entry_start,
         entry_first_pos, block_table, table_width, block_size, heads, kv_heads, scale, window, cus);
     VK_LAUNCH_CHECK();

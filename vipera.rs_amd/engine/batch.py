@@ -64,6 +64,8 @@ class StepBatch:
     num_prefill_tiles: int = 0
     num_decode_entries: int = 0
     max_decode_kv_len: int = 0
+    max_tile_reach: int = 0        # positions that the last token of the longest prompt tile sees (no window counted)
+    sum_tile_reach: int = 0        # the same, added over the prompt tiles
 
 
 @dataclass
@@ -80,6 +82,8 @@ class PackedStep:
     slots: List[int]
     max_kv_len: int
     max_decode_kv_len: int
+    max_tile_reach: int = 0
+    sum_tile_reach: int = 0
 
     def flat(self) -> np.ndarray:
         return np.concatenate([s.reshape(-1) for s in self.sections]) if self.sections else np.zeros(0, np.int32)
@@ -155,6 +159,7 @@ def pack_entries(entries: Sequence[StepEntry], cache, vocab_size: int, min_table
     # by rising number of visible positions: the attention kernel pairs long tiles with short ones
     tile_list.sort()
     tiles: List[int] = [x for _, k, off in tile_list for x in (k, off)]
+    tile_reach = [p + min(TILE_TOKENS, int(counts_all[k]) - off) for p, k, off in tile_list]  # positions a tile's last token sees
     max_decode_kv = max((int(kv_len[k]) for k in singles), default=0)
 
     tables, widths = [], []
@@ -183,7 +188,7 @@ def pack_entries(entries: Sequence[StepEntry], cache, vocab_size: int, min_table
                 sources]
     sections += tables
     return PackedStep(sections, widths, T, E, len(rows), counts_all, [int(v) for v in first], [int(v) for v in slots],
-                      int(kv_len.max()), max_decode_kv)
+                      int(kv_len.max()), max_decode_kv, max(tile_reach, default=0), sum(tile_reach))
 
 
 def batch_from_buffer(packed: PackedStep, dev: torch.Tensor) -> StepBatch:
@@ -204,7 +209,8 @@ def batch_from_buffer(packed: PackedStep, dev: torch.Tensor) -> StepBatch:
         host_counts=packed.counts, host_first_pos=packed.first, host_slots=packed.slots,
         max_count=max(packed.counts), max_kv_len=packed.max_kv_len, all_single=max(packed.counts) == 1,
         num_prefill_tiles=packed.sections[8].size // 2, num_decode_entries=packed.sections[9].size,
-        max_decode_kv_len=packed.max_decode_kv_len,
+        max_decode_kv_len=packed.max_decode_kv_len, max_tile_reach=packed.max_tile_reach,
+        sum_tile_reach=packed.sum_tile_reach,
     )
 
 

@@ -564,8 +564,10 @@ def attn_bf16_supported(q: torch.Tensor, k_cache: torch.Tensor, head_dim: int) -
 def attn_bf16_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
                       tiles: torch.Tensor, entry_start: torch.Tensor, entry_first_pos: torch.Tensor,
                       block_table: torch.Tensor, heads: int, kv_heads: int, head_dim: int, scale: float,
-                      window: int) -> None:
-    """Attention of the entries' 128-token tiles listed in ``tiles`` (pairs: entry, first token within it)."""
+                      window: int, split: bool = False) -> None:
+    """Attention of the entries' 128-token tiles listed in ``tiles`` (pairs: entry, first token within it).
+    ``split``: workgroups of sixteen waves that halve a tile's positions between them and merge at the end, where
+    the kernel in use has that form (for few tiles of very different lengths); the same result up to rounding."""
     _dev(q, k_cache, v_cache, out, tiles, entry_start, entry_first_pos, block_table)
     _need(attn_bf16_supported(q, k_cache, head_dim), "attn_bf16: operands must be bfloat16 with 16-byte rows")
     _need(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= heads * head_dim, "attention: q")
@@ -577,11 +579,11 @@ def attn_bf16_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
           and entry_start.numel() == block_table.shape[0] + 1 and entry_first_pos.numel() == block_table.shape[0],
           "attention: entry arrays")
     module = f"attn_bf16_hd{attn_bf16_padded_width(head_dim)}"
-    fn = _fn(module, "vk_attn_bf16_prefill", [_p, _ll, _p, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _f, _i, _p],
+    fn = _fn(module, "vk_attn_bf16_prefill", [_p, _ll, _p, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _f, _i, _i, _p],
              key=module + ".prefill")
     _status(fn(_ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(tiles), tiles.numel() // 2,
                _ptr(entry_start), _ptr(entry_first_pos), _ptr(block_table), block_table.shape[1], k_cache.shape[2],
-               heads, kv_heads, head_dim, float(scale), int(window), _stream()), "attn_bf16_prefill")
+               heads, kv_heads, head_dim, float(scale), int(window), 1 if split else 0, _stream()), "attn_bf16_prefill")
 
 
 def attn_bf16_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
