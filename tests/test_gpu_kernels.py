@@ -67,13 +67,43 @@ def test_gemm_bf16_every_tiling_of_the_tiled_kernel(tiling, ranges):
         kernels.gemm_bf16_force_tiling(-1)
 
 
-@pytest.mark.parametrize("tiling", [0, 2, 3, 4, 9, 7, 8, 5, 10, 11, 12])   # the last three: 128 tokens x 96, 160, 224 rows
-def test_gated_product_with_every_tiling(tiling):
+@pytest.mark.parametrize("tiling", [9, 8])
+@pytest.mark.parametrize("ranges", [1, 3])
+def test_gemm_bf16_direct_tilings_with_three_lds_stages(tiling, ranges):
+    """The 128-token tilings of the kernel that loads straight into LDS, forced to three stages (what up to 128
+    tokens take by themselves) at any number of tokens: one, two, three, four and many K steps, so that the run
+    ends in each stage, with and without a step whose loads stay in flight."""
+    from vipera_rs_amd.ops import kernels
+    shapes = [(64, 520, 64), (100, 264, 128), (128, 300, 192), (257, 520, 256), (65, 2100, 4608), (33, 1028, 1600),
+              (300, 131, 1024)]
+    try:
+        kernels.gemm_bf16_force_tiling(tiling, ranges, stages=3)
+        for m, n, k in shapes:
+            g = torch.Generator().manual_seed(m + n + k)
+            a = torch.randn(m, k, generator=g).to(torch.bfloat16).to(DEV)
+            w = torch.randn(n, k, generator=g).to(torch.bfloat16).to(DEV)
+            bias = torch.randn(n, generator=g).to(DEV)
+            product = a.double() @ w.double().T
+            for out_dtype, tol in ((torch.float32, 1e-5), (torch.bfloat16, 6e-3)):
+                out = torch.full((m, n), 7.0, dtype=out_dtype, device=DEV)
+                kernels.gemm_bf16(a, w, bias, out, skinny_limit=0)
+                assert _rel(out, product + bias.double()) < tol, (m, n, k, out_dtype)
+            base = torch.randn(m, n, generator=g).to(DEV)
+            acc = base.clone()
+            kernels.gemm_bf16(a, w, None, acc, accumulate=True, skinny_limit=0)
+            assert _rel(acc, base.double() + product) < 1e-5, (m, n, k, "accumulate")
+    finally:
+        kernels.gemm_bf16_force_tiling(-1)
+
+
+@pytest.mark.parametrize("tiling,stages", [(t, 0) for t in (0, 2, 3, 4, 9, 7, 8, 5, 10, 11, 12)]   # the last three: 128 tokens x 96, 160, 224 rows
+                         + [(t, 3) for t in (9, 8, 10, 11, 12)] + [(t, 2) for t in (9, 11)])
+def test_gated_product_with_every_tiling(tiling, stages):
     from vipera_rs_amd.ops import kernels
     from vipera_rs_amd.ops.linear import interleave_gate_up
     try:
-        kernels.gemm_bf16_force_tiling(tiling)
-        for m, inter, k in [(300, 208, 192), (2048, 528, 128), (130, 1008, 640), (70, 48, 72)]:
+        kernels.gemm_bf16_force_tiling(tiling, 1, stages)
+        for m, inter, k in [(300, 208, 192), (2048, 528, 128), (130, 1008, 640), (70, 48, 72), (64, 304, 3584), (17, 160, 64)]:
             g = torch.Generator().manual_seed(m + inter + k)
             a = torch.randn(m, k, generator=g).to(torch.bfloat16).to(DEV)
             gate = torch.randn(inter, k, generator=g).to(torch.bfloat16).to(DEV)

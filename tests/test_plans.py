@@ -29,12 +29,11 @@ def test_the_lds_shared_product_splits_k_where_rows_are_few():
 def test_past_64_tokens_the_weights_are_streamed_where_tiles_would_be_few():
     for n, k in (QKV_7B, O_7B, DOWN_7B, HEAD_7B):
         assert streams_weights(64, n, k) and not streams_weights(129, n, k)
-    for n, k in (QKV_7B, O_7B, DOWN_7B, (5120, 27648), (2048, 1536)):
-        assert streams_weights(65, n, k) and streams_weights(80, n, k)
-    assert not streams_weights(65, *HEAD_7B)               # 152,064 rows fill the tiled kernel at any token count
-    assert streams_weights(128, *O_7B) and streams_weights(128, 2048, 1536) and streams_weights(128, 1536, 8960)
-    assert not streams_weights(128, *DOWN_7B) and not streams_weights(81, *QKV_7B) and not streams_weights(96, 5120, 27648)
-    assert mid_plan(65, *DOWN_7B) == (8, 1) and mid_plan(96, *O_7B) == (4, 1) and mid_plan(128, 2048, 1536) == (4, 1)
+    for m in (65, 96, 128):                                # small weights only: the 7B output projection, the 1.5B widths
+        assert streams_weights(m, *O_7B) and streams_weights(m, 2048, 1536) and streams_weights(m, 1536, 8960)
+        assert not streams_weights(m, *DOWN_7B) and not streams_weights(m, *QKV_7B) and not streams_weights(m, *HEAD_7B)
+        assert not streams_weights(m, 5120, 27648)
+    assert mid_plan(65, 1536, 8960) == (8, 1) and mid_plan(96, *O_7B) == (4, 1) and mid_plan(128, 2048, 1536) == (4, 1)
     assert mid_plan(100, 1024, 320) == (1, 1)              # no range shorter than 256
 
 
@@ -47,8 +46,9 @@ def test_the_gated_product_goes_resident_tiled_or_lds_shared():
         assert gated_plan(m, *GATE_UP_7B) == 0             # 1184 pairs over 256 CUs: 4 or 5 each
     assert gated_plan(8, 17920, 1536) in (1, 2)            # 1.5B: 560 pairs would be 2 or 3 each, too uneven
     assert gated_plan(8, 55296, 5120) == 0
-    assert gated_plan(32, *GATE_UP_7B) in (1, 2) and gated_plan(64, *GATE_UP_7B) == 3
-    assert gated_plan(24, 55296, 5120) == 3 and gated_plan(64, 17920, 1536) in (1, 2)
+    assert gated_plan(17, *GATE_UP_7B) == 3 and gated_plan(64, *GATE_UP_7B) == 3   # past the resident kernel: tiled
+    assert gated_plan(24, 55296, 5120) == 3
+    assert gated_plan(48, 17920, 1536) in (1, 2) and gated_plan(64, 17920, 1536) == 3
     assert gated_plan(8, *GATE_UP_7B, cus=304) == 0        # 1184 pairs over 304 CUs: 3 or 4 each, 3 % above the mean
     assert gated_plan(8, *GATE_UP_7B, cus=500) != 0        # over 500: 2 or 3 each, 27 % above the mean
 

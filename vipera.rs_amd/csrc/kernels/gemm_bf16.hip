@@ -321,14 +321,23 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_tile_kernel(const __bf16* _
 //   multiply the second half.
 // K ranges must be multiples of 64 (the launcher sends other shapes to gemm_tile_kernel). Four stages of
 // 32 k, which give a load three short steps to arrive instead of one long one, were slower.
+// STAGES 3 (for up to 128 tokens, where the product is a stream of the weights and a CU's bytes in flight are
+// what bounds it): step s + 3 is requested when step s's stage is free, and the barrier of a step waits for
+// step s + 1 only, so the loads of two steps are in flight instead of one.
 constexpr int DIRECT_ROW = BK * 2;  // bytes per LDS row
 
 // Until none of the wave's vector memory loads is in flight (s_waitcnt vmcnt(0), the other counters left
 // alone). A barrier alone does not wait for loads that write LDS: the compiler's fence only waits for the
 // wave's LDS instructions.
 __device__ __forceinline__ void wait_own_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+// Until at most N of them are (loads complete in the order of their issue): s_waitcnt vmcnt(N).
+template <int N>
+__device__ __forceinline__ void wait_own_loads_but() {
+  static_assert(N >= 0 && N < 64, "vmcnt has six bits");
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | 0x0F70);
+}
 
-template <int BM, int BN, int WM, int WN, typename TC, bool ACCUMULATE, bool GATED>
+template <int BM, int BN, int WM, int WN, typename TC, bool ACCUMULATE, bool GATED, int STAGES = 2>
 __global__ __launch_bounds__(WM * WN * 64) void gemm_tile_direct_kernel(const __bf16* __restrict__ A,
                                                                           const __bf16* __restrict__ W,
                                                                           const float* __restrict__ bias,
@@ -344,7 +353,9 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_tile_direct_kernel(const __
   constexpr int A_LOADS = BM / 8 / WAVES, W_LOADS = BN / 8 / WAVES;  // load instructions per wave and step
   static_assert(BM % (8 * WAVES) == 0 && BN % (8 * WAVES) == 0, "tile rows must divide among the waves' loads");
   constexpr int STAGE = (BM + BN) * DIRECT_ROW;
-  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];  // [2][BM + BN][128]
+  constexpr int LOADS = A_LOADS + W_LOADS;
+  static_assert(STAGES == 2 || STAGES == 3, "two or three LDS stages");
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];  // [STAGES][BM + BN][128]
 
   const int total = tiles_m * tiles_n;
   const int per_xcd = (total + XCDS - 1) / XCDS;
@@ -410,14 +421,19 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_tile_direct_kernel(const __
   bf16x8 fa0[TM], fw0[TN], fa1[TM], fw1[TN];
   issue_loads(0, 0);
   if (steps > 1) issue_loads(1, 1);
-  wait_own_loads();
+  if (STAGES == 3 && steps > 2) {
+    issue_loads(2, 2);
+    wait_own_loads_but<2 * LOADS>();  // step 0 has arrived; the other two stay in flight
+  } else {
+    wait_own_loads();
+  }
   __syncthreads();
   read_fragments(0, 0, fa0, fw0);
   // Hints for the instruction order within a half step: the LDS reads and the loads go out one by one
   // between products, so that their issue hides behind the matrix core's work instead of stalling it.
   auto interleave = [](auto lds_reads, auto loads) {
-    constexpr int READS = decltype(lds_reads)::value, LOADS = decltype(loads)::value;
-    static_for<LOADS>([](auto) {
+    constexpr int READS = decltype(lds_reads)::value, LOADS_NOW = decltype(loads)::value;
+    static_for<LOADS_NOW>([](auto) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one matrix instruction
       __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one load
     });
@@ -427,25 +443,30 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_tile_direct_kernel(const __
     });
     __builtin_amdgcn_sched_group_barrier(0x008, TM * TN, 0);
   };
-  auto step = [&](int s, auto with_loads, auto with_next) {
-    const int stage = s & 1;
+  // `in_flight`: how many later steps' loads may stay in flight at the barrier (all of a step's loads that were
+  // issued before them have then arrived)
+  auto step = [&](int s, int stage, auto with_loads, auto with_next, auto in_flight) {
+    const int next_stage = stage + 1 == STAGES ? 0 : stage + 1;
     read_fragments(stage, 1, fa1, fw1);
     multiply(fa0, fw0);
     interleave(std::integral_constant<int, TM + TN>{}, std::integral_constant<int, 0>{});
     __builtin_amdgcn_sched_barrier(0);  // the products stay on this side: they cover the reads above
-    wait_own_loads();
+    wait_own_loads_but<decltype(in_flight)::value * LOADS>();
     __syncthreads();
-    if constexpr (decltype(with_loads)::value) issue_loads(stage, s + 2);
-    if constexpr (decltype(with_next)::value) read_fragments(stage ^ 1, 0, fa0, fw0);
+    if constexpr (decltype(with_loads)::value) issue_loads(stage, s + STAGES);
+    if constexpr (decltype(with_next)::value) read_fragments(next_stage, 0, fa0, fw0);
     multiply(fa1, fw1);
     interleave(std::integral_constant<int, decltype(with_next)::value ? TM + TN : 0>{},
-               std::integral_constant<int, decltype(with_loads)::value ? A_LOADS + W_LOADS : 0>{});
+               std::integral_constant<int, decltype(with_loads)::value ? LOADS : 0>{});
     __builtin_amdgcn_sched_barrier(0);
   };
-  int s = 0;
-  for (; s + 2 < steps; ++s) step(s, std::true_type{}, std::true_type{});
-  if (s + 1 < steps) step(s++, std::false_type{}, std::true_type{});
-  step(s, std::false_type{}, std::false_type{});
+  int s = 0, stage = 0;
+  auto advance = [&]() { stage = stage + 1 == STAGES ? 0 : stage + 1; };
+  for (; s + STAGES < steps; ++s, advance())   // with three stages the step after next stays in flight
+    step(s, stage, std::true_type{}, std::true_type{}, std::integral_constant<int, STAGES - 2>{});
+  for (; s + 1 < steps; ++s, advance())
+    step(s, stage, std::false_type{}, std::true_type{}, std::integral_constant<int, 0>{});
+  step(s, stage, std::false_type{}, std::false_type{}, std::integral_constant<int, 0>{});
 
   const int wave_m = m0 + wm * TM * 16, wave_n = n0 + wn * TN * 16;
   if constexpr (GATED) {
@@ -1519,24 +1540,26 @@ int launch_mid(const __bf16* A, const __bf16* W, const float* bias, TC* C, float
   return VK_UNSUPPORTED_SIZE;
 }
 
-template <bool DIRECT, int BM, int BN, int WM, int WN, typename TC, bool ACC, bool GATED>
+template <bool DIRECT, int BM, int BN, int WM, int WN, typename TC, bool ACC, bool GATED, int STAGES>
 constexpr auto tile_kernel() {
-  if constexpr (DIRECT) return gemm_tile_direct_kernel<BM, BN, WM, WN, TC, ACC, GATED>;
+  if constexpr (DIRECT) return gemm_tile_direct_kernel<BM, BN, WM, WN, TC, ACC, GATED, STAGES>;
   else return gemm_tile_kernel<BM, BN, WM, WN, TC, ACC, GATED>;
 }
 
-// DIRECT: the kernel that loads straight into LDS; K must be a multiple of 64.
-template <int BM, int BN, int WM, int WN, typename TC, bool ACC, bool GATED, bool DIRECT = false>
+// DIRECT: the kernel that loads straight into LDS; K must be a multiple of 64. STAGES: its LDS stages.
+template <int BM, int BN, int WM, int WN, typename TC, bool ACC, bool GATED, bool DIRECT = false, int STAGES = 2>
 int launch_tile_as(const __bf16* A, const __bf16* W, const float* bias, TC* C, int M, int N, int K, long long lda,
                    long long ldc, int vector_ok, int ranges, float* partial, hipStream_t s) {
-  constexpr int lds_bytes = DIRECT ? 2 * (BM + BN) * DIRECT_ROW : 2 * (BM + BN) * ROW * (int)sizeof(__bf16);
+  static_assert(DIRECT || STAGES == 2, "only the direct kernel has a third stage");
+  constexpr int lds_bytes = DIRECT ? STAGES * (BM + BN) * DIRECT_ROW : 2 * (BM + BN) * ROW * (int)sizeof(__bf16);
+  static_assert(lds_bytes <= 160 * 1024, "a CU has 160 KB of LDS");
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
   const long long total = (long long)tiles_m * tiles_n;
   const long long grid = (total + XCDS - 1) / XCDS * XCDS;
   if (grid > 0x7fffffffLL) return VK_UNSUPPORTED_SIZE;
   if (ranges <= 1 || GATED) {
     static bool configured = false;
-    auto kernel = tile_kernel<DIRECT, BM, BN, WM, WN, TC, ACC, GATED>();
+    auto kernel = tile_kernel<DIRECT, BM, BN, WM, WN, TC, ACC, GATED, STAGES>();
     if (!configured) {
       hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
       if (e != hipSuccess) return (int)e;
@@ -1550,7 +1573,7 @@ int launch_tile_as(const __bf16* A, const __bf16* W, const float* bias, TC* C, i
   // K split over workgroups: float partial sums [range, M, N], then the ranges are added in ascending order
   if constexpr (!GATED) {
     static bool configured_partial = false;
-    auto kernel = tile_kernel<DIRECT, BM, BN, WM, WN, float, false, false>();
+    auto kernel = tile_kernel<DIRECT, BM, BN, WM, WN, float, false, false, STAGES>();
     if (!configured_partial) {
       hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
       if (e != hipSuccess) return (int)e;
@@ -1571,6 +1594,7 @@ int launch_tile_as(const __bf16* A, const __bf16* W, const float* bias, TC* C, i
 
 int g_tile_config = -1;  // -1: chosen by shape; else a tiling (see launch_tile) and g_tile_ranges force a plan, for measurements
 int g_tile_ranges = 1;
+int g_tile_stages = 0;   // 0: chosen by shape; 2 or 3 force the direct kernel's LDS stages where the tiling has both
 
 // Which tiling, and into how many ranges K is split: the pair with the shortest estimated time. A full GPU
 // of 256x256 tiles runs at about 1.15 PFLOP/s with the kernel that loads straight into LDS and at 1.0
@@ -1644,26 +1668,37 @@ int launch_tile(const __bf16* A, const __bf16* W, const float* bias, TC* C, int 
   const int r = plan.ranges;
 #define VK_TILE(BMV, BNV, WMV, WNV, DIRECTV) \
   return launch_tile_as<BMV, BNV, WMV, WNV, TC, ACC, GATED, DIRECTV>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, r, partial, s)
+  // the 128-token tiles of the direct kernel with a third LDS stage: up to 128 tokens the product is a stream of
+  // the weights (with more tokens, and so more tiles per weight row, two stages measured the same or better)
+#define VK_TILE_DEEP(BMV, BNV, WMV, WNV)                                                                              \
+  {                                                                                                                  \
+    if (deep)                                                                                                        \
+      return launch_tile_as<BMV, BNV, WMV, WNV, TC, ACC, GATED, true, 3>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, r, \
+                                                                         partial, s);                                \
+    VK_TILE(BMV, BNV, WMV, WNV, true);                                                                               \
+  }
+  const bool deep = g_tile_stages ? g_tile_stages == 3 : M <= 128;
   if constexpr (GATED) {
     switch (plan.config) {
       // four waves side by side along the tokens: a wave owns all rows of the tile, an even number of 16-row
       // tiles, so gate and up rows of the same outputs meet in one wave
-      case 10: VK_TILE(128, 96, 4, 1, true);
-      case 11: VK_TILE(128, 160, 4, 1, true);
-      case 12: VK_TILE(128, 224, 4, 1, true);
+      case 10: VK_TILE_DEEP(128, 96, 4, 1);
+      case 11: VK_TILE_DEEP(128, 160, 4, 1);
+      case 12: VK_TILE_DEEP(128, 224, 4, 1);
     }
   }
   switch (plan.config) {
     case 5: VK_TILE(256, 256, 4, 2, true);
     case 6: VK_TILE(256, 192, 4, 2, true);
     case 7: VK_TILE(256, 128, 4, 2, true);
-    case 8: VK_TILE(128, 256, 2, 4, true);
-    case 9: VK_TILE(128, 128, 2, 2, true);
+    case 8: VK_TILE_DEEP(128, 256, 2, 4);
+    case 9: VK_TILE_DEEP(128, 128, 2, 2);
     case 2: VK_TILE(256, 128, 4, 2, false);
     case 3: VK_TILE(128, 256, 2, 4, false);
     case 4: VK_TILE(256, 256, 4, 4, false);
     default: VK_TILE(128, 128, 2, 2, false);
   }
+#undef VK_TILE_DEEP
 #undef VK_TILE
 }
 }  // namespace
@@ -1957,8 +1992,10 @@ extern "C" int vk_gemm_bf16_gated_scaled(const void* A, const void* W, void* C, 
                                      (hipStream_t)stream);
 }
 
-extern "C" int vk_gemm_bf16_tile_config(int tiling, int ranges) {
+extern "C" int vk_gemm_bf16_tile_config(int tiling, int ranges, int stages) {
+  if (stages != 0 && stages != 2 && stages != 3) return VK_BAD_ARGUMENT;
   g_tile_config = tiling;
   g_tile_ranges = ranges;
+  g_tile_stages = stages;
   return 0;
 }

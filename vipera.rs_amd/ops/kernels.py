@@ -540,14 +540,16 @@ TILE_TILINGS = {0: "128x128 staged", 2: "256x128 staged", 3: "128x256 staged", 4
                 10: "128x96 direct, gated only", 11: "128x160 direct, gated only", 12: "128x224 direct, gated only"}
 
 
-def gemm_bf16_force_tiling(tiling: int = -1, ranges: int = 1) -> None:
+def gemm_bf16_force_tiling(tiling: int = -1, ranges: int = 1, stages: int = 0) -> None:
     """For tests and measurements: make the tiled kernel of :func:`gemm_bf16` and :func:`gemm_bf16_gated`
     use one tiling (a key of ``TILE_TILINGS``) and split K into ``ranges``; ``-1`` gives the choice back
-    to the launcher.  A "direct" tiling falls back to its staged twin when K is no multiple of 64."""
+    to the launcher.  A "direct" tiling falls back to its staged twin when K is no multiple of 64.  ``stages``:
+    2 or 3 LDS stages for the direct 128-token tilings (0: three up to 128 tokens, else two)."""
     if tiling >= 0:
         _need(tiling in TILE_TILINGS and 1 <= ranges <= 8, "gemm_bf16_force_tiling: unknown tiling or ranges")
-    fn = _fn("gemm_bf16", "vk_gemm_bf16_tile_config", [_i, _i])
-    _status(fn(-1 if tiling < 0 else tiling, int(ranges)), "gemm_bf16_force_tiling")
+    _need(stages in (0, 2, 3), "gemm_bf16_force_tiling: stages are 0 (by shape), 2 or 3")
+    fn = _fn("gemm_bf16", "vk_gemm_bf16_tile_config", [_i, _i, _i])
+    _status(fn(-1 if tiling < 0 else tiling, int(ranges), int(stages)), "gemm_bf16_force_tiling")
 
 
 # ----------------------------------------------------------------------------------------------

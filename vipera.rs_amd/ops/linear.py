@@ -5,7 +5,7 @@ combination (the 32-bit run, or a matrix kept in 32-bit inside a bfloat16 run) g
 32-bit FMA kernel.  Among the matrix-core kernels the number of rows of ``a`` (tokens) decides:
 
 * many (prompts): the LDS-tiled kernel;
-* up to 64 (decoding), and up to 80 or 128 where that was measured faster (:func:`streams_weights`): the
+* up to 64 (decoding), and up to 128 for small weights (:func:`streams_weights`): the
   product is a stream of the weights.  Up to four tokens, or a small weight
   at up to 16 tokens, use the kernel whose waves split K inside a workgroup; otherwise the kernel that
   shares the activations through LDS, with K split over workgroups where the weight has too few rows
@@ -23,15 +23,13 @@ from . import kernels
 
 def streams_weights(m: int, n: int, k: int) -> bool:
     """Whether a bfloat16 product of ``m`` tokens runs on a weight-streaming kernel rather than the tiled one:
-    always up to 64 tokens; up to 80 for every weight but an output matrix (whose many rows fill the tiled
-    kernel as well), and up to 128 for a small weight, where 128-token tiles are too few to fill the GPU
-    (7B widths at 65 tokens: output projection 13.5 against 16.4 us, down projection 40.7 against 43.7; the 32B
-    down projection 78 against 103; 1.5B q/k/v 9.1 against 17.5; from 96 tokens on only the small weights gain)."""
+    always up to 64 tokens, and up to 128 for a small weight, whose 128-token tiles are too few to fill the GPU
+    (at 65 and 112 tokens: the 7B output projection 13.8 and 16.1 us against 16.1 and 17.4 tiled, the 1.5B q/k/v
+    9.2 and 10.9 against 17.8 and 13.9; the larger weights are as fast or faster on the tiled kernel with its
+    three LDS stages: the 7B down projection 36.3 against 41.8 at 80 tokens)."""
     if m <= 64:
         return True
-    if n >= 100_000:
-        return False
-    return m <= 80 or (m <= 128 and n * k <= 16_000_000)
+    return m <= 128 and n * k <= 16_000_000
 
 
 def mid_plan(m: int, n: int, k: int) -> Tuple[int, int]:
@@ -138,9 +136,10 @@ def gated_plan(m: int, n: int, k: int, cus: int = 256) -> int:
     pairs = n // 32
     if gated_resident_fits(m, n, k) and -(-pairs // cus) * cus <= 1.15 * pairs:
         return 0
-    if m * n * k >= 6.5e9:
-        # many tokens on a large weight: the tiled kernel (3), which reads a tile's activations once for 256
-        # weight rows, passes the LDS-shared one (7B widths from about 52 tokens, 32B from about 20, 1.5B never)
+    if n * k >= 1e8 or m * n * k >= 1.5e9:
+        # a large weight, or many tokens on a small one: the tiled kernel (3) with its three LDS stages and tiles
+        # of 96 to 224 weight rows that fill the CUs in one round passes the LDS-shared one (7B widths at 17 to 64
+        # tokens: 51 to 54 us against 57 to 71; 32B: 102 to 106 against 110 to 120; 1.5B from 64 tokens)
         return 3
     return gated_rows_per_wave(m, n)
 
