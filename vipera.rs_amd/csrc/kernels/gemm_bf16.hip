@@ -1599,7 +1599,8 @@ int g_tile_stages = 0;   // 0: chosen by shape; 2 or 3 force the direct kernel's
 // Which tiling, and into how many ranges K is split: the pair with the shortest estimated time. A full GPU
 // of 256x256 tiles runs at about 1.15 PFLOP/s with the kernel that loads straight into LDS and at 1.0
 // with the staged one (measured on the 7B shapes at 2,048 tokens); the smaller tiles reach 0.75 to 0.8 of
-// their kernel's best, 256x192 about 0.9. Workgroups run in whole rounds of one per CU (two for the 128x128
+// their kernel's best, 256x192 about 0.9, and 256x128 with its three LDS stages about 0.95 (it is what the output
+// and down projections of 512 to 2,048 tokens run on, where 256x256 tiles are too few). Workgroups run in whole rounds of one per CU (two for the 128x128
 // tile, whose LDS lets two share a CU, unless every workgroup finds a CU of its own), so a launch that fills
 // the last round badly loses that share. Splitting K
 // multiplies the workgroups, at the price of writing and re-reading float partial sums (they mostly stay
@@ -1622,7 +1623,7 @@ TilePlan choose_tile_plan(int M, int N, int K, long long partial_floats, bool di
   // that with 128 of them a tile the tiles come in more than one round and less than two (7B width at 64 tokens:
   // 296 tiles of 128 rows, two to a CU on 40 CUs, one on the others); a width of 96, 160 or 224 rows can come
   // close to one tile per CU (237 tiles of 160 rows)
-  static const Tiling straight[] = {{5, 256, 256, 1, 1.15}, {7, 256, 128, 1, 0.92}, {8, 128, 256, 1, 0.88}, {9, 128, 128, 2, 0.9},
+  static const Tiling straight[] = {{5, 256, 256, 1, 1.15}, {7, 256, 128, 1, 1.1}, {8, 128, 256, 1, 0.88}, {9, 128, 128, 2, 0.9},
                                     {6, 256, 192, 1, 1.05}, {10, 128, 96, 2, 0.85}, {11, 128, 160, 2, 0.88}, {12, 128, 224, 1, 0.88}};
   const Tiling* tilings = direct ? straight : staged;
   TilePlan best{tilings[3].config, 1};
@@ -1690,7 +1691,11 @@ int launch_tile(const __bf16* A, const __bf16* W, const float* bias, TC* C, int 
   switch (plan.config) {
     case 5: VK_TILE(256, 256, 4, 2, true);
     case 6: VK_TILE(256, 192, 4, 2, true);
-    case 7: VK_TILE(256, 128, 4, 2, true);
+    case 7:  // three stages fit this tile's LDS, and its loads per product are the most of the 256-token tiles
+      if (g_tile_stages != 2)
+        return launch_tile_as<256, 128, 4, 2, TC, ACC, GATED, true, 3>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, r,
+                                                                       partial, s);
+      VK_TILE(256, 128, 4, 2, true);
     case 8: VK_TILE_DEEP(128, 256, 2, 4);
     case 9: VK_TILE_DEEP(128, 128, 2, 2);
     case 2: VK_TILE(256, 128, 4, 2, false);
