@@ -49,6 +49,9 @@ SHAPES = {
 }
 
 
+SETTLE_STEPS = 96   # untimed decode steps between the prompts and the warm-up steps (see decode())
+
+
 def log(text):
     print(f"[bench] {text}", file=sys.stderr, flush=True)
 
@@ -152,9 +155,9 @@ def main() -> int:
         # every prompt gets a portion in every prefill step, so that all requests start decoding together
         engine = Engine(None, runner=runner, max_num_seqs=batch, max_num_batched_tokens=batch * 2048, chunk_size=2048,
                         max_model_len=ctx + 8, pipelined=not args.in_turn)
-        prompt_len = ctx - steps - warmup - 1
+        prompt_len = ctx - steps - warmup - SETTLE_STEPS - 1
         for _ in range(batch):
-            engine.add_request(tokens(prompt_len), max_new_tokens=steps + warmup + 4)
+            engine.add_request(tokens(prompt_len), max_new_tokens=steps + warmup + SETTLE_STEPS + 4)
         last = time.perf_counter()
         for guard in range(10_000):  # prefill, until every request has its first token and the next step is all decode
             if guard == 9_999 or not engine.has_work():
@@ -165,6 +168,11 @@ def main() -> int:
                 last = time.perf_counter()
             if engine.scheduler.num_waiting == 0 and report.num_batched_tokens == batch:
                 break
+        # The GPU's power management takes about 0.2 s to settle after the change from prompts to decoding: for
+        # that long every decode step takes 3.5 % longer (3.885 then 3.745 ms at batch 8, from one step to the
+        # next). These untimed steps let it settle; the warm-up steps asked for follow them.
+        for _ in range(SETTLE_STEPS):
+            engine.step()
         for _ in range(warmup - 1):
             engine.step()
         torch.cuda.synchronize()
@@ -176,6 +184,17 @@ def main() -> int:
         torch.cuda.synchronize()
         seconds = time.perf_counter() - t0
         log(f"  host microseconds per step: " + ", ".join(f"{k} {v // steps}" for k, v in engine.micros.items()))
+        # the same captured step replayed back to back, nothing else in the stream: what the GPU alone needs for it
+        graphs = getattr(runner, "graphs", None)
+        if graphs is not None and graphs.graphs:
+            captured = list(graphs.graphs.values())[-1]
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            for _ in range(8):
+                captured.graph.replay()
+            torch.cuda.synchronize()
+            log(f"  the step's graph alone, replayed back to back: {(time.perf_counter() - t1) / 8 * 1e3:.3f} ms "
+                f"(the engine's step: {seconds / steps * 1e3:.3f} ms)")
         mean_ctx = ctx - steps / 2.0
         for request in list(engine._live):
             engine.cancel(request)
@@ -213,6 +232,7 @@ def main() -> int:
             "head_dim": config.head_dim, "intermediate": I, "vocab": V, "global_batch": args.batch,
             "seq_len": ctx, "prefill_tokens": T, "block_size": args.block_size, "parallelism": "single GPU",
             "sampling": "greedy", "weights_gb": round(weight_bytes / 1e9, 2), "steps_launched_ahead": not args.in_turn,
+            "untimed_decode_steps_before_warmup": SETTLE_STEPS,
         },
         "prefill": prefill,
         "roofline": {"bound": "hbm", "achieved": round(head["gbs"], 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",

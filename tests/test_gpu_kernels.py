@@ -609,3 +609,23 @@ def test_gated_product_and_interleaved_swiglu(m, inter, k):
     plain = torch.empty(m, inter, dtype=torch.bfloat16, device=DEV)
     linear_gated(a, torch.cat([gate, up]).contiguous(), plain, False)
     assert _rel(plain, want) < 1.2e-2
+
+
+@pytest.mark.parametrize("count", [1, 3, 4, 1023, 70_000])
+def test_a_steps_words_are_fetched_from_pinned_host_memory(count):
+    """The kernel that stands for the host-to-device copy of a step's metadata: the words arrive as they are, in
+    stream order, also when the pinned buffer is written again after the stream has been drained."""
+    from vipera_rs_amd.errors import InvalidArgumentError
+    from vipera_rs_amd.ops import kernels
+    g = torch.Generator().manual_seed(count)
+    host = torch.randint(-2 ** 31, 2 ** 31 - 1, (count,), generator=g, dtype=torch.int64).to(torch.int32).pin_memory()
+    out = torch.full((count,), 7, dtype=torch.int32, device=DEV)
+    if not kernels.fetch_words(host, out):
+        pytest.skip("this runtime gives pinned host memory no device address")
+    assert torch.equal(out.cpu(), host)
+    torch.cuda.synchronize()
+    host.numpy()[:] = 5
+    assert kernels.fetch_words(host, out)
+    assert int(out.min()) == 5 and int(out.max()) == 5
+    with pytest.raises(InvalidArgumentError):
+        kernels.fetch_words(torch.zeros(count, dtype=torch.int32), out)   # pageable memory is refused on the host

@@ -17,6 +17,7 @@ from typing import Dict, Optional, Sequence, Tuple
 import numpy as np
 import torch
 
+from ..ops import kernels
 from .batch import PackedStep, StepEntry, batch_from_buffer, pack_entries
 
 BATCH_BUCKETS = (1, 2, 4, 8, 16, 24, 32, 48, 64, 96, 128, 192, 256)
@@ -112,7 +113,10 @@ class DecodeGraphs:
         captured.turn ^= 1
         staging = captured.staging[captured.turn]
         staging.numpy()[:] = flat
-        captured.buffer.copy_(staging, non_blocking=True)
+        # a kernel fetches the step's words from the pinned buffer: a copy command of this size goes to the copy
+        # engine, whose hand-over leaves the GPU idle between two steps
+        if not kernels.fetch_words(staging, captured.buffer):
+            captured.buffer.copy_(staging, non_blocking=True)
         captured.graph.replay()
         self.replays += 1
         rows = [k for k, e in enumerate(entries) if len(e.want)]

@@ -80,6 +80,23 @@ def _fn(module: str, name: str, argtypes, key: str = None):
 
 
 # ----------------------------------------------------------------------------------------------
+def fetch_words(pinned: torch.Tensor, out: torch.Tensor) -> bool:
+    """``out[:] = pinned[:]`` (int32 words) by a kernel that reads the pinned host tensor directly, in the current
+    stream.  Returns False, having done nothing, if the runtime does not give the host memory a device address
+    (the caller then copies with ``out.copy_``)."""
+    _dev(out)
+    _need(not pinned.is_cuda and pinned.is_pinned(), "fetch_words: the source must be pinned host memory")
+    _need(pinned.dtype == torch.int32 and out.dtype == torch.int32 and pinned.is_contiguous() and out.is_contiguous()
+          and pinned.numel() == out.numel(), "fetch_words: two contiguous int32 tensors of one size")
+    fn = _fn("elementwise", "vk_fetch_words", [_p, _p, _ll, _p])
+    code = fn(pinned.data_ptr(), _ptr(out), out.numel(), _stream())
+    if code == -2:
+        return False
+    _status(code, "fetch_words")
+    return True
+
+
+# ----------------------------------------------------------------------------------------------
 def embed_gather(table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor,
                  source: Optional[torch.Tensor] = None, sampled: Optional[torch.Tensor] = None) -> None:
     """``out[t, :] = table[tokens[t], :]`` widened to 32-bit.  The caller has checked the ids.
