@@ -261,8 +261,12 @@ def serving(args, config, runtime, model, shape_name, layers_full, dtype_key) ->
     runner = ModelRunner(model, runtime, args.block_size, pages, requests + 1, use_graphs=True, max_context=context)
     engine = Engine(None, runner=runner, max_num_seqs=requests, max_num_batched_tokens=budget, chunk_size=chunk,
                     max_model_len=context, pipelined=not args.in_turn)
-    # a short run first: kernel modules are compiled and loaded, decode graphs of the small buckets captured
+    # a short run first: kernel modules are compiled and loaded; then the decode steps of every size are captured,
+    # as a server does before it takes requests
     engine.generate([prompts[0][:600], prompts[1][:300]], 8)
+    started = time.perf_counter()
+    captured = engine.warm_up()
+    log(f"{captured} decode steps captured ahead in {time.perf_counter() - started:.1f} s")
     for prompt in prompts:
         engine.add_request(prompt, new_tokens)
     torch.cuda.synchronize()
@@ -291,7 +295,7 @@ def serving(args, config, runtime, model, shape_name, layers_full, dtype_key) ->
         "config": {"model": shape_name, "layers": args.layers, "layers_full": layers_full, "requests": requests,
                    "prompt_tokens": prompt_tokens, "new_tokens_each": new_tokens, "chunk_size": chunk,
                    "max_num_batched_tokens": budget, "seq_len": context, "block_size": args.block_size,
-                   "steps_launched_ahead": not args.in_turn},
+                   "steps_launched_ahead": not args.in_turn, "decode_steps_captured_ahead": captured},
         "generated_per_second": round(generated / seconds, 1), "seconds": round(seconds, 3),
     }), flush=True)
     return 0

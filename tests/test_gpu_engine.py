@@ -322,3 +322,25 @@ def test_cancel_while_a_step_is_on_its_way(folders):
             done[g.request] = g
     assert list(done) == [second] and done[second].tokens == want
     assert engine.runner.cache.check() == "" and engine.runner.cache.live_requests() == 0
+
+
+@pytest.mark.gpu
+def test_decode_steps_captured_ahead_are_the_ones_that_generation_replays():
+    """warm_up captures every batch and context bucket once; generation afterwards captures nothing more and gives
+    the tokens of an engine that captures as it goes."""
+    import tempfile
+    from helpers import CONFIG_A, make_folder, random_tokens
+    from vipera_rs_amd import Engine
+    with tempfile.TemporaryDirectory() as tmp:
+        make_folder(tmp, CONFIG_A, 5, torch.float32)
+        prompts = [random_tokens(CONFIG_A["vocab_size"], n, 70 + n) for n in (9, 30, 17)]
+        lazy = Engine(tmp, dtype="float32", max_num_seqs=4, max_model_len=300).generate(prompts, 24)
+        engine = Engine(tmp, dtype="float32", max_num_seqs=4, max_model_len=300)
+        made = engine.warm_up()
+        assert made == 3 * 2                       # batch buckets 1, 2, 4 x context buckets 256, 512
+        assert engine.warm_up() == 0               # nothing left to capture
+        graphs = engine.runner.graphs
+        before = set(graphs.graphs)
+        ahead = engine.generate(prompts, 24)
+        assert set(graphs.graphs) == before and graphs.replays > 0
+        assert [g.tokens for g in ahead] == [g.tokens for g in lazy]

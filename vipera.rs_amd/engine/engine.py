@@ -141,6 +141,17 @@ class Engine:
         self.failed = 0
         self.step_count = 0
         self.micros = {"schedule": 0, "compute": 0, "sample": 0}
+        self.max_num_seqs = int(max_num_seqs)
+
+    def warm_up(self, max_batch: Optional[int] = None, max_context: Optional[int] = None) -> int:
+        """Capture the decode steps of every batch size up to ``max_batch`` requests (default: ``max_num_seqs``)
+        and every context length up to ``max_context`` (default: the engine's limit) before the first request
+        needs them; without it a step is captured when its size first occurs, which stalls that step for tens
+        of milliseconds.  Returns the number of steps captured (0 for an engine without captured steps)."""
+        graphs = getattr(self.runner, "graphs", None)
+        if graphs is None:
+            return 0
+        return graphs.capture_ahead(int(max_batch or self.max_num_seqs), int(max_context or self.max_model_len))
 
     @staticmethod
     def _load(folder, config, runtime, block_size, num_blocks, num_slots, use_graphs, max_context) -> ModelRunner:

@@ -68,6 +68,62 @@ class DecodeGraphs:
         packed.max_kv_len = context_bucket
         return packed
 
+    def _capture(self, batch_bucket: int, context_bucket: int, words: int) -> _Captured:
+        """Warm up and capture the step of ``batch_bucket`` entries over ``context_bucket`` positions (on padding
+        entries only) and keep it; ``words``: the length of such a step's packed metadata."""
+        runner = self.runner
+        device = runner.runtime.device
+        # two pinned staging buffers, used in turn: with steps launched ahead of their results, the copy of
+        # the step before may still be waiting in the stream when the next step is packed
+        staging = [torch.empty(words, dtype=torch.int32).pin_memory() for _ in range(2)]
+        buffer = torch.empty(words, dtype=torch.int32, device=device)
+        padding = self._pack([], batch_bucket, context_bucket)
+        staging[0].numpy()[:] = padding.flat()
+        buffer.copy_(staging[0], non_blocking=True)
+        batch = batch_from_buffer(padding, buffer)
+        batch.sampled_tokens = runner.sampled_tokens
+        # an eager run first: it loads every kernel module the step needs, outside of the capture
+        runner.model.forward(batch, runner.storage)
+        torch.cuda.synchronize(device)
+        graph = torch.cuda.CUDAGraph()
+        # No garbage collection while the stream is capturing: a collected object that holds pinned or
+        # device memory, an event or another graph (an engine that is no longer used, say) would be
+        # freed through calls that are not allowed during a capture, and the process would abort.
+        # What is garbage now is collected before the capture starts.
+        gc.collect()
+        collecting = gc.isenabled()
+        gc.disable()
+        try:
+            with torch.cuda.graph(graph, pool=self.pool):
+                logits = runner.model.forward(batch, runner.storage)
+        finally:
+            if collecting:
+                gc.enable()
+        if self.pool is None:
+            self.pool = graph.pool()
+        captured = _Captured(graph, buffer, staging, batch, logits)
+        self.graphs[(batch_bucket, context_bucket)] = captured
+        return captured
+
+    def capture_ahead(self, max_batch: int, max_context: int) -> int:
+        """Capture the steps of every batch bucket up to ``max_batch`` entries and every context bucket up to
+        ``max_context`` positions that are not captured yet, so that no step of a running engine has to (a
+        capture drains the stream and takes tens of milliseconds). Returns how many were captured."""
+        top_batch = _bucket(max(1, min(max_batch, BATCH_BUCKETS[-1])), BATCH_BUCKETS)
+        top_context = self._context_bucket(max(1, min(max_context, self.max_context)))
+        made = 0
+        for batch_bucket in BATCH_BUCKETS:
+            if batch_bucket > top_batch:
+                break
+            context_bucket = 256
+            while context_bucket <= top_context:
+                if (batch_bucket, context_bucket) not in self.graphs:
+                    words = self._pack([], batch_bucket, context_bucket).flat().size
+                    self._capture(batch_bucket, context_bucket, words)
+                    made += 1
+                context_bucket *= 2
+        return made
+
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         """Logits ``[wanted, vocab]`` like the eager step; ``want`` of an entry is ``[]`` or ``[0]``."""
         runner = self.runner
@@ -79,37 +135,7 @@ class DecodeGraphs:
         key = (batch_bucket, context_bucket)
         captured = self.graphs.get(key)
         if captured is None:
-            device = runner.runtime.device
-            # two pinned staging buffers, used in turn: with steps launched ahead of their results, the copy of
-            # the step before may still be waiting in the stream when the next step is packed
-            staging = [torch.empty(flat.size, dtype=torch.int32).pin_memory() for _ in range(2)]
-            buffer = torch.empty(flat.size, dtype=torch.int32, device=device)
-            padding = self._pack([], batch_bucket, context_bucket)
-            staging[0].numpy()[:] = padding.flat()
-            buffer.copy_(staging[0], non_blocking=True)
-            batch = batch_from_buffer(padding, buffer)
-            batch.sampled_tokens = runner.sampled_tokens
-            # an eager run first: it loads every kernel module the step needs, outside of the capture
-            runner.model.forward(batch, runner.storage)
-            torch.cuda.synchronize(device)
-            graph = torch.cuda.CUDAGraph()
-            # No garbage collection while the stream is capturing: a collected object that holds pinned or
-            # device memory, an event or another graph (an engine that is no longer used, say) would be
-            # freed through calls that are not allowed during a capture, and the process would abort.
-            # What is garbage now is collected before the capture starts.
-            gc.collect()
-            collecting = gc.isenabled()
-            gc.disable()
-            try:
-                with torch.cuda.graph(graph, pool=self.pool):
-                    logits = runner.model.forward(batch, runner.storage)
-            finally:
-                if collecting:
-                    gc.enable()
-            if self.pool is None:
-                self.pool = graph.pool()
-            captured = _Captured(graph, buffer, staging, batch, logits)
-            self.graphs[key] = captured
+            captured = self._capture(batch_bucket, context_bucket, flat.size)
         captured.turn ^= 1
         staging = captured.staging[captured.turn]
         staging.numpy()[:] = flat
@@ -122,5 +148,9 @@ class DecodeGraphs:
         rows = [k for k, e in enumerate(entries) if len(e.want)]
         if len(rows) == batch_bucket:
             return captured.logits
+        if rows == list(range(len(rows))):
+            # the usual case, every entry wants its logits and the padding comes last: a view of the first rows
+            # (an index tensor made from a list is a blocking copy, which would end the launching ahead)
+            return captured.logits[:len(rows)]
         index = torch.tensor(rows, dtype=torch.long, device=captured.logits.device)
         return captured.logits.index_select(0, index)
