@@ -49,6 +49,25 @@ __device__ __forceinline__ bf16x8 zero8() {
   return z;
 }
 
+// A column's four lanes (lanes c, c + 16, c + 32, c + 48) combine their values with two lane swaps that run in the
+// vector ALU (v_permlane16_swap exchanges the odd 16-lane rows of one register with the even rows of another,
+// v_permlane32_swap the upper half of one with the lower half of another; with both registers holding v, the two
+// results hold a lane's own value and its partner's), not with two round trips through the LDS crossbar, which sat
+// in the middle of every step's chain from scores to weights.
+__device__ __forceinline__ float max_of_column(float v) {
+  auto rows = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = fmaxf(__uint_as_float(rows[0]), __uint_as_float(rows[1]));
+  auto halves = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(halves[0]), __uint_as_float(halves[1]));
+}
+// The sum in a fixed order: (lane group 0 + 1) + (2 + 3) for every lane.
+__device__ __forceinline__ float sum_of_column(float v) {
+  auto rows = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = __uint_as_float(rows[0]) + __uint_as_float(rows[1]);
+  auto halves = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(halves[0]) + __uint_as_float(halves[1]);
+}
+
 // Position -> (page index, slot in the page). Page sizes are almost always powers of two: then a shift
 // and a mask stand for the division, which would otherwise cost some thirty instructions per use, on
 // the path to every load address.
@@ -158,8 +177,7 @@ __device__ __forceinline__ void attend_range(const bf16x8 (&qf)[KS], int col_lo,
         sv[sub * 4 + j] = x;
         tile_max = fmaxf(tile_max, x);
       }
-    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, 64));
-    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
+    tile_max = max_of_column(tile_max);
     const float m_new = fmaxf(m, tile_max);
     float alpha = 1.f;
     bf16x8 pf = zero8();
@@ -387,8 +405,7 @@ __global__ __launch_bounds__(PT_THREADS) void attn_prefill_kernel(
     for (int sub = 0; sub < 4; ++sub)
 #pragma unroll
       for (int j = 0; j < 4; ++j) tile_max = fmaxf(tile_max, s[sub][j]);
-    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, 64));
-    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
+    tile_max = max_of_column(tile_max);
     const float m_new = fmaxf(m, tile_max);
     bf16x8 pf[2] = {zero8(), zero8()};
     if (__builtin_amdgcn_ballot_w64(m_new > m) != 0) {
@@ -440,8 +457,7 @@ __global__ __launch_bounds__(PT_THREADS) void attn_prefill_kernel(
       __syncthreads();
     }
   }
-  l += __shfl_xor(l, 16, 64);
-  l += __shfl_xor(l, 32, 64);
+  l = sum_of_column(l);
   if (!col_ok) return;
   const float inv = 1.f / l;
   __bf16* dst = out + (size_t)(tok0 + c) * heads * hd + (size_t)h * hd;
@@ -630,8 +646,7 @@ __global__ __launch_bounds__(SPLIT ? 2 * PT_THREADS : PT_THREADS) void attn_pref
     for (int sub = 0; sub < 4; ++sub)
 #pragma unroll
       for (int j = 0; j < 4; ++j) tile_max = fmaxf(tile_max, s[sub][j]);
-    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, 64));
-    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
+    tile_max = max_of_column(tile_max);
     const float m_new = fmaxf(m, tile_max);
     bf16x8 pf[2] = {zero8(), zero8()};
     if (__builtin_amdgcn_ballot_w64(m_new > m) != 0) {
@@ -707,8 +722,7 @@ __global__ __launch_bounds__(SPLIT ? 2 * PT_THREADS : PT_THREADS) void attn_pref
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) o[dt] = o[dt] * a0 + hand_o[(wave * DT + dt) * 64 + lane] * a1;
   }
-  l += __shfl_xor(l, 16, 64);
-  l += __shfl_xor(l, 32, 64);
+  l = sum_of_column(l);
   if (!col_ok) return;
   const float inv = 1.f / l;
   __bf16* dst = out + (size_t)(tok0 + c) * heads * hd + (size_t)h * hd;
@@ -773,8 +787,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void at
   for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
   attend_range<REGS>(qf, lo, col_ok ? pos : -1, begin, end, cv, scale, o, m, l);
-  l += __shfl_xor(l, 16, 64);
-  l += __shfl_xor(l, 32, 64);
+  l = sum_of_column(l);
   if (!col_ok) return;
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) {
