@@ -345,8 +345,10 @@ def generate_command(argv: List[str]) -> int:
     context = ctx if ctx is not None else min(config.context_limit, 2048)  # main.rs:655-663
     block_size = args.number("--block-size", 16, int)
     # one request at a time, as the reference's command line runs (main.rs:680-693)
+    # steps are launched ahead of their tokens (the engine falls back to one step at a time while a request's
+    # penalties need its tokens on the host)
     engine = Engine(folder, dtype=dtype, block_size=block_size, max_num_seqs=1, max_model_len=context,
-                    num_blocks=(context + block_size - 1) // block_size)
+                    num_blocks=(context + block_size - 1) // block_size, pipelined=True)
     started = time.perf_counter()
     json_out = "--json" in args.switches
     shown = []
