@@ -344,3 +344,26 @@ def test_decode_steps_captured_ahead_are_the_ones_that_generation_replays():
         ahead = engine.generate(prompts, 24)
         assert set(graphs.graphs) == before and graphs.replays > 0
         assert [g.tokens for g in ahead] == [g.tokens for g in lazy]
+
+
+def test_captured_steps_without_any_wait_between_them_keep_their_own_metadata():
+    """Thirty captured decode steps launched back to back, no result read in between (nothing wanted until the
+    last): every step must run with its own positions and pages, although the host is far ahead of the GPU."""
+    import tempfile
+    from vipera_rs_amd.engine.batch import StepEntry
+    from vipera_rs_amd.engine.runner import ModelRunner
+    with tempfile.TemporaryDirectory() as tmp:
+        make_folder(tmp, CONFIG_B, 3, torch.float32)
+        tokens = random_tokens(CONFIG_B["vocab_size"], 50, 9)
+        cfg, weights = qwen2_plain.load_folder(tmp)
+        want = qwen2_plain.forward(cfg, weights, tokens)[-1]
+        runner = ModelRunner.from_folder(tmp, dtype="float32", block_size=16, num_blocks=8, num_slots=2, use_graphs=True,
+                                         max_context=128)
+        runner.cache.reserve(1, 0, len(tokens))
+        runner.step([StepEntry(1, 0, tokens[:20], [])])
+        logits = None
+        for p in range(20, len(tokens)):
+            logits = runner.step([StepEntry(1, p, [tokens[p]], [0] if p == len(tokens) - 1 else [])])
+        got = logits[0].double().cpu().numpy()
+        assert np.abs(got - want).max() <= 1e-4 * np.abs(want).max()
+        assert runner.graphs.replays == 30

@@ -34,6 +34,7 @@ class _Captured:
     def __init__(self, graph, buffer, staging, batch, logits):
         self.graph, self.buffer, self.staging, self.batch, self.logits = graph, buffer, staging, batch, logits
         self.turn = 0  # which of the two staging buffers the last step used
+        self.fetched = [None, None]  # per staging buffer: the event after the GPU's last read of it
 
 
 class DecodeGraphs:
@@ -138,11 +139,18 @@ class DecodeGraphs:
             captured = self._capture(batch_bucket, context_bucket, flat.size)
         captured.turn ^= 1
         staging = captured.staging[captured.turn]
+        if captured.fetched[captured.turn] is not None:
+            # a caller that never waits for results (steps in which no logits are wanted) could be more than two
+            # steps ahead of the GPU: the buffer is not written before its last reader has run
+            captured.fetched[captured.turn].synchronize()
         staging.numpy()[:] = flat
         # a kernel fetches the step's words from the pinned buffer: a copy command of this size goes to the copy
         # engine, whose hand-over leaves the GPU idle between two steps
         if not kernels.fetch_words(staging, captured.buffer):
             captured.buffer.copy_(staging, non_blocking=True)
+        read = torch.cuda.Event()
+        read.record()
+        captured.fetched[captured.turn] = read
         captured.graph.replay()
         self.replays += 1
         rows = [k for k, e in enumerate(entries) if len(e.want)]
