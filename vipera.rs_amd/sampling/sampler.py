@@ -120,6 +120,7 @@ class BatchSampler:
         self._ids = [None, None]
         self._device_words = None
         self._turn = 0
+        self._done = [None, None]
 
     def sample(self, logits: torch.Tensor, rows: Sequence[RowRequest]) -> List[int]:
         return self.collect(self.launch(logits, rows))
@@ -133,6 +134,8 @@ class BatchSampler:
         self._penalize(logits, rows, vocab)
         self._turn ^= 1
         turn = self._turn
+        if self._done[turn] is not None:
+            self._done[turn].synchronize()   # the launch that last used this pair of pinned buffers has run
         slots = self.slot_table.shape[0]
         for r in rows:
             if not 0 <= r.slot < slots:
@@ -172,6 +175,7 @@ class BatchSampler:
         ids[:count].copy_(out, non_blocking=True)
         event = torch.cuda.Event()
         event.record()
+        self._done[turn] = event
         return PendingSample(count, ids, event)
 
     def collect(self, pending: PendingSample) -> List[int]:
