@@ -648,7 +648,6 @@ __global__ __launch_bounds__(SPLIT ? 2 * PT_THREADS : PT_THREADS) void attn_pref
       for (int j = 0; j < 4; ++j) tile_max = fmaxf(tile_max, s[sub][j]);
     tile_max = max_of_column(tile_max);
     const float m_new = fmaxf(m, tile_max);
-    bf16x8 pf[2] = {zero8(), zero8()};
     if (__builtin_amdgcn_ballot_w64(m_new > m) != 0) {
       const float alpha = (m_new > m && m > -INFINITY) ? __builtin_amdgcn_exp2f((m - m_new) * c2) : 1.f;
       l *= alpha;
@@ -656,8 +655,11 @@ __global__ __launch_bounds__(SPLIT ? 2 * PT_THREADS : PT_THREADS) void attn_pref
       for (int dt = 0; dt < DT; ++dt) o[dt] *= alpha;
       m = m_new;
     }
-    if (m_new > -INFINITY) {
-      const float mc = m_new * c2;
+    // No branch around the weights: a column that sees nothing yet has m = -inf and only masked scores, which
+    // give exp2(-inf - 0) = 0, as a masked score under a finite m does.
+    bf16x8 pf[2];
+    {
+      const float mc = m_new > -INFINITY ? m_new * c2 : 0.f;
       float sum = 0.f;
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
