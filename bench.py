@@ -74,6 +74,10 @@ def main() -> int:
                         help="instead of the headline measurement: a continuous batch of 64 requests, prompts of 128 to "
                              "8,192 random tokens in portions of 512, 256 new tokens each (the 1.5B workload; use with "
                              "--shape 1.5b --ctx 32768)")
+    parser.add_argument("--split", action="store_true",
+                        help="also run one decode step (of --batch requests at --ctx) and one prefill eagerly with a "
+                             "pair of GPU events around every kernel launch, and add the microseconds of each class of "
+                             "kernel to the line (split_decode_us, split_prefill_us)")
     parser.add_argument("--in-turn", action="store_true",
                         help="wait for a step's tokens on the host before the next step is launched")
     args = parser.parse_args()
@@ -143,7 +147,8 @@ def main() -> int:
         return dt
 
     prefill_once(10_000)
-    prefill_s = min(prefill_once(10_001 + k) for k in range(3))
+    PREFILL_RUNS = 3     # the best of this many timed runs is reported (named in `config`)
+    prefill_s = min(prefill_once(10_001 + k) for k in range(PREFILL_RUNS))
     prefill_flops = 2.0 * T * L * layer_matrix + 2.0 * V * H + L * 4.0 * config.num_attention_heads * config.head_dim \
         * (T * (T + 1) / 2)
     prefill = {"value": round(T / prefill_s, 1), "tokens": T, "ms": round(prefill_s * 1e3, 3),
@@ -232,7 +237,7 @@ def main() -> int:
             "head_dim": config.head_dim, "intermediate": I, "vocab": V, "global_batch": args.batch,
             "seq_len": ctx, "prefill_tokens": T, "block_size": args.block_size, "parallelism": "single GPU",
             "sampling": "greedy", "weights_gb": round(weight_bytes / 1e9, 2), "steps_launched_ahead": not args.in_turn,
-            "untimed_decode_steps_before_warmup": SETTLE_STEPS,
+            "untimed_decode_steps_before_warmup": SETTLE_STEPS, "prefill_is_best_of_runs": PREFILL_RUNS,
         },
         "prefill": prefill,
         "roofline": {"bound": "hbm", "achieved": round(head["gbs"], 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
@@ -240,8 +245,81 @@ def main() -> int:
         "points": {f"decode_b{b}": round(r["tok_s"], 1) for b, r in results.items() if b != args.batch},
         "points_ms": {f"decode_b{b}": round(r["ms"], 4) for b, r in results.items() if b != args.batch},
     }
+    if args.split:
+        line.update(kernel_split(args, config, runner, tokens, ctx, T))
     print(json.dumps(line), flush=True)
     return 0
+
+
+def kernel_split(args, config, runner, tokens, ctx, T):
+    """Microseconds per class of kernel for one decode step of ``--batch`` requests at context ``ctx`` and for one
+    prefill of ``T`` tokens, each the mean of five eager runs with a pair of GPU events around every launch
+    (``vipera_rs_amd.ops.profile``; the reference prints such a split as its PROFILE lines,
+    crates/vipera-backend-cpu/src/profile.rs:226-275).  The decode step reads a cache of ``ctx - 1`` positions per
+    request that no prompt has filled: its kernels' times do not depend on what the pages hold."""
+    import torch
+
+    from vipera_rs_amd.engine.batch import StepEntry
+    from vipera_rs_amd.ops.profile import KernelTimer, weight_shape
+    from vipera_rs_amd.sampling import BatchSampler, RowRequest, SamplingParams
+
+    H, V, I = config.hidden_size, config.vocab_size, config.intermediate_size
+    Q, KV = config.num_attention_heads * config.head_dim, config.num_key_value_heads * config.head_dim
+    products = {(Q + 2 * KV, H): "qkv", (H, Q): "output", (2 * I, H): "gate_up", (H, I): "down", (V, H): "head"}
+    other = {"attn_bf16_prefill": "attention", "attn_bf16_decode": "attention", "attn_generic": "attention",
+             "rmsnorm": "norms", "rope_kvwrite": "rope_kvwrite", "rope_angles": "rope_kvwrite",
+             "embed_gather": "embedding", "sample": "sampler", "swiglu": "swiglu", "fetch_words": "metadata"}
+
+    def label(name, call_args, kwargs):
+        shape = weight_shape(name, call_args)
+        if shape is not None:
+            return products.get(shape, f"product_{shape[0]}x{shape[1]}")
+        return other.get(name, name)
+
+    sampler = BatchSampler(runner.runtime.device)
+    runs = 5
+
+    def measure(entries_of, rows):
+        timer = KernelTimer(label)
+        wall = 0.0
+        for run in range(runs + 1):          # the first run loads what is not loaded yet and is not counted
+            entries = entries_of(run)
+            batch = runner.prepare(entries)
+            torch.cuda.synchronize()
+            if run == 0:
+                logits = runner.run(batch)
+                sampler.sample(logits, rows)
+                continue
+            with timer:
+                timer.hold_back()
+                start = torch.cuda.Event(enable_timing=True)
+                end = torch.cuda.Event(enable_timing=True)
+                start.record()
+                logits = runner.run(batch)
+                sampler.launch(logits, rows)
+                end.record()
+            torch.cuda.synchronize()
+            wall += start.elapsed_time(end) * 1e3
+        split = {key: round(value / runs, 1) for key, value in timer.microseconds().items()}
+        split["kernels_sum"] = round(sum(v for k, v in split.items() if k != "launches"), 1)
+        split["eager_step"] = round(wall / runs, 1)
+        return split
+
+    batch = args.batch
+    for request in range(batch):
+        runner.cache.reserve(20_000 + request, 0, ctx)
+    greedy = [RowRequest(SamplingParams(), slot=k, position=ctx) for k in range(batch)]
+    ids = tokens(batch)
+    decode = measure(lambda run: [StepEntry(20_000 + r, ctx - 1, [ids[r]], [0]) for r in range(batch)], greedy)
+    for request in range(batch):
+        runner.cache.release(20_000 + request)
+    prompt = tokens(T)
+    runner.cache.reserve(30_000, 0, T)
+    prefill = measure(lambda run: [StepEntry(30_000, 0, prompt, [T - 1])], greedy[:1])
+    runner.cache.release(30_000)
+    log("split of one decode step (us): " + ", ".join(f"{k} {v}" for k, v in decode.items()))
+    log("split of one prefill (us): " + ", ".join(f"{k} {v}" for k, v in prefill.items()))
+    return {"split_decode_us": decode, "split_prefill_us": prefill}
 
 
 def serving(args, config, runtime, model, shape_name, layers_full, dtype_key) -> int:

@@ -139,3 +139,30 @@ def test_bad_geometry_is_refused():
         CacheManager([CacheGroupSpec(0, 4)], 1)
     with pytest.raises(InvalidArgumentError):
         CacheManager([CacheGroupSpec(4, 4)], 0)
+
+
+def test_cache_groups_may_differ_in_page_size_and_pool_size():
+    """One number for every group, or one per group in the order in which the run order first needs each; a page
+    size that a mixer asks for itself stands; the engine's list has to match the number of groups."""
+    from vipera_rs_amd.cache import group_keys, group_position_bytes, plan_groups
+    from vipera_rs_amd.errors import InvalidArgumentError
+    from vipera_rs_amd.models import CacheNeed
+    from vipera_rs_amd.parts import KVCacheSpec, StateSpec
+    needs = [CacheNeed(0, KVCacheSpec(2, 16, 0), None), CacheNeed(1, KVCacheSpec(2, 16, 21), None),
+             CacheNeed(2, None, StateSpec((4,))), CacheNeed(3, KVCacheSpec(1, 32, 0, block_size=64), None),
+             CacheNeed(1, KVCacheSpec(2, 16, 21), None), CacheNeed(5, KVCacheSpec(4, 8, 0), None)]
+    assert group_keys(needs) == [(0, 0), (21, 0), (0, 64)]
+    same = plan_groups(needs, 16, 10)
+    assert [(g.block_size, g.num_blocks, g.window) for g in same] == [(16, 10, 0), (16, 10, 21), (64, 10, 0)]
+    each = plan_groups(needs, [16, 8, 32], [10, 40, 3])
+    assert [(g.block_size, g.num_blocks, g.window) for g in each] == [(16, 10, 0), (8, 40, 21), (64, 3, 0)]
+    with pytest.raises(InvalidArgumentError, match="2 values for 3 cache groups"):
+        plan_groups(needs, 16, [10, 40])
+    # bytes per cached position and group: owners only (entry 4 reads entry 1's cache)
+    assert group_position_bytes(needs, 2) == [(2 * 32 + 4 * 16) * 2, 2 * 32 * 2, 1 * 64 * 2]
+    cache = CacheManager(each, 2)
+    assert cache.reserve(7, 0, 100) is None
+    assert [cache.used_blocks(g) for g in range(3)] == [7, 13, 2] and cache.check() == ""
+    cache.advance(7, 100)                     # position 100 will see 80..100: pages 10, 11, 12 of 8 positions stay
+    assert [cache.used_blocks(g) for g in range(3)] == [7, 3, 2]
+    assert cache.allocate_micros() >= 0

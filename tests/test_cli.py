@@ -88,6 +88,58 @@ def test_plan_predicts_memory_and_refuses_what_does_not_fit(folder, tmp_path):
     assert violation["constraint"] == "device_memory" and violation["required_bytes"] > violation["available_bytes"]
 
 
+def test_plan_counts_the_weights_as_the_loader_keeps_them(tmp_path):
+    """Whatever floating-point type a folder stores, the plan's ``weight_bytes`` is the sum over the tensors of the
+    size in the dtype the loader keeps each in (planner.rs:266-430 predicts what the backend then allocates)."""
+    import vipera_rs_amd  # noqa: F401
+    from vipera_rs_amd.cli import plan_model
+    from vipera_rs_amd.config import config_from_dict
+    from vipera_rs_amd.models import declare_model
+    from vipera_rs_amd.weights import Checkpoint, kept_dtype, write_safetensors
+    specs = {s.name: s for s in declare_model(config_from_dict(CONFIG_B))}
+    source = make_folder(tmp_path / "f32", CONFIG_B, 1, torch.float32)
+    ck = Checkpoint(source)
+    tensors = {name: ck.read(name).clone() for name in ck.names()}
+    ck.close()
+    matrices = sum(t.numel() for n, t in tensors.items() if specs[n].role == "matrix")
+    vectors = sum(t.numel() for n, t in tensors.items() if specs[n].role == "vector")
+    assert matrices > 0 and vectors > 0
+    for stored in (torch.float32, torch.bfloat16, torch.float16):
+        folder = str(tmp_path / str(stored).split(".")[-1])
+        config_from_dict(CONFIG_B).save(folder)
+        write_safetensors(os.path.join(folder, "model.safetensors"), ((n, t.to(stored)) for n, t in tensors.items()))
+        for run_as, keep in (("bfloat16", False), ("bfloat16", True), ("float32", False)):
+            run_dtype = torch.float32 if run_as == "float32" else torch.bfloat16
+            want = sum(t.numel() * torch.empty(0, dtype=kept_dtype(specs[n], stored, run_dtype, keep)).element_size()
+                       for n, t in tensors.items())
+            plan = plan_model(folder, 64, 1, run_as, 16, keep_float32=keep)
+            assert plan["weight_bytes"] == want, (stored, run_as, keep)
+            kept32 = run_as == "float32" or (keep and stored == torch.float32)
+            assert want == matrices * (4 if kept32 else 2) + vectors * 4
+    # the command line says the same
+    out = run("plan", str(tmp_path / "float32"), "--ctx", "64", "--json")
+    assert json.loads(out.stdout)["weight_bytes"] == matrices * 2 + vectors * 4
+    out = run("plan", str(tmp_path / "float32"), "--ctx", "64", "--keep-float32", "--json")
+    assert json.loads(out.stdout)["weight_bytes"] == matrices * 4 + vectors * 4
+
+
+def test_a_shape_no_kernel_takes_is_refused_when_the_model_is_opened(tmp_path):
+    """A head width above the attention kernels' limit: `unsupported` (exit 2) from every subcommand that opens the
+    model, before any weight is read (the reference refuses while it reads the header, model.rs:1323-1328,
+    1367-1383; exit codes errors/lib.rs:94-104), not an internal error from the first step."""
+    wide = dict(CONFIG_B, hidden_size=64, num_attention_heads=1, num_key_value_heads=1, head_dim=272,
+                intermediate_size=32, vocab_size=40, num_hidden_layers=1)
+    folder = make_folder(tmp_path / "wide", wide, 1)
+    for command in (["model-info", folder], ["plan", folder], ["generate", folder, "--prompt-ids", "1 2 3"]):
+        out = run(*command)
+        assert out.returncode == 2, (command, out.stderr)
+        assert out.stderr.startswith("vipera: ") and "head_dim 272" in out.stderr and "limit of 256" in out.stderr
+        assert out.stdout == ""
+    # the weights are not looked at: the same refusal without them
+    os.remove(os.path.join(folder, "model.safetensors"))
+    assert "head_dim 272" in run("plan", folder).stderr
+
+
 def test_random_model_writes_a_loadable_folder(tmp_path):
     cfg_path = tmp_path / "cfg.json"
     cfg_path.write_text(json.dumps(CONFIG_B))
@@ -126,7 +178,7 @@ def test_generate_prints_token_ids_and_json(folder):
     out = run("generate", folder, "--prompt-ids", ids, "--max-tokens", "6", "--dtype", "float32", "--json")
     report = json.loads(out.stdout)
     assert report["tokens"] == want and report["prompt_tokens"] == 9 and report["generated_tokens"] == 6
-    assert report["finish"] == "length" and report["processed_tokens"] == 9 + 5 and "compute" in report["micros"]
+    assert report["finish"] == "length" and report["processed_tokens"] == 9 + 5 and set(report["micros"]) == {"schedule", "allocate", "compute", "sample"}
     seeded = [run("generate", folder, "--prompt-ids", ids, "--max-tokens", "8", "--temperature", "0.9", "--seed", "4",
                   "--dtype", "float32").stdout for _ in range(2)]
     assert seeded[0] == seeded[1] and len(seeded[0].split()) == 8

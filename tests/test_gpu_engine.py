@@ -367,3 +367,165 @@ def test_captured_steps_without_any_wait_between_them_keep_their_own_metadata():
         got = logits[0].double().cpu().numpy()
         assert np.abs(got - want).max() <= 1e-4 * np.abs(want).max()
         assert runner.graphs.replays == 30
+
+
+# --- sampling through the engine, held to an oracle outside it ------------------------------------------------------
+def _id_order_draw(logits, params, u):
+    """The draw the engine makes, from the plain sampler's parts: the kept set of the reference's cuts
+    (crates/vipera-sampler/src/lib.rs:172-232), walked in id order with ``target = u * mass`` until
+    ``target < running`` (lib.rs:234-242 with the engine's order of walking).  Returns the token and how far,
+    as a share of the mass, the target lies from the nearest edge between two kept tokens."""
+    from plain import sampler_plain as S
+    kept = sorted(S.kept_set(logits.astype(np.float32), params.temperature, params.top_k, params.top_p, params.min_p))
+    mass = sum(float(w) for _, w in kept)
+    target, running, token, edges = u * mass, 0.0, None, []
+    for candidate, weight in kept:
+        running += float(weight)
+        edges.append(running)
+        if token is None and target < running:
+            token = candidate
+    token = kept[-1][0] if token is None else token
+    margin = min(abs(target - edge) for edge in edges[:-1]) / mass if len(edges) > 1 else 1.0
+    return token, margin
+
+
+@pytest.mark.parametrize("cuts", ["none", "default"])
+@pytest.mark.parametrize("pipelined", [False, True])
+def test_seeded_sampling_through_the_engine_equals_the_plain_sampler(folders, cuts, pipelined):
+    """The second tiny configuration's workload (prompts of 1, 7, 19 and 33 tokens in portions of 6 beside decoding
+    requests, temperature 0.8, a seed per request, 10 new tokens): every token the engine draws is the one that
+    the plain forward pass, the plain sampler's kept set and the plain generator's next uniform select, token by
+    token.  A draw that walked the ids the wrong way, used a uniform one draw late, or took another request's
+    generator would pass every comparison of the engine with itself; it does not pass this one."""
+    from plain import sampler_plain as S
+    from vipera_rs_amd import SamplingParams
+    cfg, weights = qwen2_plain.load_folder(folders["B"])
+    prompts = [random_tokens(CONFIG_B["vocab_size"], n, 70 + n) for n in (1, 7, 19, 33)]
+    extra = dict(top_k=0, top_p=1.0, min_p=0.0) if cuts == "none" else {}
+    params = [SamplingParams(temperature=0.8, seed=11 + k, **extra) for k in range(4)]
+    engine = _engine(folders["B"], block_size=8, num_blocks=40, max_num_seqs=4, chunk_size=6, max_num_batched_tokens=16,
+                     pipelined=pipelined)
+    got = engine.generate(prompts, 10, params)
+    clear = 0
+    for prompt, p, generation in zip(prompts, params, got):
+        assert len(generation.tokens) == 10
+        logits = qwen2_plain.forward(cfg, weights, prompt + generation.tokens[:-1])
+        rng = S.Rng(p.seed)
+        for k, token in enumerate(generation.tokens):
+            want, margin = _id_order_draw(logits[len(prompt) - 1 + k], p, rng.next_f64())
+            if margin > 1e-4:     # the target is clear of an edge between two tokens: no rounding can move the draw
+                assert token == want, f"prompt of {len(prompt)}, seed {p.seed}: token {k} is {token}, the plain draw {want}"
+                clear += 1
+    assert clear >= 36, f"only {clear} of 40 draws were clear of an edge"
+
+
+def test_the_generator_step_in_the_sampling_kernel():
+    """xorshift64* worked by hand from state 1 (x ^= x >> 12; x ^= x << 25; x ^= x >> 27; output
+    x * 0x2545F4914F6CDD1D): the next state is 2^25 + 1 and the output 5180492295206395165, so the uniform is
+    (output >> 11) / 2^53 = 0.28083...; with masses 0.25 / 0.75 the id-order walk takes token 1, with 0.3 / 0.7
+    token 0."""
+    from vipera_rs_amd.ops import kernels
+    dev = "cuda:0"
+    u = (5180492295206395165 >> 11) / float(1 << 53)
+    assert 0.25 < u < 0.3
+    for masses, want in (((0.25, 0.75), 1), ((0.3, 0.7), 0)):
+        logits = torch.tensor([[np.log(masses[0]), np.log(masses[1])]], dtype=torch.float32, device=dev)
+        table = torch.zeros((3, 2), dtype=torch.int64, device=dev)
+        out = torch.full((1,), -7, dtype=torch.int32, device=dev)
+        one = lambda v, d: torch.tensor([v], dtype=d, device=dev)  # noqa: E731
+        kernels.sample(logits, one(1.0, torch.float32), one(0, torch.int32), one(1.0, torch.float32),
+                       one(0.0, torch.float32), None, out, slot=one(2, torch.int32), position=one(41, torch.int32),
+                       reseed=one(1, torch.int32), seed_state=one(1, torch.int64), slot_table=table)
+        assert out.item() == want
+        assert table.cpu().tolist() == [[0, 0], [0, 0], [33554433, 41]]   # the slot keeps the state after the step
+        # the next draw goes on from the slot's state: the host's generator from the same state agrees
+        kernels.sample(logits, one(1.0, torch.float32), one(0, torch.int32), one(1.0, torch.float32),
+                       one(0.0, torch.float32), None, out, slot=one(2, torch.int32), position=one(42, torch.int32),
+                       reseed=one(0, torch.int32), seed_state=one(0, torch.int64), slot_table=table)
+        from vipera_rs_amd.sampling import Rng
+        host = Rng(0)
+        host.state = 33554433
+        u2 = host.next_f64()
+        assert out.item() == (0 if u2 < masses[0] else 1) and table[2, 0].item() == host.state
+
+
+def test_a_sampler_launch_that_fails_leaves_the_other_requests_streams_alone(folders):
+    """The host books a request's draws only when the launch has gone through.  Here the launch raises once, in a
+    step in which two requests draw while a third is still in its prompt: the two fail, the third finishes with
+    exactly its solo tokens, and nothing is left held."""
+    from vipera_rs_amd import SamplingParams
+    from vipera_rs_amd.errors import InvalidArgumentError
+    prompts = [random_tokens(CONFIG_B["vocab_size"], n, 70 + n) for n in (3, 5, 40)]
+    params = [SamplingParams(temperature=0.8, seed=31 + k) for k in range(3)]
+    solo = _engine(folders["B"], block_size=8, num_blocks=16, max_num_seqs=1, chunk_size=6).generate(
+        [prompts[2]], 10, params[2])[0].tokens
+    engine = _engine(folders["B"], block_size=8, num_blocks=40, max_num_seqs=3, chunk_size=6, max_num_batched_tokens=16)
+    launch, calls = engine.sampler.launch, []
+
+    def flaky(logits, rows):
+        calls.append(len(rows))
+        if len(calls) == 3:
+            raise InvalidArgumentError("state slot 99 is outside the table")
+        return launch(logits, rows)
+
+    engine.sampler.launch = flaky
+    got = engine.generate(prompts, 10, params)
+    assert calls[2] == 2 and [g.finish for g in got] == ["error", "error", "length"]
+    assert "state slot 99" in got[0].error
+    assert got[2].tokens == solo
+    assert engine.runner.cache.check() == "" and engine.runner.cache.live_requests() == 0
+
+
+# --- preemption in the configurations and dtypes that had none ----------------------------------------------------
+def test_preemption_with_windowed_layers(folders):
+    """The fourth configuration (two cache groups: all positions, and a window of 21) with so few pages that
+    requests are preempted and recomputed: every request's tokens are its solo run's."""
+    prompts = [random_tokens(CONFIG_B["vocab_size"], n, 90 + n) for n in (30, 28, 25, 31)]
+    solo = [_engine(folders["D"], block_size=8, num_blocks=12, max_num_seqs=1).generate([p], 40)[0].tokens
+            for p in prompts]
+    engine = _engine(folders["D"], block_size=8, num_blocks=18, max_num_seqs=4, chunk_size=16)
+    got = engine.generate(prompts, 40)
+    assert engine.stats()["preemptions"] > 0
+    assert [g.tokens for g in got] == solo
+    cache = engine.runner.cache
+    assert cache.check() == "" and cache.live_requests() == 0 and len(cache.groups) == 2
+    assert [cache.free_blocks(g) for g in range(2)] == [18, 18]
+
+
+@pytest.mark.parametrize("pipelined", [False, True])
+def test_bfloat16_generation_under_preemption_follows_the_plain_implementation(folders, pipelined):
+    """bfloat16 with so few pages that requests are preempted: a recomputed request must go on as the plain
+    implementation does wherever that one's best token leads clearly."""
+    cfg, weights = qwen2_plain.load_folder(folders["B16"])
+    prompts = [random_tokens(CONFIG_B["vocab_size"], n, 90 + n) for n in (30, 28, 25, 31)]
+    engine = _engine(folders["B16"], dtype="bfloat16", block_size=16, num_blocks=10, max_num_seqs=4, chunk_size=16,
+                     pipelined=pipelined)
+    got = engine.generate(prompts, 40)
+    assert engine.stats()["preemptions"] > 0
+    checked = 0
+    for p, g in zip(prompts, got):
+        assert len(g.tokens) == 40
+        logits = qwen2_plain.forward(cfg, weights, p + g.tokens[:-1])
+        checked += assert_tokens_follow_plain(logits, len(p), g.tokens, 1e-2, f"prompt of {len(p)}")
+    assert checked > 60, "too few tokens had a clear lead to say anything"
+    assert engine.runner.cache.check() == "" and engine.runner.cache.live_requests() == 0
+
+
+def test_a_request_on_pages_that_a_request_with_nan_activations_gave_back(folders):
+    """A request whose pages hold NaN ends (here: is cancelled after its keys and values were overwritten with NaN, as
+    overflowed activations leave them) and the next request takes exactly those pages; a portion of 5 leaves most of
+    its last page unwritten.  Its tokens are those of a run on a fresh pool."""
+    prompt = random_tokens(CONFIG_B["vocab_size"], 21, 77)
+    for dtype, name in (("float32", "B"), ("bfloat16", "B16")):
+        want = _engine(folders[name], dtype=dtype, block_size=16, num_blocks=6, max_num_seqs=1).generate([prompt], 12)[0].tokens
+        engine = _engine(folders[name], dtype=dtype, block_size=16, num_blocks=6, max_num_seqs=1, chunk_size=5)
+        first = engine.add_request(random_tokens(CONFIG_B["vocab_size"], 60, 78), 30)
+        for _ in range(20):
+            engine.step()
+        assert engine.runner.cache.used_blocks(0) >= 4
+        for paged in engine.runner.storage.kv:
+            paged.k.fill_(float("nan"))
+            paged.v.fill_(float("nan"))
+        assert engine.cancel(first).finish == "cancelled" and engine.runner.cache.used_blocks(0) == 0
+        got = engine.generate([prompt], 12)[0]
+        assert got.finish == "length" and got.tokens == want, dtype

@@ -213,7 +213,7 @@ def _plain_attention(q, k, v, first_pos, window, scale):
 class _Paged:
     """A paged cache filled by hand: shuffled pages, K [page, kvh, slot, hd], V [page, kvh, hd, slot]."""
 
-    def __init__(self, seqs, kv_heads, hd, block_size, dtype, seed):
+    def __init__(self, seqs, kv_heads, hd, block_size, dtype, seed, stale_nan=False):
         g = torch.Generator().manual_seed(seed)
         self.block_size = block_size
         need = [(n + block_size - 1) // block_size for n in seqs]
@@ -221,6 +221,11 @@ class _Paged:
         order = torch.randperm(pages, generator=g).tolist()
         self.k = (torch.randn(pages, kv_heads, block_size, hd, generator=g) * 7).to(dtype)   # stale values everywhere
         self.v = (torch.randn(pages, kv_heads, hd, block_size, generator=g) * 7).to(dtype)
+        if stale_nan:
+            # what no live position occupies is not finite, as after a request whose activations overflowed gave its
+            # pages back: also the slots of a held page past the request's last position
+            self.k.fill_(float("nan"))
+            self.v.fill_(float("nan"))
         self.tables, self.keys, self.values = [], [], []
         for n, blocks in zip(seqs, need):
             table = [order.pop() for _ in range(blocks)]
@@ -261,12 +266,16 @@ ATTN_CASES = [
 
 @pytest.mark.parametrize("case", ATTN_CASES, ids=[f"h{c[0]}kv{c[1]}d{c[2]}b{c[3]}w{c[4]}" for c in ATTN_CASES])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_attention_kernels_against_plain_softmax(case, dtype):
+@pytest.mark.parametrize("stale", ["finite", "nan"])
+def test_attention_kernels_against_plain_softmax(case, dtype, stale):
+    """``stale``: what the pool holds wherever no live position lies, the rest of a request's last page included:
+    large finite numbers, or NaN (a weight of zero times NaN is NaN on the matrix cores, so such a slot must not
+    reach a product at all)."""
     from vipera_rs_amd.ops import kernels
     from vipera_rs_amd.ops.attention import decode_chunking
     heads, kv_heads, hd, bs, window, entries = case
     scale = 1.0 / math.sqrt(hd)
-    cache = _Paged([kv for kv, _ in entries], kv_heads, hd, bs, dtype, seed=heads * 100 + hd)
+    cache = _Paged([kv for kv, _ in entries], kv_heads, hd, bs, dtype, seed=heads * 100 + hd, stale_nan=stale == "nan")
     g = torch.Generator().manual_seed(hd)
     counts = [n for _, n in entries]
     T = sum(counts)
@@ -397,10 +406,11 @@ def test_decode_attention_at_the_benchmark_head_shapes(heads, kv_heads, hd, batc
     that is dropped shows."""
     from vipera_rs_amd.ops import kernels
     from vipera_rs_amd.ops.attention import decode_chunking
-    if batch == 64 and heads != 28:
-        pytest.skip("the batch of 64 runs at the 7B head shape")
     bs, scale, dtype = 16, 1.0 / math.sqrt(hd), torch.bfloat16
     lengths = [(4096, 3000, 2049, 4095, 1, 3001, 130, 4096)[e % 8] for e in range(batch)]
+    if batch == 64 and heads != 28:
+        # the other two head shapes at a quarter of the lengths: the float64 oracle is what the time goes to
+        lengths = [(1024, 750, 513, 1023, 1, 751, 130, 1024)[e % 8] for e in range(batch)]
     cache = _Paged(lengths, kv_heads, hd, bs, dtype, seed=heads)
     g = torch.Generator().manual_seed(batch)
     qkv = torch.randn(batch, (heads + 2 * kv_heads) * hd, generator=g).to(dtype)

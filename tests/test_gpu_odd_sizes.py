@@ -54,11 +54,13 @@ def test_odd_sizes_against_plain(tmp_path, name, dtype, tol, block_size):
 
 
 def test_sizes_no_kernel_takes_are_refused_with_a_clear_error(tmp_path):
-    from vipera_rs_amd.engine.batch import StepEntry
+    """When the model is opened, not at its first step: from the runner's and the engine's constructors."""
+    from vipera_rs_amd import Engine
     from vipera_rs_amd.engine.runner import ModelRunner
     from vipera_rs_amd.errors import UnsupportedError
     folder = make_folder(tmp_path / "wide", _config(64, 1, 1, 272, 32, 40, layers=1), 1)
-    runner = ModelRunner.from_folder(folder, dtype="float32", block_size=16, num_blocks=4, num_slots=1)
-    runner.cache.reserve(0, 0, 3)
-    with pytest.raises(UnsupportedError, match="head_dim 272"):
-        runner.step([StepEntry(0, 0, [1, 2, 3], [2])])
+    for dtype in ("float32", "bfloat16"):
+        with pytest.raises(UnsupportedError, match="head_dim 272"):
+            ModelRunner.from_folder(folder, dtype=dtype, block_size=16, num_blocks=4, num_slots=1)
+        with pytest.raises(UnsupportedError, match="head_dim 272"):
+            Engine(folder, dtype=dtype, block_size=16, num_blocks=4, max_num_seqs=1)

@@ -131,7 +131,7 @@ def _random_part_tensors(cls, spec, prefix, seed, runtime):
     from vipera_rs_amd.weights import kept_dtype, random_tensor
     host, device = {}, {}
     for t in cls.declare(spec, prefix):
-        if t.unused:      # a tensor a folder may hold but the part does not read
+        if t.optional:    # a tensor a folder need not hold
             continue
         value = random_tensor(t, seed, torch.float32)
         kept = kept_dtype(t, torch.float32 if runtime.dtype == torch.float32 else torch.bfloat16, runtime.dtype)
@@ -433,8 +433,10 @@ def test_a_stateful_toy_mixer_is_registered_built_and_stepped(tmp_path):
         assert at == {r: len(t) for r, t in requests.items()} and runner.cache.check() == ""
 
 
-def test_a_stateful_toy_mixer_generates_through_captured_steps_with_padding(tmp_path):
-    """Three live requests decode in a captured step of four entries.  The padding entry writes the scratch
+@pytest.mark.parametrize("pipelined", [False, True])
+def test_a_stateful_toy_mixer_generates_through_captured_steps_with_padding(tmp_path, pipelined):
+    """Three live requests decode in a captured step of four entries (``pipelined``: each step launched before the
+    tokens of the step before have reached the host, which reads them on the device).  The padding entry writes the scratch
     state row and not slot 0, which a live request holds, and the first use of a graph runs a step once: either
     fault would change a request's state and, from there on, its tokens."""
     from vipera_rs_amd import Engine
@@ -445,7 +447,9 @@ def test_a_stateful_toy_mixer_generates_through_captured_steps_with_padding(tmp_
         folder = make_folder(tmp_path / "toy", config, 8)
         cfg, w = P.load_folder(folder)
         prompts = [random_tokens(256, n, 50 + n) for n in (7, 12, 3)]
-        engine = Engine(folder, dtype="float32", block_size=8, num_blocks=24, max_num_seqs=3, use_graphs=True)
+        engine = Engine(folder, dtype="float32", block_size=8, num_blocks=24, max_num_seqs=3, use_graphs=True,
+                        pipelined=pipelined)
+        assert engine.pipelined == pipelined
         got = engine.generate(prompts, max_new_tokens=20)
         graphs = engine.runner.graphs
         assert graphs.replays >= 19 and any(bucket == 4 for bucket, _ in graphs.graphs), "no padded captured step ran"

@@ -198,6 +198,14 @@ def test_generator_vectors():
     from vipera_rs_amd.sampling import Rng
     ours, theirs = Rng(12345), S.Rng(12345)       # the engine's generator is the same generator
     assert [ours.next_f64() for _ in range(20)] == [theirs.next_f64() for _ in range(20)]
+    # the xorshift64* step itself, worked by hand from state 1: x ^= x >> 12 leaves 1, x ^= x << 25 gives
+    # 2^25 + 1 = 33554433, x ^= x >> 27 leaves it, and 33554433 * 0x2545F4914F6CDD1D mod 2^64 is the output
+    for rng in (S.Rng(0), Rng(0)):
+        rng.state = 1
+        assert rng.next_u64() == 5180492295206395165 == (33554433 * 0x2545F4914F6CDD1D) % (1 << 64)
+        assert rng.state == 33554433
+    # a wrong shift or direction changes it: the three shifts are not interchangeable
+    assert ((1 ^ (1 << 12)) * 0x2545F4914F6CDD1D) % (1 << 64) != 5180492295206395165
 
 
 def test_greedy_and_cuts():

@@ -116,8 +116,12 @@ def test_what_dtype_a_tensor_keeps():
     m, v = TensorSpec("m", (2, 2), MATRIX), TensorSpec("v", (2,), VECTOR)
     bf, f32 = torch.bfloat16, torch.float32
     assert kept_dtype(m, bf, bf) == bf            # bfloat16 stays bfloat16
-    assert kept_dtype(m, f32, bf) == f32          # a matrix stored in 32-bit stays so
+    assert kept_dtype(m, f32, bf) == bf           # a matrix takes the run's dtype whatever the file stores ...
+    assert kept_dtype(m, torch.float16, bf) == bf
+    assert kept_dtype(m, f32, bf, keep_float32=True) == f32   # ... unless 32-bit storage is asked to be kept
+    assert kept_dtype(m, torch.float16, bf, keep_float32=True) == bf
     assert kept_dtype(m, bf, f32) == f32          # the 32-bit run widens everything
+    assert kept_dtype(v, f32, bf) == f32          # a vector stored in 32-bit stays so
     assert kept_dtype(v, bf, bf) == f32           # norm weights and biases are always 32-bit
     assert kept_dtype(TensorSpec("t", (2,), "int_table"), torch.int64, bf) == torch.int32
 
@@ -149,11 +153,11 @@ def test_a_bfloat16_folder(tmp_path):
     ck.check(declare_model(config_from_dict(CONFIG_A)))
 
 
-def test_a_tied_model_may_hold_an_output_matrix_that_is_not_read(tmp_path):
+def test_a_tied_model_may_hold_an_output_matrix(tmp_path):
     cfg = config_from_dict(CONFIG_A)                        # tied embeddings
     folder = make_folder(tmp_path / "m", CONFIG_A, 0)
     specs = declare_model(cfg)
-    assert [s.name for s in specs if s.unused] == ["lm_head.weight"]
+    assert [s.name for s in specs if s.optional] == ["lm_head.weight"]
     ck = Checkpoint(folder)
     assert "lm_head.weight" not in ck.names()               # random weights do not write it
     ck.check(specs)

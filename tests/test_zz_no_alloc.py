@@ -61,6 +61,31 @@ def test_two_calls_in_a_row_the_second_smaller():
     _both(lib, 48, 1000, 2048, 4, seed=1, accumulate=True)
     _both(lib, 5, 136, 512, 2, seed=2, accumulate=False)     # finds the larger call's partial sums in the array
     _both(lib, 64, 3584, 4096, 8, seed=3, accumulate=True)   # and a larger one again
+    _both(lib, 100, 1000, 1544, 4, seed=4, accumulate=False)  # 65 to 128 tokens: the kernel's chunks of 128 along K
+    _both(lib, 7, 200, 1024, 2, seed=5, accumulate=False)
+
+
+def test_the_driver_sees_no_allocation_either():
+    """Free device memory as the driver counts it (not torch's allocator, which a hipMalloc inside the library
+    would pass by) is the same before and after a hundred calls, once the first call has run."""
+    lib = _library()
+    device = torch.device("cuda:0")
+    m, n, k, ranges = 24, 1024, 2048, 4
+    a = torch.randn(m, k).to(torch.bfloat16).to(device)
+    w = (torch.randn(n, k) * 0.05).to(torch.bfloat16).to(device)
+    out = torch.zeros(m, n, device=device)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    args = (a.data_ptr(), w.data_ptr(), None, out.data_ptr(), 0, m, n, k, k, n, 0, ranges, 1, stream)
+    assert lib.vk_gemm_bf16_mid_no_alloc(*args) == 0          # the first call on the device asks for the array's address
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    allocated_before = torch.cuda.memory_stats()["allocation.all.allocated"]
+    for _ in range(100):
+        assert lib.vk_gemm_bf16_mid_no_alloc(*args) == 0
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before
+    assert torch.cuda.memory_stats()["allocation.all.allocated"] == allocated_before
+    assert torch.allclose(out, a.float() @ w.float().T, rtol=2e-2, atol=2e-2)
 
 
 def test_sizes_beyond_the_array_are_refused():
@@ -77,5 +102,8 @@ def test_sizes_beyond_the_array_are_refused():
     status = lib.vk_gemm_bf16_mid_no_alloc(a.data_ptr(), w.data_ptr(), None, out.data_ptr(), 0, m, n, k, k, n, 0, ranges,
                                            1, stream)
     assert status == -2
+    # sizes whose product would not fit 64 bits do not slip past the check either
+    assert lib.vk_gemm_bf16_mid_no_alloc(a.data_ptr(), w.data_ptr(), None, out.data_ptr(), 0, 2 ** 31 - 1, 2 ** 31 - 1, k,
+                                         k, n, 0, 2 ** 31 - 1, 1, stream) == -2
     torch.cuda.synchronize()
     assert not out.any()

@@ -40,6 +40,7 @@ def _host():
         "vk_cache_release": ([p, u64], i),
         "vk_cache_table": ([p, u64, i, ip, i], i),
         "vk_cache_fill_tables": ([p, c.POINTER(u64), i, i, ip, i, ip, ip], i),
+        "vk_cache_allocate_nanos": ([p], u64),
         "vk_cache_slot": ([p, u64], i),
         "vk_cache_knows": ([p, u64], i),
         "vk_cache_free_blocks": ([p, i], i),
@@ -171,6 +172,10 @@ class CacheManager:
 
     def blocks_needed(self, group: int, total: int, portion: int) -> int:
         return self._lib.vk_cache_blocks_needed(self._handle, group, total, portion)
+
+    def allocate_micros(self) -> int:
+        """Microseconds spent so far in reserving, advancing and releasing, whoever asked (a scheduler, a replay)."""
+        return int(self._lib.vk_cache_allocate_nanos(self._handle) // 1000)
 
     def check(self) -> str:
         """Empty when every page and slot is free or held exactly once; else what is wrong."""

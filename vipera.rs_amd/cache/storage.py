@@ -13,7 +13,7 @@ crates/vipera-runtime/src/engine.rs:130-159, crates/vipera-sampler/src/rng.rs:13
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Dict, List, Optional, Sequence
+from typing import Dict, List, Optional, Sequence, Tuple, Union
 
 import torch
 
@@ -29,13 +29,36 @@ class PagedKV:
     block_size: int
 
 
-def plan_groups(needs, block_size: int, num_blocks: int) -> List[CacheGroupSpec]:
-    """One group per distinct retention rule among the run order's attention entries."""
-    windows: List[int] = []
+def group_key(kv) -> Tuple[int, int]:
+    """What makes two cache-owning layers share a group: the same window and the same page size asked for."""
+    return int(kv.window), int(kv.block_size)
+
+
+def group_keys(needs) -> List[Tuple[int, int]]:
+    """The groups of a run order, in the order in which its entries first need each."""
+    keys: List[Tuple[int, int]] = []
     for need in needs:
-        if need.kv is not None and need.kv.window not in windows:
-            windows.append(need.kv.window)
-    return [CacheGroupSpec(block_size, num_blocks, window) for window in windows]
+        if need.kv is not None and group_key(need.kv) not in keys:
+            keys.append(group_key(need.kv))
+    return keys
+
+
+def _per_group(value: Union[int, Sequence[int]], count: int, what: str) -> List[int]:
+    if isinstance(value, int):
+        return [value] * count
+    values = [int(v) for v in value]
+    if len(values) != count:
+        raise InvalidArgumentError(f"{what} lists {len(values)} values for {count} cache groups")
+    return values
+
+
+def plan_groups(needs, block_size: Union[int, Sequence[int]], num_blocks: Union[int, Sequence[int]]) -> List[CacheGroupSpec]:
+    """One group per distinct (window, page size asked for) among the run order's attention entries, in the order
+    of :func:`group_keys`.  ``block_size`` and ``num_blocks``: one number for every group, or one per group; a
+    page size that a mixer asks for itself (``KVCacheSpec.block_size``) stands."""
+    keys = group_keys(needs)
+    sizes, counts = _per_group(block_size, len(keys), "block_size"), _per_group(num_blocks, len(keys), "num_blocks")
+    return [CacheGroupSpec(asked or sizes[g], counts[g], window) for g, (window, asked) in enumerate(keys)]
 
 
 class CacheStorage:
@@ -53,9 +76,13 @@ class CacheStorage:
             if need.owner != index:
                 continue
             if need.kv is not None:
-                group = next((g for g, spec in enumerate(self.groups) if spec.window == need.kv.window), None)
-                if group is None:
-                    raise InvalidArgumentError(f"no cache group keeps a window of {need.kv.window}")
+                keys = group_keys(needs)
+                group = keys.index(group_key(need.kv))
+                if group >= len(self.groups) or self.groups[group].window != need.kv.window or (
+                        need.kv.block_size and self.groups[group].block_size != need.kv.block_size):
+                    raise InvalidArgumentError(
+                        f"the cache groups do not match the model: entry {index} needs a window of {need.kv.window}"
+                        + (f" in pages of {need.kv.block_size}" if need.kv.block_size else ""))
                 spec = self.groups[group]
                 k = runtime.zeros((spec.num_blocks + 1, need.kv.kv_heads, spec.block_size, need.kv.head_dim))
                 v = runtime.zeros((spec.num_blocks + 1, need.kv.kv_heads, need.kv.value_width, spec.block_size))
@@ -79,6 +106,17 @@ class CacheStorage:
                 seen.add(id(entry))
                 total += entry.k.shape[1] * (entry.k.shape[3] + entry.v.shape[2]) * entry.k.element_size()
         return total
+
+
+def group_position_bytes(needs, element: int) -> List[int]:
+    """Bytes per cached position of each group (in the order of :func:`group_keys`), over the entries of ``needs``
+    that own their storage; ``element`` is the size of a cached key or value."""
+    keys = group_keys(needs)
+    out = [0] * len(keys)
+    for index, need in enumerate(needs):
+        if need.owner == index and need.kv is not None:
+            out[keys.index(group_key(need.kv))] += need.kv.bytes_per_position(element)
+    return out
 
 
 def cache_bytes(needs, element: int):

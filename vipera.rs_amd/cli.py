@@ -23,12 +23,13 @@ vipera: inference engine for one MI355X
 
 USAGE:
     vipera model-info <model-dir> [--json]
-    vipera plan <model-dir> [--ctx N] [--batch N] [--dtype bfloat16|float32] [--block-size N] [--json]
+    vipera plan <model-dir> [--ctx N] [--batch N] [--dtype bfloat16|float32] [--block-size N] [--keep-float32]
+                [--json]
     vipera sample [--logits CSV | --logits-file PATH] [--count N] [--seed N] [--temperature F]
                   [--top-k N] [--top-p F] [--min-p F] [--repetition-penalty F] [--recent IDS] [--json]
     vipera generate <model-dir> (--prompt-ids IDS | --prompt-ids-file PATH) [--max-tokens N] [--ctx N]
                     [--dtype bfloat16|float32] [--block-size N] [--temperature F] [--top-k N] [--top-p F]
-                    [--min-p F] [--repetition-penalty F] [--seed N] [--json]
+                    [--min-p F] [--repetition-penalty F] [--seed N] [--keep-float32] [--json]
     vipera random-model <config.json> <out-dir> [--seed N] [--dtype bfloat16|float32]
     vipera --help
 
@@ -119,11 +120,14 @@ def _emit(text: str) -> None:
 
 # --- model-info -----------------------------------------------------------------------------------
 def model_summary(folder: str) -> dict:
+    import torch
+
     from .config.registry import load_config
-    from .models import declare_model
+    from .models import check_model, declare_model
     from .weights import Checkpoint
 
     config = load_config(folder)
+    check_model(config, torch.bfloat16)        # a model that no kernel takes is refused as one, not described
     checkpoint = Checkpoint(folder)
     try:
         dtypes: Dict[str, int] = {}
@@ -175,16 +179,22 @@ def model_info_command(argv: List[str]) -> int:
 
 
 # --- plan -------------------------------------------------------------------------------------------
-def plan_model(folder: str, ctx: Optional[int], batch: int, dtype: str, block_size: int) -> dict:
-    """Bytes on the device and work per step, from the configuration alone.
+def plan_model(folder: str, ctx: Optional[int], batch: int, dtype: str, block_size: int,
+               keep_float32: bool = False) -> dict:
+    """Bytes on the device and work per step, from the configuration and the tensor headers alone.
 
-    The cache costs ``2 * kv_heads * head_dim * bytes`` per position and attention layer, the
-    reference's arithmetic (crates/vipera-core/src/planner.rs:191-206).
+    The weights are counted in the dtypes the loader keeps them in (``weights.kept_bytes``: matrices in the run's
+    dtype whatever the folder stores, or with ``keep_float32`` 32-bit ones as stored), so the plan predicts what
+    loading then allocates, as the reference's planner does for its backend
+    (crates/vipera-core/src/planner.rs:266-430).  The cache costs ``2 * kv_heads * head_dim * bytes`` per position
+    and attention layer, the reference's arithmetic (planner.rs:191-206).
     """
+    import torch
+
     from .cache import cache_bytes
     from .config.registry import load_config
-    from .models import declare_cache_needs, declare_model
-    from .weights.checkpoint import MATRIX
+    from .models import check_model, declare_cache_needs, declare_model
+    from .weights.checkpoint import MATRIX, Checkpoint, kept_bytes, kept_dtype
 
     config = load_config(folder)
     if ctx is None:
@@ -195,21 +205,29 @@ def plan_model(folder: str, ctx: Optional[int], batch: int, dtype: str, block_si
     if ctx < 1 or batch < 1 or block_size < 1:
         raise InvalidArgumentError("--ctx, --batch and --block-size must be at least 1")
     element = 4 if dtype == "float32" else 2
-    weight_bytes = 0
-    matrix_elements = 0
-    head_elements = 0
-    for spec in declare_model(config):
-        if spec.unused:
-            continue
-        count = 1
-        for dim in spec.shape:
-            count *= dim
-        weight_bytes += count * (element if spec.role == MATRIX else 4)
-        if spec.role == MATRIX:
+    run_dtype = torch.float32 if dtype == "float32" else torch.bfloat16
+    specs = declare_model(config)
+    check_model(config, run_dtype)             # what no kernel takes is refused before any byte is counted
+    checkpoint = Checkpoint(folder)
+    try:
+        weight_bytes = kept_bytes(checkpoint, specs, run_dtype, keep_float32)
+        matrix_elements = matrix_bytes = 0
+        for spec in specs:
+            present = spec.name in checkpoint.tensors
+            if spec.role != MATRIX or (spec.optional and not present):
+                continue
+            count = 1
+            for dim in spec.shape:
+                count *= dim
             matrix_elements += count
+            stored = checkpoint.info(spec.name).torch_dtype if present else run_dtype
+            matrix_bytes += count * (4 if kept_dtype(spec, stored, run_dtype, keep_float32) == torch.float32 else 2)
+        head_name = f"{config.head_spec().params['name']}.weight"
+        tied = bool(config.head_spec().params.get("tied_to")) and head_name not in checkpoint.tensors
+    finally:
+        checkpoint.close()
     emb = config.embedding_spec().params
     embedding_elements = int(emb["vocab"]) * int(emb["width"])
-    tied = bool(config.head_spec().params.get("tied_to"))
     head_elements = embedding_elements
     kv_per_token, state_per_slot = cache_bytes(declare_cache_needs(config), element)
     blocks = batch * ((ctx + block_size - 1) // block_size)
@@ -218,7 +236,7 @@ def plan_model(folder: str, ctx: Optional[int], batch: int, dtype: str, block_si
     workspace = 2048 * (int(emb["width"]) * 4 + int(emb["vocab"]) * 4) + 256 * 1024 * 1024
     total = weight_bytes + kv_bytes + state_bytes + workspace + DEVICE_RESERVE
     # a decode step reads every matrix once (the embedding table only when it is also the head)
-    step_weights = (matrix_elements - (0 if tied else embedding_elements)) * element
+    step_weights = matrix_bytes * (matrix_elements - (0 if tied else embedding_elements)) // max(matrix_elements, 1)
     linear_elements = matrix_elements - embedding_elements - (0 if tied else head_elements)
     plan = {
         "dtype": dtype, "context": ctx, "batch": batch, "block_size": block_size,
@@ -239,14 +257,14 @@ def plan_model(folder: str, ctx: Optional[int], batch: int, dtype: str, block_si
 
 def plan_command(argv: List[str]) -> int:
     args = Args(argv, "plan", {"--json": False, "--ctx": True, "--batch": True, "--dtype": True,
-                               "--block-size": True}, 1)
+                               "--block-size": True, "--keep-float32": False}, 1)
     if not args.positional:
         raise UsageError("plan needs a model folder")
     dtype = args.values.get("--dtype", "bfloat16")
     if dtype not in ("bfloat16", "float32"):
         raise InvalidArgumentError(f"--dtype expects bfloat16 or float32, got \"{dtype}\"")
     plan = plan_model(args.positional[0], args.number("--ctx", None, int), args.number("--batch", 1, int), dtype,
-                      args.number("--block-size", 16, int))
+                      args.number("--block-size", 16, int), "--keep-float32" in args.switches)
     if "--json" in args.switches:
         _emit(json.dumps(plan, indent=2) + "\n")
     else:
@@ -310,7 +328,7 @@ def sample_command(argv: List[str]) -> int:
 def generate_command(argv: List[str]) -> int:
     flags = {"--json": False, "--prompt-ids": True, "--prompt-ids-file": True, "--max-tokens": True, "--ctx": True,
              "--dtype": True, "--block-size": True, "--temperature": True, "--top-k": True, "--top-p": True,
-             "--min-p": True, "--repetition-penalty": True, "--seed": True}
+             "--min-p": True, "--repetition-penalty": True, "--seed": True, "--keep-float32": False}
     args = Args(argv, "generate", flags, 1)
     if not args.positional:
         raise UsageError("generate needs a model folder")
@@ -339,6 +357,10 @@ def generate_command(argv: List[str]) -> int:
 
     folder = args.positional[0]
     config = load_config(folder)
+    import torch
+
+    from .models import check_model
+    check_model(config, torch.float32 if dtype == "float32" else torch.bfloat16)   # refused before the GPU is touched
     ctx = args.number("--ctx", None, int)
     if ctx is not None and ctx > config.context_limit:
         raise UnsupportedError(f"requested context {ctx} exceeds the model's maximum of {config.context_limit}")
@@ -348,7 +370,8 @@ def generate_command(argv: List[str]) -> int:
     # steps are launched ahead of their tokens (the engine falls back to one step at a time while a request's
     # penalties need its tokens on the host)
     engine = Engine(folder, dtype=dtype, block_size=block_size, max_num_seqs=1, max_model_len=context,
-                    num_blocks=(context + block_size - 1) // block_size, pipelined=True)
+                    num_blocks=(context + block_size - 1) // block_size, pipelined=True,
+                    keep_float32="--keep-float32" in args.switches)
     started = time.perf_counter()
     json_out = "--json" in args.switches
     shown = []

@@ -73,6 +73,8 @@ int vk_cache_fill_tables(void* handle, const unsigned long long* ids, int count,
   return -1;
 }
 
+unsigned long long vk_cache_allocate_nanos(void* handle) { return static_cast<CacheManager*>(handle)->allocate_nanos(); }
+
 int vk_cache_slot(void* handle, unsigned long long id) { return static_cast<CacheManager*>(handle)->slot(id); }
 int vk_cache_knows(void* handle, unsigned long long id) { return static_cast<CacheManager*>(handle)->knows(id) ? 1 : 0; }
 int vk_cache_free_blocks(void* handle, int group) { return static_cast<CacheManager*>(handle)->free_blocks(group); }

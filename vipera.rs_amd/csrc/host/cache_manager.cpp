@@ -50,6 +50,7 @@ int CacheManager::blocks_needed(int g, int total, int portion) const {
 }
 
 ReserveResult CacheManager::reserve(uint64_t id, int start, int total) {
+  Timed timed(&allocate_nanos_);
   if (start < 0) start = 0;
   if (total < start) total = start;
   auto found = requests_.find(id);
@@ -88,6 +89,7 @@ ReserveResult CacheManager::reserve(uint64_t id, int start, int total) {
 }
 
 void CacheManager::advance(uint64_t id, int processed) {
+  Timed timed(&allocate_nanos_);
   auto found = requests_.find(id);
   if (found == requests_.end()) return;
   for (size_t g = 0; g < groups_.size(); ++g) {
@@ -104,6 +106,7 @@ void CacheManager::advance(uint64_t id, int processed) {
 }
 
 bool CacheManager::release(uint64_t id) {
+  Timed timed(&allocate_nanos_);
   auto found = requests_.find(id);
   if (found == requests_.end()) return false;
   for (size_t g = 0; g < groups_.size(); ++g) {

@@ -12,6 +12,7 @@
 // could never fit is told so (341-346). What differs: pages are given back when a request ends
 // or when a window has moved past them, and there is no parking of finished requests.
 #pragma once
+#include <chrono>
 #include <cstdint>
 #include <map>
 #include <string>
@@ -78,6 +79,9 @@ class CacheManager {
   // Checks that every page is either free or held by exactly one table entry, and every slot
   // likewise. Returns an empty string when all is well, else what is wrong.
   std::string check() const;
+  // Nanoseconds spent so far in reserve, advance and release: the `allocate` stage of a step's timing
+  // (crates/vipera-runtime/src/pipeline.rs:251-270), whoever called them.
+  uint64_t allocate_nanos() const { return allocate_nanos_; }
 
  private:
   struct Held {
@@ -92,6 +96,16 @@ class CacheManager {
   std::map<uint64_t, Held> requests_;
   std::vector<int> empty_;
   int bad_frees_ = 0;  // pages given back that were not held: must stay 0
+  uint64_t allocate_nanos_ = 0;
+  struct Timed {  // adds the time of its scope to the manager's count
+    uint64_t* into;
+    std::chrono::steady_clock::time_point from = std::chrono::steady_clock::now();
+    explicit Timed(uint64_t* total) : into(total) {}
+    ~Timed() {
+      *into += (uint64_t)std::chrono::duration_cast<std::chrono::nanoseconds>(std::chrono::steady_clock::now() - from)
+                   .count();
+    }
+  };
 };
 
 }  // namespace vipera

@@ -49,6 +49,18 @@ __device__ __forceinline__ bf16x8 zero8() {
   return z;
 }
 
+// A V^T operand with the elements of positions at or past a range's end set to zero: of its elements 0-3 the first
+// `head` are kept, of its elements 4-7 the first `tail` (counts below 1 keep nothing, above 3 everything). Such a
+// position's weight is zero, but the slot may hold anything, also what is not finite (a page that another request
+// gave back, which the matrix instruction would turn into NaN: 0 * NaN), so the value is made zero as well. Only the
+// last tile of a range needs it.
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ bf16x8 keep_before_end(bf16x8 v, int head, int tail) {
+  auto pair = [](int kept, int e) { return kept > e + 1 ? 0xFFFFFFFFu : kept > e ? 0x0000FFFFu : 0u; };
+  const u32x4 mask = {pair(head, 0), pair(head, 2), pair(tail, 0), pair(tail, 2)};
+  return __builtin_bit_cast(bf16x8, __builtin_bit_cast(u32x4, v) & mask);
+}
+
 // A column's four lanes (lanes c, c + 16, c + 32, c + 48) combine their values with two lane swaps that run in the
 // vector ALU (v_permlane16_swap exchanges the odd 16-lane rows of one register with the even rows of another,
 // v_permlane32_swap the upper half of one with the lower half of another; with both registers holding v, the two
@@ -110,8 +122,9 @@ struct StepOperands {
 // [begin, end) reads a position inside it instead, a dim past the head width reads dim 0, a page id
 // that is not held reads page 0. None of these can reach a result: such a position's score is masked
 // before the softmax and its weight is zero, the query is zero in the padded dims and padded output
-// dims are not stored; what is read in their place is cache content of the same request, which is finite
-// (the pool starts zeroed). The block table is checked on the host before a step runs.
+// dims are not stored; what is read in their place is cache content of the same request. The group of eight V
+// positions that holds `end - 1` may reach past `end`, into slots that this request has not written: the range's
+// last step zeroes those elements (keep_before_end). The block table is checked on the host before a step runs.
 template <bool REGS>
 __device__ __forceinline__ void load_step(int kb, int begin, int end, const CacheView& cv, StepOperands& r) {
   const int lane = threadIdx.x & 63, lr = lane & 15, lg = lane >> 4;
@@ -193,10 +206,14 @@ __device__ __forceinline__ void attend_range(const bf16x8 (&qf)[KS], int col_lo,
       l = l * alpha + sum;
       m = m_new;
     }
+    // the last step of the range (known when it is compiled): V slots at or past `end` count as zero
+    constexpr bool LAST = decltype(rem_)::value == 0;
+    const int kept = end - (kb + lg * 8);
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
       o[dt] *= alpha;
-      o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.vf[dt], pf, o[dt], 0, 0, 0);
+      const bf16x8 vf = LAST ? keep_before_end(cur.vf[dt], kept, kept - 4) : cur.vf[dt];
+      o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, o[dt], 0, 0, 0);
     }
   };
   load_step<REGS>(first, begin, end, cv, ops[0]);
@@ -287,8 +304,9 @@ __global__ __launch_bounds__(PT_THREADS) void attn_prefill_kernel(
   // FAST: the page size is a power of two that divides 64. Tiles start at multiples of 64, so which page of
   // a tile a piece lies in, and where in that page, is the same for every tile: the thread keeps both, a tile's
   // page id is one table read at a clamped index, and an address is one multiply-add. Nothing is loaded
-  // conditionally: a piece outside [begin, end) reads a page of the same request inside that range (finite
-  // numbers: the pool starts zeroed), and its positions are masked, or weigh zero, for every column.
+  // conditionally: a piece outside [begin, end) reads a page of the same request inside that range, and its
+  // positions are masked, or weigh zero, for every column; the V^T operands of the tile that holds `end` are
+  // zeroed from `end` on (keep_before_end), since the slots there may hold anything.
   int k_tab[PT_PER_THREAD], v_tab[PT_PER_THREAD];          // page of the piece within a tile
   unsigned k_in[PT_PER_THREAD], v_in[PT_PER_THREAD];       // byte offset of the piece within its page
   const unsigned page_bytes = (unsigned)(kv_heads * bs * hd * 2);
@@ -428,12 +446,17 @@ __global__ __launch_bounds__(PT_THREADS) void attn_prefill_kernel(
       }
       l += sum;
     }
-    // ---- output: V^T operands from LDS
+    // ---- output: V^T operands from LDS (elements 0-3: positions 4 lg .. of a step's first 16, 4-7: of its second 16)
+    const bool tail = p0 + PT_KV > end;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
 #pragma unroll
       for (int step = 0; step < 2; ++step) {
-        const bf16x8 vf = *(const bf16x8*)(sV + (dt * 16 + lr) * PT_VROW + step * 32 + lg * 8);
+        bf16x8 vf = *(const bf16x8*)(sV + (dt * 16 + lr) * PT_VROW + step * 32 + lg * 8);
+        if (tail) {
+          const int kept = end - (p0 + step * 32 + lg * 4);
+          vf = keep_before_end(vf, kept, kept - 16);
+        }
         o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[step], o[dt], 0, 0, 0);
       }
     }
@@ -566,8 +589,9 @@ __global__ __launch_bounds__(SPLIT ? 2 * PT_THREADS : PT_THREADS) void attn_pref
 
   // Per lane and load instruction: which page of a tile its chunk lies in and where in that page; both are the
   // same for every tile, since tiles start at multiples of 64 and the page size divides 64. Nothing is loaded
-  // conditionally: a chunk outside [begin, end) reads a page of the same request inside that range (finite
-  // numbers: the pool starts zeroed), and its positions are masked, or weigh zero, for every column.
+  // conditionally: a chunk outside [begin, end) reads a page of the same request inside that range, and its
+  // positions are masked, or weigh zero, for every column; the V^T operands of the tile that holds `end` are
+  // zeroed from `end` on (keep_before_end), since the slots there may hold anything.
   int k_tab[PD_KLOADS], v_tab[PD_VLOADS];
   unsigned k_in[PD_KLOADS], v_in[PD_VLOADS];
   const unsigned page_bytes = (unsigned)(kv_heads * bs * hd * 2);
@@ -671,11 +695,16 @@ __global__ __launch_bounds__(SPLIT ? 2 * PT_THREADS : PT_THREADS) void attn_pref
       }
       l += sum;
     }
+    const bool tail = p0 + PT_KV > end;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
 #pragma unroll
       for (int st = 0; st < 2; ++st) {
-        const bf16x8 vf = *(const bf16x8*)(base + v_at[st] + dt * 16 * 128);
+        bf16x8 vf = *(const bf16x8*)(base + v_at[st] + dt * 16 * 128);
+        if (tail) {
+          const int kept = end - (p0 + st * 32 + lg * 8);
+          vf = keep_before_end(vf, kept, kept - 4);
+        }
         o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[st], o[dt], 0, 0, 0);
       }
     }

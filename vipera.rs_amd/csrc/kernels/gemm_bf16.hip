@@ -1592,6 +1592,9 @@ int launch_tile_as(const __bf16* A, const __bf16* W, const float* bias, TC* C, i
   return 0;
 }
 
+// Process-wide overrides for tests and measurements (vk_gemm_bf16_tile_config sets them): plain globals, read by
+// every launch of the tiled kernel from any thread and not synchronised. Nothing on the serving path sets them; a
+// program that does must not launch products from another thread meanwhile.
 int g_tile_config = -1;  // -1: chosen by shape; else a tiling (see launch_tile) and g_tile_ranges force a plan, for measurements
 int g_tile_ranges = 1;
 int g_tile_stages = 0;   // 0: chosen by shape; 2 or 3 force the direct kernel's LDS stages where the tiling has both
@@ -1813,8 +1816,12 @@ extern "C" int vk_gemm_bf16_mid_no_alloc(const void* A, const void* W, const flo
                                          int rows_per_wave, void* stream) {
   if (M <= 0 || N <= 0) return 0;
   if (ranges < 1) return VK_BAD_ARGUMENT;
-  // every range writes all of its M x N sums before the second kernel reads them, so nothing has to be cleared
-  if (ranges > 1 && (long long)ranges * M * N > VK_NO_ALLOC_SCRATCH_FLOATS) return VK_UNSUPPORTED_SIZE;
+  if (M > 128) return VK_UNSUPPORTED_SIZE;   // as vk_gemm_bf16_mid; checked before M enters a product
+  // every range writes all of its M x N sums before the second kernel reads them, so nothing has to be cleared;
+  // each factor is bounded before the product is formed (M <= 128), so the comparison cannot overflow
+  if (ranges > 1 && ((long long)ranges > VK_NO_ALLOC_SCRATCH_FLOATS || (long long)N > VK_NO_ALLOC_SCRATCH_FLOATS ||
+                     (long long)ranges * M * N > VK_NO_ALLOC_SCRATCH_FLOATS))
+    return VK_UNSUPPORTED_SIZE;
   int status = 0;
   float* partial = scratch_of_current_device(&status);
   if (!partial) return status;

@@ -90,12 +90,12 @@ class PackedStep:
 
 
 def pack_entries(entries: Sequence[StepEntry], cache, vocab_size: int, min_table_width: int = 1,
-                 pad_entries: int = 0, pad_page: int = -1, pad_slot: int = 0) -> PackedStep:
+                 pad_entries: int = 0, pad_slot: int = 0) -> PackedStep:
     """Check ``entries`` and lay them out for the device.
 
     The pages of every token must already be reserved in ``cache``.  ``pad_entries`` appends
-    single-token dummy entries (token 0 at position 0, every table entry ``pad_page``, state slot
-    ``pad_slot``), which a captured graph of a fixed batch size needs; their logits are computed and
+    single-token dummy entries (token 0 at position 0, every table entry the scratch page of its group, which is
+    the page past the pool's last, state slot ``pad_slot``), which a captured graph of a fixed batch size needs; their logits are computed and
     ignored, and what they write goes to the scratch page and the scratch state row, which belong to
     no request.  A step of padding only (no ``entries``) is what a graph is warmed up and captured on.
     """
@@ -180,7 +180,7 @@ def pack_entries(entries: Sequence[StepEntry], cache, vocab_size: int, min_table
                 f"request {e.request}: positions {lo}..{int(kv_len[failed]) - 1} are not all backed by pages "
                 f"in cache group {g}; reserve before the step")
         if pad_entries:
-            table[real:, :] = pad_page
+            table[real:, :] = spec.num_blocks
         tables.append(table)
         widths.append(width)
     sections = [tokens, positions, entry_of, starts, first, kv_len.astype(np.int32), slots,

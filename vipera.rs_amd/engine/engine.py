@@ -88,7 +88,8 @@ class Engine:
 
     ``model``: a folder with ``config.json`` and ``model.safetensors``.  ``dtype``: ``"bfloat16"``
     or ``"float32"``.  The cache has ``num_blocks`` pages of ``block_size`` positions per group of
-    layers; when ``num_blocks`` is absent it is sized for ``max_num_seqs`` requests of
+    layers (each one number for every group, or a list with one per group in the order in which the model's
+    layers first need each group); when ``num_blocks`` is absent it is sized for ``max_num_seqs`` requests of
     ``max_model_len`` tokens, bounded by free device memory.  ``use_graphs`` (default on) replays
     steps of single tokens as captured HIP graphs.
 
@@ -99,6 +100,9 @@ class Engine:
     dropped.  While a live request uses penalties (they look at the last tokens on the host), steps run
     one after the other as without the option.
 
+    ``keep_float32``: matrices that the folder stores in 32-bit stay in 32-bit in a bfloat16 run instead of being
+    converted to bfloat16 when they are loaded; their products then run through the 32-bit kernel.
+
     ``eager_admission``: start a waiting request as soon as its first portion finds pages, instead of only
     when all its tokens fit beside what the running requests still need (see ``csrc/host/scheduler.h``).
     """
@@ -107,7 +111,8 @@ class Engine:
                  num_blocks: Optional[int] = None, max_num_seqs: int = 8, max_num_batched_tokens: int = 2048,
                  chunk_size: int = 512, max_model_len: Optional[int] = None,
                  eos_token_ids: Optional[Sequence[int]] = None, runner: Optional[ModelRunner] = None,
-                 use_graphs: Optional[bool] = None, pipelined: bool = False, eager_admission: bool = False):
+                 use_graphs: Optional[bool] = None, pipelined: bool = False, eager_admission: bool = False,
+                 keep_float32: bool = False):
         if runner is None:
             runtime = Runtime(device, dtype)
             from ..config.registry import load_config
@@ -117,10 +122,13 @@ class Engine:
                 raise InvalidArgumentError(
                     f"requested context {limit} exceeds the model's maximum of {config.context_limit}")
             if num_blocks is None:
-                num_blocks = max_num_seqs * ((limit + block_size - 1) // block_size)
+                sizes = [block_size] if isinstance(block_size, int) else list(block_size)
+                counts = [max_num_seqs * ((limit + size - 1) // size) for size in sizes]
+                num_blocks = counts[0] if isinstance(block_size, int) else counts
             if use_graphs is None:
                 use_graphs = True
-            runner = self._load(model, config, runtime, block_size, num_blocks, max_num_seqs, use_graphs, limit)
+            runner = self._load(model, config, runtime, block_size, num_blocks, max_num_seqs, use_graphs, limit,
+                                keep_float32)
         else:  # a runner that is already set up (its model, cache and graphs are used as they are)
             config = runner.model.config
             limit = int(max_model_len or config.context_limit)
@@ -140,7 +148,11 @@ class Engine:
         self.generations = 0
         self.failed = 0
         self.step_count = 0
-        self.micros = {"schedule": 0, "compute": 0, "sample": 0}
+        # host microseconds by stage, as the reference's per-turn log keeps them (crates/vipera-runtime/src/
+        # pipeline.rs:251-270): deciding the step, reserving and giving back pages (counted by the cache manager
+        # itself, inside the scheduler's calls and outside them), packing and launching the model, sampling
+        self.micros = {"schedule": 0, "allocate": 0, "compute": 0, "sample": 0}
+        self._allocate_seen = runner.cache.allocate_micros()
         self.max_num_seqs = int(max_num_seqs)
 
     def warm_up(self, max_batch: Optional[int] = None, max_context: Optional[int] = None) -> int:
@@ -154,24 +166,31 @@ class Engine:
         return graphs.capture_ahead(int(max_batch or self.max_num_seqs), int(max_context or self.max_model_len))
 
     @staticmethod
-    def _load(folder, config, runtime, block_size, num_blocks, num_slots, use_graphs, max_context) -> ModelRunner:
-        from ..cache import cache_bytes
+    def _load(folder, config, runtime, block_size, num_blocks, num_slots, use_graphs, max_context,
+              keep_float32=False) -> ModelRunner:
+        from ..cache import cache_bytes, group_position_bytes, plan_groups
 
-        model = ModelRunner.load_model(folder, config, runtime)
+        model = ModelRunner.load_model(folder, config, runtime, keep_float32=keep_float32)
         free, _ = torch.cuda.mem_get_info(runtime.device)
         num_slots = max(num_slots, 1)
-        per_position, per_slot = cache_bytes(model.cache_needs(), 4 if runtime.dtype == torch.float32 else 2)
-        per_page = per_position * block_size
+        element = 4 if runtime.dtype == torch.float32 else 2
+        needs = model.cache_needs()
+        _, per_slot = cache_bytes(needs, element)
         room = 0.9 * free - per_slot * (num_slots + 1)       # fixed-size state first: one row per slot and a scratch row
         if room < 0:
             raise InfeasibleError(
                 f"no room for {num_slots} state slots of {per_slot} bytes in {free} free bytes of device memory")
-        if per_page and num_blocks * per_page > room:
-            fit = int(room // per_page)
-            if fit < 1:
+        groups = plan_groups(needs, block_size, num_blocks)
+        per_page = [spec.block_size * per_position
+                    for spec, per_position in zip(groups, group_position_bytes(needs, element))]
+        wanted = sum(spec.num_blocks * page for spec, page in zip(groups, per_page))
+        if wanted > room:   # every pool shrinks by the same share
+            counts = [int(spec.num_blocks * room / wanted) for spec in groups]
+            if min(counts) < 1:
                 raise InfeasibleError(
-                    f"no room for a single cache page of {per_page} bytes in {free} free bytes of device memory")
-            num_blocks = fit
+                    f"no room for a single cache page of {max(per_page)} bytes per group in {free} free bytes of "
+                    "device memory")
+            num_blocks = counts if not isinstance(num_blocks, int) else min(counts)
         return ModelRunner(model, runtime, block_size, num_blocks, num_slots, use_graphs, max_context)
 
     # --- requests ---------------------------------------------------------------------------------
@@ -205,14 +224,27 @@ class Engine:
         when the request draws for the first time in that slot (at its start, or wound forward by the draws it
         had made when it comes back after a preemption)."""
         live = self._live[entry.request]
-        seed_state = None
-        if not live.seeded:
-            seed_state = seeded_state(live.params.seed, live.draws)
-            live.seeded = True
-        if not live.params.greedy:
-            live.draws += 1
+        seed_state = None if live.seeded else seeded_state(live.params.seed, live.draws)
         return RowRequest(live.params, self.runner.cache.slot(entry.request), entry.start + len(entry.tokens), recent,
                           seed_state)
+
+    def _launch_sampling(self, logits, wanting, rows, report: StepReport):
+        """Launch the sampling of ``rows`` (one per entry of ``wanting``).  Only once the launch has gone through is
+        it booked on the host that these requests' slots hold their generators and that each drawing row has used
+        one uniform: a launch that raises leaves the host's counts where the device's generators are, and fails the
+        requests it was for.  Returns the pending sample, or None after a failure."""
+        try:
+            pending = self.sampler.launch(logits, rows)
+        except ViperaError as err:
+            for e in wanting:
+                self._fail(e.request, str(err), report)
+            return None
+        for e in wanting:
+            live = self._live[e.request]
+            live.seeded = True
+            if not live.params.greedy:
+                live.draws += 1
+        return pending
 
     def _note_preempted(self, plan, report: StepReport) -> None:
         for request in plan.preempted:
@@ -236,11 +268,12 @@ class Engine:
     def _step_ahead(self) -> StepReport:
         """Launch the next step, then take in the tokens of the step launched before it."""
         report = StepReport()
+        self._book("", 0.0)     # pages moved since the last step (requests added or cancelled) are booked first
         started = time.perf_counter()
         plan = self.scheduler.plan()
         self._note_preempted(plan, report)
         scheduled = time.perf_counter()
-        self.micros["schedule"] += int((scheduled - started) * 1e6)
+        self._book("schedule", scheduled - started)
         previous, launched = self._inflight, None
         if plan.entries:
             entries = []
@@ -267,21 +300,19 @@ class Engine:
                 self.scheduler.advance(e.request)
                 self._live[e.request].processed += len(e.tokens)
             wanting = [e for e in plan.entries if e.wants_logits]
-            if wanting:
-                rows = [self._row(e) for e in wanting]
-                pending = self.sampler.launch(logits, rows)
+            pending = self._launch_sampling(logits, wanting, [self._row(e) for e in wanting], report) if wanting else None
+            if pending is not None:
                 # the scheduler goes on as if the token were known: a placeholder stands for it until it arrives
                 reasons = [self.scheduler.append(e.request, 0, False) for e in wanting]
                 launched = _InFlight(pending, [e.request for e in wanting], reasons,
                                      {e.request: row for row, e in enumerate(wanting)})
         computed = time.perf_counter()
+        self._book("compute", computed - scheduled)
         self._inflight = previous
         if previous is not None:
             self._collect(report, newer=launched)
         self._inflight = launched
-        done = time.perf_counter()
-        self.micros["compute"] += int((computed - scheduled) * 1e6)
-        self.micros["sample"] += int((done - computed) * 1e6)
+        self._book("sample", time.perf_counter() - computed)
         return report
 
     def _collect(self, report: StepReport, newer: Optional[_InFlight] = None) -> None:
@@ -313,12 +344,23 @@ class Engine:
                 report.finished.append(Generation(request, len(live.prompt), live.generated, FINISH_NAMES[reason],
                                                   live.processed, live.preemptions))
 
+    def _book(self, stage: str, seconds: float) -> None:
+        """Book ``seconds`` of host time: what the cache manager spent on pages since the last booking is
+        ``allocate`` (it happens inside the scheduler's decisions, after a step, and when a request ends), the rest
+        goes to ``stage``."""
+        now = self.runner.cache.allocate_micros()
+        pages, self._allocate_seen = now - self._allocate_seen, now
+        self.micros["allocate"] += pages
+        if stage:
+            self.micros[stage] += max(0, int(seconds * 1e6) - pages)
+
     def _step_in_turn(self, report: StepReport) -> StepReport:
+        self._book("", 0.0)
         started = time.perf_counter()
         plan = self.scheduler.plan()
         self._note_preempted(plan, report)
         scheduled = time.perf_counter()
-        self.micros["schedule"] += int((scheduled - started) * 1e6)
+        self._book("schedule", scheduled - started)
         if not plan.entries:
             return report
         entries = [StepEntry(e.request, e.start, e.tokens, [len(e.tokens) - 1] if e.wants_logits else [])
@@ -336,12 +378,14 @@ class Engine:
             self._live[e.request].processed += len(e.tokens)
         wanting = [e for e in plan.entries if e.wants_logits]
         computed = time.perf_counter()
+        self._book("compute", computed - scheduled)
         if wanting:
             rows = []
             for e in wanting:
                 live = self._live[e.request]
                 rows.append(self._row(e, _recent_tokens(live) if live.params.penalizes else ()))
-            tokens = self.sampler.sample(logits, rows)
+            pending = self._launch_sampling(logits, wanting, rows, report)
+            tokens = self.sampler.collect(pending) if pending is not None else []
             for e, token in zip(wanting, tokens):
                 if token < 0:
                     self._fail(e.request, "the logits hold no finite value", report)
@@ -358,9 +402,7 @@ class Engine:
                     self.generations += 1
                     report.finished.append(Generation(e.request, len(live.prompt), live.generated,
                                                       FINISH_NAMES[reason], live.processed, live.preemptions))
-        done = time.perf_counter()
-        self.micros["compute"] += int((computed - scheduled) * 1e6)
-        self.micros["sample"] += int((done - computed) * 1e6)
+        self._book("sample", time.perf_counter() - computed)
         return report
 
     def _fail(self, request: int, message: str, report: StepReport) -> None:

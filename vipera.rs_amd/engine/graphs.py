@@ -60,7 +60,7 @@ class DecodeGraphs:
         cache = self.runner.cache
         width = max((context_bucket + g.block_size - 1) // g.block_size for g in cache.groups) if cache.groups else 1
         packed = pack_entries(entries, cache, self.runner.vocab_size, min_table_width=width,
-                              pad_entries=batch_bucket - len(entries), pad_page=self.runner.num_blocks,
+                              pad_entries=batch_bucket - len(entries),
                               pad_slot=self.runner.storage.scratch_slot)
         # every row's logits are computed; the caller picks the wanted ones
         packed.sections[7] = np.arange(batch_bucket, dtype=np.int32)

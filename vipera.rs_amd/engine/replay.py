@@ -18,7 +18,7 @@ from .runner import ModelRunner
 
 class Replayer:
     def __init__(self, model_dir: str, dtype: str, max_tokens: int, block_size: int = 16,
-                 device: str = "cuda:0", log: Optional[Callable[[str], None]] = None):
+                 device: str = "cuda:0", log: Optional[Callable[[str], None]] = None, keep_float32: bool = False):
         if max_tokens < 1:
             raise InvalidArgumentError(f"--max-tokens must be at least 1, got {max_tokens}")
         if block_size < 1:
@@ -33,7 +33,7 @@ class Replayer:
         if log:
             log(f"[trace_run] loading {model_dir} as {dtype}; {num_blocks} pages of {page} positions per cache group")
         self.runner = ModelRunner.from_folder(model_dir, dtype=dtype, device=device, block_size=page,
-                                              num_blocks=num_blocks, num_slots=16)
+                                              num_blocks=num_blocks, num_slots=16, keep_float32=keep_float32)
         self.ids: Dict[str, int] = {}
         self.lengths: Dict[int, int] = {}
         self.next_id = 0

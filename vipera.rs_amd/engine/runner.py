@@ -27,7 +27,10 @@ SAMPLED_CAPACITY = 1024  # rows of logits one step may be sampled for with devic
 
 
 class ModelRunner:
-    def __init__(self, model, runtime: Runtime, block_size: int, num_blocks: int, num_slots: int,
+    """``block_size`` and ``num_blocks``: positions per page and pages in the pool, one number for every cache group
+    or a list with one per group (in the order of ``cache.group_keys(model.cache_needs())``)."""
+
+    def __init__(self, model, runtime: Runtime, block_size, num_blocks, num_slots: int,
                  use_graphs: bool = False, max_context: int = 0):
         if not model.loaded:
             raise InvalidArgumentError("the model has no weights yet; load them before building a runner")
@@ -49,16 +52,20 @@ class ModelRunner:
         self.graphs = None
         if use_graphs:
             from .graphs import DecodeGraphs
-            self.graphs = DecodeGraphs(self, max_context or block_size * num_blocks)
+            longest = min((g.block_size * g.num_blocks for g in groups if g.window == 0), default=0)
+            self.graphs = DecodeGraphs(self, max_context or longest or max((g.block_size * g.num_blocks for g in groups), default=1))
 
     # --- construction helpers -----------------------------------------------------------------
     @staticmethod
-    def load_model(folder: str, config: ModelConfig, runtime: Runtime, progress=None):
-        """The model of ``config`` with the weights of ``folder`` on the runtime's device."""
+    def load_model(folder: str, config: ModelConfig, runtime: Runtime, progress=None, keep_float32: bool = False):
+        """The model of ``config`` with the weights of ``folder`` on the runtime's device.  A model with a size that
+        no kernel takes is refused when it is built, before the folder's tensors are opened.  ``keep_float32``:
+        matrices that the folder stores in 32-bit stay so in a bfloat16 run (see ``weights.kept_dtype``)."""
         model = build_model(config, runtime)
         checkpoint = Checkpoint(folder)
         try:
-            tensors = load_tensors(checkpoint, model.tensor_specs(), runtime.dtype, runtime.device, progress)
+            tensors = load_tensors(checkpoint, model.tensor_specs(), runtime.dtype, runtime.device, progress,
+                                   keep_float32)
         finally:
             checkpoint.close()
         model.load(tensors)
@@ -67,9 +74,9 @@ class ModelRunner:
     @classmethod
     def from_folder(cls, folder: str, dtype="bfloat16", device="cuda:0", block_size: int = 16,
                     num_blocks: int = 256, num_slots: int = 8, progress=None, use_graphs: bool = False,
-                    max_context: int = 0) -> "ModelRunner":
+                    max_context: int = 0, keep_float32: bool = False) -> "ModelRunner":
         runtime = Runtime(device, dtype)
-        model = cls.load_model(folder, load_config(folder), runtime, progress)
+        model = cls.load_model(folder, load_config(folder), runtime, progress, keep_float32)
         return cls(model, runtime, block_size, num_blocks, num_slots, use_graphs, max_context)
 
     # --- the step ---------------------------------------------------------------------------------
@@ -83,7 +90,11 @@ class ModelRunner:
         return self.model.forward(batch, self.storage)
 
     def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
-        """Logits ``[wanted, vocab]`` (32-bit, on the device) in the order of the entries and their ``want``."""
+        """Logits ``[wanted, vocab]`` (32-bit, on the device) in the order of the entries and their ``want``.
+
+        With captured steps the tensor may be a view of a graph's own output buffer, which the next step of the
+        same size overwrites: it holds this step's logits until the next call of ``step``, in stream order.  A
+        caller that keeps logits longer copies them."""
         if self.graphs is not None and self.graphs.wants(entries):
             self.steps += 1
             return self.graphs.step(entries)

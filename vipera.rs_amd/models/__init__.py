@@ -5,7 +5,7 @@ from .. import parts  # noqa: F401  (registers the built-in parts)
 from ..config.base import ModelConfig
 from ..config.registry import lookup_architecture
 from . import qwen2  # noqa: F401  (registers the architecture)
-from .decoder import CacheNeed, DecoderModel, declare_cache_needs, declare_model
+from .decoder import CacheNeed, DecoderModel, check_model, declare_cache_needs, declare_model
 
 
 def build_model(config: ModelConfig, runtime):
@@ -14,4 +14,4 @@ def build_model(config: ModelConfig, runtime):
     return builder(config, runtime)
 
 
-__all__ = ["CacheNeed", "DecoderModel", "build_model", "declare_cache_needs", "declare_model"]
+__all__ = ["CacheNeed", "DecoderModel", "build_model", "check_model", "declare_cache_needs", "declare_model"]

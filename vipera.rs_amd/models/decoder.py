@@ -62,6 +62,19 @@ def declare_model(config: ModelConfig) -> List[TensorSpec]:
     return specs
 
 
+def check_model(config: ModelConfig, dtype) -> None:
+    """Raise ``UnsupportedError`` if some part of ``config``'s model has a size that no kernel takes in a run of
+    ``dtype``.  Touches no GPU and reads no weight: it is what opening a model does first."""
+    emb = config.embedding_spec()
+    part_class("embedding", emb.kind).check_supported(emb, dtype)
+    for layer in config.layer_specs():
+        part_class("block", layer.block).check_supported(layer, dtype)
+    norm = config.final_norm_spec()
+    part_class("norm", norm.kind).check_supported(norm, dtype)
+    head = config.head_spec()
+    part_class("head", head.kind).check_supported(head, dtype)
+
+
 def declare_cache_needs(config: ModelConfig) -> List[CacheNeed]:
     """What every entry of ``config``'s run order keeps per request, from the configuration alone. Touches no GPU."""
     layers = config.layer_specs()
@@ -79,6 +92,7 @@ class DecoderModel:
     def __init__(self, config: ModelConfig, runtime):
         self.config = config
         self.runtime = runtime
+        check_model(config, runtime.dtype)    # sizes that no kernel takes are refused here, before weights are read
         emb, norm, head = config.embedding_spec(), config.final_norm_spec(), config.head_spec()
         self.embedding = part_class("embedding", emb.kind)(emb, "", runtime)
         self.layers = [part_class("block", spec.block)(spec, runtime) for spec in config.layer_specs()]

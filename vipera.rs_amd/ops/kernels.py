@@ -64,6 +64,11 @@ def _status(code: int, name: str) -> None:
     raise InternalError(f"{name}: HIP error {code} at launch")
 
 
+ATTENTION_MAX_HEAD_DIM = 256    # both attention kernels keep a head's dims in registers or one LDS row
+ATTENTION_MAX_HEADS = 65_535    # q, k and v heads of a token are one grid dimension of the rotation kernel
+GEMM_BF16_MAX_K = 1 << 23       # the matrix-core products form 32-bit byte offsets inside a tile of rows
+
+
 def _cache_ok(k_cache, v_cache, kv_heads: int, head_dim: int, dtype) -> bool:
     """K pages ``[pages, kv_heads, block_size, head_dim]``, V pages ``[pages, kv_heads, head_dim, block_size]``."""
     return (k_cache.dim() == 4 and v_cache.dim() == 4 and k_cache.shape[1] == kv_heads
@@ -255,8 +260,8 @@ def attn_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, 
     _need(entry_of_token.dtype == torch.int32 and entry_of_token.numel() >= num_tokens, "attention: entries")
     _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(), "attention: table")
     _need(heads % kv_heads == 0, "attention: heads must be a multiple of kv_heads")
-    if head_dim > 256:
-        raise UnsupportedError(f"attention: head_dim {head_dim} is above the kernel's limit of 256")
+    if head_dim > ATTENTION_MAX_HEAD_DIM:
+        raise UnsupportedError(f"attention: head_dim {head_dim} is above the kernels' limit of {ATTENTION_MAX_HEAD_DIM}")
     fn = _fn("attn_generic", "vk_attn_generic",
              [_p, _ll, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _i, _p])
     _status(fn(_ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(out), _dt(q, "q"), _ptr(positions),
@@ -342,9 +347,11 @@ def logit_bias(logits: torch.Tensor, rows: torch.Tensor, tokens: torch.Tensor, v
 
 # ----------------------------------------------------------------------------------------------
 def gemm_bf16_supported(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> bool:
-    """Whether the matrix-core kernels take these operands (16-byte chunks along K)."""
+    """Whether the matrix-core kernels take these operands (16-byte chunks along K, rows short enough for their
+    32-bit offsets); what they do not take goes to the 32-bit FMA kernel."""
     k = a.shape[1]
     return (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out.dtype in _DT and k % 8 == 0
+            and k < GEMM_BF16_MAX_K and a.stride(0) < GEMM_BF16_MAX_K
             and a.stride(1) == 1 and (a.stride(0) % 8 == 0 or a.shape[0] == 1) and a.data_ptr() % 16 == 0
             and w.is_contiguous() and w.data_ptr() % 16 == 0 and out.stride(1) == 1)
 

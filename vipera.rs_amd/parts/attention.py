@@ -78,6 +78,17 @@ class Attention(Mixer):
         p = spec.params
         return KVCacheSpec(int(p["kv_heads"]), int(p["head_dim"]), int(p.get("window") or 0)), None
 
+    @classmethod
+    def check_supported(cls, spec: PartSpec, dtype: torch.dtype) -> None:
+        p = spec.params
+        heads, kv_heads, head_dim = int(p["heads"]), int(p["kv_heads"]), int(p["head_dim"])
+        if head_dim > kernels.ATTENTION_MAX_HEAD_DIM:
+            raise UnsupportedError(f"attention: head_dim {head_dim} is above the kernels' limit of "
+                                   f"{kernels.ATTENTION_MAX_HEAD_DIM}")
+        if heads + 2 * kv_heads > kernels.ATTENTION_MAX_HEADS:
+            raise UnsupportedError(f"attention: {heads} query heads with {kv_heads} key/value heads are above the "
+                                   f"kernels' limit of {kernels.ATTENTION_MAX_HEADS} heads in all")
+
     fills_handoff = True
 
     def _fused(self, tokens: int, position, batch) -> Optional[str]:

@@ -41,12 +41,15 @@ from ..weights.checkpoint import TensorSpec
 @dataclass(frozen=True)
 class KVCacheSpec:
     """Keys and values in pages: per position ``kv_heads * head_dim`` keys and ``kv_heads * value_dim``
-    values (``value_dim`` 0: as wide as the keys); ``window`` 0 keeps all."""
+    values (``value_dim`` 0: as wide as the keys); ``window`` 0 keeps all.  ``block_size``: positions per page if the
+    mixer needs a page size of its own (0: the engine's).  Layers with the same window and page size share a
+    *group*: one pool of pages and one block table per request."""
 
     kv_heads: int
     head_dim: int
     window: int = 0
     value_dim: int = 0
+    block_size: int = 0
 
     @property
     def value_width(self) -> int:
@@ -85,6 +88,13 @@ class Part:
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         """Take the declared tensors (already on the device in their kept dtype)."""
+
+    @classmethod
+    def check_supported(cls, spec: PartSpec, dtype: torch.dtype) -> None:
+        """Raise :class:`~vipera_rs_amd.errors.UnsupportedError` if no kernel takes a part of ``spec`` in a run of
+        ``dtype``.  From the spec alone: it is asked when a model is opened, before any weight is read, as the
+        reference refuses what its backend cannot run while it reads the header
+        (crates/vipera-backend-cpu/src/model.rs:1323-1328, 1367-1383)."""
 
 
 @dataclass
@@ -176,6 +186,13 @@ class Block:
 
     def load(self, tensors) -> None:
         raise NotImplementedError
+
+    @classmethod
+    def check_supported(cls, spec: LayerSpec, dtype: torch.dtype) -> None:
+        """Ask every part of the layer whether the kernels take it (see :meth:`Part.check_supported`)."""
+        for family, part in (("norm", spec.mixer_norm), ("mixer", spec.mixer), ("norm", spec.ffn_norm),
+                             ("ffn", spec.ffn), ("position", spec.position)):
+            part_class(family, part.kind).check_supported(part, dtype)
 
     #: a block that sets this takes ``incoming=`` and ``outgoing=`` in ``forward`` and has ``accepts_incoming`` and
     #: ``fills_outgoing`` (see :class:`NormHandoff`: its first norm prepared by the layer before, the next layer's

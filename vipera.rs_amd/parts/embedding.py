@@ -60,14 +60,18 @@ class LMHead(Part):
 
     @classmethod
     def declare(cls, spec: PartSpec, prefix: str) -> List[TensorSpec]:
-        # with tied embeddings a folder may still hold an output matrix (a copy of the table): it is not read
+        # With tied embeddings the output matrix is optional: a folder that holds one has it used, as the reference
+        # uses `output.weight` whenever the file has it and the embedding table only otherwise (model.rs:424-425).
         return [TensorSpec(f"{prefix}{spec.params['name']}.weight",
                            (int(spec.params["vocab"]), int(spec.params["width"])), MATRIX,
-                           unused=bool(spec.params.get("tied_to")))]
+                           optional=bool(spec.params.get("tied_to")))]
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
-        name = self.tied_to if self.tied_to else f"{self.prefix}{self.spec.params['name']}"
-        self.weight = tensors[f"{name}.weight"]  # tied: the same buffer, no copy
+        own = f"{self.prefix}{self.spec.params['name']}.weight"
+        if self.tied_to and own not in tensors:
+            self.weight = tensors[f"{self.tied_to}.weight"]  # tied: the same buffer, no copy
+        else:
+            self.weight = tensors[own]
 
     def forward(self, h: torch.Tensor) -> torch.Tensor:
         logits = self.runtime.empty((h.shape[0], self.vocab), torch.float32)

@@ -18,7 +18,7 @@ import torch
 from ..errors import InvalidArgumentError, IoError, ParseError
 from .safetensors_io import SafetensorsFile, TensorInfo
 
-MATRIX = "matrix"   # kept in the run's dtype unless the file stores it in 32-bit
+MATRIX = "matrix"   # converted to the run's dtype when it is loaded (see kept_dtype)
 VECTOR = "vector"   # norm weights, biases: kept in 32-bit
 INT_TABLE = "int_table"  # integer tables: kept as int32
 
@@ -32,7 +32,7 @@ class TensorSpec:
     role: str = MATRIX
     init: str = "normal"      # "normal" N(0, std) | "one_plus_normal" 1 + N(0, std) | "zeros" | "ones"
     std: float = 0.02
-    unused: bool = False      # a folder may hold it, the model does not read it: its shape is checked, nothing is loaded
+    optional: bool = False    # a folder need not hold it; when it does, its shape is checked and it is loaded
 
 
 class WeightsError(InvalidArgumentError):
@@ -106,7 +106,7 @@ class Checkpoint:
     def check(self, specs: Iterable[TensorSpec]) -> None:
         """Raise one :class:`WeightsError` that lists everything wrong, or return."""
         wanted = {spec.name: spec for spec in specs}
-        missing = [name for name, spec in wanted.items() if name not in self.tensors and not spec.unused]
+        missing = [name for name, spec in wanted.items() if name not in self.tensors and not spec.optional]
         unexpected = [name for name in self.tensors if name not in wanted]
         wrong = []
         for name, spec in wanted.items():
@@ -122,37 +122,60 @@ class Checkpoint:
             shard.close()
 
 
-def kept_dtype(spec: TensorSpec, stored: torch.dtype, run_dtype: torch.dtype) -> torch.dtype:
+def kept_dtype(spec: TensorSpec, stored: torch.dtype, run_dtype: torch.dtype, keep_float32: bool = False) -> torch.dtype:
     """The dtype a tensor has on the device.
 
-    Matrices take the run's dtype, except that a matrix stored in 32-bit stays in
-    32-bit; vectors (norm weights, biases) are always widened to 32-bit, which is exact;
-    integer tables become int32.
+    A matrix is converted once, when it is loaded, to the run's dtype, whatever floating-point type the folder
+    stores it in (32-bit, 16-bit float or bfloat16; to bfloat16 by rounding to nearest even): the run's kernels and
+    the memory a plan predicts are then those of the run's dtype, not of the file's.  ``keep_float32``: a matrix
+    stored in 32-bit stays in 32-bit in a bfloat16 run (its products then go through the 32-bit FMA kernel, at a
+    fraction of the speed).  Vectors (norm weights, biases) are always 32-bit, which widens a 16-bit one exactly and
+    leaves a 32-bit one as it is; integer tables become int32.
     """
     if spec.role == INT_TABLE:
         return torch.int32
     if spec.role == VECTOR:
         return torch.float32
-    if stored == torch.float32 or run_dtype == torch.float32:
+    if run_dtype == torch.float32 or (keep_float32 and stored == torch.float32):
         return torch.float32
     return run_dtype
 
 
+def kept_bytes(checkpoint: Checkpoint, specs: Sequence[TensorSpec], run_dtype: torch.dtype,
+               keep_float32: bool = False) -> int:
+    """Device bytes of the tensors that :func:`load_tensors` would load from ``checkpoint``, from its headers alone.
+    A required tensor that the folder does not hold (yet) counts as if it were stored in the run's dtype."""
+    total = 0
+    for spec in specs:
+        present = spec.name in checkpoint.tensors
+        if not present and spec.optional:
+            continue
+        count = 1
+        for dim in spec.shape:
+            count *= int(dim)
+        stored = checkpoint.info(spec.name).torch_dtype if present else run_dtype
+        total += count * torch.empty(0, dtype=kept_dtype(spec, stored, run_dtype, keep_float32)).element_size()
+    return total
+
+
 def load_tensors(checkpoint: Checkpoint, specs: Sequence[TensorSpec], run_dtype: torch.dtype,
-                 device: torch.device, progress=None) -> Dict[str, torch.Tensor]:
-    """Check the folder against ``specs`` and copy every tensor to the device in its kept dtype."""
+                 device: torch.device, progress=None, keep_float32: bool = False) -> Dict[str, torch.Tensor]:
+    """Check the folder against ``specs`` and copy every tensor to the device in its kept dtype (an optional
+    tensor that the folder does not hold is left out).  A tensor goes up as it is stored and is converted on the
+    device."""
     checkpoint.check(specs)
     out: Dict[str, torch.Tensor] = {}
     for spec in specs:
-        if spec.unused:
+        if spec.name not in checkpoint.tensors:
             continue
         stored = checkpoint.read(spec.name)
-        dtype = kept_dtype(spec, stored.dtype, run_dtype)
+        dtype = kept_dtype(spec, stored.dtype, run_dtype, keep_float32)
         if not (stored.dtype.is_floating_point or spec.role == INT_TABLE):
             raise InvalidArgumentError(
                 f"tensor \"{spec.name}\" is stored as {stored.dtype}, expected a floating-point dtype"
             )
-        out[spec.name] = stored.to(device=device, dtype=dtype, copy=True).contiguous()
+        on_device = stored.to(device=device, copy=True)
+        out[spec.name] = (on_device if on_device.dtype == dtype else on_device.to(dtype)).contiguous()
         if progress is not None:
             progress(spec.name)
     return out

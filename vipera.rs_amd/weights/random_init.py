@@ -73,7 +73,7 @@ def random_tensor(spec: TensorSpec, seed: int, dtype: torch.dtype) -> torch.Tens
 
 def random_tensors(specs: Iterable[TensorSpec], seed: int, dtype: torch.dtype):
     for spec in specs:
-        if not spec.unused:
+        if not spec.optional:
             yield spec.name, random_tensor(spec, seed, dtype)
 
 
@@ -101,7 +101,7 @@ def random_device_tensors(specs: Sequence[TensorSpec], seed: int, run_dtype: tor
 
     out: Dict[str, torch.Tensor] = {}
     for spec in specs:
-        if spec.unused:
+        if spec.optional:
             continue
         dtype = kept_dtype(spec, run_dtype, run_dtype)
         tensor = torch.empty(spec.shape, dtype=dtype, device=device)
