@@ -24,6 +24,7 @@ SIGNATURES = {
     "plain_rope_kvwrite": [P, I, P, P, P, I, P, P, P, P, I, I, I, I, I, I, P],
     "plain_swiglu": [P, P, I, I, I, I, P],
     "plain_gemm_generic": [P, I, P, I, P, P, I, I, I, I, LL, LL, I, P],
+    "plain_gemm_stream": [P, P, P, P, I, I, I, I, LL, LL, I, P, LL, P],
     "plain_gemm_bf16": [P, P, P, P, I, I, I, I, LL, LL, I, I, I, P, LL, P],
     "plain_gemm_bf16_mid": [P, P, P, P, I, I, I, I, LL, LL, I, I, I, P, LL, P],
     "plain_gemm_bf16_gated": [P, P, P, I, I, I, LL, LL, I, P],
@@ -32,7 +33,8 @@ SIGNATURES = {
     "plain_gemm_bf16_qkv_rope": [P, P, P, P, I, I, I, LL, LL, P, P, P, P, P, P, I, I, I, I, I, P, I, F, P],
     "plain_gemm_bf16_mid_follow": [P, P, P, P, I, I, I, LL, LL, I, I, P, LL, P, P, LL, P, LL, I, P, P],
     "plain_gemm_bf16_mid_qkv_rope": [P, P, P, P, I, I, I, LL, LL, I, I, P, LL, P, P, P, P, P, P, I, I, I, I, I, P, I, I, F, P],
-    "plain_attn_generic": [P, LL, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, P],
+    "plain_attn_generic": [P, LL, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, P, P],
+    "plain_attn_decode_f32": [P, LL, P, P, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, P],
     "plain_attn_bf16_prefill": [P, LL, P, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, P],
     "plain_attn_bf16_decode": [P, LL, P, P, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, I, I, P],
     "plain_sample": [P, I, I, P, P, P, P, P, P, P, P, I, P, P, P, P, P, I, P],

@@ -197,6 +197,15 @@ extern "C" int plain_gemm_generic(const void* A, int a_dtype, const void* W, int
   return 0;
 }
 
+// the 32-bit weight stream for up to 64 tokens; the workspace shapes the kernel's work only
+extern "C" int plain_gemm_stream(const float* A, const float* W, const float* bias, void* C, int c_dtype, int M, int N,
+                                 int K, long long lda, long long ldc, int accumulate, float*, long long, void*) {
+  if (M <= 0 || N <= 0) return 0;
+  if (K <= 0 || M > 64 || !known(c_dtype) || lda < K || ldc < N || (accumulate && c_dtype != DT_F32)) return BAD_ARGUMENT;
+  product(A, DT_F32, W, DT_F32, bias, C, c_dtype, M, N, K, lda, ldc, accumulate != 0);
+  return 0;
+}
+
 extern "C" int plain_gemm_bf16(const void* A, const void* W, const float* bias, void* C, int c_dtype, int M, int N,
                                int K, long long lda, long long ldc, int accumulate, int, int, float*, long long,
                                void*) {
@@ -359,16 +368,36 @@ extern "C" int plain_gemm_bf16_gated_scaled(const void* A, const void* W, void* 
 extern "C" int plain_attn_generic(const void* q, long long q_stride, const void* k_cache, const void* v_cache,
                                   void* out, int dtype, const int* positions, const int* entry_of_token,
                                   const int* block_table, int table_width, int block_size, int num_tokens, int heads,
-                                  int kv_heads, int hd, float scale, int window, void*) {
+                                  int kv_heads, int hd, float scale, int window, const int* skip_single_of, void*) {
   if (num_tokens <= 0) return 0;
   if (!known(dtype) || hd <= 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads || block_size <= 0 || window < 0)
     return BAD_ARGUMENT;
   const size_t elem = dtype == DT_F32 ? 4 : 2;
-  for (int t = 0; t < num_tokens; ++t)
+  for (int t = 0; t < num_tokens; ++t) {
+    // skip_single_of: the step's entry_start; the token of an entry that holds one token is left alone
+    if (skip_single_of && skip_single_of[entry_of_token[t] + 1] - skip_single_of[entry_of_token[t]] == 1) continue;
     for (int h = 0; h < heads; ++h)
       attend((const char*)q + ((size_t)t * q_stride + (size_t)h * hd) * elem, k_cache, v_cache, dtype,
              block_table + (size_t)entry_of_token[t] * table_width, block_size, kv_heads, h / (heads / kv_heads), hd,
              scale, positions[t], window, (char*)out + ((size_t)t * heads * hd + (size_t)h * hd) * elem);
+  }
+  return 0;
+}
+
+// the 32-bit attention of single-token entries; `partial` and `chunks` shape the kernel's work only
+extern "C" int plain_attn_decode_f32(const float* q, long long q_stride, const float* k_cache, const float* v_cache,
+                                     float* out, float*, const int* entries, int num_entries, const int* entry_start,
+                                     const int* entry_first_pos, const int* block_table, int table_width,
+                                     int block_size, int heads, int kv_heads, int hd, float scale, int window, int,
+                                     void*) {
+  if (hd <= 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads || block_size <= 0 || window < 0) return BAD_ARGUMENT;
+  for (int e = 0; e < num_entries; ++e) {
+    const int entry = entries[e], t = entry_start[entry];
+    for (int h = 0; h < heads; ++h)
+      attend(q + (size_t)t * q_stride + (size_t)h * hd, k_cache, v_cache, DT_F32,
+             block_table + (size_t)entry * table_width, block_size, kv_heads, h / (heads / kv_heads), hd, scale,
+             entry_first_pos[entry], window, out + (size_t)t * heads * hd + (size_t)h * hd);
+  }
   return 0;
 }
 

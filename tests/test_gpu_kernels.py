@@ -182,16 +182,53 @@ def test_gemm_generic_against_float64(m, n, k, dtypes):
     assert _rel(out, want) < (2e-6 if dtypes[2] == torch.float32 else 6e-3)
 
 
-def test_gemm_generic_does_not_depend_on_the_batch():
+@pytest.mark.parametrize("k", [64, 200, 256, 1100, 2600])
+def test_gemm_generic_does_not_depend_on_the_batch(k):
+    """Every output element is summed in one fixed order (chains over ranges of 256 k, four ranges to a slab, slabs in
+    ascending order), whichever kernel computes it: the weight stream that takes up to 64 tokens gives bit for bit
+    the rows of the tiled kernel that takes 70, alone or in any company, with and without a bias, accumulating or not."""
     from vipera_rs_amd.ops import kernels
-    g = torch.Generator().manual_seed(2)
-    a = torch.randn(70, 136, generator=g).to(DEV)
-    w = torch.randn(90, 136, generator=g).to(DEV)
+    g = torch.Generator().manual_seed(k)
+    a = torch.randn(70, k, generator=g).to(DEV)
+    w = torch.randn(90, k, generator=g).to(DEV)
+    bias = torch.randn(90, generator=g).to(DEV)
+    base = torch.randn(70, 90, generator=g).to(DEV)
     whole = torch.empty(70, 90, device=DEV)
     kernels.gemm_generic(a, w, None, whole)
-    single = torch.empty(1, 90, device=DEV)
-    kernels.gemm_generic(a[37:38].contiguous(), w, None, single)
-    assert torch.equal(single[0], whole[37])  # bit for bit: one thread sums each element in k order
+    assert _rel(whole, a.double() @ w.double().T) < 2e-6
+    for rows in ([37], [0, 1], list(range(5, 12)), list(range(3, 36)), list(range(6, 70))):
+        part = torch.empty(len(rows), 90, device=DEV)
+        kernels.gemm_generic(a[rows].contiguous(), w, None, part)
+        assert torch.equal(part, whole[rows]), f"{len(rows)} rows"      # bit for bit
+    with_bias = torch.empty(70, 90, device=DEV)
+    kernels.gemm_generic(a, w, bias, with_bias)
+    added = base.clone()
+    kernels.gemm_generic(a, w, bias, added, accumulate=True)
+    few = base[20:28].clone()
+    kernels.gemm_generic(a[20:28], w, bias, few, accumulate=True)        # a view with a row stride of its own
+    assert torch.equal(few, added[20:28])
+    rounded = torch.empty(8, 90, dtype=torch.bfloat16, device=DEV)
+    kernels.gemm_generic(a[20:28], w, bias, rounded)
+    assert torch.equal(rounded, with_bias[20:28].to(torch.bfloat16))
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 64, 4), (3, 70, 36), (8, 3584, 1536), (9, 129, 1028), (16, 1000, 4096), (40, 200, 520),
+                                   (64, 333, 2052)])
+def test_gemm_stream_against_float64(m, n, k):
+    """The 32-bit weight stream at sizes of its own: K that ends inside a chunk of 32, a range and a slab, rows of
+    W that do not fill a workgroup's 64, every count of tokens' class."""
+    from vipera_rs_amd.ops import kernels
+    g = torch.Generator().manual_seed(m * n + k)
+    a = torch.randn(m, k, generator=g).to(DEV)
+    w = torch.randn(n, k, generator=g).to(DEV)
+    bias = torch.randn(n, generator=g).to(DEV)
+    out = torch.full((m, n), float("nan"), device=DEV)
+    kernels.gemm_generic(a, w, bias, out)
+    assert _rel(out, a.double() @ w.double().T + bias.double()) < 2e-6
+    wide = torch.zeros(m, n + 8, device=DEV)                               # an output with a row stride of its own
+    kernels.gemm_generic(a, w, None, wide[:, 4:n + 4])
+    assert _rel(wide[:, 4:n + 4], a.double() @ w.double().T) < 2e-6
+    assert float(wide[:, :4].abs().max()) == 0.0 and float(wide[:, n + 4:].abs().max()) == 0.0
 
 
 # --- attention -------------------------------------------------------------------------------------
@@ -300,6 +337,21 @@ def test_attention_kernels_against_plain_softmax(case, dtype, stale):
     out = torch.zeros(T, heads * hd, dtype=dtype, device=DEV)
     kernels.attn_generic(qkv_d, k_d, v_d, out, dev(positions), dev(entry_of), table_d, heads, kv_heads, hd, scale, window)
     assert _rel(out.cpu(), want) < tol, "32-bit-arithmetic kernel"
+
+    if dtype == torch.float32 and kernels.attn_decode_f32_supported(qkv_d, k_d, hd):
+        # single tokens on the 32-bit kernel that splits their positions, the portions on the general one
+        singles = [e for e, n in enumerate(counts) if n == 1]
+        es = dev(torch.tensor(starts, dtype=torch.int32))
+        fp = dev(torch.tensor(first, dtype=torch.int32))
+        out3 = torch.zeros(T, heads * hd, dtype=dtype, device=DEV)
+        if singles:
+            chunks = (max(entries[e][0] for e in singles) + 255) // 256 + 1      # a chunk that sees nothing, too
+            partial = torch.full((len(singles) * heads * chunks * (hd + 2),), float("nan"), device=DEV)
+            kernels.attn_decode_f32(qkv_d, k_d, v_d, out3, partial, dev(torch.tensor(singles, dtype=torch.int32)), es, fp,
+                                    table_d, heads, kv_heads, hd, scale, window, chunks)
+        kernels.attn_generic(qkv_d, k_d, v_d, out3, dev(positions), dev(entry_of), table_d, heads, kv_heads, hd, scale, window,
+                             skip_single_of=es)
+        assert _rel(out3.cpu(), want) < tol, "32-bit decode kernel beside the general one"
 
     if dtype == torch.bfloat16:
         from vipera_rs_amd.engine.batch import TILE_TOKENS

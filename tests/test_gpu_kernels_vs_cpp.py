@@ -238,6 +238,11 @@ def test_products_beside_their_twins(m, n, k):
     a, w, bias = torch.randn(m, k, generator=g), torch.randn(n, k, generator=g), torch.randn(n, generator=g)
     (got, want), = both("gemm_generic", "gemm_generic", [a, 0, w, 0, bias, torch.empty(m, n), 0, m, n, k, k, n, 0, None], [5])
     assert rel_err(got.numpy(), want.double().numpy()) < 2e-6
+    if m <= 64 and k % 4 == 0:
+        slabs = torch.empty(((k + 1023) // 1024) * m * n)
+        (got, want), = both("gemm_generic", "gemm_stream", [a, w, bias, torch.randn(m, n, generator=g), 0, m, n, k, k, n, 1, slabs,
+                                                            slabs.numel(), None], [3])
+        assert rel_err(got.numpy(), want.double().numpy()) < 2e-6
     ab, wb = a.to(torch.bfloat16), w.to(torch.bfloat16)
     for out_dtype, tol in ((torch.float32, 1e-5), (torch.bfloat16, 6e-3)):
         (got, want), = both("gemm_bf16", "gemm_bf16", [ab, wb, bias, torch.empty(m, n, dtype=out_dtype), DT[out_dtype], m, n, k, k,
@@ -285,8 +290,39 @@ def test_generic_attention_beside_its_twin(dtype, window):
     positions = i32([0, 1, 7, 8, 36, 37, 38, 255, 300])
     (got, want), = both("attn_generic", "attn_generic",
                         [qkv, qkv.shape[1], k, v, torch.empty(9, heads * hd, dtype=dtype), DT[dtype], positions, i32([0] * 9), table,
-                         table.shape[1], bs, 9, heads, kv_heads, hd, 1 / math.sqrt(hd), window, None], [4])
+                         table.shape[1], bs, 9, heads, kv_heads, hd, 1 / math.sqrt(hd), window, None, None], [4])
     assert rel_err(got.float().numpy(), want.double().numpy()) < (3e-6 if dtype == torch.float32 else 8e-3)
+
+
+@pytest.mark.parametrize("heads,kv_heads,hd,bs", [(6, 3, 48, 8), (7, 1, 128, 16), (12, 1, 64, 4), (5, 5, 256, 32)])
+@pytest.mark.parametrize("window", [0, 37])
+def test_32_bit_decode_attention_beside_its_twin(heads, kv_heads, hd, bs, window):
+    """Single-token entries at positions around the edges of a wave's 64 and a chunk's 256 positions, beside a portion
+    of a prompt that the general kernel takes in the same step (and leaves the single tokens alone)."""
+    lengths = [1, 2, 64, 65, 256, 257, 300, 777]
+    T = max(lengths)
+    k, v, table = _paged(T, kv_heads, hd, bs, torch.float32, hd + heads, entries=len(lengths) + 1)
+    g = torch.Generator().manual_seed(hd)
+    portion = 5                                      # the last entry: tokens 100..104 of a prompt
+    tokens = len(lengths) + portion
+    qkv = torch.randn(tokens, (heads + 2 * kv_heads) * hd, generator=g)
+    entry_start = i32(list(range(len(lengths) + 1)) + [tokens])
+    first_pos = i32([n - 1 for n in lengths] + [100])
+    chunks = (T + 255) // 256
+    partial = torch.full((len(lengths) * heads * chunks * (hd + 2),), float("nan"))
+    out = torch.zeros(tokens, heads * hd)
+    (got, want), = both("attn_generic", "attn_decode_f32",
+                        [qkv, qkv.shape[1], k, v, out, partial, i32(list(range(len(lengths)))), len(lengths), entry_start,
+                         first_pos, table, table.shape[1], bs, heads, kv_heads, hd, 1 / math.sqrt(hd), window, chunks, None], [4])
+    assert rel_err(got[:len(lengths)].numpy(), want[:len(lengths)].double().numpy()) < 3e-6
+    assert float(got[len(lengths):].abs().max()) == 0.0          # the portion's rows are not this kernel's
+    positions = i32([n - 1 for n in lengths] + list(range(100, 100 + portion)))
+    entry_of = i32(list(range(len(lengths))) + [len(lengths)] * portion)
+    (got, want), = both("attn_generic", "attn_generic",
+                        [qkv, qkv.shape[1], k, v, torch.zeros(tokens, heads * hd), 0, positions, entry_of, table, table.shape[1], bs,
+                         tokens, heads, kv_heads, hd, 1 / math.sqrt(hd), window, entry_start, None], [4])
+    assert rel_err(got[len(lengths):].numpy(), want[len(lengths):].double().numpy()) < 3e-6
+    assert float(got[:len(lengths)].abs().max()) == 0.0          # and the single tokens not the general kernel's
 
 
 @pytest.mark.parametrize("hd", [64, 128, 80])

@@ -138,7 +138,7 @@ def test_attention_twins_over_a_shuffled_table(window):
     out = torch.empty(T, heads * hd)
     positions, entry = torch.arange(T, dtype=torch.int32), torch.zeros(T, dtype=torch.int32)
     call("plain_attn_generic", qkv, qkv.shape[1], k_cache, v_cache, out, 0, positions, entry, table, table.shape[1], bs, T,
-         heads, kv_heads, hd, 1 / math.sqrt(hd), window, None)
+         heads, kv_heads, hd, 1 / math.sqrt(hd), window, None, None)
     assert rel_err(out.numpy(), want) < 1e-6
     # the bfloat16 entry points: a prompt cut into a portion of 13 tokens and six single tokens
     qb, kb, vb = qkv.to(torch.bfloat16), k_cache.to(torch.bfloat16), v_cache.to(torch.bfloat16)
@@ -216,7 +216,7 @@ def _forward_through_twins(cfg, w, tokens, bs=8):
              kv_heads, hd, None)
         attn = torch.empty(T, heads * hd)
         call("plain_attn_generic", qkv, width, k_cache, v_cache, attn, 0, positions, entry, table, pages, bs, T, heads,
-             kv_heads, hd, 1.0 / math.sqrt(hd), P.layer_window(cfg, i), None)
+             kv_heads, hd, 1.0 / math.sqrt(hd), P.layer_window(cfg, i), None, None)
         call("plain_gemm_generic", attn, 0, f(p + "self_attn.o_proj.weight"), 0, None, x, 0, T, H, heads * hd, heads * hd, H, 1,
              None)
         call("plain_rmsnorm", x, f(p + "post_attention_layernorm.weight"), None, h, 0, T, H, float(cfg["rms_norm_eps"]), None)

@@ -235,9 +235,17 @@ def gemm_generic(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor],
         _need(bias.dtype == torch.float32 and bias.numel() == n and bias.is_contiguous(), "gemm: bias must be float32 [n]")
     if accumulate:
         _need(out.dtype == torch.float32, "gemm: accumulation needs a float32 output")
-    fn = _fn("gemm_generic", "vk_gemm_generic", [_p, _i, _p, _i, _p, _p, _i, _i, _i, _i, _ll, _ll, _i, _p])
     lda = a.stride(0) if m > 1 else max(a.stride(0), k)
     ldc = out.stride(0) if m > 1 else max(out.stride(0), n)
+    if (m <= 64 and a.dtype == torch.float32 and w.dtype == torch.float32 and k >= 4 and k % 4 == 0 and lda % 4 == 0
+            and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0 and k < 65535 * 1024):
+        # up to 64 tokens in 32-bit: a stream of the weights (the same sums in the same order as the tiled kernel)
+        slabs = _split_k_workspace(a.device, ((k + 1023) // 1024) * m * n, "stream")
+        fn = _fn("gemm_generic", "vk_gemm_stream", [_p, _p, _p, _p, _i, _i, _i, _i, _ll, _ll, _i, _p, _ll, _p])
+        _status(fn(_ptr(a), _ptr(w), _ptr(bias), _ptr(out), _dt(out, "out"), m, n, k, lda, ldc, 1 if accumulate else 0,
+                   _ptr(slabs), slabs.numel(), _stream()), "gemm_stream")
+        return
+    fn = _fn("gemm_generic", "vk_gemm_generic", [_p, _i, _p, _i, _p, _p, _i, _i, _i, _i, _ll, _ll, _i, _p])
     _status(fn(_ptr(a), _dt(a, "a"), _ptr(w), _dt(w, "w"), _ptr(bias), _ptr(out), _dt(out, "out"), m, n, k, lda, ldc,
                1 if accumulate else 0, _stream()), "gemm_generic")
 
@@ -245,13 +253,18 @@ def gemm_generic(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor],
 # ----------------------------------------------------------------------------------------------
 def attn_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
                  positions: torch.Tensor, entry_of_token: torch.Tensor, block_table: torch.Tensor,
-                 heads: int, kv_heads: int, head_dim: int, scale: float, window: int) -> None:
+                 heads: int, kv_heads: int, head_dim: int, scale: float, window: int,
+                 skip_single_of: Optional[torch.Tensor] = None) -> None:
     """Causal GQA over the paged cache for every token of the step, in 32-bit arithmetic.
 
     ``q``: a view ``[tokens, >= heads * head_dim]`` whose row holds the query heads first (the fused
-    qkv buffer qualifies); ``out``: ``[tokens, heads * head_dim]``.
+    qkv buffer qualifies); ``out``: ``[tokens, heads * head_dim]``.  ``skip_single_of``: the step's
+    ``entry_start``; tokens of entries that hold one token are then left alone (for :func:`attn_decode_f32`).
     """
-    _dev(q, k_cache, v_cache, out, positions, entry_of_token, block_table)
+    _dev(q, k_cache, v_cache, out, positions, entry_of_token, block_table, skip_single_of)
+    if skip_single_of is not None:
+        _need(skip_single_of.dtype == torch.int32 and skip_single_of.numel() == block_table.shape[0] + 1,
+              "attention: entry_start must hold one offset per entry and the end")
     num_tokens = out.shape[0]
     _need(q.dim() == 2 and q.shape[0] == num_tokens and q.stride(1) == 1 and q.shape[1] >= heads * head_dim, "attention: q")
     _need(out.shape == (num_tokens, heads * head_dim) and out.is_contiguous() and out.dtype == q.dtype, "attention: out")
@@ -263,10 +276,49 @@ def attn_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, 
     if head_dim > ATTENTION_MAX_HEAD_DIM:
         raise UnsupportedError(f"attention: head_dim {head_dim} is above the kernels' limit of {ATTENTION_MAX_HEAD_DIM}")
     fn = _fn("attn_generic", "vk_attn_generic",
-             [_p, _ll, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _i, _p])
+             [_p, _ll, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _i, _p, _p])
     _status(fn(_ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(out), _dt(q, "q"), _ptr(positions),
                _ptr(entry_of_token), _ptr(block_table), block_table.shape[1], k_cache.shape[2], num_tokens, heads,
-               kv_heads, head_dim, float(scale), int(window), _stream()), "attn_generic")
+               kv_heads, head_dim, float(scale), int(window), _ptr(skip_single_of), _stream()), "attn_generic")
+
+
+ATTN_DECODE_F32_CHUNK = 256   # positions of one workgroup of attn_decode_f32 (the kernel's DEC_CHUNK)
+
+
+def attn_decode_f32_supported(q: torch.Tensor, k_cache: torch.Tensor, head_dim: int) -> bool:
+    """Whether :func:`attn_decode_f32` takes the operands: all 32-bit, a head width and pages that are multiples
+    of 4, 16-byte rows."""
+    return (q.dtype == torch.float32 and k_cache.dtype == torch.float32 and head_dim % 4 == 0
+            and head_dim <= ATTENTION_MAX_HEAD_DIM and k_cache.shape[2] % 4 == 0 and q.stride(0) % 4 == 0
+            and q.data_ptr() % 16 == 0)
+
+
+def attn_decode_f32(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
+                    partial: torch.Tensor, entries: torch.Tensor, entry_start: torch.Tensor,
+                    entry_first_pos: torch.Tensor, block_table: torch.Tensor, heads: int, kv_heads: int,
+                    head_dim: int, scale: float, window: int, chunks: int) -> None:
+    """32-bit attention of the single-token entries listed in ``entries``; their positions are split into
+    ``chunks`` of :data:`ATTN_DECODE_F32_CHUNK`, which must cover the longest visible range."""
+    _dev(q, k_cache, v_cache, out, partial, entries, entry_start, entry_first_pos, block_table)
+    _need(attn_decode_f32_supported(q, k_cache, head_dim), "attn_decode_f32: 32-bit operands, head width and pages "
+          "that are multiples of 4")
+    _need(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= heads * head_dim, "attention: q")
+    _need(out.shape == (q.shape[0], heads * head_dim) and out.is_contiguous() and out.dtype == q.dtype, "attention: out")
+    _need(_cache_ok(k_cache, v_cache, kv_heads, head_dim, q.dtype), "attention: cache shape or dtype")
+    count = entries.numel()
+    _need(entries.dtype == torch.int32 and entries.is_contiguous(), "attention: entries")
+    _need(partial.dtype == torch.float32 and partial.is_contiguous()
+          and partial.numel() >= count * heads * chunks * (head_dim + 2), "attention: workspace too small")
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(), "attention: table")
+    _need(entry_start.dtype == torch.int32 and entry_first_pos.dtype == torch.int32
+          and entry_start.numel() == block_table.shape[0] + 1 and entry_first_pos.numel() == block_table.shape[0],
+          "attention: entry arrays")
+    _need(heads % kv_heads == 0 and chunks >= 1, "attention: heads must be a multiple of kv_heads")
+    fn = _fn("attn_generic", "vk_attn_decode_f32",
+             [_p, _ll, _p, _p, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _f, _i, _i, _p])
+    _status(fn(_ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(partial), _ptr(entries), count,
+               _ptr(entry_start), _ptr(entry_first_pos), _ptr(block_table), block_table.shape[1], k_cache.shape[2],
+               heads, kv_heads, head_dim, float(scale), int(window), int(chunks), _stream()), "attn_decode_f32")
 
 
 # ----------------------------------------------------------------------------------------------
