@@ -12,7 +12,9 @@ def test_few_tokens_stream_the_weights_with_k_split_inside_a_workgroup():
     for n, k in (QKV_7B, O_7B, DOWN_7B, HEAD_7B):
         assert streams_in_wave_order(1, n, k) and streams_in_wave_order(4, n, k)
     assert streams_in_wave_order(16, *QKV_7B) and streams_in_wave_order(16, *O_7B)
-    assert not streams_in_wave_order(8, *DOWN_7B)          # a long K: activations are shared through LDS instead
+    assert streams_in_wave_order(8, *DOWN_7B)              # up to 8 tokens also with a long K: no second kernel for K ranges
+    assert streams_in_wave_order(8, 1536, 8960)
+    assert not streams_in_wave_order(9, *DOWN_7B)          # past 8 tokens activations are shared through LDS instead
     assert not streams_in_wave_order(8, *HEAD_7B)          # many rows: likewise
     assert not streams_in_wave_order(17, *QKV_7B)
 
@@ -44,13 +46,14 @@ def test_the_gated_product_goes_resident_tiled_or_lds_shared():
     assert not gated_resident_fits(8, 37888, 3584 + 64)    # K in whole chunks of 256 only
     for m in (1, 8, 16):
         assert gated_plan(m, *GATE_UP_7B) == 0             # 1184 pairs over 256 CUs: 4 or 5 each
-    assert gated_plan(8, 17920, 1536) in (1, 2)            # 1.5B: 560 pairs would be 2 or 3 each, too uneven
+    assert gated_plan(8, 17920, 1536) == 0                 # 1.5B: 560 pairs are 2 or 3 each; as fast, and the norm before it is free
     assert gated_plan(8, 55296, 5120) == 0
     assert gated_plan(17, *GATE_UP_7B) == 3 and gated_plan(64, *GATE_UP_7B) == 3   # past the resident kernel: tiled
     assert gated_plan(24, 55296, 5120) == 3
     assert gated_plan(48, 17920, 1536) in (1, 2) and gated_plan(64, 17920, 1536) == 3
     assert gated_plan(8, *GATE_UP_7B, cus=304) == 0        # 1184 pairs over 304 CUs: 3 or 4 each, 3 % above the mean
-    assert gated_plan(8, *GATE_UP_7B, cus=500) != 0        # over 500: 2 or 3 each, 27 % above the mean
+    assert gated_plan(8, *GATE_UP_7B, cus=500) == 0        # over 500: 2 or 3 each, 27 % above the mean
+    assert gated_plan(8, 4096, 1024, cus=256) != 0         # 128 pairs over 256 CUs: half of them would have none
 
 
 def test_q_k_v_of_17_to_64_tokens_rotates_in_the_kernel_that_adds_its_ranges():

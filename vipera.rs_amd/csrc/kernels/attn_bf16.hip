@@ -833,95 +833,77 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void at
   }
 }
 
-// Merge the chunks of one (entry, head): M = max m_c; out = sum_c acc_c e^(m_c - M) / sum_c l_c e^(m_c - M),
-// chunks in ascending order (layer.cu:443-467). One wave per (entry, head): the chunk weights are worked
-// out in parallel over the chunks (their sum by a fixed tree), then every lane owns output dims.
+// Merge the chunks of one (entry, head): M = max m_c; out = sum_c acc_c e^(m_c - M) / sum_c l_c e^(m_c - M)
+// (layer.cu:443-467). One workgroup of four waves per (entry, head). The kernel is a few memory round trips long
+// and nothing else, so everything it reads is requested at its start, before anything is computed: the token's
+// row, the chunks' (max, sum), and of the weighted sums the first four chunks of every thread, which with up to
+// 4 * parts chunks is all of them. Thread -> (part, four output dims); part p sums the chunks p, p + parts, ...
+// in ascending order, and the parts are added in ascending order: one fixed order for a given head width and
+// number of chunks.
 constexpr int MAX_CHUNKS = 128;
-__global__ __launch_bounds__(64) void attn_combine_kernel(const float* __restrict__ partial, __bf16* __restrict__ out,
-                                                          const int* __restrict__ entries,
-                                                          const int* __restrict__ entry_start, int heads, int hd,
-                                                          int chunks) {
+constexpr int CB_THREADS = 256;
+__global__ __launch_bounds__(CB_THREADS) void attn_combine_kernel(const float* __restrict__ partial,
+                                                                  __bf16* __restrict__ out,
+                                                                  const int* __restrict__ entries,
+                                                                  const int* __restrict__ entry_start, int heads, int hd,
+                                                                  int chunks) {
   __shared__ float weight[MAX_CHUNKS];
-  __shared__ f32x4 part_sum[64];
-  const int slot = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  __shared__ float wave_best[4], wave_total[4];
+  __shared__ f32x4 part_sum[CB_THREADS];
+  const int slot = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const size_t stride = hd + 2;
   const float* src = partial + ((size_t)slot * heads + h) * chunks * stride;
-  // lane -> (part, four output dims); part p sums the chunks c = p, p + parts, ... ; parts are added in order
-  const int quads = hd / 4;                         // hd is a multiple of 8
-  const int parts = quads >= 64 ? 1 : 64 / quads;
-  // Everything this wave reads is requested before anything is computed: the token's row, the chunks' (max, sum)
-  // and the first four chunks of each lane's sums. With a few chunks that is all of them, and the kernel is one
-  // round trip to memory instead of one per chunk behind the weights.
+  const int quads = hd / 4;                               // hd is a multiple of 8 and at most 256
+  const int parts = CB_THREADS / quads;                   // at least 4
+  const int quad = tid % quads, part = tid / quads;
+  const bool active = part < parts;
   constexpr int AHEAD = 4;
   const int token = entry_start[entries[slot]];
-  const int quad0 = parts > 1 ? lane % quads : lane, part0 = parts > 1 ? lane / quads : 0;
-  const bool active0 = quad0 < quads && part0 < parts;
   f32x4 ahead[AHEAD];
 #pragma unroll
   for (int u = 0; u < AHEAD; ++u) {
-    const int c = min(part0 + u * parts, chunks - 1);   // a clamped chunk's value is not used
-    ahead[u] = *(const f32x4*)(src + (size_t)c * stride + min(quad0, quads - 1) * 4);
+    const int c = min(part + u * parts, chunks - 1);      // a clamped chunk's value is not used
+    ahead[u] = *(const f32x4*)(src + (size_t)c * stride + quad * 4);
   }
-  float mc[MAX_CHUNKS / 64], lc[MAX_CHUNKS / 64];
-  float best = -INFINITY;
-#pragma unroll
-  for (int i = 0; i < MAX_CHUNKS / 64; ++i) {
-    const int c = lane + 64 * i;
-    mc[i] = c < chunks ? src[(size_t)c * stride + hd] : -INFINITY;
-    lc[i] = c < chunks ? src[(size_t)c * stride + hd + 1] : 0.f;
-    best = fmaxf(best, mc[i]);
-  }
-  best = wave_max(best);
-  float total = 0.f;
-#pragma unroll
-  for (int i = 0; i < MAX_CHUNKS / 64; ++i) {
-    const float w = mc[i] > -INFINITY ? __expf(mc[i] - best) : 0.f;
-    const int c = lane + 64 * i;
-    if (c < chunks) weight[c] = w;
-    total += w * lc[i];
-  }
-  total = wave_sum(total);
+  // chunk tid's (max, sum): MAX_CHUNKS <= CB_THREADS
+  const float mc = tid < chunks ? src[(size_t)tid * stride + hd] : -INFINITY;
+  const float lc = tid < chunks ? src[(size_t)tid * stride + hd + 1] : 0.f;
+  float best = wave_max(mc);
+  if (lane == 0) wave_best[wave] = best;
   __syncthreads();
-  const float inv = 1.f / total;
-  __bf16* dst = out + (size_t)token * heads * hd + (size_t)h * hd;
-  for (int q0 = 0; q0 < quads; q0 += 64) {
-    const int quad = q0 + quad0;
-    const int part = part0;
-    const bool active = quad < quads && part < parts;
-    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-    if (active) {
-      int c = part;
-      if (q0 == 0 && active0) {   // the chunks requested ahead
+  best = fmaxf(fmaxf(wave_best[0], wave_best[1]), fmaxf(wave_best[2], wave_best[3]));
+  const float w = mc > -INFINITY ? __expf(mc - best) : 0.f;
+  if (tid < chunks) weight[tid] = w;
+  const float mine = wave_sum(w * lc);
+  if (lane == 0) wave_total[wave] = mine;
+  __syncthreads();
+  const float inv = 1.f / (((wave_total[0] + wave_total[1]) + wave_total[2]) + wave_total[3]);
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  if (active) {
+    int c = part;
 #pragma unroll
-        for (int u = 0; u < AHEAD; ++u, c += parts) {
-          if (c >= chunks) break;
-          const float w = weight[c];
+    for (int u = 0; u < AHEAD; ++u, c += parts) {
+      if (c >= chunks) break;
+      const float wc = weight[c];
 #pragma unroll
-          for (int j = 0; j < 4; ++j) acc[j] += w != 0.f ? ahead[u][j] * w : 0.f;   // an empty chunk holds stale numbers
-        }
-      }
-      for (; c < chunks; c += parts) {
-        const float w = weight[c];
-        const f32x4 v = *(const f32x4*)(src + (size_t)c * stride + quad * 4);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) acc[j] += w != 0.f ? v[j] * w : 0.f;
-      }
+      for (int j = 0; j < 4; ++j) acc[j] += wc != 0.f ? ahead[u][j] * wc : 0.f;   // an empty chunk holds stale numbers
     }
-    if (parts > 1) {
-      __syncthreads();
-      part_sum[lane] = acc;
-      __syncthreads();
-      if (part == 0 && active) {
-        acc = part_sum[quad];
-        for (int p = 1; p < parts; ++p) acc += part_sum[p * quads + quad];
-      }
-    }
-    if (part == 0 && active) {
-      bf16x4 r;
+    for (; c < chunks; c += parts) {
+      const float wc = weight[c];
+      const f32x4 v = *(const f32x4*)(src + (size_t)c * stride + quad * 4);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) r[j] = (__bf16)(acc[j] * inv);
-      *(bf16x4*)(dst + quad * 4) = r;
+      for (int j = 0; j < 4; ++j) acc[j] += wc != 0.f ? v[j] * wc : 0.f;
     }
+  }
+  part_sum[tid] = acc;
+  __syncthreads();
+  if (tid < quads) {
+    acc = part_sum[tid];
+    for (int p = 1; p < parts; ++p) acc += part_sum[p * quads + tid];
+    bf16x4 r;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) r[j] = (__bf16)(acc[j] * inv);
+    *(bf16x4*)(out + (size_t)token * heads * hd + (size_t)h * hd + tid * 4) = r;
   }
 }
 }  // namespace
@@ -1014,7 +996,7 @@ extern "C" int vk_attn_bf16_decode(const void* q, long long q_stride, const void
                              kv_heads, hd, scale, window, chunk, head_blocks, dense);
   VK_LAUNCH_CHECK();
   dim3 cgrid(num_entries, heads);
-  attn_combine_kernel<<<cgrid, 64, 0, s>>>(partial, (__bf16*)out, entries, entry_start, heads, hd, chunks);
+  attn_combine_kernel<<<cgrid, CB_THREADS, 0, s>>>(partial, (__bf16*)out, entries, entry_start, heads, hd, chunks);
   VK_LAUNCH_CHECK();
   return 0;
 }

@@ -1331,11 +1331,19 @@ __global__ void gemm_reduce_kernel(const float* __restrict__ partial, const floa
   const int m = (int)(idx / quads), n = (int)(idx % quads) * 4;
   f32x4 sum = {0.f, 0.f, 0.f, 0.f};
   const bool whole = n + 3 < N && (N & 3) == 0;
-  for (int r = 0; r < ranges; ++r) {
-    const float* src = partial + ((size_t)r * M + m) * N + n;
-    if (whole) {
-      sum += *(const f32x4*)src;
-    } else {
+  if (whole) {
+    // the first eight ranges are requested together (a clamped range is not added), the others one by one
+    constexpr int AHEAD = 8;
+    f32x4 ahead[AHEAD];
+#pragma unroll
+    for (int r = 0; r < AHEAD; ++r) ahead[r] = *(const f32x4*)(partial + ((size_t)min(r, ranges - 1) * M + m) * N + n);
+#pragma unroll
+    for (int r = 0; r < AHEAD; ++r)
+      if (r < ranges) sum += ahead[r];
+    for (int r = AHEAD; r < ranges; ++r) sum += *(const f32x4*)(partial + ((size_t)r * M + m) * N + n);
+  } else {
+    for (int r = 0; r < ranges; ++r) {
+      const float* src = partial + ((size_t)r * M + m) * N + n;
 #pragma unroll
       for (int j = 0; j < 4; ++j)
         if (n + j < N) sum[j] += src[j];
@@ -1357,25 +1365,50 @@ __global__ __launch_bounds__(256) void gemm_reduce_follow_kernel(const float* __
   if (n < N) {
     f32x4 sum = {0.f, 0.f, 0.f, 0.f};
     const bool whole = n + 3 < N && vector_ok;
-    for (int r = 0; r < ranges; ++r) {
-      const float* src = partial + ((size_t)r * M + m) * N + n;
-      if (whole) {
-        sum += *(const f32x4*)src;
-      } else {
+    if (whole) {
+      // Everything the thread reads is requested before anything is added: the first eight ranges' sums, the old
+      // residual, the gain and the bias. The kernel is a few memory round trips long and little else, and a
+      // load that waits behind an addition is one more of them.
+      constexpr int AHEAD = 8;
+      f32x4 ahead[AHEAD];
+#pragma unroll
+      for (int r = 0; r < AHEAD; ++r)
+        ahead[r] = *(const f32x4*)(partial + ((size_t)min(r, ranges - 1) * M + m) * N + n);   // a clamped range is not added
+      float* at = C + (size_t)m * ldc + n;
+      const f32x4 old = *(const f32x4*)at;
+      const f32x4 gain = *(const f32x4*)(follow.gain + n);
+      const f32x4 b = bias ? *(const f32x4*)(bias + n) : f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int r = 0; r < AHEAD; ++r)
+        if (r < ranges) sum += ahead[r];
+      for (int r = AHEAD; r < ranges; ++r) sum += *(const f32x4*)(partial + ((size_t)r * M + m) * N + n);
+      f32x4 x;
+      bf16x4 scaled;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        x[j] = sum[j] + b[j] + old[j];
+        scaled[j] = (__bf16)(x[j] * gain[j]);
+        squares += x[j] * x[j];
+      }
+      *(f32x4*)at = x;
+      *(bf16x4*)(follow.scaled + (size_t)m * follow.ld_scaled + n) = scaled;
+    } else {
+      for (int r = 0; r < ranges; ++r) {
+        const float* src = partial + ((size_t)r * M + m) * N + n;
 #pragma unroll
         for (int j = 0; j < 4; ++j)
           if (n + j < N) sum[j] += src[j];
       }
-    }
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-      if (n + j < N) {
-        float* at = C + (size_t)m * ldc + n + j;
-        const float x = sum[j] + (bias ? bias[n + j] : 0.f) + *at;
-        *at = x;
-        follow.scaled[(size_t)m * follow.ld_scaled + n + j] = (__bf16)(x * follow.gain[n + j]);
-        squares += x * x;
-      }
+      for (int j = 0; j < 4; ++j)
+        if (n + j < N) {
+          float* at = C + (size_t)m * ldc + n + j;
+          const float x = sum[j] + (bias ? bias[n + j] : 0.f) + *at;
+          *at = x;
+          follow.scaled[(size_t)m * follow.ld_scaled + n + j] = (__bf16)(x * follow.gain[n + j]);
+          squares += x * x;
+        }
+    }
   }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) squares += __shfl_xor(squares, off);
@@ -1408,10 +1441,29 @@ __global__ __launch_bounds__(256) void gemm_reduce_rope_kernel(const float* __re
   const int d0 = rotated ? (u % quads) * 4 : ((u - rotated_units) % (hd / 4)) * 4;
   const int lo_col = head * hd + d0, hi_col = lo_col + half;
   f32x4 lo = {0.f, 0.f, 0.f, 0.f}, hi = {0.f, 0.f, 0.f, 0.f};
-  for (int range = 0; range < ranges; ++range) {
-    const float* src = partial + ((size_t)range * M + m) * N;
-    lo += *(const f32x4*)(src + lo_col);
-    if (rotated) hi += *(const f32x4*)(src + hi_col);
+  {
+    // the first four ranges of both halves are requested together (a clamped range is not added; a v head reads
+    // its own columns twice), the others one by one
+    constexpr int AHEAD = 4;
+    f32x4 ahead_lo[AHEAD], ahead_hi[AHEAD];
+    const int hi_at = rotated ? hi_col : lo_col;
+#pragma unroll
+    for (int range = 0; range < AHEAD; ++range) {
+      const float* src = partial + ((size_t)min(range, ranges - 1) * M + m) * N;
+      ahead_lo[range] = *(const f32x4*)(src + lo_col);
+      ahead_hi[range] = *(const f32x4*)(src + hi_at);
+    }
+#pragma unroll
+    for (int range = 0; range < AHEAD; ++range)
+      if (range < ranges) {
+        lo += ahead_lo[range];
+        hi += ahead_hi[range];
+      }
+    for (int range = AHEAD; range < ranges; ++range) {
+      const float* src = partial + ((size_t)range * M + m) * N;
+      lo += *(const f32x4*)(src + lo_col);
+      hi += *(const f32x4*)(src + hi_at);
+    }
   }
   if (r.sumsq) {
     float squares = 0.f;

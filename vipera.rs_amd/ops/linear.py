@@ -49,8 +49,11 @@ def mid_plan(m: int, n: int, k: int) -> Tuple[int, int]:
 
 
 def streams_in_wave_order(m: int, n: int, k: int) -> bool:
-    """Whether a bfloat16 product of ``m`` tokens runs on the kernel whose waves split K inside a workgroup."""
-    return m <= 4 or (m <= 16 and n < 16_384 and k < 8_192)
+    """Whether a bfloat16 product of ``m`` tokens runs on the kernel whose waves split K inside a workgroup: up to 4
+    tokens always; up to 8 where the weight has few rows, also with a long K (every workgroup reads all activations,
+    but there is no second kernel that adds K ranges: the down projection at 8 tokens 30.2 against 28.2 + 4.9 us at
+    the 7B widths, 12.1 against 11.1 + 6.2 at the 1.5B widths); up to 16 with a short K as well."""
+    return m <= 4 or (m <= 8 and n < 16_384) or (m <= 16 and n < 16_384 and k < 8_192)
 
 
 def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
@@ -130,11 +133,12 @@ def gated_rows_per_wave(m: int, n: int) -> int:
 def gated_plan(m: int, n: int, k: int, cus: int = 256) -> int:
     """What :func:`kernels.gemm_bf16_gated` is asked for at up to 64 tokens: 0, the kernel with resident
     activations and one workgroup per CU, where it takes the shape and the pairs of 16 gate and 16 up rows
-    divide evenly enough over the ``cus`` workgroups (the busiest within 15 % of the mean: at 7B and 32B
-    widths it measured 2 to 7 % faster than the LDS-shared kernel, at the 1.5B width, 2 or 3 pairs a
-    workgroup, 5 % slower); else the LDS-shared kernel with one or two tiles per wave."""
+    divide evenly enough over the ``cus`` workgroups (the busiest within 40 % of the mean: at 7B and 32B
+    widths it measured 2 to 7 % faster than the LDS-shared kernel; at the 1.5B width, 2 or 3 pairs a
+    workgroup, the two measure alike, 15.9 against 15.7 us at 8 tokens, and the resident kernel can divide by the
+    norm before it, which saves that norm's kernel); else the LDS-shared kernel with one or two tiles per wave."""
     pairs = n // 32
-    if gated_resident_fits(m, n, k) and -(-pairs // cus) * cus <= 1.15 * pairs:
+    if gated_resident_fits(m, n, k) and -(-pairs // cus) * cus <= 1.4 * pairs:
         return 0
     if n * k >= 1e8 or m * n * k >= 1.5e9:
         # a large weight, or many tokens on a small one: the tiled kernel (3) with its three LDS stages and tiles
