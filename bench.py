@@ -21,6 +21,7 @@ import argparse
 import json
 import os
 import sys
+import threading
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
@@ -56,6 +57,19 @@ def log(text):
     print(f"[bench] {text}", file=sys.stderr, flush=True)
 
 
+def still_running(every_seconds: float = 60.0) -> None:
+    """A line on stderr every minute for as long as the program runs: a 32-bit step over the prompts of a large
+    batch takes minutes, and a run that prints nothing for long looks hung to whoever watches it."""
+    started = time.perf_counter()
+
+    def beat():
+        while True:
+            time.sleep(every_seconds)
+            log(f"  still running, {time.perf_counter() - started:.0f} s")
+
+    threading.Thread(target=beat, daemon=True).start()
+
+
 def main() -> int:
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -84,6 +98,8 @@ def main() -> int:
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this engine runs on a single MI355X, so --gpus {args.gpus} is not run")
         return 2
+
+    still_running()
 
     import torch
 

@@ -107,6 +107,49 @@ def test_rope_and_cache_write(dtype, hd, rotary_dim):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("hd,rotary_dim,bs", [(128, 128, 16), (64, 32, 8), (48, 48, 24), (32, 16, 16)])
+def test_rope_of_a_large_step_writes_what_the_small_step_kernel_writes(dtype, hd, rotary_dim, bs):
+    """With the step's table of sines the kernel takes eight tokens a workgroup and, where they are eight
+    consecutive positions of one request from a multiple of eight on, writes the value pages eight slots at a time.
+    Portions that start anywhere, a request without a page, a last group of fewer tokens: q, k and both caches
+    hold bit for bit what the kernel of the small steps leaves (which the test above holds to the plain rotation)."""
+    from vipera_rs_amd.ops import kernels
+    from vipera_rs_amd.parts.rotary import neox_inverse_frequencies
+    heads, kv_heads = 5, 2
+    portions = [(8, 32), (5, 13), (0, 3), (64, 16), (16, 8), (3, 5)]      # (first position, tokens) per entry
+    positions = [first + i for first, count in portions for i in range(count)]
+    entry_of = [e for e, (_, count) in enumerate(portions) for _ in range(count)]
+    width = 96 // bs + 1
+    table = torch.full((len(portions), width), -1, dtype=torch.int32)
+    order = torch.randperm(len(portions) * width, generator=torch.Generator().manual_seed(bs)).view(len(portions), width)
+    for e, (first, count) in enumerate(portions):
+        for block in range(first // bs, (first + count - 1) // bs + 1):
+            table[e, block] = int(order[e, block])
+    table[4, 16 // bs] = -1                                              # this request's tokens are not kept
+    pages = len(portions) * width
+    g = torch.Generator().manual_seed(hd + bs)
+    qkv = torch.randn(len(positions), (heads + 2 * kv_heads) * hd, generator=g).to(dtype)
+    inv = torch.from_numpy(neox_inverse_frequencies(rotary_dim, 10000.0)).to(DEV)
+    pos_d = torch.tensor(positions, dtype=torch.int32, device=DEV)
+    entry_d = torch.tensor(entry_of, dtype=torch.int32, device=DEV)
+    results = []
+    for angles in (None, kernels.rope_angles(pos_d, inv, len(positions))):
+        q_d = qkv.clone().to(DEV)
+        k_d = torch.zeros(pages, kv_heads, bs, hd, dtype=dtype, device=DEV)
+        v_d = torch.zeros(pages, kv_heads, hd, bs, dtype=dtype, device=DEV)
+        kernels.rope_kvwrite(q_d, pos_d, inv, rotary_dim, k_d, v_d, entry_d, table.to(DEV), heads, kv_heads, hd, angles)
+        results.append((q_d, k_d, v_d))
+    for small, large in zip(*results):
+        assert torch.equal(small, large)
+    assert float(results[1][2].abs().max()) > 0.0
+    # without a cache (a layer that reads another layer's) only q and k are rotated
+    q_only = qkv.clone().to(DEV)
+    kernels.rope_kvwrite(q_only, pos_d, inv, rotary_dim, None, None, entry_d, None, heads, kv_heads, hd,
+                         kernels.rope_angles(pos_d, inv, len(positions)))
+    assert torch.equal(q_only, results[0][0])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_swiglu_kernel(dtype):
     from vipera_rs_amd.ops import kernels
     gate_up = (torch.randn(7, 2 * 200) * 4).to(dtype).to(DEV)

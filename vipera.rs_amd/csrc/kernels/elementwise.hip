@@ -230,64 +230,121 @@ __global__ __launch_bounds__(ROPE_HEADS_PER_BLOCK * 64) void rope_kvwrite_kernel
   }
 }
 
-// The same work with 16 bytes per thread: a thread owns V consecutive dims of one head (V = 8 bfloat16 or 4 floats).
-// A chunk in the first half of the rotated dims rotates with its partner half a rotation width further on; a chunk
-// past the rotated dims of a key head is copied to the cache; a chunk of a value head is scattered into the
-// transposed page. Per element the arithmetic is that of rope_kvwrite_kernel. Needs head width, rotated width and
-// its half to be multiples of V.
+// The same work with 16 bytes per access, for steps of many tokens (the sines come from the step's table): a
+// workgroup owns ROPE_GROUP consecutive tokens of the batch, a wave one of them. A lane owns V consecutive dims
+// (V = 8 bfloat16 or 4 floats) in the first half of the rotated dims of a q or k head and their partners half a
+// rotation width further on; with 64 lanes a wave covers 64 / (half / V) heads at a time, one contiguous stretch of
+// the token's row, and keeps its sines across the heads where its chunk stays the same. Dims of a key head past
+// the rotated ones are copied to the cache. Value heads: where the group's tokens are eight consecutive positions
+// of one request that begin at a multiple of eight (the inside of a prompt's portion), a thread takes V dims of
+// all eight tokens, transposes them in registers and writes, per dim, the eight slots of the transposed page as
+// one stretch (the 7B prompt of 2,048 tokens: 131,072 stores of 16 bytes instead of a million of two); any other
+// group scatters element by element. Per element the arithmetic is that of rope_kvwrite_kernel. Needs head
+// width, rotated width and its half to be multiples of V.
+constexpr int ROPE_GROUP = 8;
 template <typename T>
-__global__ __launch_bounds__(256) void rope_kvwrite_vector_kernel(
-    T* __restrict__ qkv, const int* __restrict__ positions, const float* __restrict__ inv_freq,
-    const float2* __restrict__ angles, int rotary_dim, T* __restrict__ k_cache, T* __restrict__ v_cache,
-    const int* __restrict__ entry_of_token, const int* __restrict__ block_table, int table_width, int block_size,
-    int heads, int kv_heads, int hd, int total_heads) {
+__global__ __launch_bounds__(ROPE_GROUP * 64) void rope_kvwrite_vector_kernel(
+    T* __restrict__ qkv, const int* __restrict__ positions, const float2* __restrict__ angles, int rotary_dim,
+    T* __restrict__ k_cache, T* __restrict__ v_cache, const int* __restrict__ entry_of_token,
+    const int* __restrict__ block_table, int table_width, int block_size, int heads, int kv_heads, int hd,
+    int num_tokens) {
   constexpr int V = 16 / (int)sizeof(T);
   typedef T vec_t __attribute__((ext_vector_type(V)));
-  const int chunks = hd / V;
-  const int unit = blockIdx.y * blockDim.x + threadIdx.x;
-  if (unit >= total_heads * chunks) return;
-  const int t = blockIdx.x, head = unit / chunks, i0 = (unit % chunks) * V;
-  const int pos = positions[t];
-  T* h = qkv + (size_t)t * (heads + 2 * kv_heads) * hd + (size_t)head * hd;
-  const bool is_q = head < heads, is_k = !is_q && head < heads + kv_heads;
-  const int half = rotary_dim / 2;
-  int page = -1;
-  if (!is_q && k_cache != nullptr) page = block_table[(size_t)entry_of_token[t] * table_width + pos / block_size];
-  const int slot = pos % block_size;
-  if (is_q || is_k) {
-    const size_t k_at = is_k && page >= 0 ? (((size_t)page * kv_heads + (head - heads)) * block_size + slot) * hd : 0;
-    if (i0 < half) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int t0 = blockIdx.x * ROPE_GROUP, t = t0 + wave;
+  const int half = rotary_dim / 2, row = (heads + 2 * kv_heads) * hd;
+  if (t < num_tokens) {
+    const int pos = positions[t];
+    int page = -1;
+    if (k_cache != nullptr) page = block_table[(size_t)entry_of_token[t] * table_width + pos / block_size];
+    const int slot = pos % block_size;
+    T* token = qkv + (size_t)t * row;
+    const int chunks = half / V, items = (heads + kv_heads) * chunks;
+    const bool same_chunk = 64 % chunks == 0;  // then u % chunks is the same in every round
+    float sn[V], cs[V];
+    for (int u = lane; u < items; u += 64) {
+      const int head = u / chunks, i0 = (u % chunks) * V;
+      if (!same_chunk || u == lane) {
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+          const float2 sc = angles[(size_t)t * half + i0 + j];
+          sn[j] = sc.x;
+          cs[j] = sc.y;
+        }
+      }
+      T* h = token + (size_t)head * hd;
       const vec_t lo = *(const vec_t*)(h + i0), hi = *(const vec_t*)(h + i0 + half);
       vec_t a, b;
 #pragma unroll
       for (int j = 0; j < V; ++j) {
-        float sn, cs;
-        if (angles) {
-          const float2 sc = angles[(size_t)t * half + i0 + j];
-          sn = sc.x;
-          cs = sc.y;
-        } else {
-          sincosf((float)pos * inv_freq[i0 + j], &sn, &cs);
-        }
-        const float l = to_float<T>(lo[j]), u = to_float<T>(hi[j]);
-        a[j] = from_float<T>(l * cs - u * sn);
-        b[j] = from_float<T>(l * sn + u * cs);
+        const float l = to_float<T>(lo[j]), w = to_float<T>(hi[j]);
+        a[j] = from_float<T>(l * cs[j] - w * sn[j]);
+        b[j] = from_float<T>(l * sn[j] + w * cs[j]);
       }
       *(vec_t*)(h + i0) = a;
       *(vec_t*)(h + i0 + half) = b;
-      if (is_k && page >= 0) {
-        *(vec_t*)(k_cache + k_at + i0) = a;
-        *(vec_t*)(k_cache + k_at + i0 + half) = b;
+      if (head >= heads && page >= 0) {
+        T* at = k_cache + (((size_t)page * kv_heads + (head - heads)) * block_size + slot) * hd;
+        *(vec_t*)(at + i0) = a;
+        *(vec_t*)(at + i0 + half) = b;
       }
-    } else if (i0 >= rotary_dim && is_k && page >= 0) {
-      *(vec_t*)(k_cache + k_at + i0) = *(const vec_t*)(h + i0);
     }
-  } else if (page >= 0) {
-    const int kvh = head - heads - kv_heads;
-    const size_t v_at = (((size_t)page * kv_heads + kvh) * hd + i0) * block_size + slot;
-    const vec_t v = *(const vec_t*)(h + i0);
+    if (rotary_dim < hd && page >= 0) {  // the dims of the key heads that are not rotated
+      const int tail = (hd - rotary_dim) / V;
+      for (int u = lane; u < kv_heads * tail; u += 64) {
+        const int kvh = u / tail, i0 = rotary_dim + (u % tail) * V;
+        *(vec_t*)(k_cache + (((size_t)page * kv_heads + kvh) * block_size + slot) * hd + i0) =
+            *(const vec_t*)(token + (size_t)(heads + kvh) * hd + i0);
+      }
+    }
+  }
+  if (k_cache == nullptr) return;
+  // the value heads of the group's tokens
+  const int v_chunks = hd / V, v_items = kv_heads * v_chunks;
+  bool whole = t0 + ROPE_GROUP <= num_tokens && (block_size & 7) == 0;
+  int first = 0, entry = 0;
+  if (whole) {
+    first = positions[t0];
+    entry = entry_of_token[t0];
+    whole = (first & 7) == 0;
 #pragma unroll
-    for (int j = 0; j < V; ++j) v_cache[v_at + (size_t)j * block_size] = v[j];
+    for (int j = 1; j < ROPE_GROUP; ++j)
+      whole = whole && positions[t0 + j] == first + j && entry_of_token[t0 + j] == entry;
+  }
+  if (whole) {
+    const int page = block_table[(size_t)entry * table_width + first / block_size];
+    if (page < 0) return;
+    const int slot = first % block_size;
+    for (int u = threadIdx.x; u < v_items; u += ROPE_GROUP * 64) {
+      const int kvh = u / v_chunks, i0 = (u % v_chunks) * V;
+      vec_t of_token[ROPE_GROUP];
+#pragma unroll
+      for (int j = 0; j < ROPE_GROUP; ++j)
+        of_token[j] = *(const vec_t*)(qkv + (size_t)(t0 + j) * row + (size_t)(heads + kv_heads + kvh) * hd + i0);
+      T* at = v_cache + (((size_t)page * kv_heads + kvh) * hd + i0) * block_size + slot;
+#pragma unroll
+      for (int d = 0; d < V; ++d)
+#pragma unroll
+        for (int part = 0; part < ROPE_GROUP / V; ++part) {
+          vec_t slots;
+#pragma unroll
+          for (int j = 0; j < V; ++j) slots[j] = of_token[part * V + j][d];
+          *(vec_t*)(at + (size_t)d * block_size + part * V) = slots;
+        }
+    }
+    return;
+  }
+  const int count = min(ROPE_GROUP, num_tokens - t0);
+  for (int u = threadIdx.x; u < count * v_items; u += ROPE_GROUP * 64) {
+    const int tt = t0 + u / v_items, item = u % v_items;
+    const int kvh = item / v_chunks, i0 = (item % v_chunks) * V;
+    const int pos = positions[tt];
+    const int page = block_table[(size_t)entry_of_token[tt] * table_width + pos / block_size];
+    if (page < 0) continue;
+    const vec_t v = *(const vec_t*)(qkv + (size_t)tt * row + (size_t)(heads + kv_heads + kvh) * hd + i0);
+    T* at = v_cache + (((size_t)page * kv_heads + kvh) * hd + i0) * block_size + pos % block_size;
+#pragma unroll
+    for (int j = 0; j < V; ++j) at[(size_t)j * block_size] = v[j];
   }
 }
 
@@ -306,19 +363,18 @@ extern "C" int vk_rope_kvwrite(void* qkv, int dtype, const int* positions, const
   {  // 16 bytes per thread where the widths allow it and the sines come from the step's table (a step of many
      // tokens); computing eight sines in a row per thread is slower than one per lane (measured with 8 tokens)
     const int v = dtype == DT_F32 ? 4 : 8;
-    const bool aligned = ((uintptr_t)qkv & 15) == 0 && ((uintptr_t)k_cache & 15) == 0;
-    if ((dtype == DT_F32 || dtype == DT_BF16) && angles != nullptr && aligned && hd % v == 0 && rotary_dim % v == 0 &&
+    const bool aligned = (((uintptr_t)qkv | (uintptr_t)k_cache | (uintptr_t)v_cache) & 15) == 0;
+    if ((dtype == DT_F32 || dtype == DT_BF16) && angles != nullptr && aligned && rotary_dim > 0 && hd % v == 0 && rotary_dim % v == 0 &&
         (rotary_dim / 2) % v == 0) {
-      const int units = total_heads * (hd / v);
-      const dim3 vgrid(num_tokens, (units + 255) / 256);
+      const unsigned groups = (unsigned)((num_tokens + ROPE_GROUP - 1) / ROPE_GROUP);
       if (dtype == DT_F32)
-        rope_kvwrite_vector_kernel<float><<<vgrid, 256, 0, s>>>(
-            (float*)qkv, positions, inv_freq, (const float2*)angles, rotary_dim, (float*)k_cache, (float*)v_cache,
-            entry_of_token, block_table, table_width, block_size, heads, kv_heads, hd, total_heads);
+        rope_kvwrite_vector_kernel<float><<<groups, ROPE_GROUP * 64, 0, s>>>(
+            (float*)qkv, positions, (const float2*)angles, rotary_dim, (float*)k_cache, (float*)v_cache, entry_of_token,
+            block_table, table_width, block_size, heads, kv_heads, hd, num_tokens);
       else
-        rope_kvwrite_vector_kernel<bf16_t><<<vgrid, 256, 0, s>>>(
-            (bf16_t*)qkv, positions, inv_freq, (const float2*)angles, rotary_dim, (bf16_t*)k_cache, (bf16_t*)v_cache,
-            entry_of_token, block_table, table_width, block_size, heads, kv_heads, hd, total_heads);
+        rope_kvwrite_vector_kernel<bf16_t><<<groups, ROPE_GROUP * 64, 0, s>>>(
+            (bf16_t*)qkv, positions, (const float2*)angles, rotary_dim, (bf16_t*)k_cache, (bf16_t*)v_cache,
+            entry_of_token, block_table, table_width, block_size, heads, kv_heads, hd, num_tokens);
       VK_LAUNCH_CHECK();
       return 0;
     }

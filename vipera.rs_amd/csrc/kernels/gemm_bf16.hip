@@ -1655,8 +1655,8 @@ int g_tile_stages = 0;   // 0: chosen by shape; 2 or 3 force the direct kernel's
 // of 256x256 tiles runs at about 1.15 PFLOP/s with the kernel that loads straight into LDS and at 1.0
 // with the staged one (measured on the 7B shapes at 2,048 tokens); the smaller tiles reach 0.75 to 0.8 of
 // their kernel's best, 256x192 about 0.9, and 256x128 with its three LDS stages about 0.95 (it is what the output
-// and down projections of 512 to 2,048 tokens run on, where 256x256 tiles are too few). Workgroups run in whole rounds of one per CU (two for the 128x128
-// tile, whose LDS lets two share a CU, unless every workgroup finds a CU of its own), so a launch that fills
+// and down projections of 512 to 2,048 tokens run on, where 256x256 tiles are too few). Workgroups run in whole rounds of one per CU (two where
+// the LDS of the tile's stages lets two share a CU: the 128x128 tile and its narrower kin with two stages, unless every workgroup finds a CU of its own), so a launch that fills
 // the last round badly loses that share. Splitting K
 // multiplies the workgroups, at the price of writing and re-reading float partial sums (they mostly stay
 // in the caches: about 6 TB/s) and one more launch; each range keeps at least 512 of K. The estimate ranks
@@ -1664,6 +1664,8 @@ int g_tile_stages = 0;   // 0: chosen by shape; 2 or 3 force the direct kernel's
 // Ties go to the larger tile and to fewer ranges.
 struct TilePlan { int config, ranges; };
 int g_compute_units = 0;
+// the 128-token tiles of the direct kernel run with a third LDS stage for up to 128 tokens (see launch_tile)
+bool tile_is_deep(int M) { return g_tile_stages ? g_tile_stages == 3 : M <= 128; }
 TilePlan choose_tile_plan(int M, int N, int K, long long partial_floats, bool direct, bool gated = false) {
   if (g_compute_units == 0) {
     int device = 0, count = 0;
@@ -1672,14 +1674,14 @@ TilePlan choose_tile_plan(int M, int N, int K, long long partial_floats, bool di
       count = 256;
     g_compute_units = count;
   }
-  struct Tiling { int config, tokens, rows, resident; double speed; };
-  static const Tiling staged[] = {{4, 256, 256, 1, 1.0}, {2, 256, 128, 1, 0.8}, {3, 128, 256, 1, 0.8}, {0, 128, 128, 2, 0.75}};
+  struct Tiling { int config, tokens, rows; double speed; };
+  static const Tiling staged[] = {{4, 256, 256, 1.0}, {2, 256, 128, 0.8}, {3, 128, 256, 0.8}, {0, 128, 128, 0.75}};
   // the last three (the gated product of up to 128 tokens only): the weight of a feed-forward has so many rows
   // that with 128 of them a tile the tiles come in more than one round and less than two (7B width at 64 tokens:
   // 296 tiles of 128 rows, two to a CU on 40 CUs, one on the others); a width of 96, 160 or 224 rows can come
   // close to one tile per CU (237 tiles of 160 rows)
-  static const Tiling straight[] = {{5, 256, 256, 1, 1.15}, {7, 256, 128, 1, 1.1}, {8, 128, 256, 1, 0.88}, {9, 128, 128, 2, 0.9},
-                                    {6, 256, 192, 1, 1.05}, {10, 128, 96, 2, 0.85}, {11, 128, 160, 2, 0.88}, {12, 128, 224, 1, 0.88}};
+  static const Tiling straight[] = {{5, 256, 256, 1.15}, {7, 256, 128, 1.1}, {8, 128, 256, 0.88}, {9, 128, 128, 0.9},
+                                    {6, 256, 192, 1.05}, {10, 128, 96, 0.85}, {11, 128, 160, 0.88}, {12, 128, 224, 0.88}};
   const Tiling* tilings = direct ? straight : staged;
   TilePlan best{tilings[3].config, 1};
   double best_time = 1e30;
@@ -1689,10 +1691,14 @@ TilePlan choose_tile_plan(int M, int N, int K, long long partial_floats, bool di
     if (M <= 128 && t.tokens > 128) continue;
     if (M > 128 && t.tokens == 128 && t.rows == 256) continue;  // with many tokens the wide side goes to the tokens
     const long long groups = (long long)((M + t.tokens - 1) / t.tokens) * ((N + t.rows - 1) / t.rows);
+    // how many workgroups share a CU follows from the LDS of the stages that will be launched (at most two)
+    const int stages = !direct ? 2 : t.tokens == 128 ? (tile_is_deep(M) ? 3 : 2) : (t.config == 7 && g_tile_stages != 2 ? 3 : 2);
+    const int lds_bytes = stages * (t.tokens + t.rows) * (direct ? 128 : 144);
+    const int resident = lds_bytes * 2 <= 160 * 1024 ? 2 : 1;
     for (int ranges = 1; ranges <= 8; ranges *= 2) {
       if (ranges > 1 && (K / ranges < 512 || (long long)ranges * M * N > partial_floats)) break;
       // workgroups that all find a CU of their own do not share one, however many would fit
-      const long long slots = groups * ranges <= g_compute_units ? g_compute_units : (long long)g_compute_units * t.resident;
+      const long long slots = groups * ranges <= g_compute_units ? g_compute_units : (long long)g_compute_units * resident;
       const long long rounds = (groups * ranges + slots - 1) / slots;
       const double fill = (double)(groups * ranges) / ((double)rounds * slots);
       double time = flops / (1e15 * t.speed * fill);
@@ -1733,7 +1739,7 @@ int launch_tile(const __bf16* A, const __bf16* W, const float* bias, TC* C, int 
                                                                          partial, s);                                \
     VK_TILE(BMV, BNV, WMV, WNV, true);                                                                               \
   }
-  const bool deep = g_tile_stages ? g_tile_stages == 3 : M <= 128;
+  const bool deep = tile_is_deep(M);
   if constexpr (GATED) {
     switch (plan.config) {
       // four waves side by side along the tokens: a wave owns all rows of the tile, an even number of 16-row
