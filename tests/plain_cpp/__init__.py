@@ -30,6 +30,7 @@ SIGNATURES = {
     "plain_gemm_bf16_gated": [P, P, P, I, I, I, LL, LL, I, P],
     "plain_gemm_bf16_follow": [P, P, P, P, I, I, I, LL, LL, P, P, LL, P, LL, P, P],
     "plain_gemm_bf16_gated_scaled": [P, P, P, I, I, I, LL, LL, P, I, F, P],
+    "plain_gemm_bf16_gated_tile_scaled": [P, P, P, I, I, I, LL, LL, P, I, I, F, P],
     "plain_gemm_bf16_qkv_rope": [P, P, P, P, I, I, I, LL, LL, P, P, P, P, P, P, I, I, I, I, I, P, I, F, P],
     "plain_gemm_bf16_mid_follow": [P, P, P, P, I, I, I, LL, LL, I, I, P, LL, P, P, LL, P, LL, I, P, P],
     "plain_gemm_bf16_mid_qkv_rope": [P, P, P, P, I, I, I, LL, LL, I, I, P, LL, P, P, P, P, P, P, I, I, I, I, I, P, I, I, F, P],

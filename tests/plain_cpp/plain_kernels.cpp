@@ -364,6 +364,32 @@ extern "C" int plain_gemm_bf16_gated_scaled(const void* A, const void* W, void* 
   return 0;
 }
 
+// The gated product on the tiled kernel on such a scaled input, for any number of tokens.
+extern "C" int plain_gemm_bf16_gated_tile_scaled(const void* A, const void* W, void* C, int M, int N, int K,
+                                                 long long lda, long long ldc, const float* sumsq, int groups, int stride,
+                                                 float eps, void*) {
+  if (M <= 0 || N <= 0) return 0;
+  if (K <= 0 || lda < K || (N & 31) || ldc < N / 2 || groups <= 0 || stride < M) return BAD_ARGUMENT;
+  for (int m = 0; m < M; ++m) {
+    double squares = 0.0;
+    for (int g = 0; g < groups; ++g) squares += (double)sumsq[(size_t)g * stride + m];
+    const double inv = 1.0 / std::sqrt(squares / (double)K + (double)eps);
+    for (int i = 0; i < N / 2; ++i) {
+      const int gate_row = (i / 16) * 32 + i % 16, up_row = gate_row + 16;
+      double gate = 0.0, up = 0.0;
+      for (int k = 0; k < K; ++k) {
+        const double a = load(A, DT_BF16, (size_t)m * lda + k);
+        gate += a * (double)load(W, DT_BF16, (size_t)gate_row * K + k);
+        up += a * (double)load(W, DT_BF16, (size_t)up_row * K + k);
+      }
+      gate *= inv;
+      up *= inv;
+      store(C, DT_BF16, (size_t)m * ldc + i, (float)(up * (gate / (1.0 + std::exp(-gate)))));
+    }
+  }
+  return 0;
+}
+
 // --- attention over the paged cache ----------------------------------------------------------------------------
 extern "C" int plain_attn_generic(const void* q, long long q_stride, const void* k_cache, const void* v_cache,
                                   void* out, int dtype, const int* positions, const int* entry_of_token,

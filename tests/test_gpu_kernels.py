@@ -616,7 +616,7 @@ def test_the_norm_split_between_the_products_around_it(m, width, k_in, inter):
     eps = 1e-5
     x = x0.clone()
     scaled = torch.empty(m, width, dtype=torch.bfloat16, device=DEV)
-    sumsq = torch.full((kernels.follow_sumsq_floats(width),), 7.0, device=DEV)
+    sumsq = torch.full((kernels.follow_sumsq_floats(width, m),), 7.0, device=DEV)
     groups = kernels.gemm_bf16_follow(a, w_o, None, x, gain, scaled, sumsq)
     want_x = x0.double() + a.double() @ w_o.double().T
     assert _rel(x, want_x) < 1e-5
@@ -638,6 +638,59 @@ def test_the_norm_split_between_the_products_around_it(m, width, k_in, inter):
     out3 = torch.empty(m, inter, dtype=torch.bfloat16, device=DEV)
     kernels.gemm_bf16_gated(h3, fused, out3, 0)
     assert _rel(out, out3.double()) < 1.2e-2
+
+
+@pytest.mark.parametrize("tiling", [-1, 0, 2, 3, 4, 9, 7, 8, 5, 10, 11, 12])
+@pytest.mark.parametrize("m,width,k_in,inter", [(64, 520, 1024, 16 * 21), (33, 1032, 1536, 16 * 40), (17, 264, 2048, 16 * 9),
+                                               (300, 3584, 512, 16 * 64), (5, 200, 0, 16 * 30)])
+def test_the_tiled_gated_product_divides_by_the_norm_before_it(tiling, m, width, k_in, inter):
+    """17 to 64 tokens: the residual product whose K is split over workgroups leaves bfloat16(x * g) and the sums of
+    squares (the kernel that adds its ranges does), and the tiled gated product divides gate and up by the root
+    mean square.  Every tiling of both tiled kernels; sums of squares made by hand too (k_in 0), for token counts
+    and group counts that no product before the norm produces.  Against 64-bit, as the kernels it replaces."""
+    from vipera_rs_amd.ops import kernels
+    from vipera_rs_amd.ops.linear import interleave_gate_up
+    g = torch.Generator().manual_seed(m + width + k_in)
+    gain = (1 + 0.2 * torch.randn(width, generator=g)).to(DEV)
+    gate = (torch.randn(inter, width, generator=g) / width ** 0.5).to(torch.bfloat16).to(DEV)
+    up = (torch.randn(inter, width, generator=g) / width ** 0.5).to(torch.bfloat16).to(DEV)
+    fused = interleave_gate_up(gate, up)
+    eps = 1e-5
+    stride = kernels.follow_stride(m)
+    x0 = (torch.randn(m, width, generator=g) * 2).to(DEV)
+    x0[m // 2, 3] = 60.0                                      # one row with a far larger mean square
+    if k_in and m <= 64:
+        a = torch.randn(m, k_in, generator=g).to(torch.bfloat16).to(DEV)
+        w_o = (torch.randn(width, k_in, generator=g) / k_in ** 0.5).to(torch.bfloat16).to(DEV)
+        x = x0.clone()
+        scaled = torch.full((m, width), 7.0, dtype=torch.bfloat16, device=DEV)
+        sumsq = torch.full((kernels.follow_sumsq_floats(width, m),), 7.0, device=DEV)
+        groups = kernels.gemm_bf16_mid_follow(a, w_o, None, x, 2, 1, gain, scaled, sumsq)
+        want_x = x0.double() + a.double() @ w_o.double().T
+        assert _rel(x, want_x) < 1e-5
+    else:  # 37 groups of uneven shares of each row's squares
+        x, want_x = x0, x0.double()
+        scaled = (x0 * gain).to(torch.bfloat16)
+        groups = 37
+        shares = torch.rand(groups, m, generator=g).to(DEV).double() + 0.1
+        shares = shares / shares.sum(0, keepdim=True) * (want_x ** 2).sum(-1)
+        sumsq = torch.full((groups * stride,), 7.0, device=DEV)
+        sumsq.view(groups, stride)[:, :m] = shares.float()
+    try:
+        kernels.gemm_bf16_force_tiling(tiling)
+        act = torch.full((m, inter), 7.0, dtype=torch.bfloat16, device=DEV)
+        kernels.gemm_bf16_gated_tile_scaled(scaled, fused, act, sumsq, groups, eps)
+        h = want_x * torch.rsqrt((want_x ** 2).mean(-1, keepdim=True) + eps) * gain.double()
+        gd, ud = h @ gate.double().T, h @ up.double().T
+        want = ud * (gd / (1 + torch.exp(-gd)))
+        assert _rel(act, want) < 1.2e-2
+        h3 = torch.empty(m, width, dtype=torch.bfloat16, device=DEV)       # the two kernels it replaces are as far
+        kernels.rmsnorm(x, gain, eps, h3)                                  # from the 64-bit result, each on its side
+        act3 = torch.empty_like(act)
+        kernels.gemm_bf16_gated(h3, fused, act3, 3)
+        assert _rel(act3, want) < 1.2e-2 and _rel(act, act3.double()) < 2.4e-2
+    finally:
+        kernels.gemm_bf16_force_tiling(-1)
 
 
 @pytest.mark.parametrize("m,inter,k", [(1, 32, 64), (5, 48, 96), (8, 18944, 512), (16, 176, 200), (33, 128, 264), (64, 1024, 256),

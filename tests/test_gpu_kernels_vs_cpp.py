@@ -141,7 +141,7 @@ def test_the_first_norm_of_a_layer_split_between_the_layers(m, width, k_in, head
     gain = 1 + 0.2 * torch.randn(width, generator=g)
     w = (torch.randn(n, width, generator=g) / math.sqrt(width)).to(torch.bfloat16)
     bias = torch.randn(n, generator=g)
-    floats = kernels.follow_sumsq_floats(width)
+    floats = kernels.follow_sumsq_floats(width, m)
     groups_d, groups_h = ctypes.c_int(0), ctypes.c_int(0)
     if split:
         partial = torch.empty(4 * 64 * width)
@@ -220,6 +220,29 @@ def test_split_qkv_product_that_rotates_while_it_adds_its_ranges(m, heads, kv_he
     kernels.gemm_bf16_mid_qkv_rope(dev[0], dev[1], dev[2], fused, 2, 1, dev[13], dev[14], kc2, vc2, dev[17], dev[18], heads,
                                    kv_heads, hd)
     assert torch.equal(fused, qkv) and torch.equal(kc2, kc) and torch.equal(vc2, vc)
+
+
+@pytest.mark.parametrize("m,width,inter,groups", [(70, 264, 16 * 9, 5), (300, 520, 16 * 21, 56), (17, 200, 16 * 6, 1)])
+def test_the_tiled_gated_product_on_a_scaled_input_beside_its_twin(m, width, inter, groups):
+    from vipera_rs_amd.ops import kernels
+    from vipera_rs_amd.ops.linear import interleave_gate_up
+    g = torch.Generator().manual_seed(m + width)
+    x = torch.randn(m, width, generator=g) * 2
+    gain = 1 + 0.2 * torch.randn(width, generator=g)
+    scaled = (x * gain).to(torch.bfloat16)
+    stride = kernels.follow_stride(m)
+    sumsq = torch.full((groups, stride), 3.0)
+    shares = torch.rand(groups, m, generator=g) + 0.1
+    sumsq[:, :m] = shares / shares.sum(0, keepdim=True) * (x ** 2).sum(-1)
+    gate = (torch.randn(inter, width, generator=g) / math.sqrt(width)).to(torch.bfloat16)
+    up = (torch.randn(inter, width, generator=g) / math.sqrt(width)).to(torch.bfloat16)
+    args = [scaled, interleave_gate_up(gate, up), torch.empty(m, inter, dtype=torch.bfloat16), m, 2 * inter, width, width, inter,
+            sumsq, groups, stride, 1e-5, None]
+    (got, want), = both("gemm_bf16", "gemm_bf16_gated_tile_scaled", args, [2])
+    assert rel_err(got.float().numpy(), want.double().numpy()) < 8e-3
+    h = x.double() * torch.rsqrt((x.double() ** 2).mean(-1, keepdim=True) + 1e-5) * gain.double()
+    gd, ud = h @ gate.double().T, h @ up.double().T
+    assert rel_err(got.float().numpy(), (ud * (gd / (1 + torch.exp(-gd)))).numpy()) < 1.2e-2
 
 
 def _kernel_with_pointer(name):

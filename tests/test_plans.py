@@ -63,10 +63,11 @@ def test_q_k_v_of_17_to_64_tokens_rotates_in_the_kernel_that_adds_its_ranges():
 
 
 def test_room_for_the_sums_of_squares():
-    assert follow_stride(16) == 16 and follow_stride(17) == 64
+    assert follow_stride(16) == 16 and follow_stride(17) == 64 and follow_stride(64) == 64
+    assert follow_stride(65) == 128 and follow_stride(2048) == 2048
     for n in (16, 64, 1000, 3584, 8192):
-        assert follow_sumsq_floats(n) >= ((n + 7) // 8) * 16           # a workgroup per 8 columns, 16 tokens
-        assert follow_sumsq_floats(n) >= ((n + 1023) // 1024) * 64     # a workgroup per 1,024 columns, 64 tokens
+        assert follow_sumsq_floats(n, 16) >= ((n + 7) // 8) * 16          # a workgroup per 8 columns, 16 tokens
+        assert follow_sumsq_floats(n, 64) >= ((n + 1023) // 1024) * 64    # a workgroup per 1,024 columns, 64 tokens
 
 
 def test_decode_attention_chunks():

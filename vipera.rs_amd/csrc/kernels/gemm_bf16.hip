@@ -173,6 +173,84 @@ constexpr int BK = 64;
 constexpr int ROW = BK + 8;  // elements per LDS row: 144 bytes
 constexpr int XCDS = 8;
 
+// The second half of an RMS norm that is split between the products around it (see FollowNorm), in a tiled
+// product, for any number of tokens: the input is x * gain as the product before the norm left it, and the 32-bit
+// sums of token m are multiplied by 1 / sqrt(sum over the groups of sumsq[group * stride + m] / K + eps) before
+// bias and activation. The first half stays with the kernels of up to 64 tokens: in the tiled kernel's epilogue it
+// was measured too (x * gain and the squares of each wave's columns written beside the residual) and saves
+// nothing from 128 to 2,048 tokens, where the norm kernel it replaces moves little more than the epilogue adds.
+struct TileNorm {
+  const float* sumsq = nullptr;
+  int groups = 0, stride = 0;
+  float eps = 0.f;
+};
+
+// At the start of a tile kernel the THREADS / BM threads of a token each add every
+// (THREADS / BM)-th group, in ascending order, and leave their part in part_sums[part * BM + token] (a token past M
+// takes the last one's, which nothing uses). A thread requests 32 groups at a time at clamped addresses before it
+// adds any: one round trip to memory for up to 64 groups on two threads, behind the tile's first operand requests,
+// where a loop of a load and an addition at a time cost the gate/up product of 2,048 tokens 69 us of 437. The
+// barrier before the first product makes the parts visible; tile_norm_factor adds them in ascending order.
+template <int BM, int THREADS>
+__device__ __forceinline__ void tile_norm_parts(const TileNorm& norm, int m0, int M, int tid, float* part_sums) {
+  static_assert(THREADS % BM == 0, "whole threads per token");
+  constexpr int PER = THREADS / BM, AHEAD = 32;
+  if (!norm.sumsq) return;
+  const int token = tid % BM, part = tid / BM;
+  const float* of_token = norm.sumsq + min(m0 + token, M - 1);
+  float squares = 0.f;
+  for (int base = part; base < norm.groups; base += AHEAD * PER) {
+    float ahead[AHEAD];
+#pragma unroll
+    for (int j = 0; j < AHEAD; ++j) ahead[j] = of_token[(size_t)min(base + j * PER, norm.groups - 1) * norm.stride];
+#pragma unroll
+    for (int j = 0; j < AHEAD; ++j)
+      if (base + j * PER < norm.groups) squares += ahead[j];
+  }
+  part_sums[part * BM + token] = squares;
+}
+template <int BM, int THREADS>
+__device__ __forceinline__ float tile_norm_factor(const TileNorm& norm, const float* part_sums, int token, int K) {
+  float squares = 0.f;
+#pragma unroll
+  for (int part = 0; part < THREADS / BM; ++part) squares += part_sums[part * BM + token];
+  return 1.0f / sqrtf(squares / (float)K + norm.eps);
+}
+
+// What a wave of a tile kernel does with its sums: acc[tn][tm] holds, in lane (lr, lg), outputs
+// [wave_n + tn * 16 + lg * 4, + 4) of token wave_m + tm * 16 + lr. `part_sums`: see tile_norm_parts; `wave_token`:
+// the wave's first token within the tile.
+template <int BM, int THREADS, int TM, int TN, typename TC, bool ACCUMULATE, bool GATED>
+__device__ __forceinline__ void tile_epilogue(f32x4 (&acc)[TN][TM], TC* __restrict__ C, long long ldc, int M, int N,
+                                              int K, const float* __restrict__ bias, bool vector_ok, int wave_m,
+                                              int wave_n, int lr, int lg, const TileNorm& norm,
+                                              const float* part_sums, int wave_token) {
+  if (norm.sumsq) {
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm) {
+      const float inv = tile_norm_factor<BM, THREADS>(norm, part_sums, wave_token + tm * 16 + lr, K);
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn) acc[tn][tm] *= inv;
+    }
+  }
+  if constexpr (GATED) {
+    // N counts fused rows (pairs of 16-row tiles: gate, up); the output has N / 2 columns
+    static_assert(!GATED || TN % 2 == 0, "a wave must own whole gate/up pairs");
+#pragma unroll
+    for (int pair = 0; pair < TN / 2; ++pair)
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm)
+        store_gated((__bf16*)C, ldc, wave_m + tm * 16 + lr, (wave_n + pair * 32) / 2 + lg * 4, M, N / 2,
+                    acc[2 * pair][tm], acc[2 * pair + 1][tm]);
+    return;
+  }
+#pragma unroll
+  for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm)
+      store4<TC, ACCUMULATE>(C, ldc, wave_m + tm * 16 + lr, wave_n + tn * 16 + lg * 4, M, N, acc[tn][tm], bias, vector_ok);
+}
+
 // BM x BN: output tile of a workgroup (tokens x weight rows); WM x WN: its grid of waves. A wave owns
 // (BM / WM) x (BN / WN) outputs as TM x TN instruction tiles.
 template <int BM, int BN, int WM, int WN, typename TC, bool ACCUMULATE, bool GATED>
@@ -181,7 +259,8 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_tile_kernel(const __bf16* _
                                                                    const float* __restrict__ bias, TC* __restrict__ C,
                                                                    int M, int N, int K, long long lda, long long ldc,
                                                                    int tiles_m, int tiles_n, int vector_ok,
-                                                                   int k_per_range, long long range_stride) {
+                                                                   int k_per_range, long long range_stride,
+                                                                   TileNorm norm) {
   // gridDim.y > 1: K is split into ranges of k_per_range (a multiple of 64); range r writes its partial
   // sums to C + r * range_stride and a second kernel adds the ranges
   const int k_begin = blockIdx.y * k_per_range, k_end = min(K, k_begin + k_per_range);
@@ -256,7 +335,9 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_tile_kernel(const __bf16* _
   };
 
   const int steps = (k_end - k_begin + BK - 1) / BK;
+  __shared__ float part_sums[THREADS];
   load_global(k_begin);
+  tile_norm_parts<BM, THREADS>(norm, m0, M, tid, part_sums);
   store_lds(0);
   __syncthreads();
   for (int s = 0; s < steps; ++s) {
@@ -281,24 +362,9 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_tile_kernel(const __bf16* _
     __syncthreads();
   }
 
-  const int wave_m = m0 + wm * TM * 16, wave_n = n0 + wn * TN * 16;
-  if constexpr (GATED) {
-    // N counts fused rows (pairs of 16-row tiles: gate, up); the output has N / 2 columns
-    static_assert(!GATED || TN % 2 == 0, "a wave must own whole gate/up pairs");
-#pragma unroll
-    for (int pair = 0; pair < TN / 2; ++pair)
-#pragma unroll
-      for (int tm = 0; tm < TM; ++tm)
-        store_gated((__bf16*)C, ldc, wave_m + tm * 16 + lr, (wave_n + pair * 32) / 2 + lg * 4, M, N / 2,
-                    acc[2 * pair][tm], acc[2 * pair + 1][tm]);
-  } else {
-#pragma unroll
-    for (int tn = 0; tn < TN; ++tn)
-#pragma unroll
-      for (int tm = 0; tm < TM; ++tm)
-        store4<TC, ACCUMULATE>(C, ldc, wave_m + tm * 16 + lr, wave_n + tn * 16 + lg * 4, M, N, acc[tn][tm], bias,
-                               vector_ok != 0);
-  }
+  tile_epilogue<BM, THREADS, TM, TN, TC, ACCUMULATE, GATED>(acc, C, ldc, M, N, K, bias, vector_ok != 0,
+                                                            m0 + wm * TM * 16, n0 + wn * TN * 16, lr, lg, norm,
+                                                            part_sums, wm * TM * 16);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -344,7 +410,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_tile_direct_kernel(const __
                                                                           TC* __restrict__ C, int M, int N, int K,
                                                                           long long lda, long long ldc, int tiles_m,
                                                                           int tiles_n, int vector_ok, int k_per_range,
-                                                                          long long range_stride) {
+                                                                          long long range_stride, TileNorm norm) {
   typedef __attribute__((address_space(3))) void* lds_ptr;
   const int k_begin = blockIdx.y * k_per_range, k_end = min(K, k_begin + k_per_range);
   C += (size_t)blockIdx.y * range_stride;
@@ -419,10 +485,12 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_tile_direct_kernel(const __
 
   const int steps = (k_end - k_begin) / BK;
   bf16x8 fa0[TM], fw0[TN], fa1[TM], fw1[TN];
+  __shared__ float part_sums[WAVES * 64];
   issue_loads(0, 0);
   if (steps > 1) issue_loads(1, 1);
+  if (STAGES == 3 && steps > 2) issue_loads(2, 2);
+  tile_norm_parts<BM, WAVES * 64>(norm, m0, M, tid, part_sums);  // behind the first requests, before the first wait
   if (STAGES == 3 && steps > 2) {
-    issue_loads(2, 2);
     wait_own_loads_but<2 * LOADS>();  // step 0 has arrived; the other two stay in flight
   } else {
     wait_own_loads();
@@ -468,23 +536,9 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_tile_direct_kernel(const __
     step(s, stage, std::false_type{}, std::true_type{}, std::integral_constant<int, 0>{});
   step(s, stage, std::false_type{}, std::false_type{}, std::integral_constant<int, 0>{});
 
-  const int wave_m = m0 + wm * TM * 16, wave_n = n0 + wn * TN * 16;
-  if constexpr (GATED) {
-    static_assert(!GATED || TN % 2 == 0, "a wave must own whole gate/up pairs");
-#pragma unroll
-    for (int pair = 0; pair < TN / 2; ++pair)
-#pragma unroll
-      for (int tm = 0; tm < TM; ++tm)
-        store_gated((__bf16*)C, ldc, wave_m + tm * 16 + lr, (wave_n + pair * 32) / 2 + lg * 4, M, N / 2,
-                    acc[2 * pair][tm], acc[2 * pair + 1][tm]);
-  } else {
-#pragma unroll
-    for (int tn = 0; tn < TN; ++tn)
-#pragma unroll
-      for (int tm = 0; tm < TM; ++tm)
-        store4<TC, ACCUMULATE>(C, ldc, wave_m + tm * 16 + lr, wave_n + tn * 16 + lg * 4, M, N, acc[tn][tm], bias,
-                               vector_ok != 0);
-  }
+  tile_epilogue<BM, WAVES * 64, TM, TN, TC, ACCUMULATE, GATED>(acc, C, ldc, M, N, K, bias, vector_ok != 0,
+                                                               m0 + wm * TM * 16, n0 + wn * TN * 16, lr, lg, norm,
+                                                               part_sums, wm * TM * 16);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1601,10 +1655,10 @@ constexpr auto tile_kernel() {
 // DIRECT: the kernel that loads straight into LDS; K must be a multiple of 64. STAGES: its LDS stages.
 template <int BM, int BN, int WM, int WN, typename TC, bool ACC, bool GATED, bool DIRECT = false, int STAGES = 2>
 int launch_tile_as(const __bf16* A, const __bf16* W, const float* bias, TC* C, int M, int N, int K, long long lda,
-                   long long ldc, int vector_ok, int ranges, float* partial, hipStream_t s) {
+                   long long ldc, int vector_ok, int ranges, float* partial, hipStream_t s, const TileNorm& norm) {
   static_assert(DIRECT || STAGES == 2, "only the direct kernel has a third stage");
   constexpr int lds_bytes = DIRECT ? STAGES * (BM + BN) * DIRECT_ROW : 2 * (BM + BN) * ROW * (int)sizeof(__bf16);
-  static_assert(lds_bytes <= 160 * 1024, "a CU has 160 KB of LDS");
+  static_assert(lds_bytes + WM * WN * 64 * 4 <= 160 * 1024, "a CU has 160 KB of LDS (the stages and the norm's sums)");
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
   const long long total = (long long)tiles_m * tiles_n;
   const long long grid = (total + XCDS - 1) / XCDS * XCDS;
@@ -1618,7 +1672,7 @@ int launch_tile_as(const __bf16* A, const __bf16* W, const float* bias, TC* C, i
       configured = true;
     }
     kernel<<<(int)grid, WM * WN * 64, lds_bytes, s>>>(A, W, bias, C, M, N, K, lda, ldc, tiles_m, tiles_n, vector_ok, K,
-                                                      0);
+                                                      0, norm);
     VK_LAUNCH_CHECK();
     return 0;
   }
@@ -1635,7 +1689,7 @@ int launch_tile_as(const __bf16* A, const __bf16* W, const float* bias, TC* C, i
     const int used = (K + k_per_range - 1) / k_per_range;
     kernel<<<dim3((unsigned)grid, used), WM * WN * 64, lds_bytes, s>>>(A, W, nullptr, partial, M, N, K, lda, N, tiles_m,
                                                                        tiles_n, (N & 3) == 0 ? 1 : 0, k_per_range,
-                                                                       (long long)M * N);
+                                                                       (long long)M * N, norm);
     VK_LAUNCH_CHECK();
     const long long threads = (long long)M * ((N + 3) / 4);
     gemm_reduce_kernel<TC, ACC><<<(int)((threads + 255) / 256), 256, 0, s>>>(partial, bias, C, M, N, ldc, used, vector_ok);
@@ -1717,7 +1771,8 @@ TilePlan choose_tile_plan(int M, int N, int K, long long partial_floats, bool di
 // 256x192 (2,048 tokens x 4,608 rows are 192 such tiles for 256 CUs, against 144 of 256x256).
 template <typename TC, bool ACC, bool GATED = false>
 int launch_tile(const __bf16* A, const __bf16* W, const float* bias, TC* C, int M, int N, int K, long long lda,
-                long long ldc, int vector_ok, float* partial, long long partial_floats, hipStream_t s) {
+                long long ldc, int vector_ok, float* partial, long long partial_floats, hipStream_t s,
+                const TileNorm& norm = TileNorm{}) {
   const bool direct = (K & 63) == 0;
   TilePlan plan = choose_tile_plan(M, N, K, (GATED || !partial) ? 0 : partial_floats, direct, GATED);
   if (g_tile_config >= 0) plan = TilePlan{g_tile_config, g_tile_ranges > 1 && !GATED && partial ? g_tile_ranges : 1};
@@ -1729,14 +1784,15 @@ int launch_tile(const __bf16* A, const __bf16* W, const float* bias, TC* C, int 
   }
   const int r = plan.ranges;
 #define VK_TILE(BMV, BNV, WMV, WNV, DIRECTV) \
-  return launch_tile_as<BMV, BNV, WMV, WNV, TC, ACC, GATED, DIRECTV>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, r, partial, s)
+  return launch_tile_as<BMV, BNV, WMV, WNV, TC, ACC, GATED, DIRECTV>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, r, partial, s, \
+                                                                     norm)
   // the 128-token tiles of the direct kernel with a third LDS stage: up to 128 tokens the product is a stream of
   // the weights (with more tokens, and so more tiles per weight row, two stages measured the same or better)
 #define VK_TILE_DEEP(BMV, BNV, WMV, WNV)                                                                              \
   {                                                                                                                  \
     if (deep)                                                                                                        \
       return launch_tile_as<BMV, BNV, WMV, WNV, TC, ACC, GATED, true, 3>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, r, \
-                                                                         partial, s);                                \
+                                                                         partial, s, norm);                          \
     VK_TILE(BMV, BNV, WMV, WNV, true);                                                                               \
   }
   const bool deep = tile_is_deep(M);
@@ -1755,7 +1811,7 @@ int launch_tile(const __bf16* A, const __bf16* W, const float* bias, TC* C, int 
     case 7:  // three stages fit this tile's LDS, and its loads per product are the most of the 256-token tiles
       if (g_tile_stages != 2)
         return launch_tile_as<256, 128, 4, 2, TC, ACC, GATED, true, 3>(A, W, bias, C, M, N, K, lda, ldc, vector_ok, r,
-                                                                       partial, s);
+                                                                       partial, s, norm);
       VK_TILE(256, 128, 4, 2, true);
     case 8: VK_TILE_DEEP(128, 256, 2, 4);
     case 9: VK_TILE_DEEP(128, 128, 2, 2);
@@ -2060,6 +2116,25 @@ extern "C" int vk_gemm_bf16_gated_scaled(const void* A, const void* W, void* C, 
   if (groups > 512) return VK_UNSUPPORTED_SIZE;  // a thread adds two groups
   return launch_resident_gated<true>((const __bf16*)A, (const __bf16*)W, (__bf16*)C, M, N, K, lda, ldc, sumsq, groups, eps,
                                      (hipStream_t)stream);
+}
+
+// vk_gemm_bf16_gated on the tiled kernel for any number of tokens, with A = x * gain of the norm before and gate
+// and up divided by the root mean square that `sumsq` (`groups` groups of `stride` floats) and `eps` give.
+extern "C" int vk_gemm_bf16_gated_tile_scaled(const void* A, const void* W, void* C, int M, int N, int K, long long lda,
+                                              long long ldc, const float* sumsq, int groups, int stride, float eps,
+                                              void* stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (K <= 0 || (K & 7) || (lda & 7) || lda < K || (N & 31) || ldc < N / 2 || !sumsq || groups <= 0 || stride < M)
+    return VK_BAD_ARGUMENT;
+  if (((uintptr_t)A & 15) || ((uintptr_t)W & 15)) return VK_BAD_ARGUMENT;
+  if (K >= (1 << 23) || lda >= (1 << 23)) return VK_UNSUPPORTED_SIZE;
+  TileNorm norm;
+  norm.sumsq = sumsq;
+  norm.groups = groups;
+  norm.stride = stride;
+  norm.eps = eps;
+  return launch_tile<__bf16, false, true>((const __bf16*)A, (const __bf16*)W, nullptr, (__bf16*)C, M, N, K, lda, ldc, 0,
+                                          nullptr, 0, (hipStream_t)stream, norm);
 }
 
 extern "C" int vk_gemm_bf16_tile_config(int tiling, int ranges, int stages) {

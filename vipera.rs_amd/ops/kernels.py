@@ -489,10 +489,17 @@ def gemm_bf16_follow_supported(a: torch.Tensor, w: torch.Tensor, out: torch.Tens
             and out.is_contiguous() and gemm_bf16_supported(a, w, out))
 
 
-def follow_sumsq_floats(n: int) -> int:
+def follow_stride(tokens: int) -> int:
+    """Floats per group of the sums of squares that the first half of a split norm leaves for ``tokens`` rows: 16 for
+    up to 16 tokens, else the tokens rounded up to a multiple of 64."""
+    return 16 if tokens <= 16 else (tokens + 63) // 64 * 64
+
+
+def follow_sumsq_floats(n: int, tokens: int) -> int:
     """Floats that the sums of squares of :func:`gemm_bf16_follow` and :func:`gemm_bf16_mid_follow` may take for an
-    output of ``n`` columns (16 per workgroup that owns at least 8 columns, or 64 per 1,024 columns)."""
-    return max(((n + 7) // 8) * 16, ((n + 1023) // 1024) * 64)
+    output of ``n`` columns and ``tokens`` rows (16 per workgroup that owns at least 8 columns, or a
+    :func:`follow_stride` per 1,024 columns)."""
+    return max(((n + 7) // 8) * 16, ((n + 1023) // 1024) * follow_stride(tokens))
 
 
 def gemm_bf16_follow(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
@@ -507,7 +514,7 @@ def gemm_bf16_follow(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tens
     _need(gemm_bf16_follow_supported(a, w, out), "gemm_bf16_follow: bfloat16 operands, a float32 output, at most 16 tokens")
     _need(scaled.dtype == torch.bfloat16 and scaled.is_contiguous(), "gemm_bf16_follow: scaled must be bfloat16 [m, n]")
     _need(gain.dtype == torch.float32 and gain.numel() == n and gain.is_contiguous(), "gemm_bf16_follow: gain must be float32 [n]")
-    _need(sumsq.dtype == torch.float32 and sumsq.is_contiguous() and sumsq.numel() >= follow_sumsq_floats(n),
+    _need(sumsq.dtype == torch.float32 and sumsq.is_contiguous() and sumsq.numel() >= follow_sumsq_floats(n, m),
           "gemm_bf16_follow: sumsq is too small")
     if bias is not None:
         _need(bias.dtype == torch.float32 and bias.numel() == n and bias.is_contiguous(), "gemm: bias must be float32 [n]")
@@ -519,11 +526,6 @@ def gemm_bf16_follow(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tens
     _status(fn(_ptr(a), _ptr(w), _ptr(bias), _ptr(out), m, n, k, lda, n, _ptr(gain), _ptr(scaled), n, _ptr(sumsq),
                sumsq.numel(), ctypes.byref(groups), _stream()), "gemm_bf16_follow")
     return int(groups.value)
-
-
-def follow_stride(tokens: int) -> int:
-    """Floats per group of the sums of squares that :func:`gemm_bf16_mid_follow` leaves for ``tokens`` rows."""
-    return 16 if tokens <= 16 else 64
 
 
 def gemm_bf16_mid_follow(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
@@ -541,7 +543,7 @@ def gemm_bf16_mid_follow(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.
           "gemm_bf16_mid_follow: bfloat16 operands and a float32 output")
     _need(scaled.dtype == torch.bfloat16 and scaled.is_contiguous(), "gemm_bf16_mid_follow: scaled must be bfloat16 [m, n]")
     _need(gain.dtype == torch.float32 and gain.numel() == n and gain.is_contiguous(), "gemm_bf16_mid_follow: gain")
-    _need(sumsq.dtype == torch.float32 and sumsq.is_contiguous() and sumsq.numel() >= follow_sumsq_floats(n),
+    _need(sumsq.dtype == torch.float32 and sumsq.is_contiguous() and sumsq.numel() >= follow_sumsq_floats(n, m),
           "gemm_bf16_mid_follow: sumsq is too small")
     if bias is not None:
         _need(bias.dtype == torch.float32 and bias.numel() == n and bias.is_contiguous(), "gemm: bias must be float32 [n]")
@@ -617,6 +619,27 @@ def gemm_bf16_gated_scaled(scaled: torch.Tensor, w: torch.Tensor, out: torch.Ten
     fn = _fn("gemm_bf16", "vk_gemm_bf16_gated_scaled", [_p, _p, _p, _i, _i, _i, _ll, _ll, _p, _i, _f, _p])
     _status(fn(_ptr(scaled), _ptr(w), _ptr(out), m, n, k, lda, ldc, _ptr(sumsq), int(groups), float(eps), _stream()),
             "gemm_bf16_gated_scaled")
+
+
+def gemm_bf16_gated_tile_scaled(scaled: torch.Tensor, w: torch.Tensor, out: torch.Tensor, sumsq: torch.Tensor,
+                                groups: int, eps: float) -> None:
+    """:func:`gemm_bf16_gated` on the tiled kernel, for any number of tokens, on the first half of a split norm:
+    ``scaled`` is ``x * gain`` in bfloat16, and gate and up are divided by the root mean square of ``x`` (from the
+    ``groups`` sums of squares, :func:`follow_stride` floats each, and ``eps``) before the activation."""
+    _dev(scaled, w, out, sumsq)
+    m, k = scaled.shape
+    n = w.shape[0]
+    _need(w.shape[1] == k and out.shape == (m, n // 2) and n % 32 == 0, "gemm_gated: shapes")
+    _need(gemm_bf16_supported(scaled, w, out) and out.dtype == torch.bfloat16, "gemm_gated: operands must be bfloat16")
+    stride = follow_stride(m)
+    _need(sumsq.dtype == torch.float32 and sumsq.is_contiguous() and groups >= 1 and sumsq.numel() >= groups * stride,
+          "gemm_bf16_gated_tile_scaled: sumsq")
+    lda = scaled.stride(0) if m > 1 else max(scaled.stride(0), k)
+    lda = lda if lda % 8 == 0 else k
+    ldc = out.stride(0) if m > 1 else max(out.stride(0), n // 2)
+    fn = _fn("gemm_bf16", "vk_gemm_bf16_gated_tile_scaled", [_p, _p, _p, _i, _i, _i, _ll, _ll, _p, _i, _i, _f, _p])
+    _status(fn(_ptr(scaled), _ptr(w), _ptr(out), m, n, k, lda, ldc, _ptr(sumsq), int(groups), stride, float(eps), _stream()),
+            "gemm_bf16_gated_tile_scaled")
 
 
 TILE_TILINGS = {0: "128x128 staged", 2: "256x128 staged", 3: "128x256 staged", 4: "256x256 staged",

@@ -17,7 +17,7 @@ from ..config.base import PartSpec
 from ..errors import InvalidArgumentError, UnsupportedError
 from ..ops import kernels
 from ..ops.attention import paged_attention
-from ..ops.linear import linear, split_qkv_plan, streams_in_wave_order
+from ..ops.linear import linear, linear_follow, split_qkv_plan, streams_in_wave_order
 from ..weights.checkpoint import MATRIX, VECTOR, TensorSpec
 from .base import KVCacheSpec, Mixer, register_mixer
 
@@ -149,12 +149,10 @@ class Attention(Mixer):
         attn = self.runtime.empty((tokens, self.q_width))
         paged_attention(qkv, cache.k, cache.v, attn, batch, table, self.heads, self.kv_heads, self.head_dim,
                         self.scale, self.window)
-        if (handoff is not None and attn.dtype == torch.bfloat16 and self.w_o.dtype == torch.bfloat16
-                and streams_in_wave_order(tokens, *self.w_o.shape)
-                and kernels.gemm_bf16_follow_supported(attn, self.w_o, residual)):
+        if handoff is not None:
             # the output product also prepares the norm that follows (its gained copy of the residual, its squares)
-            handoff.groups = kernels.gemm_bf16_follow(attn, self.w_o, self.b_o, residual, handoff.gain, handoff.scaled,
-                                                      handoff.sumsq)
+            # where its kernel can; 0 groups say that it could not
+            handoff.groups = linear_follow(attn, self.w_o, self.b_o, residual, handoff.gain, handoff.scaled, handoff.sumsq)
         else:
             linear(attn, self.w_o, self.b_o, residual, accumulate=True)
 

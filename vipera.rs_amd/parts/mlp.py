@@ -48,19 +48,29 @@ class GatedMLP(FeedForward):
         self.w_gate_up = interleave_gate_up(gate, up) if self.interleaved else _cat([gate, up])
         self.w_down = tensors[base + "down_proj.weight"]
 
+    def _dividing_plan(self, tokens: int):
+        """0 or 3 where the gate/up product of ``tokens`` rows runs on a kernel that can divide by the norm in front
+        of it (the kernel with resident activations, the tiled kernel), else None."""
+        if not (self.interleaved and self.w_gate_up.dtype == torch.bfloat16 and self.runtime.dtype == torch.bfloat16):
+            return None
+        if tokens > 64:  # no product before the norm leaves its first half for more than 64 tokens
+            return None
+        plan = gated_plan(tokens, *self.w_gate_up.shape, kernels.compute_units(self.w_gate_up.device))
+        return plan if plan in (0, 3) and (plan == 3 or tokens <= 16) else None
+
     def accepts_handoff(self, tokens: int) -> bool:
-        # where the gate/up product is the kernel with resident activations, which can divide by the norm itself
-        return (self.interleaved and self.w_gate_up.dtype == torch.bfloat16 and self.runtime.dtype == torch.bfloat16
-                and tokens <= 16 and gated_plan(tokens, *self.w_gate_up.shape,
-                                                kernels.compute_units(self.w_gate_up.device)) == 0)
+        return self._dividing_plan(tokens) is not None
 
     fills_handoff = True
 
     def forward(self, h, batch, residual, handoff=None, outgoing=None) -> None:
         tokens = residual.shape[0]
         act = self.runtime.empty((tokens, self.inter))
-        if handoff is not None:
+        if handoff is not None and self._dividing_plan(tokens) == 0:
             kernels.gemm_bf16_gated_scaled(handoff.scaled, self.w_gate_up, act, handoff.sumsq, handoff.groups, handoff.eps)
+        elif handoff is not None:
+            kernels.gemm_bf16_gated_tile_scaled(handoff.scaled, self.w_gate_up, act, handoff.sumsq, handoff.groups,
+                                                handoff.eps)
         else:
             linear_gated(h, self.w_gate_up, act, self.interleaved)
         if outgoing is not None:

@@ -34,7 +34,7 @@ class RMSNorm(Norm):
         if self.runtime.dtype != torch.bfloat16 or self.weight is None or self.weight.dtype != torch.float32:
             return None
         return NormHandoff(self.weight, self.eps, self.runtime.empty((tokens, self.width)),
-                           torch.empty(kernels.follow_sumsq_floats(self.width), dtype=torch.float32,
+                           torch.empty(kernels.follow_sumsq_floats(self.width, tokens), dtype=torch.float32,
                                        device=self.weight.device))
 
     def forward(self, x, out=None, rows=None):
