@@ -446,12 +446,12 @@ extern "C" int plain_attn_bf16_prefill(const void* q, long long q_stride, const 
   return 0;
 }
 
-// entries: the entries that hold exactly one token; `partial`, `chunk` and `chunks` shape the kernel's work only
+// entries: the entries that hold exactly one token; `partial`, `chunk`, `chunks` and `join` shape the kernel's work only
 extern "C" int plain_attn_bf16_decode(const void* q, long long q_stride, const void* k_cache, const void* v_cache,
                                       void* out, float*, const int* entries, int num_entries, const int* entry_start,
                                       const int* entry_first_pos, const int* block_table, int table_width,
                                       int block_size, int heads, int kv_heads, int hd, float scale, int window, int,
-                                      int, int dense, void*) {
+                                      int, int dense, int, void*) {
   if (hd <= 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads || block_size <= 0 || window < 0) return BAD_ARGUMENT;
   for (int e = 0; e < num_entries; ++e) {
     // dense: entry e is the e-th single-token entry and holds token e

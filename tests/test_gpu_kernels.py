@@ -376,6 +376,12 @@ def test_attention_kernels_against_plain_softmax(case, dtype, stale):
                 kernels.attn_bf16_decode(qkv_d, k_d, v_d, out2, partial, dev(torch.tensor(singles, dtype=torch.int32)),
                                          es, fp, table_d, heads, kv_heads, hd, scale, window, chunk, chunks)
                 assert _rel(out2.cpu(), want) < tol, f"matrix-core kernels, chunk {chunk}"
+                if chunks <= kernels.ATTN_DECODE_JOINED_CHUNKS:   # a workgroup that takes all chunks and merges them itself
+                    joined = out2.clone()
+                    joined[[starts[e] for e in singles]] = 7.0
+                    kernels.attn_bf16_decode(qkv_d, k_d, v_d, joined, None, dev(torch.tensor(singles, dtype=torch.int32)),
+                                             es, fp, table_d, heads, kv_heads, hd, scale, window, chunk, chunks, join=True)
+                    assert _rel(joined.cpu(), want) < tol, f"matrix-core kernels, chunk {chunk}, joined"
         assert _rel(out2.cpu(), want) < tol, "matrix-core kernels"
 
 
@@ -412,6 +418,11 @@ def test_decode_attention_over_thousands_of_positions(window):
             kernels.attn_bf16_decode(qkv_d, k_d, v_d, out, partial, singles, es, fp, table_d, heads, kv_heads, hd, scale,
                                      window, chunk, chunks, dense=dense)
             assert _rel(out.cpu(), want) < 1.2e-2, f"chunk {chunk}, dense {dense}"
+            if chunks <= kernels.ATTN_DECODE_JOINED_CHUNKS:
+                out = torch.zeros(len(lengths), heads * hd, dtype=dtype, device=DEV)
+                kernels.attn_bf16_decode(qkv_d, k_d, v_d, out, None, singles, es, fp, table_d, heads, kv_heads, hd, scale,
+                                         window, chunk, chunks, dense=dense, join=True)
+                assert _rel(out.cpu(), want) < 1.2e-2, f"chunk {chunk}, dense {dense}, joined"
 
 
 def _plain_attention_by_head(q, k, v, first_pos, window, scale):
@@ -457,7 +468,7 @@ def test_decode_attention_at_the_benchmark_head_shapes(heads, kv_heads, hd, batc
     In every entry one far key is made to stand out for the first head of each group, so that a chunk or a page
     that is dropped shows."""
     from vipera_rs_amd.ops import kernels
-    from vipera_rs_amd.ops.attention import decode_chunking
+    from vipera_rs_amd.ops.attention import decode_chunking, joins_decode_chunks
     bs, scale, dtype = 16, 1.0 / math.sqrt(hd), torch.bfloat16
     lengths = [(4096, 3000, 2049, 4095, 1, 3001, 130, 4096)[e % 8] for e in range(batch)]
     if batch == 64 and heads != 28:
@@ -503,6 +514,11 @@ def test_decode_attention_at_the_benchmark_head_shapes(heads, kv_heads, hd, batc
         kernels.attn_bf16_decode(qkv_d, k_d, v_d, dense, partial, singles, es, fp, dev(table), heads, kv_heads, hd, scale, 0,
                                  chunk, chunks, dense=True)
         assert torch.equal(dense, out)
+        if joins_decode_chunks(chunks, batch, kv_heads, (group + 15) // 16, 256):   # what the engine does at batch 64
+            joined = torch.zeros(batch, heads * hd, dtype=dtype, device=DEV)
+            kernels.attn_bf16_decode(qkv_d, k_d, v_d, joined, None, singles, es, fp, dev(table), heads, kv_heads, hd, scale,
+                                     0, chunk, chunks, dense=True, join=True)
+            assert _rel(joined.cpu(), want) < 1.2e-2, f"visible {visible}: chunk {chunk} x {chunks}, joined"
     out = torch.zeros(batch, heads * hd, dtype=dtype, device=DEV)
     kernels.attn_generic(qkv_d, k_d, v_d, out, fp, singles, dev(cache.table), heads, kv_heads, hd, scale, 0)
     assert _rel(out.cpu(), want) < 1.2e-2, "32-bit-arithmetic kernel on the bfloat16 cache"

@@ -368,12 +368,13 @@ def test_matrix_core_attention_beside_its_twins(hd, window):
         assert rel_err(got[:count].float().numpy(), want[:count].double().numpy()) < 8e-3
     chunk, chunks = 128, 4
     partial = torch.empty(1 * heads * chunks * (hd + 2))
-    (got, want), = both(module, "attn_bf16_decode",
-                        [qkv, qkv.shape[1], k, v, torch.zeros(T, heads * hd, dtype=torch.bfloat16), partial, i32([1]), 1, entry_start,
-                         first_pos, table, table.shape[1], bs, heads, kv_heads, hd, 1 / math.sqrt(hd), window, chunk, chunks, 0,
-                         None],
-                        [4])
-    assert rel_err(got[count:].float().numpy(), want[count:].double().numpy()) < 8e-3
+    for join in (0, 1):                           # a workgroup per chunk and a merge kernel, or one that merges its waves' chunks
+        (got, want), = both(module, "attn_bf16_decode",
+                            [qkv, qkv.shape[1], k, v, torch.zeros(T, heads * hd, dtype=torch.bfloat16), None if join else partial,
+                             i32([1]), 1, entry_start, first_pos, table, table.shape[1], bs, heads, kv_heads, hd,
+                             1 / math.sqrt(hd), window, chunk, chunks, 0, join, None],
+                            [4])
+        assert rel_err(got[count:].float().numpy(), want[count:].double().numpy()) < 8e-3
 
 
 def test_sampling_kernels_beside_their_twins():

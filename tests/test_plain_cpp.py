@@ -149,7 +149,7 @@ def test_attention_twins_over_a_shuffled_table(window):
     for t in range(13, T):   # each later token as an entry of its own that reads the same pages
         call("plain_attn_bf16_decode", qb, qb.shape[1], kb, vb, low, None, torch.tensor([0], dtype=torch.int32), 1,
              torch.tensor([t, t + 1], dtype=torch.int32), torch.tensor([t], dtype=torch.int32), table, table.shape[1], bs,
-             heads, kv_heads, hd, 1 / math.sqrt(hd), window, 128, 1, 0, None)
+             heads, kv_heads, hd, 1 / math.sqrt(hd), window, 128, 1, 0, 0, None)
     exact = P.attention(qb[:, :heads * hd].double().numpy().reshape(T, heads, hd),
                         kb.double().numpy()[pages].transpose(0, 2, 1, 3).reshape(-1, kv_heads, hd)[:T],
                         vb.double().numpy()[pages].transpose(0, 3, 1, 2).reshape(-1, kv_heads, hd)[:T], window=window)

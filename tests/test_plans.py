@@ -15,6 +15,8 @@ def test_few_tokens_stream_the_weights_with_k_split_inside_a_workgroup():
     assert streams_in_wave_order(8, *DOWN_7B)              # up to 8 tokens also with a long K: no second kernel for K ranges
     assert streams_in_wave_order(8, 1536, 8960)
     assert not streams_in_wave_order(9, *DOWN_7B)          # past 8 tokens activations are shared through LDS instead
+    assert not streams_in_wave_order(1, 5120, 27648) and not streams_in_wave_order(8, 5120, 27648)   # the 32B down projection
+    assert streams_in_wave_order(1, 152064, 5120) and streams_in_wave_order(8, 5120, 5120)
     assert not streams_in_wave_order(8, *HEAD_7B)          # many rows: likewise
     assert not streams_in_wave_order(17, *QKV_7B)
 
@@ -22,6 +24,8 @@ def test_few_tokens_stream_the_weights_with_k_split_inside_a_workgroup():
 def test_the_lds_shared_product_splits_k_where_rows_are_few():
     assert mid_plan(8, *DOWN_7B) == (4, 1)                 # 56 row blocks x 4 ranges fill 256 CUs
     assert mid_plan(64, *DOWN_7B) == (9, 2)                # many tokens and a long K: two tiles per wave, 28 row blocks x 9
+    assert mid_plan(32, 5120, 27648) == (6, 2) and mid_plan(31, 5120, 27648) == (3, 1)
+    assert mid_plan(64, 1536, 8960) == (10, 1)             # few rows: one tile per wave, 24 row blocks x 10
     assert mid_plan(8, *HEAD_7B) == (1, 1) and mid_plan(64, *HEAD_7B) == (1, 2)
     assert mid_plan(64, *QKV_7B) == (3, 1) and mid_plan(64, *O_7B) == (4, 1)
     ranges, _ = mid_plan(64, 2048, 1536)                   # 1.5B q/k/v: no range shorter than 512

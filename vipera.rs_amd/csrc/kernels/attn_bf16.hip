@@ -774,14 +774,22 @@ __global__ __launch_bounds__(SPLIT ? 2 * PT_THREADS : PT_THREADS) void attn_pref
 // one key head. Chunk c covers positions [c * chunk, (c + 1) * chunk) of the visible range and leaves
 // (max, sum, weighted sum) in `partial`: [entry, head, chunk, hd + 2] floats. REGS: a chunk spans at most
 // 64 pages, whose ids the wave reads once.
-template <bool REGS>
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void attn_decode_kernel(
+// JOINED: grid (entries, kv_heads * head_blocks), a workgroup of `chunks` waves (at most JOINED_WAVES), wave c
+// taking chunk c; the waves leave (max, sum, weighted sum) in LDS and merge them there, wave w the output tiles
+// w, w + chunks, ... in ascending order of the chunks, and write `out` themselves: no `partial`, no second kernel.
+// For steps whose (entry, key head) pairs alone fill the GPU (64 requests x 4 key heads), where the chunks only
+// serve to keep several waves on a CU.
+constexpr int JOINED_WAVES = 8;
+template <bool REGS, bool JOINED>
+__global__ __launch_bounds__(JOINED ? JOINED_WAVES * 64 : 64) __attribute__((amdgpu_waves_per_eu(2))) void attn_decode_kernel(
     const __bf16* __restrict__ q, long long q_stride, const __bf16* __restrict__ k_cache,
-    const __bf16* __restrict__ v_cache, float* __restrict__ partial, const int* __restrict__ entries,
-    const int* __restrict__ entry_start, const int* __restrict__ entry_first_pos,
+    const __bf16* __restrict__ v_cache, float* __restrict__ partial, __bf16* __restrict__ out,
+    const int* __restrict__ entries, const int* __restrict__ entry_start, const int* __restrict__ entry_first_pos,
     const int* __restrict__ block_table, int table_width, int block_size, int heads, int kv_heads, int hd,
     float scale, int window, int chunk, int head_blocks, int dense) {
   const int lane = threadIdx.x & 63, lr = lane & 15, lg = lane >> 4;
+  const int wave = JOINED ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) : 0;
+  const int chunk_index = JOINED ? wave : blockIdx.z, chunks = JOINED ? (int)(blockDim.x >> 6) : (int)gridDim.z;
   // dense: entry i is slot i and holds token i (a step of single tokens only), which saves two reads that the
   // position, and with it every other read, would wait for
   const int slot = blockIdx.x, entry = dense ? slot : entries[slot];
@@ -792,35 +800,74 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void at
   // without a window a chunk's first page does not depend on the position: its page ids are asked for beside it
   int early_pages = -1;
   if (REGS && window == 0)
-    early_pages = block_table[(size_t)entry * table_width + min(ps.page(blockIdx.z * chunk) + lane, table_width - 1)];
+    early_pages = block_table[(size_t)entry * table_width + min(ps.page(chunk_index * chunk) + lane, table_width - 1)];
   const int pos = entry_first_pos[entry];
   const int lo = (window > 0 && pos + 1 > window) ? pos + 1 - window : 0;
-  const int begin = max(lo, blockIdx.z * chunk), end = min(pos + 1, (blockIdx.z + 1) * chunk);
+  const int begin = max(lo, chunk_index * chunk), end = min(pos + 1, (chunk_index + 1) * chunk);
   const int head_in_group = hb * 16 + lr;
   const bool col_ok = head_in_group < group;
   const int h = kvh * group + head_in_group;
-  float* dst = partial + (((size_t)slot * heads + (col_ok ? h : 0)) * gridDim.z + blockIdx.z) * (hd + 2);
-  if (begin >= end) {  // nothing of this chunk is visible
-    if (col_ok && lg == 0) {
-      dst[hd] = -INFINITY;
-      dst[hd + 1] = 0.f;
-    }
-    return;
-  }
-  bf16x8 qf[KS];
-  load_q(col_ok ? q + (size_t)token * q_stride + (size_t)h * hd : nullptr, hd, qf);
-  CacheView cv{k_cache, v_cache, block_table + (size_t)entry * table_width, table_width, ps,
-               kv_heads, hd, kvh, ps.page(begin), early_pages};
-  if (REGS && window != 0) {
-    const int index = cv.page0 + lane;
-    if (index <= ps.page(end - 1) && index < table_width) cv.pages = cv.table[index];
-  }
+  float* dst = partial + (((size_t)slot * heads + (col_ok ? h : 0)) * chunks + chunk_index) * (hd + 2);
   f32x4 o[DT];
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
-  attend_range<REGS>(qf, lo, col_ok ? pos : -1, begin, end, cv, scale, o, m, l);
-  l = sum_of_column(l);
+  if (begin >= end) {  // nothing of this chunk is visible
+    if constexpr (!JOINED) {
+      if (col_ok && lg == 0) {
+        dst[hd] = -INFINITY;
+        dst[hd + 1] = 0.f;
+      }
+      return;
+    }
+  } else {
+    bf16x8 qf[KS];
+    load_q(col_ok ? q + (size_t)token * q_stride + (size_t)h * hd : nullptr, hd, qf);
+    CacheView cv{k_cache, v_cache, block_table + (size_t)entry * table_width, table_width, ps,
+                 kv_heads, hd, kvh, ps.page(begin), early_pages};
+    if (REGS && window != 0) {
+      const int index = cv.page0 + lane;
+      if (index <= ps.page(end - 1) && index < table_width) cv.pages = cv.table[index];
+    }
+    attend_range<REGS>(qf, lo, col_ok ? pos : -1, begin, end, cv, scale, o, m, l);
+    l = sum_of_column(l);
+  }
+  if constexpr (JOINED) {
+    extern __shared__ __attribute__((aligned(16))) float joined_lds[];
+    f32x4* sums = (f32x4*)joined_lds;                              // [chunks][DT][64]
+    float* max_sum = joined_lds + (size_t)chunks * DT * 64 * 4;    // [chunks][16][2]
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) sums[(wave * DT + dt) * 64 + lane] = o[dt];
+    if (lg == 0) {
+      max_sum[(wave * 16 + lr) * 2] = m;
+      max_sum[(wave * 16 + lr) * 2 + 1] = l;
+    }
+    __syncthreads();
+    // out = sum_c acc_c e^(m_c - M) / sum_c l_c e^(m_c - M) with M = max m_c, as attn_combine_kernel merges
+    float best = -INFINITY;
+    for (int c = 0; c < chunks; ++c) best = fmaxf(best, max_sum[(c * 16 + lr) * 2]);
+    float total = 0.f;
+    for (int c = 0; c < chunks; ++c) {
+      const float mc = max_sum[(c * 16 + lr) * 2];
+      total += (mc > -INFINITY ? __expf(mc - best) : 0.f) * max_sum[(c * 16 + lr) * 2 + 1];
+    }
+    const float inv = 1.f / total;
+    for (int dt = wave; dt < DT; dt += chunks) {
+      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+      for (int c = 0; c < chunks; ++c) {
+        const float mc = max_sum[(c * 16 + lr) * 2];
+        if (mc > -INFINITY) acc += sums[(c * DT + dt) * 64 + lane] * __expf(mc - best);   // an empty chunk adds nothing
+      }
+      const int d = dt * 16 + lg * 4;
+      if (col_ok && d < hd) {
+        bf16x4 r;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) r[j] = (__bf16)(acc[j] * inv);
+        *(bf16x4*)(out + (size_t)token * heads * hd + (size_t)h * hd + d) = r;
+      }
+    }
+    return;
+  }
   if (!col_ok) return;
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) {
@@ -973,27 +1020,47 @@ extern "C" int vk_attn_bf16_prefill(const void* q, long long q_stride, const voi
 
 // entries: indices of the step's entries that hold exactly one token. partial: at least
 // num_entries * heads * chunks * (hd + 2) floats. `chunks` must cover the longest visible range:
-// chunks * chunk >= longest position + 1.
+// chunks * chunk >= longest position + 1. `join` nonzero: one workgroup of `chunks` waves (at most 8) per entry and
+// key head merges its chunks itself and writes `out`; `partial` is not used and may be null.
 extern "C" int vk_attn_bf16_decode(const void* q, long long q_stride, const void* k_cache, const void* v_cache,
                                    void* out, float* partial, const int* entries, int num_entries,
                                    const int* entry_start, const int* entry_first_pos, const int* block_table,
                                    int table_width, int block_size, int heads, int kv_heads, int hd, float scale,
-                                   int window, int chunk, int chunks, int dense, void* stream) {
+                                   int window, int chunk, int chunks, int dense, int join, void* stream) {
   if (num_entries <= 0) return 0;
   if (hd <= 0 || hd > HDP || (hd & 7) || block_size <= 0 || (block_size & 7) || heads <= 0 || kv_heads <= 0 ||
       heads % kv_heads || (q_stride & 7) || window < 0 || chunk < 32 || (chunk & 31) || chunks <= 0 ||
       chunks > MAX_CHUNKS)
     return VK_UNSUPPORTED_SIZE;
+  if (join && chunks > JOINED_WAVES) return VK_UNSUPPORTED_SIZE;
+  if (!join && !partial) return VK_BAD_ARGUMENT;
   const int group = heads / kv_heads, head_blocks = (group + 15) / 16;
   if (kv_heads * head_blocks > 65535 || heads > 65535) return VK_UNSUPPORTED_SIZE;
   hipStream_t s = (hipStream_t)stream;
-  dim3 grid(num_entries, kv_heads * head_blocks, chunks);
   // pages a chunk can touch: chunks start at multiples of `chunk`, which need not be page edges
   const int chunk_pages = chunk % block_size == 0 ? chunk / block_size : chunk / block_size + 2;
-  auto kernel = chunk_pages <= 64 ? attn_decode_kernel<true> : attn_decode_kernel<false>;
+  if (join) {
+    auto kernel = chunk_pages <= 64 ? attn_decode_kernel<true, true> : attn_decode_kernel<false, true>;
+    const int lds_bytes = chunks * (DT * 64 * 16 + 16 * 2 * 4);
+    static bool configured[2] = {false, false};
+    if (!configured[chunk_pages <= 64]) {
+      hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         JOINED_WAVES * (DT * 64 * 16 + 16 * 2 * 4));
+      if (e != hipSuccess) return (int)e;
+      configured[chunk_pages <= 64] = true;
+    }
+    kernel<<<dim3(num_entries, kv_heads * head_blocks), chunks * 64, lds_bytes, s>>>(
+        (const __bf16*)q, q_stride, (const __bf16*)k_cache, (const __bf16*)v_cache, nullptr, (__bf16*)out, entries,
+        entry_start, entry_first_pos, block_table, table_width, block_size, heads, kv_heads, hd, scale, window, chunk,
+        head_blocks, dense);
+    VK_LAUNCH_CHECK();
+    return 0;
+  }
+  dim3 grid(num_entries, kv_heads * head_blocks, chunks);
+  auto kernel = chunk_pages <= 64 ? attn_decode_kernel<true, false> : attn_decode_kernel<false, false>;
   kernel<<<grid, 64, 0, s>>>((const __bf16*)q, q_stride, (const __bf16*)k_cache, (const __bf16*)v_cache, partial,
-                             entries, entry_start, entry_first_pos, block_table, table_width, block_size, heads,
-                             kv_heads, hd, scale, window, chunk, head_blocks, dense);
+                             (__bf16*)out, entries, entry_start, entry_first_pos, block_table, table_width, block_size,
+                             heads, kv_heads, hd, scale, window, chunk, head_blocks, dense);
   VK_LAUNCH_CHECK();
   dim3 cgrid(num_entries, heads);
   attn_combine_kernel<<<cgrid, CB_THREADS, 0, s>>>(partial, (__bf16*)out, entries, entry_start, heads, hd, chunks);

@@ -695,13 +695,19 @@ def attn_bf16_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
                heads, kv_heads, head_dim, float(scale), int(window), 1 if split else 0, _stream()), "attn_bf16_prefill")
 
 
+ATTN_DECODE_JOINED_CHUNKS = 8   # waves of a workgroup that merges its chunks itself
+
+
 def attn_bf16_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
                      partial: torch.Tensor, entries: torch.Tensor, entry_start: torch.Tensor,
                      entry_first_pos: torch.Tensor, block_table: torch.Tensor, heads: int, kv_heads: int,
-                     head_dim: int, scale: float, window: int, chunk: int, chunks: int, dense: bool = False) -> None:
+                     head_dim: int, scale: float, window: int, chunk: int, chunks: int, dense: bool = False,
+                     join: bool = False) -> None:
     """Attention of the single-token entries listed in ``entries``, positions split into ``chunks`` of ``chunk``.
     ``dense``: the step holds single-token entries only, so entry i is the i-th of them and holds token i; the
-    kernel then need not look either up."""
+    kernel then need not look either up.  ``join``: one workgroup per entry and key head takes all chunks (at most
+    ``ATTN_DECODE_JOINED_CHUNKS``), a wave each, and merges them itself; ``partial`` is then not used and may be
+    None."""
     _dev(q, k_cache, v_cache, out, partial, entries, entry_start, entry_first_pos, block_table)
     _need(attn_bf16_supported(q, k_cache, head_dim), "attn_bf16: operands must be bfloat16 with 16-byte rows")
     _need(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= heads * head_dim, "attention: q")
@@ -709,17 +715,20 @@ def attn_bf16_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     _need(_cache_ok(k_cache, v_cache, kv_heads, head_dim, q.dtype), "attention: cache shape or dtype")
     count = entries.numel()
     _need(entries.dtype == torch.int32 and entries.is_contiguous(), "attention: entries")
-    _need(partial.dtype == torch.float32 and partial.is_contiguous()
-          and partial.numel() >= count * heads * chunks * (head_dim + 2), "attention: workspace too small")
+    if join:
+        _need(chunks <= ATTN_DECODE_JOINED_CHUNKS, "attention: too many chunks for one workgroup")
+    else:
+        _need(partial is not None and partial.dtype == torch.float32 and partial.is_contiguous()
+              and partial.numel() >= count * heads * chunks * (head_dim + 2), "attention: workspace too small")
     _need(chunk >= 32 and chunk % 32 == 0 and chunks >= 1, "attention: chunk must be a multiple of 32")
     _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(), "attention: table")
     module = f"attn_bf16_hd{attn_bf16_padded_width(head_dim)}"
     fn = _fn(module, "vk_attn_bf16_decode",
-             [_p, _ll, _p, _p, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _f, _i, _i, _i, _i, _p], key=module + ".decode")
+             [_p, _ll, _p, _p, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _f, _i, _i, _i, _i, _i, _p], key=module + ".decode")
     _status(fn(_ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(partial), _ptr(entries), count,
                _ptr(entry_start), _ptr(entry_first_pos), _ptr(block_table), block_table.shape[1], k_cache.shape[2],
                heads, kv_heads, head_dim, float(scale), int(window), int(chunk), int(chunks), 1 if dense else 0,
-               _stream()),
+               1 if join else 0, _stream()),
             "attn_bf16_decode")
 
 

@@ -42,17 +42,24 @@ def mid_plan(m: int, n: int, k: int) -> Tuple[int, int]:
         return (2, 1) if m > 16 else (1, 1)
     # few weight rows: split K while the workgroups still fit the 256 CUs at once (one more range was
     # measured a third slower), each range at least two chunks long
-    # with many tokens and a long K, two tiles per wave and twice the ranges measured a tenth faster
-    rows_per_wave = 2 if m > 32 and k >= 8_192 else 1
+    # with many tokens, a long K and enough rows, two tiles per wave and twice the ranges measured a tenth faster (the
+    # 32B down projection at 32 tokens 54.7 against 60.6 us); with few rows one tile and fewer ranges (the 1.5B down
+    # projection at 64 tokens 13.0 against 15.7)
+    rows_per_wave = 2 if m >= 32 and k >= 8_192 and n >= 2_048 else 1
     row_blocks = (n + 64 * rows_per_wave - 1) // (64 * rows_per_wave)
     return max(1, min(k // 512, 256 // row_blocks)), rows_per_wave
 
 
 def streams_in_wave_order(m: int, n: int, k: int) -> bool:
     """Whether a bfloat16 product of ``m`` tokens runs on the kernel whose waves split K inside a workgroup: up to 4
-    tokens always; up to 8 where the weight has few rows, also with a long K (every workgroup reads all activations,
+    tokens; up to 8 where the weight has few rows, also with a long K (every workgroup reads all activations,
     but there is no second kernel that adds K ranges: the down projection at 8 tokens 30.2 against 28.2 + 4.9 us at
-    the 7B widths, 12.1 against 11.1 + 6.2 at the 1.5B widths); up to 16 with a short K as well."""
+    the 7B widths, 12.1 against 11.1 + 6.2 at the 1.5B widths); up to 16 with a short K as well.  Not for a weight
+    of few rows and more than 100 M elements, whose workgroups would each stream most of a megabyte through four
+    waves (the 32B down projection, 5,120 x 27,648: 62.2 us against 50.7 + 5 with K split over workgroups at one
+    token, 67.9 against 52.2 + 5 at eight)."""
+    if n < 16_384 and n * k > 100_000_000:
+        return False
     return m <= 4 or (m <= 8 and n < 16_384) or (m <= 16 and n < 16_384 and k < 8_192)
 
 
