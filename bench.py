@@ -282,7 +282,7 @@ def kernel_split(args, config, runner, tokens, ctx, T):
     H, V, I = config.hidden_size, config.vocab_size, config.intermediate_size
     Q, KV = config.num_attention_heads * config.head_dim, config.num_key_value_heads * config.head_dim
     products = {(Q + 2 * KV, H): "qkv", (H, Q): "output", (2 * I, H): "gate_up", (H, I): "down", (V, H): "head"}
-    other = {"attn_bf16_prefill": "attention", "attn_bf16_decode": "attention", "attn_generic": "attention", "attn_decode_f32": "attention",
+    other = {"attn_bf16_prefill": "attention", "attn_bf16_decode": "attention", "attn_generic": "attention", "attn_decode_f32": "attention", "attn_prefill_f32": "attention",
              "rmsnorm": "norms", "rope_kvwrite": "rope_kvwrite", "rope_angles": "rope_kvwrite",
              "embed_gather": "embedding", "sample": "sampler", "swiglu": "swiglu", "fetch_words": "metadata"}
 

@@ -36,6 +36,7 @@ SIGNATURES = {
     "plain_gemm_bf16_mid_qkv_rope": [P, P, P, P, I, I, I, LL, LL, I, I, P, LL, P, P, P, P, P, P, I, I, I, I, I, P, I, I, F, P],
     "plain_attn_generic": [P, LL, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, P, P],
     "plain_attn_decode_f32": [P, LL, P, P, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, P],
+    "plain_attn_prefill_f32": [P, LL, P, P, P, P, I, I, P, P, P, I, I, I, I, I, F, I, P],
     "plain_attn_bf16_prefill": [P, LL, P, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, P],
     "plain_attn_bf16_decode": [P, LL, P, P, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, I, I, I, P],
     "plain_sample": [P, I, I, P, P, P, P, P, P, P, P, I, P, P, P, P, P, I, P],

@@ -427,6 +427,26 @@ extern "C" int plain_attn_decode_f32(const float* q, long long q_stride, const f
   return 0;
 }
 
+// tiles: pairs (entry, first token of the tile within the entry), `tile_tokens` tokens per tile
+extern "C" int plain_attn_prefill_f32(const float* q, long long q_stride, const float* k_cache, const float* v_cache,
+                                      float* out, const int* tiles, int num_tiles, int tile_tokens,
+                                      const int* entry_start, const int* entry_first_pos, const int* block_table,
+                                      int table_width, int block_size, int heads, int kv_heads, int hd, float scale,
+                                      int window, void*) {
+  if (hd <= 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads || block_size <= 0 || window < 0 || tile_tokens <= 0)
+    return BAD_ARGUMENT;
+  for (int tile = 0; tile < num_tiles; ++tile) {
+    const int entry = tiles[2 * tile], off = tiles[2 * tile + 1];
+    const int tok0 = entry_start[entry], count = entry_start[entry + 1] - tok0;
+    for (int i = off; i < std::min(off + tile_tokens, count); ++i)
+      for (int h = 0; h < heads; ++h)
+        attend(q + (size_t)(tok0 + i) * q_stride + (size_t)h * hd, k_cache, v_cache, DT_F32,
+               block_table + (size_t)entry * table_width, block_size, kv_heads, h / (heads / kv_heads), hd, scale,
+               entry_first_pos[entry] + i, window, out + (size_t)(tok0 + i) * heads * hd + (size_t)h * hd);
+  }
+  return 0;
+}
+
 // tiles: pairs (entry, first token of the tile within the entry), 128 tokens per tile
 extern "C" int plain_attn_bf16_prefill(const void* q, long long q_stride, const void* k_cache, const void* v_cache,
                                        void* out, const int* tiles, int num_tiles, const int* entry_start,

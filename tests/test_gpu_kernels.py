@@ -283,6 +283,16 @@ class _Paged:
         self.table = torch.full((len(seqs), width), -1, dtype=torch.int32)
         for i, t in enumerate(self.tables):
             self.table[i, :len(t)] = torch.tensor(t, dtype=torch.int32)
+        self.spare = order.pop()        # a page that no request holds
+
+    def with_pages_given_back(self, first_visible):
+        """The table after a window has passed: the blocks of entry i that lie wholly before position
+        ``first_visible[i]`` name a page that nobody holds (in the engine their id is -1, which must not be followed;
+        a kernel that reads such a block here reads what the spare page holds, NaN in the tests that say so)."""
+        table = self.table.clone()
+        for i, first in enumerate(first_visible):
+            table[i, :first // self.block_size] = self.spare
+        return table
 
 
 ATTN_CASES = [
@@ -331,7 +341,9 @@ def test_attention_kernels_against_plain_softmax(case, dtype, stale):
                                                          first[e], window, scale)
     want = want.view(T, heads * hd)
     dev = lambda t: t.to(DEV)  # noqa: E731
-    qkv_d, k_d, v_d, table_d = dev(qkv), dev(cache.k), dev(cache.v), dev(cache.table)
+    # with a window, the pages that the first token of an entry no longer sees have been given back
+    table = cache.with_pages_given_back([max(0, first[e] + 1 - window) for e in range(len(entries))]) if window else cache.table
+    qkv_d, k_d, v_d, table_d = dev(qkv), dev(cache.k), dev(cache.v), dev(table)
     tol = 2e-6 if dtype == torch.float32 else 1.2e-2
 
     out = torch.zeros(T, heads * hd, dtype=dtype, device=DEV)
@@ -352,6 +364,17 @@ def test_attention_kernels_against_plain_softmax(case, dtype, stale):
         kernels.attn_generic(qkv_d, k_d, v_d, out3, dev(positions), dev(entry_of), table_d, heads, kv_heads, hd, scale, window,
                              skip_single_of=es)
         assert _rel(out3.cpu(), want) < tol, "32-bit decode kernel beside the general one"
+        if kernels.attn_prefill_f32_supported(qkv_d, k_d, hd):
+            # the portions on the 32-bit kernel that walks the positions in LDS tiles; tiles of 128 or of 64 tokens
+            for tile_tokens in (128, 64):
+                tiles = [x for e, n in enumerate(counts) if n > 1 for off in range(0, n, tile_tokens) for x in (e, off)]
+                rows = [t for e, n in enumerate(counts) if n > 1 for t in range(starts[e], starts[e + 1])]
+                out4 = torch.full((T, heads * hd), float("nan"), dtype=dtype, device=DEV)
+                kernels.attn_prefill_f32(qkv_d, k_d, v_d, out4, dev(torch.tensor(tiles, dtype=torch.int32)), tile_tokens, es,
+                                         fp, table_d, heads, kv_heads, hd, scale, window)
+                assert _rel(out4.cpu()[rows], want[rows]) < tol, f"32-bit prompt kernel, tiles of {tile_tokens}"
+                others = [t for t in range(T) if t not in set(rows)]
+                assert bool(torch.isnan(out4.cpu()[others]).all()), "the prompt kernel wrote a single token's row"
 
     if dtype == torch.bfloat16:
         from vipera_rs_amd.engine.batch import TILE_TOKENS

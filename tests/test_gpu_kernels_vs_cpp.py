@@ -348,6 +348,25 @@ def test_32_bit_decode_attention_beside_its_twin(heads, kv_heads, hd, bs, window
     assert float(got[:len(lengths)].abs().max()) == 0.0          # and the single tokens not the general kernel's
 
 
+@pytest.mark.parametrize("heads,kv_heads,hd,bs", [(6, 3, 48, 8), (7, 1, 128, 16), (4, 2, 16, 4), (3, 3, 112, 32)])
+@pytest.mark.parametrize("window", [0, 90])
+def test_32_bit_prompt_attention_beside_its_twin(heads, kv_heads, hd, bs, window):
+    """A portion of 300 tokens after 200 cached ones (its first tile begins inside a tile of positions, its last is
+    short) and a second portion of 3 tokens from position 0, beside a single token that is not this kernel's."""
+    first, count = 200, 300
+    k, v, table = _paged(first + count, kv_heads, hd, bs, torch.float32, hd + heads, entries=3)
+    g = torch.Generator().manual_seed(hd + 2)
+    T = count + 3 + 1
+    qkv = torch.randn(T, (heads + 2 * kv_heads) * hd, generator=g)
+    entry_start, first_pos = i32([0, count, count + 3, count + 4]), i32([first, 0, 77])
+    tiles = i32([0, 256, 1, 0, 0, 0, 0, 128])     # any order of the tiles
+    (got, want), = both("attn_generic", "attn_prefill_f32",
+                        [qkv, qkv.shape[1], k, v, torch.zeros(T, heads * hd), tiles, 4, 128, entry_start, first_pos, table,
+                         table.shape[1], bs, heads, kv_heads, hd, 1 / math.sqrt(hd), window, None], [4])
+    assert rel_err(got[:count + 3].numpy(), want[:count + 3].double().numpy()) < 3e-6
+    assert float(got[count + 3:].abs().max()) == 0.0
+
+
 @pytest.mark.parametrize("hd", [64, 128, 80])
 @pytest.mark.parametrize("window", [0, 150])
 def test_matrix_core_attention_beside_its_twins(hd, window):

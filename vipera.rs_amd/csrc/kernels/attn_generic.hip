@@ -156,32 +156,47 @@ __global__ __launch_bounds__(256) void attn_decode_f32_kernel(
                                              : f32x4{0.f, 0.f, 0.f, 0.f};
     }
   if (wave_sees) {
-    for (int it = 0; it < DEC_WAVE / 4; ++it) {
-      const int p = wave_begin + it * 4 + ps;
-      const int pc = min(max(p, lo), pos);       // a position outside the range reads one inside it; its score is masked
-      const float* row = k_cache + (((size_t)table[pc / block_size] * kv_heads + kvh) * block_size + pc % block_size) * hd;
-      float dot[HB];
+    // Eight steps of four positions at a time: their page ids are requested together, then their K rows, and only
+    // then is anything multiplied. A step at a time (look up the page, wait, fetch the row, wait, multiply) made
+    // the kernel sixteen pairs of round trips long: 96 us a layer for 134 MB at the 7B shape. No load sits behind
+    // a condition: a dim past the head width reads the last four dims again (its q is zero).
+    constexpr int AHEAD = 8;
+    for (int it0 = 0; it0 < DEC_WAVE / 4; it0 += AHEAD) {
+      int at[AHEAD], page[AHEAD];
 #pragma unroll
-      for (int h = 0; h < HB; ++h) dot[h] = 0.f;
+      for (int b = 0; b < AHEAD; ++b) {
+        const int p = wave_begin + (it0 + b) * 4 + ps;
+        at[b] = min(max(p, lo), pos);   // a position outside the range reads one inside it; its score is masked
+        page[b] = table[at[b] / block_size];
+      }
+      f32x4 k4[AHEAD][QC];
 #pragma unroll
-      for (int i = 0; i < QC; ++i) {
-        const int d = c * 4 + 64 * i;
-        if (d < hd) {
-          const f32x4 k4 = *(const f32x4*)(row + d);
+      for (int b = 0; b < AHEAD; ++b) {
+        const float* row = k_cache + (((size_t)page[b] * kv_heads + kvh) * block_size + at[b] % block_size) * hd;
 #pragma unroll
-          for (int h = 0; h < HB; ++h) {
-            dot[h] = fmaf(qr[h][i][0], k4[0], dot[h]);
-            dot[h] = fmaf(qr[h][i][1], k4[1], dot[h]);
-            dot[h] = fmaf(qr[h][i][2], k4[2], dot[h]);
-            dot[h] = fmaf(qr[h][i][3], k4[3], dot[h]);
-          }
-        }
+        for (int i = 0; i < QC; ++i) k4[b][i] = *(const f32x4*)(row + min(c * 4 + 64 * i, hd - 4));
       }
 #pragma unroll
-      for (int h = 0; h < HB; ++h) {
+      for (int b = 0; b < AHEAD; ++b) {
+        const int p = wave_begin + (it0 + b) * 4 + ps;
+        float dot[HB];
 #pragma unroll
-        for (int off = 1; off < 16; off <<= 1) dot[h] += __shfl_xor(dot[h], off, WAVE);
-        if (c == 0) sw[wave][h][it * 4 + ps] = (p >= lo && p <= pos) ? dot[h] * scale : -INFINITY;
+        for (int h = 0; h < HB; ++h) dot[h] = 0.f;
+#pragma unroll
+        for (int i = 0; i < QC; ++i)
+#pragma unroll
+          for (int h = 0; h < HB; ++h) {
+            dot[h] = fmaf(qr[h][i][0], k4[b][i][0], dot[h]);
+            dot[h] = fmaf(qr[h][i][1], k4[b][i][1], dot[h]);
+            dot[h] = fmaf(qr[h][i][2], k4[b][i][2], dot[h]);
+            dot[h] = fmaf(qr[h][i][3], k4[b][i][3], dot[h]);
+          }
+#pragma unroll
+        for (int h = 0; h < HB; ++h) {
+#pragma unroll
+          for (int off = 1; off < 16; off <<= 1) dot[h] += __shfl_xor(dot[h], off, WAVE);
+          if (c == 0) sw[wave][h][(it0 + b) * 4 + ps] = (p >= lo && p <= pos) ? dot[h] * scale : -INFINITY;
+        }
       }
     }
   }
@@ -206,31 +221,37 @@ __global__ __launch_bounds__(256) void attn_decode_f32_kernel(
 #pragma unroll
     for (int i = 0; i < OD; ++i) o[h][i] = 0.f;
   if (wave_sees) {
+    // the four quads' pages first, then their values, no load behind a condition: a quad of which the token sees
+    // nothing reads the quad of its own position instead (whose page is held) and counts as zeros
+    const float* quad[4];
+    bool sees[4][4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int p0 = wave_begin + (qs + 4 * j) * 4;             // four positions of one page
-      if (p0 > pos || p0 + 3 < lo) continue;
-      bool sees[4];
+      const bool any = p0 <= pos && p0 + 3 >= lo;
+      const int from = any ? p0 : (pos & ~3);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) sees[e] = p0 + e >= lo && p0 + e <= pos;
-      const float* page = v_cache + ((size_t)table[p0 / block_size] * kv_heads + kvh) * hd * block_size + p0 % block_size;
+      for (int e = 0; e < 4; ++e) sees[j][e] = any && p0 + e >= lo && p0 + e <= pos;
+      quad[j] = v_cache + ((size_t)table[from / block_size] * kv_heads + kvh) * hd * block_size + from % block_size;
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      f32x4 v4[OD];
+#pragma unroll
+      for (int i = 0; i < OD; ++i) v4[i] = *(const f32x4*)(quad[j] + (size_t)min(dg + 16 * i, hd - 1) * block_size);
       f32x4 w4[HB];
 #pragma unroll
       for (int h = 0; h < HB; ++h) w4[h] = *(const f32x4*)&sw[wave][h][(qs + 4 * j) * 4];
 #pragma unroll
       for (int i = 0; i < OD; ++i) {
-        const int d = dg + 16 * i;
-        if (d < hd) {
-          f32x4 v4 = *(const f32x4*)(page + (size_t)d * block_size);
 #pragma unroll
-          for (int e = 0; e < 4; ++e) v4[e] = sees[e] ? v4[e] : 0.f;
+        for (int e = 0; e < 4; ++e) v4[i][e] = sees[j][e] ? v4[i][e] : 0.f;
 #pragma unroll
-          for (int h = 0; h < HB; ++h) {
-            o[h][i] = fmaf(w4[h][0], v4[0], o[h][i]);
-            o[h][i] = fmaf(w4[h][1], v4[1], o[h][i]);
-            o[h][i] = fmaf(w4[h][2], v4[2], o[h][i]);
-            o[h][i] = fmaf(w4[h][3], v4[3], o[h][i]);
-          }
+        for (int h = 0; h < HB; ++h) {   // a dim past the head width adds into a sum that is never stored
+          o[h][i] = fmaf(w4[h][0], v4[i][0], o[h][i]);
+          o[h][i] = fmaf(w4[h][1], v4[i][1], o[h][i]);
+          o[h][i] = fmaf(w4[h][2], v4[i][2], o[h][i]);
+          o[h][i] = fmaf(w4[h][3], v4[i][3], o[h][i]);
         }
       }
     }
@@ -299,6 +320,188 @@ __global__ __launch_bounds__(64) void attn_combine_f32_kernel(const float* __res
     }
     out[(size_t)token * heads * hd + (size_t)h * hd + d] = from_float<T>(total / sum);
   }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Prompt portions in 32-bit. The general kernel gives every (token, query head) a workgroup that walks all of the
+// token's positions alone: 2,048 tokens x 28 heads read the cache 58 GB over per layer. Here a workgroup owns 64
+// consecutive tokens of one entry and one query head and walks the positions in tiles of 64 that begin at
+// multiples of 64 (so which positions share a tile, and with it a token's arithmetic, depends on the position alone,
+// not on how the prompt was cut): the K tile and the V^T tile go into LDS as they lie in the pages (rows padded by 16
+// bytes, so that sixteen lanes reading sixteen consecutive rows spread over the banks), slots past the last
+// position of the tile's tokens as zeros (a weight of zero times whatever a free slot holds must stay zero), and so
+// are positions before the first one that the tile's first token sees: a window has passed them, and their page
+// may have been given back (its id in the table is then -1 and must not be followed).
+//   scores   thread (ty, tx) of 16 x 16 owns tokens 4 ty .. 4 ty + 3 and positions tx, tx + 16, tx + 32, tx + 48: a
+//            dot product is an FMA chain over the head width in ascending order;
+//   softmax  online over the tiles (crates/vipera-backend-cpu/src/model.rs:1840-1857 is the plain form): a row's
+//            maximum and sum over the sixteen lanes that share it in a fixed tree, library-grade exp;
+//   output   the weights go through LDS; thread (ty, tx) owns the same four tokens and dims tx, tx + 16, ...: an
+//            FMA chain over the tile's positions in ascending order.
+// Head widths that are multiples of 16 up to 128 (the tiles of a wider head do not fit a CU's LDS) and pages of a
+// multiple of 4 positions; anything else stays with the general kernel.
+constexpr int PF_TILE = 64;
+template <int DPT>   // the head width is 16 * DPT
+__global__ __launch_bounds__(256) void attn_prefill_f32_kernel(
+    const float* __restrict__ q, long long q_stride, const float* __restrict__ k_cache,
+    const float* __restrict__ v_cache, float* __restrict__ out, const int* __restrict__ tiles,
+    const int* __restrict__ entry_start, const int* __restrict__ entry_first_pos, const int* __restrict__ block_table,
+    int table_width, int block_size, int heads, int kv_heads, float scale, int window, int tile_tokens) {
+  typedef float f32x4 __attribute__((ext_vector_type(4)));
+  constexpr int HD = 16 * DPT, QROW = HD + 4, VROW = PF_TILE + 4;
+  extern __shared__ __attribute__((aligned(16))) float pf_lds[];
+  float* q_s = pf_lds;                     // [64][QROW]
+  float* k_s = q_s + PF_TILE * QROW;       // [64][QROW]
+  float* v_s = k_s + PF_TILE * QROW;       // [HD][VROW], transposed as in the pages
+  float* p_s = v_s + HD * VROW;            // [64][VROW]
+  const int parts = tile_tokens / PF_TILE;                 // workgroups per tile of the step's list
+  // the list comes with the tiles that see most positions last; workgroups start in the order of their index, and the
+  // long ones should start first, so that the short ones fill the gaps at the end
+  const int index = gridDim.x - 1 - blockIdx.x;
+  const int tile = index / parts, part = index % parts, h = blockIdx.y;
+  const int entry = tiles[2 * tile], offset = tiles[2 * tile + 1] + part * PF_TILE;
+  const int count = entry_start[entry + 1] - entry_start[entry];
+  if (offset >= count) return;
+  const int rows = min(PF_TILE, count - offset);
+  const int tok0 = entry_start[entry] + offset, pos0 = entry_first_pos[entry] + offset;
+  const int last_pos = pos0 + rows - 1;
+  const int kvh = h / (heads / kv_heads);
+  const int* table = block_table + (size_t)entry * table_width;
+  const int tid = threadIdx.x, ty = tid >> 4, tx = tid & 15;
+
+  for (int i = tid; i < PF_TILE * (HD / 4); i += 256) {
+    const int r = i / (HD / 4), c = (i % (HD / 4)) * 4;
+    f32x4 v = {0.f, 0.f, 0.f, 0.f};
+    if (r < rows) v = *(const f32x4*)(q + (size_t)(tok0 + r) * q_stride + (size_t)h * HD + c);
+    *(f32x4*)(q_s + r * QROW + c) = v;
+  }
+  float m[4], l[4], o[4][DPT];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    m[i] = -INFINITY;
+    l[i] = 0.f;
+#pragma unroll
+    for (int j = 0; j < DPT; ++j) o[i][j] = 0.f;
+  }
+  const int lowest = (window > 0 && pos0 + 1 > window) ? pos0 + 1 - window : 0;   // the first token's first position
+  for (int kv0 = lowest / PF_TILE * PF_TILE; kv0 <= last_pos; kv0 += PF_TILE) {
+    __syncthreads();   // the tile before has been read
+    for (int i = tid; i < PF_TILE * (HD / 4); i += 256) {
+      const int r = i / (HD / 4), c = (i % (HD / 4)) * 4, p = kv0 + r;
+      f32x4 v = {0.f, 0.f, 0.f, 0.f};
+      if (p >= lowest && p <= last_pos)   // below `lowest` the window has passed: the page may have been given back
+        v = *(const f32x4*)(k_cache + (((size_t)table[p / block_size] * kv_heads + kvh) * block_size + p % block_size) * HD + c);
+      *(f32x4*)(k_s + r * QROW + c) = v;
+    }
+    for (int i = tid; i < HD * (PF_TILE / 4); i += 256) {
+      const int d = i / (PF_TILE / 4), c = (i % (PF_TILE / 4)) * 4, p = kv0 + c;   // four positions of one page
+      f32x4 v = {0.f, 0.f, 0.f, 0.f};
+      if (p + 3 >= lowest && p <= last_pos) {   // the four share a page, which is held if any of them is visible
+        v = *(const f32x4*)(v_cache + (((size_t)table[p / block_size] * kv_heads + kvh) * HD + d) * block_size + p % block_size);
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (p + e < lowest || p + e > last_pos) v[e] = 0.f;
+      }
+      *(f32x4*)(v_s + d * VROW + c) = v;
+    }
+    __syncthreads();
+    float s[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) s[i][j] = 0.f;
+    for (int c = 0; c < HD; c += 4) {
+      f32x4 qv[4], kv[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) qv[i] = *(const f32x4*)(q_s + (4 * ty + i) * QROW + c);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) kv[j] = *(const f32x4*)(k_s + (tx + 16 * j) * QROW + c);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          s[i][j] = fmaf(qv[i][0], kv[j][0], s[i][j]);
+          s[i][j] = fmaf(qv[i][1], kv[j][1], s[i][j]);
+          s[i][j] = fmaf(qv[i][2], kv[j][2], s[i][j]);
+          s[i][j] = fmaf(qv[i][3], kv[j][3], s[i][j]);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int qpos = pos0 + 4 * ty + i;
+      const int first = (window > 0 && qpos + 1 > window) ? qpos + 1 - window : 0;
+      float best = -INFINITY;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int p = kv0 + tx + 16 * j;
+        const bool sees = 4 * ty + i < rows && p <= qpos && p >= first;
+        s[i][j] = sees ? s[i][j] * scale : -INFINITY;
+        best = fmaxf(best, s[i][j]);
+      }
+#pragma unroll
+      for (int off = 1; off < 16; off <<= 1) best = fmaxf(best, __shfl_xor(best, off));
+      const float m_new = fmaxf(m[i], best);
+      float sum = 0.f;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float w = s[i][j] > -INFINITY ? expf(s[i][j] - m_new) : 0.f;
+        p_s[(4 * ty + i) * VROW + tx + 16 * j] = w;
+        sum += w;
+      }
+#pragma unroll
+      for (int off = 1; off < 16; off <<= 1) sum += __shfl_xor(sum, off);
+      const float rescale = m[i] > -INFINITY ? expf(m[i] - m_new) : 0.f;   // nothing seen so far: the sums are zero
+      l[i] = l[i] * rescale + sum;
+      m[i] = m_new;
+#pragma unroll
+      for (int j = 0; j < DPT; ++j) o[i][j] *= rescale;
+    }
+    __syncthreads();
+    for (int c = 0; c < PF_TILE; c += 4) {
+      f32x4 pv[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) pv[i] = *(const f32x4*)(p_s + (4 * ty + i) * VROW + c);
+#pragma unroll
+      for (int j = 0; j < DPT; ++j) {
+        const f32x4 vv = *(const f32x4*)(v_s + (tx + 16 * j) * VROW + c);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          o[i][j] = fmaf(pv[i][0], vv[0], o[i][j]);
+          o[i][j] = fmaf(pv[i][1], vv[1], o[i][j]);
+          o[i][j] = fmaf(pv[i][2], vv[2], o[i][j]);
+          o[i][j] = fmaf(pv[i][3], vv[3], o[i][j]);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    if (4 * ty + i >= rows) continue;
+    float* dst = out + (size_t)(tok0 + 4 * ty + i) * heads * HD + (size_t)h * HD;
+#pragma unroll
+    for (int j = 0; j < DPT; ++j) dst[tx + 16 * j] = o[i][j] / l[i];
+  }
+}
+
+template <int DPT>
+int launch_prefill_f32(dim3 grid, hipStream_t s, const float* q, long long q_stride, const float* k_cache,
+                       const float* v_cache, float* out, const int* tiles, const int* entry_start,
+                       const int* entry_first_pos, const int* block_table, int table_width, int block_size, int heads,
+                       int kv_heads, float scale, int window, int tile_tokens) {
+  constexpr int HD = 16 * DPT;
+  constexpr int lds_bytes = (2 * PF_TILE * (HD + 4) + HD * (PF_TILE + 4) + PF_TILE * (PF_TILE + 4)) * 4;
+  static_assert(lds_bytes <= 160 * 1024, "a CU has 160 KB of LDS");
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute((const void*)attn_prefill_f32_kernel<DPT>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    if (e != hipSuccess) return (int)e;
+    configured = true;
+  }
+  attn_prefill_f32_kernel<DPT><<<grid, 256, lds_bytes, s>>>(q, q_stride, k_cache, v_cache, out, tiles, entry_start,
+                                                            entry_first_pos, block_table, table_width, block_size,
+                                                            heads, kv_heads, scale, window, tile_tokens);
+  return 0;
 }
 
 template <int HB, int QC>
@@ -380,6 +583,36 @@ extern "C" int vk_attn_decode_f32(const float* q, long long q_stride, const floa
 #undef VK_DEC
   VK_LAUNCH_CHECK();
   attn_combine_f32_kernel<float><<<dim3(num_entries, heads), 64, 0, s>>>(partial, out, entries, entry_start, heads, hd, chunks);
+  VK_LAUNCH_CHECK();
+  return 0;
+}
+
+// Attention of the step's prompt portions in 32-bit: float q, cache and out. tiles: pairs (entry, first token of the
+// tile within the entry), `tile_tokens` tokens a tile (a multiple of 64), as vk_attn_bf16_prefill takes them. Head
+// widths that are multiples of 16 up to 128, pages of a multiple of 4 positions.
+extern "C" int vk_attn_prefill_f32(const float* q, long long q_stride, const float* k_cache, const float* v_cache,
+                                   float* out, const int* tiles, int num_tiles, int tile_tokens, const int* entry_start,
+                                   const int* entry_first_pos, const int* block_table, int table_width, int block_size,
+                                   int heads, int kv_heads, int hd, float scale, int window, void* stream) {
+  if (num_tiles <= 0) return 0;
+  if (hd <= 0 || hd > 128 || (hd & 15) || block_size <= 0 || (block_size & 3) || (q_stride & 3)) return VK_UNSUPPORTED_SIZE;
+  if (heads <= 0 || kv_heads <= 0 || heads % kv_heads != 0 || heads > 65535 || table_width <= 0 || window < 0 ||
+      tile_tokens <= 0 || tile_tokens % PF_TILE)
+    return VK_BAD_ARGUMENT;
+  if (((uintptr_t)q & 15) || ((uintptr_t)k_cache & 15) || ((uintptr_t)v_cache & 15)) return VK_BAD_ARGUMENT;
+  const long long groups = (long long)num_tiles * (tile_tokens / PF_TILE);
+  if (groups > 0x7fffffffLL) return VK_UNSUPPORTED_SIZE;
+  hipStream_t s = (hipStream_t)stream;
+  dim3 grid((unsigned)groups, heads);
+  int status = 0;
+#define VK_PF(DPTV)                                                                                                  \
+  case DPTV:                                                                                                         \
+    status = launch_prefill_f32<DPTV>(grid, s, q, q_stride, k_cache, v_cache, out, tiles, entry_start, entry_first_pos, \
+                                      block_table, table_width, block_size, heads, kv_heads, scale, window, tile_tokens); \
+    break;
+  switch (hd / 16) { VK_PF(1) VK_PF(2) VK_PF(3) VK_PF(4) VK_PF(5) VK_PF(6) VK_PF(7) VK_PF(8) }
+#undef VK_PF
+  if (status != 0) return status;
   VK_LAUNCH_CHECK();
   return 0;
 }

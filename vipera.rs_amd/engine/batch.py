@@ -62,6 +62,7 @@ class StepBatch:
     max_kv_len: int = 0
     all_single: bool = False
     num_prefill_tiles: int = 0
+    prefill_tile_tokens: int = TILE_TOKENS   # tokens of one entry of `prefill_tiles`
     num_decode_entries: int = 0
     max_decode_kv_len: int = 0
     max_tile_reach: int = 0        # positions that the last token of the longest prompt tile sees (no window counted)

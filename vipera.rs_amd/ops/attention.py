@@ -3,8 +3,8 @@
 A bfloat16 run whose head width and page size allow 16-byte reads uses the matrix-core kernels: one
 launch for the tiles of multi-token entries (prompt portions), one (plus the merge) for the entries
 that hold a single token, whose positions are split into chunks.  The 32-bit run has a split kernel for
-single tokens too (chunks of 256 positions); its prompt portions, and everything of odd sizes, use the
-general 32-bit kernel, which serves both kinds alike.
+single tokens too (chunks of 256 positions) and a tiled one for prompt portions (64 tokens of a head a
+workgroup); everything of odd sizes uses the general 32-bit kernel, which serves both kinds alike.
 """
 from __future__ import annotations
 
@@ -73,17 +73,21 @@ def paged_attention(qkv, k_cache, v_cache, out, batch, table, heads, kv_heads, h
                                      batch.entry_first_pos, table, heads, kv_heads, head_dim, scale, window, chunk,
                                      chunks, dense=batch.all_single, join=join)
         return
-    if batch.num_decode_entries and kernels.attn_decode_f32_supported(qkv, k_cache, head_dim):
-        # the 32-bit run: single tokens on the kernel that splits their positions into chunks and shares the reads
-        # among the query heads of a key head; prompt portions, if the step has any, on the general kernel
+    # the 32-bit run: single tokens on the kernel that splits their positions into chunks and shares the reads among
+    # the query heads of a key head, prompt portions on the kernel that walks the positions in LDS tiles; what
+    # either does not take (odd widths, pages that are no multiple of 4) is left to the general kernel
+    singles = bool(batch.num_decode_entries) and kernels.attn_decode_f32_supported(qkv, k_cache, head_dim)
+    portions = bool(batch.num_prefill_tiles) and kernels.attn_prefill_f32_supported(qkv, k_cache, head_dim)
+    if singles:
         chunks = (batch.max_decode_kv_len + kernels.ATTN_DECODE_F32_CHUNK - 1) // kernels.ATTN_DECODE_F32_CHUNK
         partial = torch.empty(batch.num_decode_entries * heads * chunks * (head_dim + 2), dtype=torch.float32,
                               device=qkv.device)
         kernels.attn_decode_f32(qkv, k_cache, v_cache, out, partial, batch.decode_entries, batch.entry_start,
                                 batch.entry_first_pos, table, heads, kv_heads, head_dim, scale, window, chunks)
-        if batch.num_prefill_tiles:
-            kernels.attn_generic(qkv, k_cache, v_cache, out, batch.positions, batch.entry_of_token, table, heads,
-                                 kv_heads, head_dim, scale, window, skip_single_of=batch.entry_start)
-        return
-    kernels.attn_generic(qkv, k_cache, v_cache, out, batch.positions, batch.entry_of_token, table, heads, kv_heads,
-                         head_dim, scale, window)
+    if portions:
+        kernels.attn_prefill_f32(qkv, k_cache, v_cache, out, batch.prefill_tiles, batch.prefill_tile_tokens,
+                                 batch.entry_start, batch.entry_first_pos, table, heads, kv_heads, head_dim, scale, window)
+    if (batch.num_decode_entries and not singles) or (batch.num_prefill_tiles and not portions):
+        # the general kernel can leave out the single tokens, not the portions: those it then computes again
+        kernels.attn_generic(qkv, k_cache, v_cache, out, batch.positions, batch.entry_of_token, table, heads, kv_heads,
+                             head_dim, scale, window, skip_single_of=batch.entry_start if singles else None)

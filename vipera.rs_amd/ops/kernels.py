@@ -321,6 +321,43 @@ def attn_decode_f32(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                heads, kv_heads, head_dim, float(scale), int(window), int(chunks), _stream()), "attn_decode_f32")
 
 
+ATTN_PREFILL_F32_MAX_HEAD_DIM = 128   # the K, V and weight tiles of a wider head do not fit a CU's LDS
+
+
+def attn_prefill_f32_supported(q: torch.Tensor, k_cache: torch.Tensor, head_dim: int) -> bool:
+    """Whether :func:`attn_prefill_f32` takes the operands: all 32-bit, a head width that is a multiple of 16 and
+    at most 128, pages of a multiple of 4 positions, 16-byte rows."""
+    return (q.dtype == torch.float32 and k_cache.dtype == torch.float32 and head_dim % 16 == 0
+            and head_dim <= ATTN_PREFILL_F32_MAX_HEAD_DIM and k_cache.shape[2] % 4 == 0 and q.stride(0) % 4 == 0
+            and q.data_ptr() % 16 == 0)
+
+
+def attn_prefill_f32(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
+                     tiles: torch.Tensor, tile_tokens: int, entry_start: torch.Tensor, entry_first_pos: torch.Tensor,
+                     block_table: torch.Tensor, heads: int, kv_heads: int, head_dim: int, scale: float,
+                     window: int) -> None:
+    """32-bit attention of the entries' tiles listed in ``tiles`` (pairs: entry, first token within it; ``tile_tokens``
+    tokens a tile, a multiple of 64): 64 tokens of one head a workgroup, the positions in LDS tiles of 64."""
+    _dev(q, k_cache, v_cache, out, tiles, entry_start, entry_first_pos, block_table)
+    _need(attn_prefill_f32_supported(q, k_cache, head_dim), "attn_prefill_f32: 32-bit operands, a head width that is a "
+          "multiple of 16 up to 128, pages of a multiple of 4 positions")
+    _need(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= heads * head_dim, "attention: q")
+    _need(out.shape == (q.shape[0], heads * head_dim) and out.is_contiguous() and out.dtype == q.dtype, "attention: out")
+    _need(_cache_ok(k_cache, v_cache, kv_heads, head_dim, q.dtype), "attention: cache shape or dtype")
+    _need(tiles.dtype == torch.int32 and tiles.numel() % 2 == 0 and tiles.is_contiguous(), "attention: tiles")
+    _need(tile_tokens >= 64 and tile_tokens % 64 == 0, "attention: tokens of a tile must be a multiple of 64")
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(), "attention: table")
+    _need(entry_start.dtype == torch.int32 and entry_first_pos.dtype == torch.int32
+          and entry_start.numel() == block_table.shape[0] + 1 and entry_first_pos.numel() == block_table.shape[0],
+          "attention: entry arrays")
+    _need(heads % kv_heads == 0, "attention: heads must be a multiple of kv_heads")
+    fn = _fn("attn_generic", "vk_attn_prefill_f32",
+             [_p, _ll, _p, _p, _p, _p, _i, _i, _p, _p, _p, _i, _i, _i, _i, _i, _f, _i, _p])
+    _status(fn(_ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(tiles), tiles.numel() // 2,
+               int(tile_tokens), _ptr(entry_start), _ptr(entry_first_pos), _ptr(block_table), block_table.shape[1],
+               k_cache.shape[2], heads, kv_heads, head_dim, float(scale), int(window), _stream()), "attn_prefill_f32")
+
+
 # ----------------------------------------------------------------------------------------------
 SAMPLE_SLICES = 32
 SAMPLE_SLICES_FROM = 32_768   # columns from which a row's best logit is searched in slices

@@ -23,7 +23,7 @@ from . import kernels
 #: bindings that launch kernels, by name; what is not listed (shape predicates, workspaces) is left alone
 LAUNCHERS = (
     "fetch_words", "embed_gather", "rmsnorm", "rope_angles", "rope_kvwrite", "swiglu", "fill_normal", "gemm_generic",
-    "attn_generic", "attn_decode_f32", "sample", "penalize", "logit_bias", "gemm_bf16", "gemm_bf16_qkv_rope", "gemm_bf16_follow",
+    "attn_generic", "attn_decode_f32", "attn_prefill_f32", "sample", "penalize", "logit_bias", "gemm_bf16", "gemm_bf16_qkv_rope", "gemm_bf16_follow",
     "gemm_bf16_mid_follow", "gemm_bf16_mid_qkv_rope", "gemm_bf16_gated_scaled", "attn_bf16_prefill",
     "attn_bf16_decode", "gemm_bf16_mid", "gemm_bf16_gated", "gemm_bf16_gated_tile_scaled",
 )
