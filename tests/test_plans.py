@@ -49,14 +49,14 @@ def test_the_gated_product_goes_resident_tiled_or_lds_shared():
     assert gated_resident_fits(8, 55296, 5120)
     assert not gated_resident_fits(8, 37888, 3584 + 64)    # K in whole chunks of 256 only
     for m in (1, 8, 16):
-        assert gated_plan(m, *GATE_UP_7B) == 0             # 1184 pairs over 256 CUs: 4 or 5 each
-    assert gated_plan(8, 17920, 1536) == 0                 # 1.5B: 560 pairs are 2 or 3 each; as fast, and the norm before it is free
+        assert gated_plan(m, *GATE_UP_7B) == 0             # 18,944 outputs over 256 CUs: 72 or 76 each
+    assert gated_plan(8, 17920, 1536) == 0                 # 1.5B: 8,960 outputs are 32 or 36 each, and the norm before it is free
     assert gated_plan(8, 55296, 5120) == 0
     assert gated_plan(17, *GATE_UP_7B) == 3 and gated_plan(64, *GATE_UP_7B) == 3   # past the resident kernel: tiled
     assert gated_plan(24, 55296, 5120) == 3
     assert gated_plan(48, 17920, 1536) in (1, 2) and gated_plan(64, 17920, 1536) == 3
-    assert gated_plan(8, *GATE_UP_7B, cus=304) == 0        # 1184 pairs over 304 CUs: 3 or 4 each, 3 % above the mean
-    assert gated_plan(8, *GATE_UP_7B, cus=500) == 0        # over 500: 2 or 3 each, 27 % above the mean
+    assert gated_plan(8, *GATE_UP_7B, cus=304) == 0        # over 304 CUs: 60 or 64 outputs each
+    assert gated_plan(8, *GATE_UP_7B, cus=500) == 0        # over 500: 36 or 40 each, 6 % above the mean
     assert gated_plan(8, 4096, 1024, cus=256) != 0         # 128 pairs over 256 CUs: half of them would have none
 
 

@@ -1165,9 +1165,14 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const __bf16* __restrict_
 
 // ---------------------------------------------------------------------------------------------
 // The gated product of up to 16 tokens with the activations resident in LDS. The launch has one workgroup
-// per CU (its LDS request keeps a second one away) and cuts the weight's pairs of 16 gate and 16 up rows
-// into as many contiguous runs, so every CU pulls the same number of bytes to within one pair: with a
-// fixed tile per workgroup the CUs that get one workgroup more than the others set the time. A workgroup
+// per CU (its LDS request keeps a second one away) and cuts the outputs into as many contiguous runs of a multiple
+// of four, so every CU pulls the same number of bytes to within four gate and four up rows: with a
+// fixed tile per workgroup the CUs that get one workgroup more than the others set the time, and with runs of
+// whole pairs of 16 gate and 16 up rows the busiest CU still had 8 % more than the mean at the 7B width (4 or 5
+// pairs) and 37 % at the 1.5B width (2 or 3). A run's pairs are its own: pair p of a run holds the outputs
+// begin + 16 p .. + 15, whichever rows of the weight those are (a lane's row is that of its output, and the rows of
+// two neighbouring pairs of the weight lie 32 apart whatever the output), and in a run's last pair the lanes past
+// its end request nothing. A workgroup
 // copies the activations into LDS once (all of K), and from then on its four waves do not meet: the run's
 // (pair, chunk of 256 k) units are cut into four equal stretches, a wave streams its stretch of weights
 // from HBM straight into operand registers, SETS register sets deep (two, three and four measured the
@@ -1199,31 +1204,41 @@ __global__ __launch_bounds__(256) void gemm_resident_gated_kernel(const __bf16* 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lr = lane & 15, lg = lane >> 4;
-  const int chunks = K / RES_CHUNK, pairs = N / 32;
-  const int p_begin = (int)((long long)pairs * blockIdx.x / gridDim.x);
-  const int p_end = (int)((long long)pairs * (blockIdx.x + 1) / gridDim.x);
-  const int units = (p_end - p_begin) * chunks;
+  const int chunks = K / RES_CHUNK, quads = N / 8;   // N / 2 outputs, four at a time
+  const int o_begin = (int)((long long)quads * blockIdx.x / gridDim.x) * 4;
+  const int o_end = (int)((long long)quads * (blockIdx.x + 1) / gridDim.x) * 4;
+  const int run_pairs = (o_end - o_begin + 15) / 16;
+  const int last_rows = o_end - o_begin - 16 * (run_pairs - 1);   // outputs of the run's last pair
+  const int units = run_pairs * chunks;
   auto bound = [&](int w) { return (int)((long long)units * w / 4); };
   const int u0 = bound(wave), u1 = bound(wave + 1), count = u1 - u0;
   const int first_pair = u0 / chunks, first_chunk = u0 % chunks;  // within the workgroup's run
 
-  const size_t w_first_row = (size_t)(p_begin + first_pair) * 32;
+  // the lane's output in the wave's first pair, and its gate row in the weight (the up row lies 16 further on)
+  const int o_first = o_begin + 16 * first_pair;
+  const int o_lane = o_first + lr;
+  const size_t w_first_row = (size_t)(o_first / 16) * 32;           // the first row any lane of the wave needs
+  const int row_lane = (o_lane / 16) * 32 + o_lane % 16 - (int)w_first_row;
   const BufferView w_view = buffer_view(W + w_first_row * K, (unsigned long long)(N - w_first_row) * K * 2);
   unsigned w_off[2];
 #pragma unroll
-  for (int rt = 0; rt < 2; ++rt) w_off[rt] = (unsigned)(((rt * 16 + lr) * K + lg * 8) * 2);
+  for (int rt = 0; rt < 2; ++rt) w_off[rt] = (unsigned)(((size_t)(rt * 16 + row_lane) * K + lg * 8) * 2);
   unsigned load_off = (unsigned)first_chunk * RES_CHUNK * 2;
-  int load_c = first_chunk;
+  int load_c = first_chunk, load_p = first_pair;
   const unsigned pair_skip = 62u * (unsigned)K;  // from the end of a pair's first row to the start of the next pair
+  const bool past_end = lr >= last_rows;         // in the run's last pair this lane's row belongs to the next run
   bf16x8 w[SETS][2][8];
   auto load_next = [&](bf16x8 (&dst)[2][8]) {
+    // an offset past the view's end reads zero and fetches nothing
+    const bool dead = past_end && load_p == run_pairs - 1;
 #pragma unroll
     for (int rt = 0; rt < 2; ++rt)
 #pragma unroll
-      for (int i = 0; i < 8; ++i) dst[rt][i] = w_view.load(w_off[rt] + load_off + i * 64);
+      for (int i = 0; i < 8; ++i) dst[rt][i] = w_view.load(dead ? 0xFFFFFFF0u : w_off[rt] + load_off + i * 64);
     load_off += RES_CHUNK * 2;
     if (++load_c == chunks) {
       load_c = 0;
+      ++load_p;
       load_off += pair_skip;
     }
   };
@@ -1284,7 +1299,7 @@ __global__ __launch_bounds__(256) void gemm_resident_gated_kernel(const __bf16* 
   bool first_part = true, from_start = first_chunk == 0;
   auto flush = [&](bool to_end) {  // the sums of units [from_start ? 0 : first_chunk, mul_c) of pair mul_p
     if (from_start && to_end) {
-      store_gated(C, ldc, lr, (p_begin + mul_p) * 16 + lg * 4, M, N / 2, acc[0] * inv, acc[1] * inv);
+      store_gated(C, ldc, lr, o_begin + mul_p * 16 + lg * 4, M, o_end, acc[0] * inv, acc[1] * inv);
     } else {
       f32x4* dst = partial + (wave * 2 + (first_part ? 0 : 1)) * 2 * 64;
       dst[lane] = acc[0];
@@ -1340,7 +1355,7 @@ __global__ __launch_bounds__(256) void gemm_resident_gated_kernel(const __bf16* 
         gate += theirs[lane];
         up += theirs[64 + lane];
       }
-      store_gated(C, ldc, lr, (p_begin + p) * 16 + lg * 4, M, N / 2, gate * inv, up * inv);
+      store_gated(C, ldc, lr, o_begin + p * 16 + lg * 4, M, o_end, gate * inv, up * inv);
     }
   }
 }
@@ -1368,8 +1383,8 @@ int launch_resident_gated(const __bf16* A, const __bf16* W, __bf16* C, int M, in
   const int cus = compute_units();
   const int pairs = N / 32;
   const int groups = pairs < cus ? pairs : cus;
-  // byte offsets from a wave's first pair are 32-bit
-  if (((long long)(pairs / groups) + 2) * 64 * K >= (1ll << 31)) return VK_UNSUPPORTED_SIZE;
+  // byte offsets from the first row that a wave needs are 32-bit: its run's pairs and one more, 64 rows each
+  if (((long long)(pairs / groups) + 4) * 64 * K >= (1ll << 31)) return VK_UNSUPPORTED_SIZE;
   kernel<<<groups, 256, lds_bytes, s>>>(A, W, C, M, N, K, lda, ldc, sumsq, norm_groups, eps);
   VK_LAUNCH_CHECK();
   return 0;

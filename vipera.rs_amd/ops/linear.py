@@ -139,13 +139,13 @@ def gated_rows_per_wave(m: int, n: int) -> int:
 
 def gated_plan(m: int, n: int, k: int, cus: int = 256) -> int:
     """What :func:`kernels.gemm_bf16_gated` is asked for at up to 64 tokens: 0, the kernel with resident
-    activations and one workgroup per CU, where it takes the shape and the pairs of 16 gate and 16 up rows
-    divide evenly enough over the ``cus`` workgroups (the busiest within 40 % of the mean: at 7B and 32B
-    widths it measured 2 to 7 % faster than the LDS-shared kernel; at the 1.5B width, 2 or 3 pairs a
-    workgroup, the two measure alike, 15.9 against 15.7 us at 8 tokens, and the resident kernel can divide by the
-    norm before it, which saves that norm's kernel); else the LDS-shared kernel with one or two tiles per wave."""
-    pairs = n // 32
-    if gated_resident_fits(m, n, k) and -(-pairs // cus) * cus <= 1.4 * pairs:
+    activations and one workgroup per CU, where it takes the shape and the outputs, four at a time, divide evenly
+    enough over the ``cus`` workgroups (every CU with a pair of 16-row tiles at least, the busiest within 10 % of the
+    mean: at 7B and 32B widths it measured 2 to 7 % faster than the LDS-shared kernel when its runs were still whole
+    pairs, and it can divide by the norm before it, which saves that norm's kernel); else the LDS-shared kernel with
+    one or two tiles per wave."""
+    pairs, quads = n // 32, n // 8
+    if gated_resident_fits(m, n, k) and pairs >= cus and -(-quads // cus) * cus <= 1.1 * quads:
         return 0
     if n * k >= 1e8 or m * n * k >= 1.5e9:
         # a large weight, or many tokens on a small one: the tiled kernel (3) with its three LDS stages and tiles
