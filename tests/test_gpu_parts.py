@@ -739,6 +739,99 @@ def test_a_routed_feed_forward_and_another_position_encoding(tmp_path):
         unregister("position", "tilt")
 
 
+def test_a_position_part_with_per_head_norms_of_q_and_k(tmp_path):
+    """What the reference hooks in before the rotation for architectures that have it (per-head RMS norms of q and k,
+    crates/vipera-backend-cpu/src/model.rs:312-313, 630-645) needs no change to the attention part: a position
+    encoding declares tensors of its own and changes q and k in place before they reach the cache.  Layer 0 gets such
+    a part from this file (norm per head with a weight of the head's width, then the NeoX rotation); layer 1 stays
+    as it is, fused rotation and all."""
+    from vipera_rs_amd.config import (LayerSpec, PartSpec, Qwen2Config, register_architecture, unregister_architecture)
+    from vipera_rs_amd.engine.batch import StepEntry
+    from vipera_rs_amd.engine.runner import ModelRunner
+    from vipera_rs_amd.models.decoder import DecoderModel
+    from vipera_rs_amd.parts import PositionEncoding, register_position, unregister
+    from vipera_rs_amd.parts.rotary import neox_inverse_frequencies
+    from vipera_rs_amd.weights import VECTOR, TensorSpec
+
+    class NormedRotary(PositionEncoding):
+        @classmethod
+        def declare(cls, spec, prefix):
+            hd = int(spec.params["head_dim"])
+            return [TensorSpec(f"{prefix}self_attn.{n}_norm.weight", (hd,), VECTOR, "one_plus_normal", std=0.3) for n in "qk"]
+
+        def load(self, tensors):
+            self.gain = {n: tensors[f"{self.prefix}self_attn.{n}_norm.weight"].float() for n in "qk"}
+            hd = int(self.spec.params["head_dim"])
+            self.inv = torch.from_numpy(neox_inverse_frequencies(hd, float(self.spec.params["base"]))).to(self.runtime.device)
+            self.eps = float(self.spec.params["eps"])
+
+        def apply(self, qkv, batch, heads, kv_heads, head_dim):
+            angle = batch.positions.float()[:, None] * self.inv[None, :]          # 32-bit, as the rotation kernels have it
+            sin, cos = torch.sin(angle)[:, None, :], torch.cos(angle)[:, None, :]
+            at = 0
+            for name, count in (("q", heads), ("k", kv_heads)):
+                x = qkv[:, at:at + count * head_dim].float().view(-1, count, head_dim)
+                x = x * torch.rsqrt((x * x).mean(-1, keepdim=True) + self.eps) * self.gain[name]
+                lo, hi = x[..., :head_dim // 2], x[..., head_dim // 2:]
+                x = torch.cat([lo * cos - hi * sin, lo * sin + hi * cos], dim=-1)
+                qkv[:, at:at + count * head_dim] = x.reshape(-1, count * head_dim).to(qkv.dtype)
+                at += count * head_dim
+
+    class NormedConfig(Qwen2Config):
+        architecture = "ToyNormedForCausalLM"
+
+        def layer_specs(self) -> List[LayerSpec]:
+            specs = super().layer_specs()
+            first = specs[0]
+            position = PartSpec("normed_rotary", {"head_dim": self.head_dim, "base": self.rope_theta, "eps": 1e-6})
+            specs[0] = LayerSpec(first.block, first.mixer, first.ffn, first.mixer_norm, first.ffn_norm, position, first.prefix)
+            return specs
+
+    def plain(cfg, w, tokens):
+        cfg = P.normalize_config(cfg)
+        T = len(tokens)
+        heads, kv_heads, hd = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+        x = w["model.embed_tokens.weight"][np.asarray(tokens)]
+        h = P.rms_norm(x, w["model.layers.0.input_layernorm.weight"], cfg["rms_norm_eps"])
+        a = "model.layers.0.self_attn."
+        q = P.linear(h, w[a + "q_proj.weight"], w.get(a + "q_proj.bias")).reshape(T, heads, hd)
+        k = P.linear(h, w[a + "k_proj.weight"], w.get(a + "k_proj.bias")).reshape(T, kv_heads, hd)
+        v = P.linear(h, w[a + "v_proj.weight"], w.get(a + "v_proj.bias")).reshape(T, kv_heads, hd)
+        q = P.rms_norm(q, w[a + "q_norm.weight"], 1e-6)            # over a head's width, one weight for all heads
+        k = P.rms_norm(k, w[a + "k_norm.weight"], 1e-6)
+        q = np.stack([P.rope_neox(q[t], t, cfg["rope_theta"]) for t in range(T)])
+        k = np.stack([P.rope_neox(k[t], t, cfg["rope_theta"]) for t in range(T)])
+        x = x + P.linear(P.attention(q, k, v, window=0).reshape(T, heads * hd), w[a + "o_proj.weight"])
+        h = P.rms_norm(x, w["model.layers.0.post_attention_layernorm.weight"], cfg["rms_norm_eps"])
+        x = x + P.swiglu_mlp(h, *(w[f"model.layers.0.mlp.{n}_proj.weight"] for n in ("gate", "up", "down")))
+        h = P.rms_norm(x, w["model.layers.1.input_layernorm.weight"], cfg["rms_norm_eps"])
+        x = x + P.attention_block(h, w, "model.layers.1.self_attn.", cfg, 0)
+        h = P.rms_norm(x, w["model.layers.1.post_attention_layernorm.weight"], cfg["rms_norm_eps"])
+        x = x + P.swiglu_mlp(h, *(w[f"model.layers.1.mlp.{n}_proj.weight"] for n in ("gate", "up", "down")))
+        return P.linear(P.rms_norm(x, w["model.norm.weight"], cfg["rms_norm_eps"]), w["model.embed_tokens.weight"])
+
+    register_position("normed_rotary", NormedRotary)
+    register_architecture("ToyNormedForCausalLM", NormedConfig, lambda config, runtime: DecoderModel(config, runtime))
+    try:
+        folder = make_folder(tmp_path / "normed", dict(CONFIG_A, architectures=["ToyNormedForCausalLM"]), 9)
+        cfg, w = P.load_folder(folder)
+        assert w["model.layers.0.self_attn.q_norm.weight"].shape == (P.normalize_config(cfg)["head_dim"],)
+        assert "model.layers.1.self_attn.q_norm.weight" not in w
+        tokens = random_tokens(256, 30, 5)
+        want = plain(cfg, w, tokens)
+        for dtype, tol in (("float32", 1e-4), ("bfloat16", 3e-2)):
+            runner = ModelRunner.from_folder(folder, dtype=dtype, block_size=8, num_blocks=16, num_slots=2)
+            rows, at = [], 0
+            for size in (11, 1, 1, 9, 2, 6):
+                runner.cache.reserve(0, at, at + size)
+                rows.append(runner.step([StepEntry(0, at, tokens[at:at + size], list(range(size)))]).float().cpu().numpy())
+                at += size
+            assert rel_err(np.concatenate(rows), want) < tol, dtype
+    finally:
+        unregister_architecture("ToyNormedForCausalLM")
+        unregister("position", "normed_rotary")
+
+
 def test_a_toy_feed_forward_takes_a_norm_handed_to_it(tmp_path):
     """A feed-forward defined here accepts a handed-off norm (`parts.NormHandoff`): for steps of up to 16 tokens
     the attention before it leaves `x * gain` and its workgroups' sums of squares instead of the norm running
