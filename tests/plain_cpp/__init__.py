@@ -37,7 +37,7 @@ SIGNATURES = {
     "plain_attn_generic": [P, LL, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, P, P],
     "plain_attn_decode_f32": [P, LL, P, P, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, P],
     "plain_attn_prefill_f32": [P, LL, P, P, P, P, I, I, P, P, P, I, I, I, I, I, F, I, P],
-    "plain_attn_bf16_prefill": [P, LL, P, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, P],
+    "plain_attn_bf16_prefill": [P, LL, P, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, P, LL, I, I, P],
     "plain_attn_bf16_decode": [P, LL, P, P, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, I, I, I, P],
     "plain_sample": [P, I, I, P, P, P, P, P, P, P, P, I, P, P, P, P, P, I, P],
     "plain_penalize": [P, I, P, P, P, P, P, P, I, P],

@@ -447,12 +447,13 @@ extern "C" int plain_attn_prefill_f32(const float* q, long long q_stride, const 
   return 0;
 }
 
-// tiles: pairs (entry, first token of the tile within the entry), 128 tokens per tile
+// tiles: pairs (entry, first token of the tile within the entry), 128 tokens per tile; `split`, the workspace and the
+// chunking shape the kernel's work only
 extern "C" int plain_attn_bf16_prefill(const void* q, long long q_stride, const void* k_cache, const void* v_cache,
                                        void* out, const int* tiles, int num_tiles, const int* entry_start,
                                        const int* entry_first_pos, const int* block_table, int table_width,
                                        int block_size, int heads, int kv_heads, int hd, float scale, int window,
-                                       int, void*) {
+                                       int, float*, long long, int, int, void*) {
   if (hd <= 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads || block_size <= 0 || window < 0) return BAD_ARGUMENT;
   for (int tile = 0; tile < num_tiles; ++tile) {
     const int entry = tiles[2 * tile], off = tiles[2 * tile + 1];

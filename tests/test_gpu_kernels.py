@@ -388,6 +388,13 @@ def test_attention_kernels_against_plain_softmax(case, dtype, stale):
                                       table_d, heads, kv_heads, hd, scale, window, split=True)
             rows = [t for e, n in enumerate(counts) if n > 1 for t in range(starts[e], starts[e + 1])]
             assert _rel(halved.cpu()[rows], want[rows]) < tol, "matrix-core prompt kernel, halved"
+            reach = max(kv for kv, n in entries if n > 1)
+            for chunk_tiles in (1, 2):          # a tile's positions in chunks of 64 and of 128, merged by a second kernel
+                chunked = torch.zeros(T, heads * hd, dtype=dtype, device=DEV)
+                kernels.attn_bf16_prefill(qkv_d, k_d, v_d, chunked, dev(torch.tensor(tiles, dtype=torch.int32)), es, fp,
+                                          table_d, heads, kv_heads, hd, scale, window, chunk_tiles=chunk_tiles,
+                                          max_chunks=-(-((reach + 63) // 64) // chunk_tiles))
+                assert _rel(chunked.cpu()[rows], want[rows]) < tol, f"matrix-core prompt kernel, chunks of {chunk_tiles}"
             kernels.attn_bf16_prefill(qkv_d, k_d, v_d, out2, dev(torch.tensor(tiles, dtype=torch.int32)), es, fp,
                                       table_d, heads, kv_heads, hd, scale, window)
         if singles:

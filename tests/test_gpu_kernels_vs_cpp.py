@@ -380,11 +380,17 @@ def test_matrix_core_attention_beside_its_twins(hd, window):
     qkv = torch.randn(T, (heads + 2 * kv_heads) * hd, generator=g).to(torch.bfloat16)
     entry_start, first_pos = i32([0, count, count + 1]), i32([first, 499])
     tiles = i32([0, 256, 0, 0, 0, 128])           # any order of the tiles
-    for split in (0, 1):                          # one workgroup per tile, or its positions halved between sixteen waves
+    padded = kernels.attn_bf16_padded_width(hd)
+    # one workgroup per tile; its positions halved between sixteen waves; or cut into chunks of 128 and of 192
+    # positions, a workgroup each, that a second kernel merges (where the width has the kernel for it)
+    for split, chunk_tiles in ((0, 0), (1, 0), (0, 2), (0, 3)):
+        max_chunks = -(-((first + count + 63) // 64) // chunk_tiles) if chunk_tiles else 0
+        partial = torch.full((3 * heads * max_chunks * 128 * (padded + 4),), float("nan")) if chunk_tiles else None
         (got, want), = both(module, "attn_bf16_prefill",
                             [qkv, qkv.shape[1], k, v, torch.zeros(T, heads * hd, dtype=torch.bfloat16), tiles, 3, entry_start,
-                             first_pos, table, table.shape[1], bs, heads, kv_heads, hd, 1 / math.sqrt(hd), window, split, None], [4])
-        assert rel_err(got[:count].float().numpy(), want[:count].double().numpy()) < 8e-3
+                             first_pos, table, table.shape[1], bs, heads, kv_heads, hd, 1 / math.sqrt(hd), window, split,
+                             partial, partial.numel() if chunk_tiles else 0, chunk_tiles, max_chunks, None], [4])
+        assert rel_err(got[:count].float().numpy(), want[:count].double().numpy()) < 8e-3, (split, chunk_tiles)
     chunk, chunks = 128, 4
     partial = torch.empty(1 * heads * chunks * (hd + 2))
     for join in (0, 1):                           # a workgroup per chunk and a merge kernel, or one that merges its waves' chunks

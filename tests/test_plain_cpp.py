@@ -145,7 +145,7 @@ def test_attention_twins_over_a_shuffled_table(window):
     low = torch.zeros(T, heads * hd, dtype=torch.bfloat16)
     call("plain_attn_bf16_prefill", qb, qb.shape[1], kb, vb, low, torch.tensor([0, 0], dtype=torch.int32), 1,
          torch.tensor([0, 13], dtype=torch.int32), torch.tensor([0], dtype=torch.int32), table, table.shape[1], bs, heads,
-         kv_heads, hd, 1 / math.sqrt(hd), window, 0, None)
+         kv_heads, hd, 1 / math.sqrt(hd), window, 0, None, 0, 0, 0, None)
     for t in range(13, T):   # each later token as an entry of its own that reads the same pages
         call("plain_attn_bf16_decode", qb, qb.shape[1], kb, vb, low, None, torch.tensor([0], dtype=torch.int32), 1,
              torch.tensor([t, t + 1], dtype=torch.int32), torch.tensor([t], dtype=torch.int32), table, table.shape[1], bs,

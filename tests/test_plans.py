@@ -74,6 +74,17 @@ def test_room_for_the_sums_of_squares():
         assert follow_sumsq_floats(n, 64) >= ((n + 1023) // 1024) * 64    # a workgroup per 1,024 columns, 64 tokens
 
 
+def test_prompt_tiles_in_chunks_for_models_of_few_heads():
+    from vipera_rs_amd.ops.attention import chunks_prompt_tiles
+    one_prompt = sum(128 * t for t in range(1, 17))                     # positions that the 16 tiles of 2,048 tokens see
+    assert chunks_prompt_tiles(16, 12, 2048, one_prompt, 256) is None   # 12 heads, one short prompt: the halved tiles
+    assert chunks_prompt_tiles(16, 28, 2048, one_prompt, 256) is None   # 448 items: more than the CUs
+    # four portions of 512 tokens that end at positions 1,000 to 8,000: 192 items, the deepest 125 steps long
+    assert chunks_prompt_tiles(16, 12, 8000, 4 * (1000 + 3000 + 5000 + 8000), 256) == (25, 5)
+    assert chunks_prompt_tiles(16, 12, 4096, 16 * 3900, 256) is None    # all about equally deep: nothing to balance
+    assert chunks_prompt_tiles(0, 12, 0, 0, 256) is None
+
+
 def test_decode_attention_chunks():
     assert decode_chunking(4096, 8, 4, 1) == (256, 16)     # 8 requests x 4 key heads x 16 chunks = 512 waves
     assert decode_chunking(4096, 64, 4, 1) == (1024, 4)

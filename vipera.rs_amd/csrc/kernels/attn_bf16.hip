@@ -515,6 +515,13 @@ __global__ __launch_bounds__(PT_THREADS) void attn_prefill_kernel(
 // (max, sum, weighted sum) are merged through LDS at the end. For a step with few work items of very different
 // lengths (one long prompt): a CU then works on its longest item with all sixteen waves instead of being left
 // with one workgroup of eight once the short neighbour has finished.
+//
+// CHUNKED (not with SPLIT): grid (tiles x heads x max_chunks); a tile's 64-position steps are cut into chunks of
+// `chunk_tiles`, a workgroup of eight waves takes one chunk (one that the tile does not have ends at once), and
+// where a tile has more than one chunk the workgroups leave (max, sum, weighted sum) of their columns in `partial`,
+// [tile, head, chunk, 128 columns, hd + 4] floats, for attn_prefill_merge_kernel to merge in ascending order. For a
+// model of few heads, whose (tile, head) items are fewer than the CUs and as long as their prompts: the 1.5B shape
+// has 12 heads, and four portions of 512 tokens are 192 items of which the one deepest in its prompt sets the time.
 #if HDP == 64 || HDP == 128 || HDP == 256
 #define VK_PREFILL_DIRECT 1
 constexpr int PD_ROWB = HDP * 2;                        // bytes of a K row in LDS
@@ -534,13 +541,16 @@ __device__ __forceinline__ int k_swizzle(int r) {
   return PD_C == 8 ? ((((r >> 3) & 1) << 2) | (r & 3)) : ((((r >> 3) & 3) << 2) | (r & 3));
 }
 
-template <bool SPLIT>
+constexpr int PD_PARTIAL_ROW = HDP + 4;   // floats of a column's partial result: the weighted sum, max, sum, and padding to 16 bytes
+
+template <bool SPLIT, bool CHUNKED = false>
 __global__ __launch_bounds__(SPLIT ? 2 * PT_THREADS : PT_THREADS) void attn_prefill_direct_kernel(
     const __bf16* __restrict__ q, long long q_stride, const __bf16* __restrict__ k_cache,
     const __bf16* __restrict__ v_cache, __bf16* __restrict__ out, const int* __restrict__ tiles,
     const int* __restrict__ entry_start, const int* __restrict__ entry_first_pos,
     const int* __restrict__ block_table, int table_width, int block_size, int heads, int kv_heads, float scale,
-    int window, int cus) {
+    int window, int cus, float* __restrict__ partial, int chunk_tiles, int max_chunks) {
+  static_assert(!(SPLIT && CHUNKED), "a chunk is taken by a workgroup of eight waves");
   typedef __attribute__((address_space(3))) void* lds_ptr;
   typedef __attribute__((address_space(1))) const void* global_ptr;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];  // [2][K tile | V^T tile]
@@ -551,9 +561,12 @@ __global__ __launch_bounds__(SPLIT ? 2 * PT_THREADS : PT_THREADS) void attn_pref
   unsigned char* lds_half = lds_raw + half * 2 * PD_STAGE;
   // work items as in attn_prefill_kernel: long ones first, paired with short ones on a CU (SPLIT: one
   // workgroup per CU, longest first)
-  const int total = (int)gridDim.x, round = blockIdx.x / cus;
+  const int total = CHUNKED ? (int)gridDim.x / max_chunks : (int)gridDim.x, round = blockIdx.x / cus;
   const int taken = (round >> 1) * cus + blockIdx.x % cus;
-  const int item = SPLIT ? total - 1 - (int)blockIdx.x : (round & 1) ? taken : total - 1 - taken;
+  // CHUNKED: the chunks of one (tile, head) are neighbours, the tiles that see most positions come first
+  const int chunk = CHUNKED ? (int)blockIdx.x % max_chunks : 0;
+  const int item = CHUNKED ? total - 1 - (int)blockIdx.x / max_chunks
+                           : SPLIT ? total - 1 - (int)blockIdx.x : (round & 1) ? taken : total - 1 - taken;
   const int tile = item / heads;
   const int entry = tiles[2 * tile], tile_off = tiles[2 * tile + 1];
   const int h = item % heads, kvh = h / (heads / kv_heads);
@@ -567,6 +580,10 @@ __global__ __launch_bounds__(SPLIT ? 2 * PT_THREADS : PT_THREADS) void attn_pref
   const int tile_first_pos = first_pos + tile_off;
   const int begin = (window > 0 && tile_first_pos + 1 > window) ? tile_first_pos + 1 - window : 0;
   const int end = tile_first_pos + tile_cols;
+  const int first_tile = begin & ~(PT_KV - 1);
+  const int all_tiles = (end - first_tile + PT_KV - 1) / PT_KV;
+  const int chunks = CHUNKED ? (all_tiles + chunk_tiles - 1) / chunk_tiles : 1;
+  if (CHUNKED && chunk >= chunks) return;   // the whole workgroup, before any barrier
 
   const int q_off = tile_off + wave * 16;
   const int c = q_off + lr;
@@ -712,11 +729,9 @@ __global__ __launch_bounds__(SPLIT ? 2 * PT_THREADS : PT_THREADS) void attn_pref
 
   // this half's tiles: all of them, or with SPLIT the first or the second half of them (both halves pass the
   // same number of barriers)
-  const int first_tile = begin & ~(PT_KV - 1);
-  const int all_tiles = (end - first_tile + PT_KV - 1) / PT_KV;
-  const int steps = SPLIT ? (all_tiles + 1) / 2 : all_tiles;
+  const int steps = CHUNKED ? min(chunk_tiles, all_tiles - chunk * chunk_tiles) : SPLIT ? (all_tiles + 1) / 2 : all_tiles;
   const int my_tiles = half ? all_tiles - steps : steps;
-  const int my_first = first_tile + (half ? steps * PT_KV : 0);
+  const int my_first = first_tile + (CHUNKED ? chunk * chunk_tiles * PT_KV : half ? steps * PT_KV : 0);
   lookup(my_first);
   if (my_tiles > 0) issue(0);
   lookup(my_first + PT_KV);
@@ -757,6 +772,16 @@ __global__ __launch_bounds__(SPLIT ? 2 * PT_THREADS : PT_THREADS) void attn_pref
   }
   l = sum_of_column(l);
   if (!col_ok) return;
+  if (CHUNKED && chunks > 1) {  // a column that sees nothing of this chunk leaves a maximum of -inf and sums of zero
+    float* dst = partial + ((((size_t)tile * heads + h) * max_chunks + chunk) * PT_TOKENS + (wave * 16 + lr)) * PD_PARTIAL_ROW;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) *(f32x4*)(dst + dt * 16 + lg * 4) = o[dt];
+    if (lg == 0) {
+      dst[hd] = m;
+      dst[hd + 1] = l;
+    }
+    return;
+  }
   const float inv = 1.f / l;
   __bf16* dst = out + (size_t)(tok0 + c) * heads * hd + (size_t)h * hd;
 #pragma unroll
@@ -766,6 +791,64 @@ __global__ __launch_bounds__(SPLIT ? 2 * PT_THREADS : PT_THREADS) void attn_pref
     for (int j = 0; j < 4; ++j) r[j] = (__bf16)(o[dt][j] * inv);
     *(bf16x4*)(dst + dt * 16 + lg * 4) = r;
   }
+}
+
+// The chunks of attn_prefill_direct_kernel<false, true> merged: grid (tiles, heads, 128 * HDP / 4 / 256), a thread
+// four dims of one column. The maxima are raw scores (the kernel scales inside its exponentials); the chunks are
+// folded in ascending order, acc = acc 2^((M - M') c) + acc_c 2^((m_c - M') c) with M' the larger of the running
+// maximum M and m_c, the sums likewise, four chunks requested at a time. A tile of one chunk was written by the
+// kernel itself.
+__global__ __launch_bounds__(256) void attn_prefill_merge_kernel(const float* __restrict__ partial, __bf16* __restrict__ out,
+                                                                 const int* __restrict__ tiles,
+                                                                 const int* __restrict__ entry_start,
+                                                                 const int* __restrict__ entry_first_pos, int heads,
+                                                                 float scale, int window, int chunk_tiles, int max_chunks) {
+  constexpr int hd = HDP, QUADS = HDP / 4, AHEAD = 4;
+  const int tile = blockIdx.x, h = blockIdx.y;
+  const int entry = tiles[2 * tile], tile_off = tiles[2 * tile + 1];
+  const int tok0 = entry_start[entry], count = entry_start[entry + 1] - tok0;
+  const int tile_cols = min(PT_TOKENS, count - tile_off);
+  const int tile_first_pos = entry_first_pos[entry] + tile_off;
+  const int begin = (window > 0 && tile_first_pos + 1 > window) ? tile_first_pos + 1 - window : 0;
+  const int end = tile_first_pos + tile_cols;
+  const int first_tile = begin & ~(PT_KV - 1);
+  const int all_tiles = (end - first_tile + PT_KV - 1) / PT_KV;
+  const int chunks = (all_tiles + chunk_tiles - 1) / chunk_tiles;
+  if (chunks <= 1) return;
+  const int at = blockIdx.z * 256 + threadIdx.x;
+  const int col = at / QUADS, quad = at % QUADS;
+  if (col >= tile_cols) return;
+  const float c2 = scale * 1.44269504088896341f;
+  const size_t chunk_stride = (size_t)PT_TOKENS * PD_PARTIAL_ROW;
+  const float* of_col = partial + ((size_t)tile * heads + h) * max_chunks * chunk_stride + (size_t)col * PD_PARTIAL_ROW;
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  float total = 0.f, best = -INFINITY;
+  for (int ch0 = 0; ch0 < chunks; ch0 += AHEAD) {
+    float mc[AHEAD], lc[AHEAD];
+    f32x4 oc[AHEAD];
+#pragma unroll
+    for (int j = 0; j < AHEAD; ++j) {   // a clamped chunk is not folded in
+      const float* src = of_col + (size_t)min(ch0 + j, chunks - 1) * chunk_stride;
+      mc[j] = src[hd];
+      lc[j] = src[hd + 1];
+      oc[j] = *(const f32x4*)(src + quad * 4);
+    }
+#pragma unroll
+    for (int j = 0; j < AHEAD; ++j)
+      if (ch0 + j < chunks && mc[j] > -INFINITY) {
+        const float both = fmaxf(best, mc[j]);
+        const float keep = best > -INFINITY ? __builtin_amdgcn_exp2f((best - both) * c2) : 0.f;
+        const float take = __builtin_amdgcn_exp2f((mc[j] - both) * c2);
+        acc = acc * keep + oc[j] * take;
+        total = total * keep + lc[j] * take;
+        best = both;
+      }
+  }
+  const float inv = 1.f / total;
+  bf16x4 r;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) r[j] = (__bf16)(acc[j] * inv);
+  *(bf16x4*)(out + (size_t)(tok0 + tile_off + col) * heads * hd + (size_t)h * hd + quad * 4) = r;
 }
 #endif
 
@@ -961,11 +1044,15 @@ extern "C" int vk_attn_bf16_hdp() { return HDP; }
 // number of positions a tile sees, rising (any order gives the same result). split: nonzero asks for workgroups
 // of sixteen waves that halve a tile's positions between them, where the kernel in use has that form (few tiles
 // of very different lengths); the result is the same up to rounding.
+// chunk_tiles > 0 (with the kernel that loads straight into LDS; ignored otherwise): a tile's steps of 64 positions
+// are cut into chunks of that many, a workgroup each, of which no tile has more than `max_chunks`; `partial` holds
+// num_tiles * heads * max_chunks * 128 * (padded head width + 4) floats.
 extern "C" int vk_attn_bf16_prefill(const void* q, long long q_stride, const void* k_cache, const void* v_cache,
                                     void* out, const int* tiles, int num_tiles, const int* entry_start,
                                     const int* entry_first_pos, const int* block_table, int table_width,
                                     int block_size, int heads, int kv_heads, int hd, float scale, int window,
-                                    int split, void* stream) {
+                                    int split, float* partial, long long partial_floats, int chunk_tiles,
+                                    int max_chunks, void* stream) {
   if (num_tiles <= 0) return 0;
   if (hd <= 0 || hd > HDP || (hd & 7) || block_size <= 0 || (block_size & 7) || heads <= 0 || kv_heads <= 0 ||
       heads % kv_heads || (q_stride & 7) || window < 0)
@@ -991,6 +1078,28 @@ extern "C" int vk_attn_bf16_prefill(const void* q, long long q_stride, const voi
   }
   if ((long long)num_tiles * heads > 0x7fffffffLL) return VK_UNSUPPORTED_SIZE;
 #ifdef VK_PREFILL_DIRECT
+  if (fast && hd == HDP && block_size >= 8 && chunk_tiles > 0) {  // the kernel that loads straight into LDS, in chunks
+    if (max_chunks <= 0 || !partial || ((uintptr_t)partial & 15) ||
+        (long long)num_tiles * heads * max_chunks * PT_TOKENS * PD_PARTIAL_ROW > partial_floats)
+      return VK_BAD_ARGUMENT;
+    if ((long long)num_tiles * heads * max_chunks > 0x7fffffffLL) return VK_UNSUPPORTED_SIZE;
+    auto chunked = attn_prefill_direct_kernel<false, true>;
+    static bool chunked_configured = false;
+    if (!chunked_configured) {
+      hipError_t e = hipFuncSetAttribute((const void*)chunked, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * PD_STAGE);
+      if (e != hipSuccess) return (int)e;
+      chunked_configured = true;
+    }
+    chunked<<<num_tiles * heads * max_chunks, PT_THREADS, 2 * PD_STAGE, (hipStream_t)stream>>>(
+        (const __bf16*)q, q_stride, (const __bf16*)k_cache, (const __bf16*)v_cache, (__bf16*)out, tiles, entry_start,
+        entry_first_pos, block_table, table_width, block_size, heads, kv_heads, scale, window, cus, partial,
+        chunk_tiles, max_chunks);
+    VK_LAUNCH_CHECK();
+    attn_prefill_merge_kernel<<<dim3(num_tiles, heads, PT_TOKENS * (HDP / 4) / 256), 256, 0, (hipStream_t)stream>>>(
+        partial, (__bf16*)out, tiles, entry_start, entry_first_pos, heads, scale, window, chunk_tiles, max_chunks);
+    VK_LAUNCH_CHECK();
+    return 0;
+  }
   if (fast && hd == HDP && block_size >= 8) {  // the kernel that loads straight into LDS
     const bool halves = split != 0 && PD_CAN_SPLIT;
     auto direct = attn_prefill_direct_kernel<false>;
@@ -1006,7 +1115,7 @@ extern "C" int vk_attn_bf16_prefill(const void* q, long long q_stride, const voi
     }
     direct<<<num_tiles * heads, halves ? 2 * PT_THREADS : PT_THREADS, direct_lds, (hipStream_t)stream>>>(
         (const __bf16*)q, q_stride, (const __bf16*)k_cache, (const __bf16*)v_cache, (__bf16*)out, tiles, entry_start,
-        entry_first_pos, block_table, table_width, block_size, heads, kv_heads, scale, window, cus);
+        entry_first_pos, block_table, table_width, block_size, heads, kv_heads, scale, window, cus, nullptr, 0, 1);
     VK_LAUNCH_CHECK();
     return 0;
   }

@@ -53,13 +53,47 @@ def halves_prompt_tiles(num_tiles: int, heads: int, longest: int, total: int, cu
     return items <= cus or (items <= 2 * cus and longest * num_tiles >= 1.25 * total)
 
 
+PROMPT_CHUNK_MIN_TILES = 8   # a chunk of a prompt tile's positions is at least 512 long
+
+
+def chunks_prompt_tiles(num_tiles: int, heads: int, longest: int, total: int, cus: int):
+    """``(chunk_tiles, max_chunks)`` if the prompt kernel should cut every tile's positions into chunks of
+    ``chunk_tiles`` steps of 64, a workgroup each, and merge them with a second kernel, else None.  For a model of
+    few heads, whose (tile, head) items are fewer than the CUs (12 heads and four portions of 512 tokens are 192
+    items) and as long as their prompts, so that the one deepest in its prompt sets the time.  The chunks are sized
+    to give every CU about two workgroups (sizes for one to six measured the same); a tile's partial results (128
+    columns x head width in 32-bit per chunk) go through memory, which is why the chunks are no shorter than 512
+    positions.  Chosen where an estimate says it pays: a workgroup of sixteen waves that halves a tile takes about
+    1.45 us per step of 64 positions, two workgroups of eight on a CU 2.9 us each, the chunked launch measured 1.6
+    times its ideal, and the merge costs 9 us (the 1.5B shape: a continuous batch with prompts of up to 8,192
+    tokens 2.56 to 2.45 s; one prompt of 2,048 tokens stays with the halved tiles, 47 against 55 us a layer)."""
+    items = num_tiles * heads
+    if items <= 0 or items > cus:
+        return None
+    steps = (total + 63) // 64 * heads                       # steps of 64 positions over all items
+    chunk_tiles = max(PROMPT_CHUNK_MIN_TILES, -(-steps // (2 * cus)))
+    longest_steps = (longest + 63) // 64
+    if longest_steps < 2 * chunk_tiles:
+        return None
+    halved = 1.45 * longest_steps
+    chunked = 1.6 * max(2.9 * chunk_tiles, 1.45 * steps / cus) + 9.0
+    if halved < 1.25 * chunked:
+        return None
+    return chunk_tiles, -(-longest_steps // chunk_tiles)
+
+
 def paged_attention(qkv, k_cache, v_cache, out, batch, table, heads, kv_heads, head_dim, scale, window) -> None:
     if kernels.attn_bf16_supported(qkv, k_cache, head_dim):
         if batch.num_prefill_tiles:
-            split = halves_prompt_tiles(batch.num_prefill_tiles, heads, batch.max_tile_reach, batch.sum_tile_reach,
-                                        kernels.compute_units(qkv.device))
+            cus = kernels.compute_units(qkv.device)
+            chunked = None
+            if kernels.attn_bf16_prefill_loads_directly(k_cache, kv_heads, head_dim):
+                chunked = chunks_prompt_tiles(batch.num_prefill_tiles, heads, batch.max_tile_reach, batch.sum_tile_reach, cus)
+            split = chunked is None and halves_prompt_tiles(batch.num_prefill_tiles, heads, batch.max_tile_reach,
+                                                            batch.sum_tile_reach, cus)
             kernels.attn_bf16_prefill(qkv, k_cache, v_cache, out, batch.prefill_tiles, batch.entry_start,
-                                      batch.entry_first_pos, table, heads, kv_heads, head_dim, scale, window, split)
+                                      batch.entry_first_pos, table, heads, kv_heads, head_dim, scale, window, split,
+                                      *(chunked or (0, 0)))
         if batch.num_decode_entries:
             group = heads // kv_heads
             visible = batch.max_decode_kv_len

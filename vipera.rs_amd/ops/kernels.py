@@ -707,13 +707,26 @@ def attn_bf16_supported(q: torch.Tensor, k_cache: torch.Tensor, head_dim: int) -
             and q.stride(0) % 8 == 0 and q.data_ptr() % 16 == 0)
 
 
+def attn_bf16_prefill_loads_directly(k_cache: torch.Tensor, kv_heads: int, head_dim: int) -> bool:
+    """Whether prompt attention runs on the kernel that loads K and V tiles straight into LDS (which alone can cut a
+    tile's positions into chunks): a head width of 64, 128 or 256 and pages of 8, 16, 32 or 64 positions."""
+    block_size = k_cache.shape[2]
+    return (head_dim in (64, 128, 256) and block_size in (8, 16, 32, 64)
+            and kv_heads * block_size * head_dim * 2 < 2 ** 32)
+
+
+ATTN_PREFILL_PARTIAL_ROW_EXTRA = 4   # floats beside the padded head width in a column's partial result
+
+
 def attn_bf16_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
                       tiles: torch.Tensor, entry_start: torch.Tensor, entry_first_pos: torch.Tensor,
                       block_table: torch.Tensor, heads: int, kv_heads: int, head_dim: int, scale: float,
-                      window: int, split: bool = False) -> None:
+                      window: int, split: bool = False, chunk_tiles: int = 0, max_chunks: int = 0) -> None:
     """Attention of the entries' 128-token tiles listed in ``tiles`` (pairs: entry, first token within it).
     ``split``: workgroups of sixteen waves that halve a tile's positions between them and merge at the end, where
-    the kernel in use has that form (for few tiles of very different lengths); the same result up to rounding."""
+    the kernel in use has that form (for few tiles of very different lengths); the same result up to rounding.
+    ``chunk_tiles`` > 0 (where :func:`attn_bf16_prefill_loads_directly`): a tile's steps of 64 positions are cut into
+    chunks of that many, a workgroup each, and a second kernel merges them; no tile may have more than ``max_chunks``."""
     _dev(q, k_cache, v_cache, out, tiles, entry_start, entry_first_pos, block_table)
     _need(attn_bf16_supported(q, k_cache, head_dim), "attn_bf16: operands must be bfloat16 with 16-byte rows")
     _need(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= heads * head_dim, "attention: q")
@@ -724,12 +737,23 @@ def attn_bf16_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     _need(entry_start.dtype == torch.int32 and entry_first_pos.dtype == torch.int32
           and entry_start.numel() == block_table.shape[0] + 1 and entry_first_pos.numel() == block_table.shape[0],
           "attention: entry arrays")
+    num_tiles = tiles.numel() // 2
+    partial = None
+    if chunk_tiles > 0 and attn_bf16_prefill_loads_directly(k_cache, kv_heads, head_dim):
+        _need(max_chunks >= 1, "attention: max_chunks")
+        partial = torch.empty(num_tiles * heads * max_chunks * 128 * (head_dim + ATTN_PREFILL_PARTIAL_ROW_EXTRA),
+                              dtype=torch.float32, device=q.device)
+    else:
+        chunk_tiles = max_chunks = 0
     module = f"attn_bf16_hd{attn_bf16_padded_width(head_dim)}"
-    fn = _fn(module, "vk_attn_bf16_prefill", [_p, _ll, _p, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _f, _i, _i, _p],
+    fn = _fn(module, "vk_attn_bf16_prefill",
+             [_p, _ll, _p, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _f, _i, _i, _p, _ll, _i, _i, _p],
              key=module + ".prefill")
-    _status(fn(_ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(tiles), tiles.numel() // 2,
+    _status(fn(_ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(tiles), num_tiles,
                _ptr(entry_start), _ptr(entry_first_pos), _ptr(block_table), block_table.shape[1], k_cache.shape[2],
-               heads, kv_heads, head_dim, float(scale), int(window), 1 if split else 0, _stream()), "attn_bf16_prefill")
+               heads, kv_heads, head_dim, float(scale), int(window), 1 if split else 0, _ptr(partial),
+               partial.numel() if partial is not None else 0, int(chunk_tiles), int(max_chunks), _stream()),
+            "attn_bf16_prefill")
 
 
 ATTN_DECODE_JOINED_CHUNKS = 8   # waves of a workgroup that merges its chunks itself
