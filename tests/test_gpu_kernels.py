@@ -576,17 +576,20 @@ def test_prompt_attention_at_the_benchmark_head_shapes(heads, kv_heads, hd):
     dev = lambda t: t.to(DEV)  # noqa: E731
     tiles = [(first[e] + off, e, off) for e, n in enumerate(counts) for off in range(0, n, TILE_TOKENS)]
     tiles = [x for _, e, off in sorted(tiles) for x in (e, off)]                # as the engine orders them
-    for split in (False, True):
+    # whole tiles, tiles in halves, and tiles in chunks of 8 and of 5 steps of 64 positions (the last chunk short)
+    for split, chunk_tiles in ((False, 0), (True, 0), (False, 8), (False, 5)):
         out = torch.zeros(T, heads * hd, dtype=dtype, device=DEV)
+        max_chunks = -(-(4096 // 64) // chunk_tiles) if chunk_tiles else 0
         kernels.attn_bf16_prefill(dev(qkv), dev(cache.k), dev(cache.v), out, dev(torch.tensor(tiles, dtype=torch.int32)),
                                   dev(torch.tensor(starts, dtype=torch.int32)), dev(torch.tensor(first, dtype=torch.int32)),
-                                  dev(cache.table), heads, kv_heads, hd, scale, 0, split=split)
+                                  dev(cache.table), heads, kv_heads, hd, scale, 0, split=split,
+                                  chunk_tiles=chunk_tiles, max_chunks=max_chunks)
         got = out.cpu()
-        assert _rel(got, want) < 1.2e-2
+        assert _rel(got, want) < 1.2e-2, (split, chunk_tiles)
         # row by row too: the first tokens of a prompt see few keys, their outputs are large and would hide a fault
         # in a late row of small outputs
         rows = (got.double() - want).abs().amax(dim=1) / want.abs().amax(dim=1)
-        assert float(rows.max()) < 3e-2, (split, int(rows.argmax()))
+        assert float(rows.max()) < 3e-2, (split, chunk_tiles, int(rows.argmax()))
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
