@@ -39,9 +39,20 @@ QWEN25_7B = {
 }
 
 
-# the other two Qwen2.5 shapes, for measurements beside the headline one (--shape)
+# the other Qwen2.5 shapes, for measurements beside the headline one (--shape); the sizes are those of the published
+# config.json of each model
 SHAPES = {
     "7b": ("Qwen2.5-7B shape", QWEN25_7B),
+    "0.5b": ("Qwen2.5-0.5B shape", dict(QWEN25_7B, num_hidden_layers=24, hidden_size=896, num_attention_heads=14,
+                                        num_key_value_heads=2, intermediate_size=4864, vocab_size=151936,
+                                        tie_word_embeddings=True, max_window_layers=21)),
+    "3b": ("Qwen2.5-3B shape", dict(QWEN25_7B, num_hidden_layers=36, hidden_size=2048, num_attention_heads=16,
+                                    num_key_value_heads=2, intermediate_size=11008, vocab_size=151936,
+                                    tie_word_embeddings=True, max_window_layers=70)),
+    "14b": ("Qwen2.5-14B shape", dict(QWEN25_7B, num_hidden_layers=48, hidden_size=5120, num_attention_heads=40,
+                                      num_key_value_heads=8, intermediate_size=13824, max_window_layers=48)),
+    "72b": ("Qwen2.5-72B shape", dict(QWEN25_7B, num_hidden_layers=80, hidden_size=8192, num_attention_heads=64,
+                                      num_key_value_heads=8, intermediate_size=29568, max_window_layers=70)),
     "1.5b": ("Qwen2.5-1.5B shape", dict(QWEN25_7B, num_hidden_layers=28, hidden_size=1536, num_attention_heads=12,
                                         num_key_value_heads=2, intermediate_size=8960, vocab_size=151936,
                                         tie_word_embeddings=True, max_window_layers=21)),

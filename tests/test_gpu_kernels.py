@@ -626,7 +626,9 @@ def test_attention_finds_one_far_key_among_hundreds(dtype):
 @pytest.mark.parametrize("m,n,k", [(1, 48, 64), (7, 300, 96), (8, 3584, 512), (16, 200, 1544), (17, 331, 520), (33, 1000, 264),
                                    (64, 520, 1024), (48, 130, 72), (64, 4608, 3584),
                                    # past 64 tokens K is walked in chunks of 128: K with a rest, K shorter than a chunk
-                                   (65, 331, 520), (80, 1000, 264), (97, 200, 1544), (128, 3584, 1024), (113, 130, 72)])
+                                   (65, 331, 520), (80, 1000, 264), (97, 200, 1544), (128, 3584, 1024), (113, 130, 72),
+                                   # weight rows a multiple of 4 KB apart: the workgroups start at different chunks
+                                   (8, 1100, 2048), (40, 2100, 4096), (100, 1100, 2048)])
 @pytest.mark.parametrize("ranges,rows_per_wave", [(1, 1), (1, 2), (3, 1), (8, 2), (2, 110), (1, 114), (3, 109)])
 def test_gemm_mid_against_float64(m, n, k, ranges, rows_per_wave):
     from vipera_rs_amd.ops import kernels
@@ -646,7 +648,7 @@ def test_gemm_mid_against_float64(m, n, k, ranges, rows_per_wave):
 
 
 @pytest.mark.parametrize("m,width,k_in,inter", [(8, 3584, 512, 18944), (1, 256, 64, 32), (16, 512, 1024, 16 * 1000),
-                                               (5, 768, 264, 16 * 41), (3, 1024, 3584, 16 * 300)])
+                                               (5, 768, 264, 16 * 41), (3, 1024, 3584, 16 * 300), (8, 896, 512, 4864)])
 def test_the_norm_split_between_the_products_around_it(m, width, k_in, inter):
     """x += a Wo^T, h = rms_norm(x) * g, out = up(h) * silu(gate(h)) as two kernels: the first also leaves
     bfloat16(x * g) and its workgroups' sums of squares, the second adds those and divides gate and up by the
@@ -747,7 +749,12 @@ def test_the_tiled_gated_product_divides_by_the_norm_before_it(tiling, m, width,
                                        # the resident kernel: one pair on four waves, fewer units than waves, runs of
                                        # uneven length, a wave's stretch inside one pair, many pairs per workgroup
                                        (1, 16, 256), (3, 48, 256), (16, 16 * 37, 512), (5, 16 * 1000, 1024), (8, 16 * 257, 3584),
-                                       (16, 16 * 300, 4352), (2, 16 * 4111, 768), (7, 32, 2048)])
+                                       (16, 16 * 300, 4352), (2, 16 * 4111, 768), (7, 32, 2048),
+                                       # weight rows a multiple of 4 KB apart (the LDS-shared kernel's workgroups
+                                       # start at different chunks)
+                                       (6, 16 * 70, 2048), (40, 16 * 70, 4096),
+                                       # 256 does not divide K: the resident kernel walks chunks of 128
+                                       (8, 4864, 896), (3, 48, 128), (16, 16 * 37, 384)])
 def test_gated_product_and_interleaved_swiglu(m, inter, k):
     from vipera_rs_amd.ops import kernels
     from vipera_rs_amd.ops.linear import gated_resident_fits, interleave_gate_up, linear_gated

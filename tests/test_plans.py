@@ -17,6 +17,9 @@ def test_few_tokens_stream_the_weights_with_k_split_inside_a_workgroup():
     assert not streams_in_wave_order(9, *DOWN_7B)          # past 8 tokens activations are shared through LDS instead
     assert not streams_in_wave_order(1, 5120, 27648) and not streams_in_wave_order(8, 5120, 27648)   # the 32B down projection
     assert streams_in_wave_order(1, 152064, 5120) and streams_in_wave_order(8, 5120, 5120)
+    # the 14B down projection: two rounds of small workgroups that would each read all activations
+    assert streams_in_wave_order(4, 5120, 13824) and not streams_in_wave_order(5, 5120, 13824)
+    assert streams_in_wave_order(8, 8192, 8192) and streams_in_wave_order(8, 10240, 8192)     # 72B: two whole rounds, or more
     assert not streams_in_wave_order(8, *HEAD_7B)          # many rows: likewise
     assert not streams_in_wave_order(17, *QKV_7B)
 
@@ -26,6 +29,7 @@ def test_the_lds_shared_product_splits_k_where_rows_are_few():
     assert mid_plan(64, *DOWN_7B) == (9, 2)                # many tokens and a long K: two tiles per wave, 28 row blocks x 9
     assert mid_plan(32, 5120, 27648) == (6, 2) and mid_plan(31, 5120, 27648) == (3, 1)
     assert mid_plan(64, 1536, 8960) == (10, 1)             # few rows: one tile per wave, 24 row blocks x 10
+    assert mid_plan(32, 2048, 11008) == (8, 1) and mid_plan(8, 5120, 13824) == (3, 1)     # the 3B and 14B down projections
     assert mid_plan(8, *HEAD_7B) == (1, 1) and mid_plan(64, *HEAD_7B) == (1, 2)
     assert mid_plan(64, *QKV_7B) == (3, 1) and mid_plan(64, *O_7B) == (4, 1)
     ranges, _ = mid_plan(64, 2048, 1536)                   # 1.5B q/k/v: no range shorter than 512
@@ -47,7 +51,8 @@ def test_the_gated_product_goes_resident_tiled_or_lds_shared():
     assert gated_resident_fits(16, *GATE_UP_7B) and not gated_resident_fits(17, *GATE_UP_7B)
     assert not gated_resident_fits(16, 55296, 5120)        # 32B: 16 tokens x 5120 do not fit a CU's LDS
     assert gated_resident_fits(8, 55296, 5120)
-    assert not gated_resident_fits(8, 37888, 3584 + 64)    # K in whole chunks of 256 only
+    assert not gated_resident_fits(8, 37888, 3584 + 64)    # K in whole chunks of 128 only
+    assert gated_resident_fits(8, 9728, 896) and gated_plan(8, 9728, 896) == 0     # the 0.5B width: chunks of 128
     for m in (1, 8, 16):
         assert gated_plan(m, *GATE_UP_7B) == 0             # 18,944 outputs over 256 CUs: 72 or 76 each
     assert gated_plan(8, 17920, 1536) == 0                 # 1.5B: 8,960 outputs are 32 or 36 each, and the norm before it is free

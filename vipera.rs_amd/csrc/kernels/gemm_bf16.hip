@@ -1094,25 +1094,37 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const __bf16* __restrict_
   // is multiplied (SETS register sets: three while registers allow three waves a SIMD, else two), the activations
   // of chunk c + 1 wait in registers until the barrier frees their LDS buffer, those of chunk c + 2 are
   // requested right after it.
+  // Where the weight's rows lie a multiple of 4 KB apart, the range's chunks are taken in a rotated order, chunk
+  // (c + turn) % whole at place c, with a turn of its own for each of the workgroups that share an XCD (every
+  // eighth): workgroups with equal shares walk K in step, and with such a K all rows of the weight put the same
+  // chunk on the same memory channels (8,192 x 8,192 at 8 tokens: 35.5 us without the turn, between 25.3 us at
+  // K = 7,680 and 28.3 at 8,704; 25.2 with it). Not otherwise: other row lengths showed no such loss, and in
+  // step the workgroups of an XCD read the same activations at the same time, out of L2.
   const int whole = (k_end - k_begin) / CHUNK;
+  const bool turned = whole > 0 && (K & 2047) == 0;
+  const int turn = turned ? (int)((blockIdx.x + blockIdx.y * gridDim.x) >> 3) % whole : 0;
+  auto k_at = [&](int c) {  // c up to the pipeline's depth past the range: such requests read what is not used
+    int j = c + turn;
+    if (j >= whole) j -= whole;
+    return k_begin + j * CHUNK;
+  };
   int buf = 0;
   constexpr int NEED = SETS - 1 > 2 ? SETS - 1 : 2;
   auto chunk = [&](auto set_, auto rem_, int c) {
     constexpr int SET = decltype(set_)::value, REM = decltype(rem_)::value;  // REM chunks follow (capped)
-    const int k0 = k_begin + c * CHUNK;
-    if constexpr (REM >= SETS - 1) load_weights(k0 + (SETS - 1) * CHUNK, w[(SET + SETS - 1) % SETS]);
+    if constexpr (REM >= SETS - 1) load_weights(k_at(c + SETS - 1), w[(SET + SETS - 1) % SETS]);
     multiply(w[SET], buf);
     if constexpr (REM >= 1) store_acts(buf ^ 1);
     __syncthreads();
-    if constexpr (REM >= 2) load_acts(k0 + 2 * CHUNK);
+    if constexpr (REM >= 2) load_acts(k_at(c + 2));
     buf ^= 1;
   };
   if (whole > 0) {
     // requests past the range (fewer chunks than the pipeline is deep) read weights that are not used
-    load_acts(k_begin);
-    static_for<SETS - 1>([&](auto j) { load_weights(k_begin + j.value * CHUNK, w[j.value]); });
+    load_acts(k_at(0));
+    static_for<SETS - 1>([&](auto j) { load_weights(k_at(j.value), w[j.value]); });
     store_acts(0);
-    load_acts(k_begin + CHUNK);
+    load_acts(k_at(1));
     __syncthreads();
     run_pipeline<SETS, NEED>(chunk, whole);
   }
@@ -1178,11 +1190,11 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const __bf16* __restrict_
 // from HBM straight into operand registers, SETS register sets deep (two, three and four measured the
 // same), across pair boundaries without draining. Where a stretch begins or ends inside a pair the wave leaves its partial sums in LDS, and the
 // wave that holds the pair's first unit adds the parts in wave order: the order of the sums depends on N,
-// K and the number of workgroups only. K must be a multiple of 256.
+// K and the number of workgroups only. K must be a multiple of 128: chunks of 256, or of 128 where 256 does not
+// divide K (a width of 896).
 #ifndef VK_RESIDENT_SETS
 #define VK_RESIDENT_SETS 3
 #endif
-constexpr int RES_CHUNK = 256;
 constexpr int RES_PARTIAL_BYTES = 4 * 2 * 2 * 64 * 16;  // [wave][first or last pair of its stretch][gate, up][lane]
 constexpr int RES_NORM_BYTES = 4 * 16 * 4;               // [wave][token]: sums of squares (SCALED)
 constexpr int RES_HEAD_BYTES = RES_PARTIAL_BYTES + RES_NORM_BYTES;
@@ -1190,7 +1202,7 @@ constexpr int RES_HEAD_BYTES = RES_PARTIAL_BYTES + RES_NORM_BYTES;
 // SCALED: the activations are x * gain of a norm whose division is still to come (see FollowNorm): the sums of
 // squares of `groups` workgroups, 16 floats each, are added here in a fixed order (a thread takes every 256th
 // workgroup, then the block's tree), and 1 / sqrt(mean + eps) scales gate and up before the activation.
-template <int SETS, bool SCALED>
+template <int SETS, bool SCALED, int RES_CHUNK = 256>
 __global__ __launch_bounds__(256) void gemm_resident_gated_kernel(const __bf16* __restrict__ A,
                                                                   const __bf16* __restrict__ W,
                                                                   __bf16* __restrict__ C, int M, int N, int K,
@@ -1223,23 +1235,31 @@ __global__ __launch_bounds__(256) void gemm_resident_gated_kernel(const __bf16* 
   unsigned w_off[2];
 #pragma unroll
   for (int rt = 0; rt < 2; ++rt) w_off[rt] = (unsigned)(((size_t)(rt * 16 + row_lane) * K + lg * 8) * 2);
-  unsigned load_off = (unsigned)first_chunk * RES_CHUNK * 2;
+  // Where the weight's rows lie a multiple of 4 KB apart, a pair's chunks are taken in a rotated order, chunk
+  // (c + turn) % chunks at place c, with a turn of its own for each of the workgroups that share an XCD (every
+  // eighth): runs of equal length move through their pairs in step, and with such a K all rows of the weight put
+  // the same chunk on the same memory channels (the 3B width, 2,048: 26.3 us without the turn, between 18.7 us
+  // at K = 1,792 and 23.3 at 2,304; 22.4 with it). Other widths lost a microsecond in fifty to the turn.
+  const int turn = (K & 2047) == 0 ? (int)(blockIdx.x >> 3) % chunks : 0;
+  int load_at = (first_chunk + turn) % chunks;   // the chunk of the weight's rows that the next request reads
+  unsigned pair_off = 0;                         // bytes from the wave's first pair to the pair of the next request
   int load_c = first_chunk, load_p = first_pair;
-  const unsigned pair_skip = 62u * (unsigned)K;  // from the end of a pair's first row to the start of the next pair
   const bool past_end = lr >= last_rows;         // in the run's last pair this lane's row belongs to the next run
-  bf16x8 w[SETS][2][8];
-  auto load_next = [&](bf16x8 (&dst)[2][8]) {
+  constexpr int KSTEPS = RES_CHUNK / 32;
+  bf16x8 w[SETS][2][KSTEPS];
+  auto load_next = [&](bf16x8 (&dst)[2][KSTEPS]) {
     // an offset past the view's end reads zero and fetches nothing
     const bool dead = past_end && load_p == run_pairs - 1;
 #pragma unroll
     for (int rt = 0; rt < 2; ++rt)
 #pragma unroll
-      for (int i = 0; i < 8; ++i) dst[rt][i] = w_view.load(dead ? 0xFFFFFFF0u : w_off[rt] + load_off + i * 64);
-    load_off += RES_CHUNK * 2;
+      for (int i = 0; i < KSTEPS; ++i)
+        dst[rt][i] = w_view.load(dead ? 0xFFFFFFF0u : w_off[rt] + pair_off + (unsigned)load_at * (RES_CHUNK * 2) + i * 64);
+    if (++load_at == chunks) load_at = 0;
     if (++load_c == chunks) {
       load_c = 0;
       ++load_p;
-      load_off += pair_skip;
+      pair_off += 64u * (unsigned)K;
     }
   };
 
@@ -1296,6 +1316,7 @@ __global__ __launch_bounds__(256) void gemm_resident_gated_kernel(const __bf16* 
   const __bf16* a_lane = acts + token * row_elems + lg * 8;
   f32x4 acc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
   int mul_c = first_chunk, mul_p = first_pair;
+  int mul_at = (first_chunk + turn) % chunks;   // the chunk of the activations that goes with the next unit
   bool first_part = true, from_start = first_chunk == 0;
   auto flush = [&](bool to_end) {  // the sums of units [from_start ? 0 : first_chunk, mul_c) of pair mul_p
     if (from_start && to_end) {
@@ -1311,15 +1332,16 @@ __global__ __launch_bounds__(256) void gemm_resident_gated_kernel(const __bf16* 
     mul_c = 0;
     ++mul_p;
   };
-  auto multiply = [&](const bf16x8 (&wf)[2][8]) {
-    const __bf16* a = a_lane + mul_c * RES_CHUNK;
+  auto multiply = [&](const bf16x8 (&wf)[2][KSTEPS]) {
+    const __bf16* a = a_lane + mul_at * RES_CHUNK;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < KSTEPS; ++i) {
       const bf16x8 av = *(const bf16x8*)(a + i * 32);
       acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[0][i], av, acc[0], 0, 0, 0);
       acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[1][i], av, acc[1], 0, 0, 0);
     }
     ++mul_c;
+    if (++mul_at == chunks) mul_at = 0;
   };
   auto step = [&](auto set_, auto rem_, int) {
     constexpr int SET = decltype(set_)::value, REM = decltype(rem_)::value;
@@ -1362,7 +1384,7 @@ __global__ __launch_bounds__(256) void gemm_resident_gated_kernel(const __bf16* 
 
 // Whether the resident kernel takes the shape, and the LDS it asks for (0: it does not).
 int resident_lds_bytes(int M, int N, int K) {
-  if (M > 16 || (K % RES_CHUNK) || (N & 31)) return 0;
+  if (M > 16 || (K % 128) || (N & 31)) return 0;
   const long long need = RES_HEAD_BYTES + (long long)M * (K + 8) * 2;
   if (need > 160 * 1024) return 0;
   return (int)(need > 82 * 1024 ? need : 82 * 1024);  // more than half a CU's LDS: one workgroup per CU
@@ -1373,12 +1395,15 @@ int launch_resident_gated(const __bf16* A, const __bf16* W, __bf16* C, int M, in
                           long long ldc, const float* sumsq, int norm_groups, float eps, hipStream_t s) {
   const int lds_bytes = resident_lds_bytes(M, N, K);
   if (!lds_bytes) return VK_UNSUPPORTED_SIZE;
-  auto kernel = gemm_resident_gated_kernel<VK_RESIDENT_SETS, SCALED>;
-  static bool configured = false;
-  if (!configured) {
+  // chunks of 128 where 256 does not divide K, with one register set more: as many bytes on their way
+  const bool halves = K % 256 != 0;
+  auto kernel = halves ? gemm_resident_gated_kernel<VK_RESIDENT_SETS + 1, SCALED, 128>
+                       : gemm_resident_gated_kernel<VK_RESIDENT_SETS, SCALED, 256>;
+  static bool configured[2] = {false, false};
+  if (!configured[halves]) {
     hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (e != hipSuccess) return (int)e;
-    configured = true;
+    configured[halves] = true;
   }
   const int cus = compute_units();
   const int pairs = N / 32;
@@ -1962,7 +1987,7 @@ extern "C" int vk_gemm_bf16_mid_no_alloc(const void* A, const void* W, const flo
 // interleaved in groups of 16 (see store_gated). bfloat16 in and out; N a multiple of 32.
 // More than 64 tokens: the tiled kernel; up to 64: the LDS-shared kernel with one K range and `rows_per_wave`
 // (1 or 2) tiles of 16 rows per wave, or with `rows_per_wave` 0 the kernel that keeps the activations resident
-// in LDS (up to 16 tokens, K a multiple of 256, tokens x K within LDS; anything else is refused), or with
+// in LDS (up to 16 tokens, K a multiple of 128, tokens x K within LDS; anything else is refused), or with
 // `rows_per_wave` 3 the tiled kernel.
 extern "C" int vk_gemm_bf16_gated(const void* A, const void* W, void* C, int M, int N, int K, long long lda,
                                   long long ldc, int rows_per_wave, void* stream) {

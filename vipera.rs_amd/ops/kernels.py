@@ -858,7 +858,7 @@ def gemm_bf16_gated(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, rows_pe
     """``out = up * silu(gate)`` where ``[gate, up] = a @ w.T`` and ``w`` interleaves gate and up rows in
     groups of 16.  ``out``: ``[tokens, w.shape[0] / 2]`` bfloat16.  ``rows_per_wave`` (up to 64 tokens): 1 or
     2 tiles per wave of the LDS-shared kernel, 0 for the kernel with resident activations (up to 16
-    tokens, K a multiple of 256, ``tokens x K`` within LDS; refused otherwise), 3 for the tiled kernel that
+    tokens, K a multiple of 128, ``tokens x K`` within LDS; refused otherwise), 3 for the tiled kernel that
     more than 64 tokens always take."""
     _dev(a, w, out)
     m, k = a.shape

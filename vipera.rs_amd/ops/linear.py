@@ -44,21 +44,26 @@ def mid_plan(m: int, n: int, k: int) -> Tuple[int, int]:
     # measured a third slower), each range at least two chunks long
     # with many tokens, a long K and enough rows, two tiles per wave and twice the ranges measured a tenth faster (the
     # 32B down projection at 32 tokens 54.7 against 60.6 us); with few rows one tile and fewer ranges (the 1.5B down
-    # projection at 64 tokens 13.0 against 15.7)
-    rows_per_wave = 2 if m >= 32 and k >= 8_192 and n >= 2_048 else 1
+    # projection at 64 tokens 13.0 against 15.7, the 3B one, 2,048 x 11,008, at 32 tokens 14.6 against 16.6)
+    rows_per_wave = 2 if m >= 32 and k >= 8_192 and n >= 3_072 else 1
     row_blocks = (n + 64 * rows_per_wave - 1) // (64 * rows_per_wave)
     return max(1, min(k // 512, 256 // row_blocks)), rows_per_wave
 
 
-def streams_in_wave_order(m: int, n: int, k: int) -> bool:
+def streams_in_wave_order(m: int, n: int, k: int, cus: int = 256) -> bool:
     """Whether a bfloat16 product of ``m`` tokens runs on the kernel whose waves split K inside a workgroup: up to 4
     tokens; up to 8 where the weight has few rows, also with a long K (every workgroup reads all activations,
     but there is no second kernel that adds K ranges: the down projection at 8 tokens 30.2 against 28.2 + 4.9 us at
     the 7B widths, 12.1 against 11.1 + 6.2 at the 1.5B widths); up to 16 with a short K as well.  Not for a weight
     of few rows and more than 100 M elements, whose workgroups would each stream most of a megabyte through four
     waves (the 32B down projection, 5,120 x 27,648: 62.2 us against 50.7 + 5 with K split over workgroups at one
-    token, 67.9 against 52.2 + 5 at eight)."""
+    token, 67.9 against 52.2 + 5 at eight).  Nor past 4 tokens for a long K whose 16-row workgroups are more than
+    one round over the ``cus`` CUs and less than two: the launch then makes two rounds of workgroups of ten rows or
+    so, each of which reads all activations, nearly as many bytes again as the weights (the 14B down projection,
+    5,120 x 13,824, at 8 tokens: 37.8 us against 29.7 + 2.5)."""
     if n < 16_384 and n * k > 100_000_000:
+        return False
+    if m > 4 and k >= 8_192 and cus < (n + 15) // 16 < 2 * cus:
         return False
     return m <= 4 or (m <= 8 and n < 16_384) or (m <= 16 and n < 16_384 and k < 8_192)
 
@@ -119,8 +124,8 @@ RESIDENT_LDS_BYTES = 160 * 1024 - (16 * 1024 + 256)   # what the resident kernel
 
 def gated_resident_fits(m: int, n: int, k: int) -> bool:
     """Whether the gated kernel that keeps all activations in LDS takes the shape: up to 16 tokens, K in
-    whole chunks of 256, and ``tokens x (K + 8)`` bfloat16 values within a CU's LDS."""
-    return m <= 16 and k % 256 == 0 and n % 32 == 0 and m * (k + 8) * 2 <= RESIDENT_LDS_BYTES
+    whole chunks of 128, and ``tokens x (K + 8)`` bfloat16 values within a CU's LDS."""
+    return m <= 16 and k % 128 == 0 and n % 32 == 0 and m * (k + 8) * 2 <= RESIDENT_LDS_BYTES
 
 
 def gated_rows_per_wave(m: int, n: int) -> int:
