@@ -58,6 +58,8 @@ def test_the_gated_product_goes_resident_tiled_or_lds_shared():
     assert gated_plan(8, 17920, 1536) == 0                 # 1.5B: 8,960 outputs are 32 or 36 each, and the norm before it is free
     assert gated_plan(8, 55296, 5120) == 0
     assert gated_plan(17, *GATE_UP_7B) == 3 and gated_plan(64, *GATE_UP_7B) == 3   # past the resident kernel: tiled
+    assert gated_plan(32, 59136, 8192) == 2 and gated_plan(33, 59136, 8192) == 3   # 72B: LDS-shared up to 32 tokens
+    assert gated_plan(8, 59136, 8192) == 0
     assert gated_plan(24, 55296, 5120) == 3
     assert gated_plan(48, 17920, 1536) in (1, 2) and gated_plan(64, 17920, 1536) == 3
     assert gated_plan(8, *GATE_UP_7B, cus=304) == 0        # over 304 CUs: 60 or 64 outputs each

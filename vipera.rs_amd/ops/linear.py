@@ -152,6 +152,11 @@ def gated_plan(m: int, n: int, k: int, cus: int = 256) -> int:
     pairs, quads = n // 32, n // 8
     if gated_resident_fits(m, n, k) and pairs >= cus and -(-quads // cus) * cus <= 1.1 * quads:
         return 0
+    if m <= 32 and k % 2048 == 0 and n * k >= 4e8:
+        # the largest weights with rows a multiple of 4 KB apart, where the LDS-shared kernel's workgroups start at
+        # different chunks: it streams them faster than the tiled one (72B, 59,136 x 8,192, at 17 to 32 tokens: 164
+        # to 171 us against 185; at 64 the norm's own kernel, which only the tiled one saves, makes them even)
+        return gated_rows_per_wave(m, n)
     if n * k >= 1e8 or m * n * k >= 1.5e9:
         # a large weight, or many tokens on a small one: the tiled kernel (3) with its three LDS stages and tiles
         # of 96 to 224 weight rows that fill the CUs in one round passes the LDS-shared one (7B widths at 17 to 64
