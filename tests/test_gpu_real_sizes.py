@@ -34,10 +34,30 @@ def real(tmp_path_factory):
 
 @pytest.mark.parametrize("dtype,tol", [("float32", 1e-4), ("bfloat16", 3e-2)])
 def test_real_layer_sizes_under_every_cut(real, dtype, tol):
+    folder, want = real[dtype]
+    _under_every_cut(folder, want, real["tokens"], dtype, tol)
+
+
+# hidden 896 is no multiple of 256 and has heads of width 64; rows of 2,048 values lie 4 KB apart, which the
+# weight-streaming kernels answer with a different first chunk for every workgroup
+OTHER_WIDTHS = {
+    "0.5b": dict(hidden_size=896, num_attention_heads=14, num_key_value_heads=2, intermediate_size=4864),
+    "3b": dict(hidden_size=2048, num_attention_heads=16, num_key_value_heads=2, intermediate_size=11008),
+}
+
+
+@pytest.mark.parametrize("name", sorted(OTHER_WIDTHS))
+def test_the_layer_sizes_of_two_other_models_under_every_cut(tmp_path, name):
+    config = dict(CONFIG_7B_LAYER, **OTHER_WIDTHS[name])
+    tokens = random_tokens(1000, 150, 31)
+    folder = make_folder(tmp_path / name, config, 5, torch.bfloat16)
+    cfg, w = P.load_folder(folder)
+    _under_every_cut(folder, P.forward(cfg, w, tokens), tokens, "bfloat16", 3e-2)
+
+
+def _under_every_cut(folder, want, tokens, dtype, tol):
     from vipera_rs_amd.engine.batch import StepEntry
     from vipera_rs_amd.engine.runner import ModelRunner
-    folder, want = real[dtype]
-    tokens = real["tokens"]
     runner = ModelRunner.from_folder(folder, dtype=dtype, block_size=16, num_blocks=40, num_slots=4)
     # whole
     runner.cache.reserve(0, 0, len(tokens))
