@@ -9,7 +9,7 @@ combination (the 32-bit run, or a matrix kept in 32-bit inside a bfloat16 run) g
   product is a stream of the weights.  Up to four tokens, or a small weight
   at up to 16 tokens, use the kernel whose waves split K inside a workgroup; otherwise the kernel that
   shares the activations through LDS, with K split over workgroups where the weight has too few rows
-  to fill the GPU otherwise.  The thresholds were measured on the 1.5B, 7B and 32B shapes on an MI355X.  The gated
+  to fill the GPU otherwise.  The thresholds were measured on the seven Qwen2.5 shapes (0.5B to 72B) on an MI355X.  The gated
   product of up to 16 tokens keeps all activations in LDS and gives every CU the same share of rows.
 """
 from __future__ import annotations
