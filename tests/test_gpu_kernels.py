@@ -212,6 +212,47 @@ def test_gemm_generic_does_not_depend_on_the_batch(k):
     assert torch.equal(rounded, with_bias[20:28].to(torch.bfloat16))
 
 
+@pytest.mark.parametrize("m,n,k", [(1024, 1024, 520), (1030, 1100, 1027), (1500, 905, 258), (1153, 1025, 2052)])
+def test_the_wide_tiles_of_gemm_generic_sum_in_the_same_order(m, n, k):
+    """128 rows and more on enough tiles take 128 x 128 tiles with 8 x 8 outputs a thread: against 64-bit, and bit
+    for bit the rows that the 64 x 64 tiles give 70 rows at a time and the weight stream 33 at a time; with a bias,
+    accumulating, into bfloat16, from bfloat16 activations, and with rows that start off a 16-byte boundary."""
+    from vipera_rs_amd.ops import kernels
+    g = torch.Generator().manual_seed(m + n + k)
+    a = torch.randn(m, k, generator=g).to(DEV)
+    w = torch.randn(n, k, generator=g).to(DEV)
+    bias = torch.randn(n, generator=g).to(DEV)
+    base = torch.randn(m, n, generator=g).to(DEV)
+    whole = torch.full((m, n), float("nan"), device=DEV)
+    kernels.gemm_generic(a, w, bias, whole)
+    assert _rel(whole, a.double() @ w.double().T + bias.double()) < 2e-6
+    for rows in (70, 33):
+        for start in (0, 128 * 3 + 5, m - rows):
+            part = torch.empty(rows, n, device=DEV)
+            kernels.gemm_generic(a[start:start + rows], w, bias, part)
+            assert torch.equal(part, whole[start:start + rows]), (rows, start)       # bit for bit
+    added = base.clone()
+    kernels.gemm_generic(a, w, bias, added, accumulate=True)
+    few = base[200:270].clone()
+    kernels.gemm_generic(a[200:270], w, bias, few, accumulate=True)
+    assert torch.equal(few, added[200:270])
+    rounded = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
+    kernels.gemm_generic(a, w, bias, rounded)
+    assert torch.equal(rounded, whole.to(torch.bfloat16))
+    half = a.to(torch.bfloat16)                                   # bfloat16 activations on a 32-bit weight
+    mixed = torch.empty(m, n, device=DEV)
+    kernels.gemm_generic(half, w, bias, mixed)
+    again = torch.empty(m, n, device=DEV)
+    kernels.gemm_generic(half.float(), w, bias, again)
+    assert torch.equal(mixed, again)
+    shifted = torch.zeros(m, k + 3, device=DEV)                   # rows 4 (k + 3) bytes apart, from a 4-byte offset
+    shifted[:, 1:k + 1] = a
+    out = torch.zeros(m, n + 8, device=DEV)
+    kernels.gemm_generic(shifted[:, 1:k + 1], w, bias, out[:, 4:n + 4])
+    assert torch.equal(out[:, 4:n + 4], whole)
+    assert float(out[:, :4].abs().max()) == 0.0 and float(out[:, n + 4:].abs().max()) == 0.0
+
+
 @pytest.mark.parametrize("m,n,k", [(1, 64, 4), (3, 70, 36), (8, 3584, 1536), (9, 129, 1028), (16, 1000, 4096), (40, 200, 520),
                                    (64, 333, 2052)])
 def test_gemm_stream_against_float64(m, n, k):

@@ -17,13 +17,15 @@
 //     never ends at -0);
 //   * the element is +0 + s0 + s1 + ... over its slabs in ascending order, then + bias, then,
 //     when accumulating, old + that.
-// Two kernels follow it. gemm_stream_kernel, for up to 64 rows of A in 32-bit operands, is a stream
+// Three kernels follow it. gemm_stream_kernel, for up to 64 rows of A in 32-bit operands, is a stream
 // of the weights: the product of a few tokens is bound by the bytes of W. gemm_generic_kernel is a
-// plain tiled product for everything else.
+// plain tiled product for everything else, gemm_generic_wide_kernel its twin with larger tiles for
+// 128 rows of A and more.
 #include "common.h"
 
 namespace {
 constexpr int RANGE_K = 256, SLAB_RANGES = 4, SLAB_K = RANGE_K * SLAB_RANGES;
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
 // ---------------------------------------------------------------------------------------------
 // The tiled product: any operand types, any M. A thread owns a 4 x 4 block of outputs and walks K in
@@ -108,9 +110,152 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const TA* __restrict_
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// The same product for 128 rows of A and more (prompts): a 128 x 128 tile, a thread owns 8 x 8 outputs (rows
+// 4 ty .. + 3 and 64 + 4 ty .. + 3, columns likewise with tx), so that a step of k costs four 16-byte LDS reads for
+// 64 FMAs where the 4 x 4 block above pays two for 16 and is bound by LDS as much as by arithmetic. The next
+// 16 k of both operands are on their way from memory into registers while this tile's are multiplied, and go
+// into the other half of a double LDS buffer: one barrier per 16 k. Every output element's sums are those of
+// the kernel above, in the same order.
+constexpr int WIDE = 128, WIDE_ROW = WIDE + 4;
+
+template <typename T>
+__device__ __forceinline__ void fetch4(const T* __restrict__ base, long long ld, int row, int rows, int k, int K,
+                                       bool vector_ok, float (&dst)[4]) {
+  if (row < rows && k + 3 < K && vector_ok) {
+    if constexpr (sizeof(T) == 4) {
+      const f32x4_t v = *(const f32x4_t*)(base + (size_t)row * ld + k);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) dst[e] = v[e];
+      return;
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < 4; ++e) dst[e] = (row < rows && k + e < K) ? to_float<T>(base[(size_t)row * ld + k + e]) : 0.f;
+}
+
+template <typename TA, typename TW, typename TC, bool ACCUMULATE>
+__global__ __launch_bounds__(256) void gemm_generic_wide_kernel(const TA* __restrict__ A, const TW* __restrict__ W,
+                                                                const float* __restrict__ bias, TC* __restrict__ C,
+                                                                int M, int N, int K, long long lda, long long ldc,
+                                                                int a_vector_ok, int w_vector_ok) {
+  __shared__ __attribute__((aligned(16))) float As[2][BK][WIDE_ROW];
+  __shared__ __attribute__((aligned(16))) float Ws[2][BK][WIDE_ROW];
+  const int tid = threadIdx.x;
+  const int m0 = blockIdx.y * WIDE, n0 = blockIdx.x * WIDE;
+  const int ty = tid / 16, tx = tid % 16;
+  float acc[8][8], slab[8][8], total[8][8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[i][j] = slab[i][j] = total[i][j] = 0.f;
+
+  // a thread stages rows tid / 4 and 64 + tid / 4 of both operands, k (tid % 4) * 4 .. + 3 of the tile
+  const int lr = tid / 4, lk = (tid % 4) * 4;
+  float ra[2][4], rw[2][4];
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      fetch4<TA>(A, lda, m0 + h * 64 + lr, M, k0 + lk, K, a_vector_ok, ra[h]);
+      fetch4<TW>(W, K, n0 + h * 64 + lr, N, k0 + lk, K, w_vector_ok, rw[h]);
+    }
+  };
+  auto stage = [&](int buf) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        As[buf][lk + e][h * 64 + lr] = ra[h][e];
+        Ws[buf][lk + e][h * 64 + lr] = rw[h][e];
+      }
+  };
+  fetch(0);
+  stage(0);
+  __syncthreads();
+  int buf = 0;
+  for (int k0 = 0; k0 < K; k0 += BK) {
+    const bool more = k0 + BK < K;
+    if (more) fetch(k0 + BK);
+#pragma unroll 4
+    for (int kk = 0; kk < BK; ++kk) {
+      float a[8], w[8];
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const f32x4_t av = *(const f32x4_t*)&As[buf][kk][h * 64 + ty * 4];
+        const f32x4_t wv = *(const f32x4_t*)&Ws[buf][kk][h * 64 + tx * 4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          a[h * 4 + e] = av[e];
+          w[h * 4 + e] = wv[e];
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[i][j] = fmaf(a[i], w[j], acc[i][j]);
+    }
+    if (more) stage(buf ^ 1);
+    __syncthreads();
+    buf ^= 1;
+    const int done = k0 + BK;
+    if (done % RANGE_K == 0 || done >= K) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          slab[i][j] += acc[i][j];
+          acc[i][j] = 0.f;
+        }
+    }
+    if (done % SLAB_K == 0 || done >= K) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          total[i][j] += slab[i][j];
+          slab[i][j] = 0.f;
+        }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int m = m0 + (i / 4) * 64 + ty * 4 + i % 4;
+    if (m >= M) continue;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int n = n0 + (j / 4) * 64 + tx * 4 + j % 4;
+      if (n >= N) continue;
+      float v = total[i][j];
+      if (bias) v += bias[n];
+      TC* dst = C + (size_t)m * ldc + n;
+      if (ACCUMULATE)
+        *dst = from_float<TC>(to_float<TC>(*dst) + v);
+      else
+        *dst = from_float<TC>(v);
+    }
+  }
+}
+
 template <typename TA, typename TW, typename TC>
 int launch(const void* A, const void* W, const float* bias, void* C, int M, int N, int K, long long lda,
            long long ldc, int accumulate, hipStream_t s) {
+  // the wide tiles where they are enough to occupy a quarter of the GPU at least (2,048 x 37,888 x 3,584: 7.9 ms
+  // against 15.1, 90 % of the rate of unpacked FMAs; 200 x 1,000 x 520, 16 tiles: 107 us against 81)
+  const long long wide_tiles = (long long)((M + WIDE - 1) / WIDE) * ((N + WIDE - 1) / WIDE);
+  if (M >= WIDE && N >= WIDE && wide_tiles >= 64) {
+    dim3 grid((N + WIDE - 1) / WIDE, (M + WIDE - 1) / WIDE);
+    // 16-byte loads where every row of an operand starts on a 16-byte boundary
+    const int a_ok = sizeof(TA) == 4 && ((uintptr_t)A % 16 == 0) && lda % 4 == 0;
+    const int w_ok = sizeof(TW) == 4 && ((uintptr_t)W % 16 == 0) && K % 4 == 0;
+    if (accumulate)
+      gemm_generic_wide_kernel<TA, TW, TC, true><<<grid, 256, 0, s>>>((const TA*)A, (const TW*)W, bias, (TC*)C, M, N, K, lda,
+                                                                      ldc, a_ok, w_ok);
+    else
+      gemm_generic_wide_kernel<TA, TW, TC, false><<<grid, 256, 0, s>>>((const TA*)A, (const TW*)W, bias, (TC*)C, M, N, K, lda,
+                                                                       ldc, a_ok, w_ok);
+    VK_LAUNCH_CHECK();
+    return 0;
+  }
   dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM);
   if (accumulate)
     gemm_generic_kernel<TA, TW, TC, true><<<grid, 256, 0, s>>>((const TA*)A, (const TW*)W, bias, (TC*)C, M, N, K, lda, ldc);
@@ -134,7 +279,6 @@ int launch(const void* A, const void* W, const float* bias, void* C, int M, int 
 // multiplies the other, and the waves do not wait for one another until the end of the range.
 constexpr int STREAM_ROWS = 64, SUB_K = 32, W_STAGE = STREAM_ROWS * SUB_K * 4, W_LOADS = W_STAGE / 1024;
 
-typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) void* lds_ptr;
 typedef __attribute__((address_space(1))) const void* global_ptr;
 
