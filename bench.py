@@ -99,6 +99,9 @@ def main() -> int:
                         help="instead of the headline measurement: a continuous batch of 64 requests, prompts of 128 to "
                              "8,192 random tokens in portions of 512, 256 new tokens each (the 1.5B workload; use with "
                              "--shape 1.5b --ctx 32768)")
+    parser.add_argument("--cache-share", type=float, default=1.0,
+                        help="with --serving: the cache pool as a share of the pages that all requests need together "
+                             "(below 1 the scheduler has to hold requests back, and preempts when pages run out)")
     parser.add_argument("--split", action="store_true",
                         help="also run one decode step (of --batch requests at --ctx) and one prefill eagerly with a "
                              "pair of GPU events around every kernel launch, and add the microseconds of each class of "
@@ -361,8 +364,9 @@ def serving(args, config, runtime, model, shape_name, layers_full, dtype_key) ->
     gen = torch.Generator().manual_seed(1)
     lengths = torch.randint(128, 8193, (requests,), generator=gen).tolist()
     prompts = [torch.randint(0, config.vocab_size, (n,), generator=gen).tolist() for n in lengths]
-    pages = sum((n + new_tokens + args.block_size - 1) // args.block_size + 1 for n in lengths)
-    context = max(args.ctx, max(lengths) + new_tokens)   # the longest request has to fit
+    needed = [(n + new_tokens + args.block_size - 1) // args.block_size + 1 for n in lengths]
+    pages = max(int(sum(needed) * args.cache_share), max(needed) + 1)   # the longest request has to fit
+    context = max(args.ctx, max(lengths) + new_tokens)
     runner = ModelRunner(model, runtime, args.block_size, pages, requests + 1, use_graphs=True, max_context=context)
     engine = Engine(None, runner=runner, max_num_seqs=requests, max_num_batched_tokens=budget, chunk_size=chunk,
                     max_model_len=context, pipelined=not args.in_turn)
@@ -400,7 +404,9 @@ def serving(args, config, runtime, model, shape_name, layers_full, dtype_key) ->
         "config": {"model": shape_name, "layers": args.layers, "layers_full": layers_full, "requests": requests,
                    "prompt_tokens": prompt_tokens, "new_tokens_each": new_tokens, "chunk_size": chunk,
                    "max_num_batched_tokens": budget, "seq_len": context, "block_size": args.block_size,
-                   "steps_launched_ahead": not args.in_turn, "decode_steps_captured_ahead": captured},
+                   "steps_launched_ahead": not args.in_turn, "decode_steps_captured_ahead": captured,
+                   "cache_pages": pages, "cache_share": args.cache_share,
+                   "preemptions": engine.stats()["preemptions"]},
         "generated_per_second": round(generated / seconds, 1), "seconds": round(seconds, 3),
     }), flush=True)
     return 0
