@@ -32,6 +32,7 @@
 // Reference for what is computed: crates/vipera-backend-cpu/src/model.rs:1005-1031 (batched products,
 // bias after the product); the idea of reading a weight row once for many tokens is that of the
 // reference's batched matvec (crates/vipera-backend-gpu/src/q4k_matvec_q8_batch.cu:40-116).
+#include <cmath>
 #include <mutex>
 
 #include "common.h"
@@ -1756,6 +1757,13 @@ int g_tile_stages = 0;   // 0: chosen by shape; 2 or 3 force the direct kernel's
 // in the caches: about 6 TB/s) and one more launch; each range keeps at least 512 of K. The estimate ranks
 // the plans as measurements at 128 to 2,048 tokens do. Few tokens keep the token side of the tile at 128.
 // Ties go to the larger tile and to fewer ranges.
+// Past 128 tokens the estimate is fitted to a sweep of every tiling and split over the q/k/v, output, down and
+// gate/up products of the seven Qwen2.5 shapes at 256 to 2,048 tokens (the plan it picks is within 1 % of the
+// fastest on average and 10 % at worst; with a share of time lost in proportion to the unfilled share it was 3
+// and 32 %): a launch that fills its rounds to a share f runs at f^0.6 of the full rate, not f, because the
+// CUs that are at work run faster when others are idle (what is limited is the chip, not the CU); a workgroup
+// alone on a CU that could hold two runs at 0.75 of its share; the 128x128 tile on eight waves is worth 1.0 and
+// 256x192 1.1; a split costs 2 us beside its bytes.
 struct TilePlan { int config, ranges; };
 int g_compute_units = 0;
 // the 128-token tiles of the direct kernel run with a third LDS stage for up to 128 tokens (see launch_tile)
@@ -1780,6 +1788,7 @@ TilePlan choose_tile_plan(int M, int N, int K, long long partial_floats, bool di
   TilePlan best{tilings[3].config, 1};
   double best_time = 1e30;
   const double flops = 2.0 * M * N * (double)K, output_bytes = 4.0 * M * N;
+  const bool many = M > 128 && direct;   // the fitted estimate
   for (int i = 0; i < (direct ? (gated && M <= 128 ? 8 : 5) : 4); ++i) {
     const Tiling& t = tilings[i];
     if (M <= 128 && t.tokens > 128) continue;
@@ -1795,8 +1804,16 @@ TilePlan choose_tile_plan(int M, int N, int K, long long partial_floats, bool di
       const long long slots = groups * ranges <= g_compute_units ? g_compute_units : (long long)g_compute_units * resident;
       const long long rounds = (groups * ranges + slots - 1) / slots;
       const double fill = (double)(groups * ranges) / ((double)rounds * slots);
-      double time = flops / (1e15 * t.speed * fill);
-      if (ranges > 1) time += (2.0 * ranges + 1.0) * output_bytes / 6e12 + 4e-6;
+      double speed = t.speed, share = fill, launch = 4e-6;
+      if (many) {
+        if (t.config == 9) speed = 1.0;
+        if (t.config == 6) speed = 1.1;
+        if (resident == 2 && groups * ranges <= g_compute_units) speed *= 0.75;
+        share = pow(fill, 0.6);
+        launch = 2e-6;
+      }
+      double time = flops / (1e15 * speed * share);
+      if (ranges > 1) time += (2.0 * ranges + 1.0) * output_bytes / 6e12 + launch;
       if (time < best_time * (1.0 - 1e-9)) {
         best_time = time;
         best = TilePlan{t.config, ranges};
