@@ -1758,12 +1758,12 @@ int g_tile_stages = 0;   // 0: chosen by shape; 2 or 3 force the direct kernel's
 // the plans as measurements at 128 to 2,048 tokens do. Few tokens keep the token side of the tile at 128.
 // Ties go to the larger tile and to fewer ranges.
 // Past 128 tokens the estimate is fitted to a sweep of every tiling and split over the q/k/v, output, down and
-// gate/up products of the seven Qwen2.5 shapes at 256 to 2,048 tokens (the plan it picks is within 1 % of the
-// fastest on average and 10 % at worst; with a share of time lost in proportion to the unfilled share it was 3
-// and 32 %): a launch that fills its rounds to a share f runs at f^0.6 of the full rate, not f, because the
-// CUs that are at work run faster when others are idle (what is limited is the chip, not the CU); a workgroup
-// alone on a CU that could hold two runs at 0.75 of its share; the 128x128 tile on eight waves is worth 1.0 and
-// 256x192 1.1; a split costs 2 us beside its bytes.
+// gate/up products of the seven Qwen2.5 shapes at 160 to 4,096 tokens (the plans it picks cost 1 % more time than
+// the fastest ones together, 15 % at worst; with a share of time lost in proportion to the unfilled share it was
+// 4 and 47 %): the work is that of whole tiles; a launch that fills its rounds to a share f runs at f^0.6 of the
+// full rate, not f, because the CUs that are at work run faster when others are idle (what is limited is the
+// chip, not the CU); a workgroup alone on a CU that could hold two runs at 0.75 of its share; the 128x128 tile on
+// eight waves is worth 0.95, 256x128 1.05 and 256x192 1.1; a range of a split costs three passes over the output.
 struct TilePlan { int config, ranges; };
 int g_compute_units = 0;
 // the 128-token tiles of the direct kernel run with a third LDS stage for up to 128 tokens (see launch_tile)
@@ -1804,16 +1804,18 @@ TilePlan choose_tile_plan(int M, int N, int K, long long partial_floats, bool di
       const long long slots = groups * ranges <= g_compute_units ? g_compute_units : (long long)g_compute_units * resident;
       const long long rounds = (groups * ranges + slots - 1) / slots;
       const double fill = (double)(groups * ranges) / ((double)rounds * slots);
-      double speed = t.speed, share = fill, launch = 4e-6;
+      double time;
       if (many) {
-        if (t.config == 9) speed = 1.0;
-        if (t.config == 6) speed = 1.1;
+        double speed = t.config == 9 ? 0.95 : t.config == 6 ? 1.1 : t.config == 7 ? 1.05 : t.speed;
         if (resident == 2 && groups * ranges <= g_compute_units) speed *= 0.75;
-        share = pow(fill, 0.6);
-        launch = 2e-6;
+        // the work of whole tiles: rows past M or N are multiplied like the others
+        const double tile_flops = 2.0 * (double)groups * t.tokens * t.rows * (double)K;
+        time = tile_flops / (1e15 * speed * pow(fill, 0.6));
+        if (ranges > 1) time += (3.0 * ranges + 1.0) * output_bytes / 6e12;
+      } else {
+        time = flops / (1e15 * t.speed * fill);
+        if (ranges > 1) time += (2.0 * ranges + 1.0) * output_bytes / 6e12 + 4e-6;
       }
-      double time = flops / (1e15 * speed * share);
-      if (ranges > 1) time += (2.0 * ranges + 1.0) * output_bytes / 6e12 + launch;
       if (time < best_time * (1.0 - 1e-9)) {
         best_time = time;
         best = TilePlan{t.config, ranges};
