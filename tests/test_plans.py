@@ -45,6 +45,7 @@ def test_past_64_tokens_the_weights_are_streamed_where_tiles_would_be_few():
         assert not streams_weights(m, 5120, 27648)
     assert mid_plan(65, 1536, 8960) == (8, 1) and mid_plan(96, *O_7B) == (4, 1) and mid_plan(128, 2048, 1536) == (4, 1)
     assert mid_plan(100, 1024, 320) == (1, 1)              # no range shorter than 256
+    assert mid_plan(65, 896, 4864) == (8, 1)               # the 0.5B down projection
 
 
 def test_the_gated_product_goes_resident_tiled_or_lds_shared():

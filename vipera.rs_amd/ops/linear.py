@@ -34,8 +34,9 @@ def streams_weights(m: int, n: int, k: int) -> bool:
 
 def mid_plan(m: int, n: int, k: int) -> Tuple[int, int]:
     """``(ranges of K, 16-row tiles per wave)`` for the LDS-shared kernel."""
-    if m > 64:  # measured at 65, 96 and 128 tokens: one tile per wave; eight ranges of a long K, else four
-        return max(1, min(8 if k >= 8_192 else 4, k // 256)), 1
+    if m > 64:  # measured at 65, 96 and 128 tokens: one tile per wave; eight ranges of a long K, else four (the 0.5B
+        # down projection, 896 x 4,864, at 65 tokens: 10.7 us with eight ranges, 14.2 with four)
+        return max(1, min(8 if k >= 4_096 else 4, k // 256)), 1
     if n >= 100_000:
         return (1, 2) if m > 16 else (1, 1)
     if n >= 16_384:
