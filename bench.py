@@ -306,7 +306,7 @@ def kernel_split(args, config, runner, tokens, ctx, T):
             return products.get(shape, f"product_{shape[0]}x{shape[1]}")
         return other.get(name, name)
 
-    sampler = BatchSampler(runner.runtime.device)
+    sampler = BatchSampler(runner.runtime.device, slots=max(64, args.batch))
     runs = 5
 
     def measure(entries_of, rows):

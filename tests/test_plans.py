@@ -102,6 +102,16 @@ def test_decode_attention_chunks():
     assert chunks <= 128 and chunk * chunks >= 1 << 20 and chunk % 32 == 0
 
 
+def test_one_workgroup_takes_all_chunks_of_a_request_and_key_head_where_those_fill_the_gpu():
+    from vipera_rs_amd.ops.attention import joins_decode_chunks
+    assert joins_decode_chunks(4, 64, 4, 1, 256) and joins_decode_chunks(4, 128, 4, 1, 256)
+    assert not joins_decode_chunks(16, 8, 4, 1, 256)        # 32 pairs for 256 CUs
+    assert not joins_decode_chunks(16, 64, 4, 1, 256)       # more chunks than a workgroup has waves
+    # a few more pairs than CUs: the CUs with two workgroups would set the time
+    assert not joins_decode_chunks(4, 72, 4, 1, 256) and not joins_decode_chunks(4, 40, 8, 1, 256)
+    assert not joins_decode_chunks(4, 96, 4, 1, 256) and joins_decode_chunks(4, 112, 4, 1, 256)
+
+
 def test_prompt_tiles_are_halved_between_sixteen_waves_only_where_a_cu_would_be_left_with_one_workgroup():
     from vipera_rs_amd.ops.attention import halves_prompt_tiles
     reach = [128 * (t + 1) for t in range(16)]                       # one prompt of 2,048 tokens

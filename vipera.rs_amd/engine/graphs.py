@@ -23,8 +23,9 @@ from .batch import PackedStep, StepEntry, batch_from_buffer, pack_entries
 # Padded batch sizes of the captured steps. A padding entry sees no positions, but its row of activations is read by
 # every workgroup of the products that stream weights in wave order (up to 8 tokens), so 5 and 6 requests have a
 # size of their own below 8 (the 7B shape: 5 requests as 8 took 3.60 ms a step, as 6 they take 3.48; 4 take 3.37),
-# and 9 to 12 one below 16 (9 requests 3.93 to 3.84 ms).
-BATCH_BUCKETS = (1, 2, 4, 6, 8, 12, 16, 24, 32, 48, 64, 96, 128, 192, 256)
+# and 9 to 12 one below 16 (9 requests 3.93 to 3.84 ms). Past 64 the sizes are 16 apart, then 32: a step of 96 tokens
+# costs what 96 cost in every product (72 requests as 96 took 8.02 ms, as 80 they take 7.69).
+BATCH_BUCKETS = (1, 2, 4, 6, 8, 12, 16, 24, 32, 48, 64, 80, 96, 112, 128, 160, 192, 224, 256)
 
 
 def _bucket(value: int, buckets: Sequence[int]) -> Optional[int]:

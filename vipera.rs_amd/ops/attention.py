@@ -36,8 +36,14 @@ def joins_decode_chunks(chunks: int, num_entries: int, kv_heads: int, head_block
     """Whether one workgroup per (entry, key head) takes all chunks, a wave each, and merges them itself instead of
     a workgroup per chunk and a second kernel: where those pairs alone fill the GPU (64 requests x 4 key heads on 256
     CUs), so that the chunks only serve to keep several waves on a CU; the merge kernel and the chunks' round trip
-    through memory are saved (4.9 us a layer at the 7B head shape)."""
-    return chunks <= kernels.ATTN_DECODE_JOINED_CHUNKS and num_entries * kv_heads * head_blocks >= 0.8 * cus
+    through memory are saved (4.9 us a layer at the 7B head shape).  Not where the pairs are a few more than the CUs:
+    the CUs with two workgroups then set the time (72 requests x 4 key heads at 4,096 positions: 141 us joined, 124
+    with a workgroup per chunk; 96 requests: 157 and 155; from 112 on joined is ahead again; a captured step of 96
+    entries also serves 65 to 95 requests)."""
+    pairs = num_entries * kv_heads * head_blocks
+    if cus < pairs < 1.55 * cus:
+        return False
+    return chunks <= kernels.ATTN_DECODE_JOINED_CHUNKS and pairs >= 0.8 * cus
 
 
 def halves_prompt_tiles(num_tiles: int, heads: int, longest: int, total: int, cus: int) -> bool:
