@@ -250,7 +250,7 @@ def test_a_captured_step_of_many_requests_rotates_by_the_positions_of_each_repla
         assert torch.equal(outs[0], outs[1]), f"replay {step} differs from the eager step"
         for r in prompts:
             lengths[r] += 1
-    assert runners[1].graphs.replays == 6 and list(runners[1].graphs.graphs) == [(192, 256)]
+    assert runners[1].graphs.replays == 6 and list(runners[1].graphs.graphs) == [(160, 256)]
 
 
 # --- steps launched ahead of their tokens ---------------------------------------------------------------------------
