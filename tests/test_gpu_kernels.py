@@ -590,6 +590,21 @@ def test_decode_attention_at_the_benchmark_head_shapes(heads, kv_heads, hd, batc
             kernels.attn_bf16_decode(qkv_d, k_d, v_d, joined, None, singles, es, fp, dev(table), heads, kv_heads, hd, scale,
                                      0, chunk, chunks, dense=True, join=True)
             assert _rel(joined.cpu(), want) < 1.2e-2, f"visible {visible}: chunk {chunk} x {chunks}, joined"
+    # the long chunks of many requests at long contexts, over a table as wide as theirs
+    visible = 4 * _context_bucket(longest)
+    table = torch.full((batch, (visible + bs - 1) // bs), -1, dtype=torch.int32)
+    table[:, :cache.table.shape[1]] = cache.table
+    for chunk in (2048, 4096):
+        chunks = (visible + chunk - 1) // chunk
+        out = torch.zeros(batch, heads * hd, dtype=dtype, device=DEV)
+        partial = torch.full((batch * heads * chunks * (hd + 2),), float("nan"), device=DEV)
+        kernels.attn_bf16_decode(qkv_d, k_d, v_d, out, partial, singles, es, fp, dev(table), heads, kv_heads, hd, scale, 0,
+                                 chunk, chunks, dense=True)
+        assert _rel(out.cpu(), want) < 1.2e-2, f"visible {visible}: chunk {chunk} x {chunks}"
+        joined = torch.zeros(batch, heads * hd, dtype=dtype, device=DEV)
+        kernels.attn_bf16_decode(qkv_d, k_d, v_d, joined, None, singles, es, fp, dev(table), heads, kv_heads, hd, scale,
+                                 0, chunk, chunks, dense=True, join=True)
+        assert _rel(joined.cpu(), want) < 1.2e-2, f"visible {visible}: chunk {chunk} x {chunks}, joined"
     out = torch.zeros(batch, heads * hd, dtype=dtype, device=DEV)
     kernels.attn_generic(qkv_d, k_d, v_d, out, fp, singles, dev(cache.table), heads, kv_heads, hd, scale, 0)
     assert _rel(out.cpu(), want) < 1.2e-2, "32-bit-arithmetic kernel on the bfloat16 cache"

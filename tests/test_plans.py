@@ -98,6 +98,10 @@ def test_decode_attention_chunks():
     assert decode_chunking(4096, 64, 4, 1) == (1024, 4)
     assert decode_chunking(4096, 1, 4, 1) == (128, 32)     # never below 128 positions a chunk
     assert decode_chunking(100, 1, 4, 1) == (128, 1)
+    # many requests at long contexts: longer chunks while they still make 2,048 waves
+    assert decode_chunking(32768, 64, 4, 1) == (4096, 8) and decode_chunking(16384, 64, 4, 1) == (2048, 8)
+    assert decode_chunking(8192, 64, 4, 1) == (1024, 8) and decode_chunking(32768, 16, 4, 1) == (1024, 32)
+    assert decode_chunking(32768, 64, 2, 1) == (2048, 16)
     chunk, chunks = decode_chunking(1 << 20, 1, 1, 1)      # never more than 128 chunks
     assert chunks <= 128 and chunk * chunks >= 1 << 20 and chunk % 32 == 0
 
