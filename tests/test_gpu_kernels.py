@@ -67,6 +67,34 @@ def test_gemm_bf16_every_tiling_of_the_tiled_kernel(tiling, ranges):
         kernels.gemm_bf16_force_tiling(-1)
 
 
+@pytest.mark.parametrize("tiling", [0, 9, 7, 5, 6])
+def test_the_tiled_kernel_computes_the_same_in_every_order_of_its_tiles(tiling):
+    """The workgroups walk the tiles in blocks of a few rows of tiles (chosen by shape, forced here): every tile is
+    computed once whatever the block height, also where the last block has fewer rows and where the launch has
+    more workgroups than tiles."""
+    from vipera_rs_amd.ops import kernels
+    g = torch.Generator().manual_seed(tiling)
+    m, n, k = 1100, 1300, 192
+    a = torch.randn(m, k, generator=g).to(torch.bfloat16).to(DEV)
+    w = torch.randn(n, k, generator=g).to(torch.bfloat16).to(DEV)
+    want = a.double() @ w.double().T
+    outs = []
+    try:
+        for ranges in (1, 3):
+            kernels.gemm_bf16_force_tiling(tiling, ranges)
+            for rows in (0, 1, 2, 4, 5, 7, 50):
+                kernels.gemm_bf16_force_tile_group(rows)
+                out = torch.full((m, n), 7.0, device=DEV)
+                kernels.gemm_bf16(a, w, None, out)
+                assert _rel(out, want) < 1e-5, (ranges, rows)
+                outs.append(out)
+            assert all(torch.equal(outs[0], o) for o in outs[1:]), ranges
+            outs.clear()
+    finally:
+        kernels.gemm_bf16_force_tile_group(0)
+        kernels.gemm_bf16_force_tiling(-1)
+
+
 @pytest.mark.parametrize("tiling", [9, 8])
 @pytest.mark.parametrize("ranges", [1, 3])
 def test_gemm_bf16_direct_tilings_with_three_lds_stages(tiling, ranges):

@@ -252,6 +252,36 @@ __device__ __forceinline__ void tile_epilogue(f32x4 (&acc)[TN][TM], TC* __restri
       store4<TC, ACCUMULATE>(C, ldc, wave_m + tm * 16 + lr, wave_n + tn * 16 + lg * 4, M, N, acc[tn][tm], bias, vector_ok);
 }
 
+// Which tile the `logical`-th workgroup of a launch owns. An XCD gets a contiguous run of logical numbers, and the
+// tiles of a run share that XCD's L2: the numbers walk blocks of `group_m` tile rows, down the rows of a block first
+// and then along its columns, so that a run covers few rows of tiles of A and few of W at the same time (a run of
+// 28 tiles of 256 x 128 as 4 x 7 reads 1,024 rows of A and 896 of W at every step of K, as 8 x 3.5 2,048 and 448:
+// a quarter fewer bytes into L2). The last block may have fewer rows.
+__device__ __forceinline__ void tile_of(int logical, int tiles_m, int tiles_n, int group_m, int* tile_m, int* tile_n) {
+  const int block = logical / (group_m * tiles_n);
+  const int first_row = block * group_m;
+  const int rows = min(group_m, tiles_m - first_row);
+  const int within = logical - block * group_m * tiles_n;
+  *tile_n = within / rows;
+  *tile_m = first_row + within % rows;
+}
+
+// Tile rows per block for tile_of: the count that makes the `per_xcd` tiles that an XCD works on at one time read
+// the fewest rows of A and W together, rows x BM + ceil(per_xcd / rows) x BN (4,096 tokens: the 7B gate/up product
+// 921 to 884 us, the 72B q/k/v product 663 to 558; at 2,048 tokens, eight rows of tiles, within 2 % either way).
+inline int tile_group_rows(int tiles_m, long long per_xcd, int BM, int BN) {
+  int best = 1;
+  long long best_cost = -1;
+  for (int rows = 1; rows <= tiles_m; ++rows) {
+    const long long cost = (long long)rows * BM + (per_xcd + rows - 1) / rows * BN;
+    if (best_cost < 0 || cost < best_cost) {
+      best = rows;
+      best_cost = cost;
+    }
+  }
+  return best;
+}
+
 // BM x BN: output tile of a workgroup (tokens x weight rows); WM x WN: its grid of waves. A wave owns
 // (BM / WM) x (BN / WN) outputs as TM x TN instruction tiles.
 template <int BM, int BN, int WM, int WN, typename TC, bool ACCUMULATE, bool GATED>
@@ -259,7 +289,8 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_tile_kernel(const __bf16* _
                                                                    const __bf16* __restrict__ W,
                                                                    const float* __restrict__ bias, TC* __restrict__ C,
                                                                    int M, int N, int K, long long lda, long long ldc,
-                                                                   int tiles_m, int tiles_n, int vector_ok,
+                                                                   int tiles_m, int tiles_n, int group_m,
+                                                                   int vector_ok,
                                                                    int k_per_range, long long range_stride,
                                                                    TileNorm norm) {
   // gridDim.y > 1: K is split into ranges of k_per_range (a multiple of 64); range r writes its partial
@@ -279,8 +310,8 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_tile_kernel(const __bf16* _
   const int per_xcd = (total + XCDS - 1) / XCDS;
   const int logical = (blockIdx.x % XCDS) * per_xcd + blockIdx.x / XCDS;
   if (logical >= total) return;
-  // tiles of one column panel of W (all m for one n) are neighbours
-  const int tile_n = logical / tiles_m, tile_m = logical % tiles_m;
+  int tile_m, tile_n;
+  tile_of(logical, tiles_m, tiles_n, group_m, &tile_m, &tile_n);
   const int m0 = tile_m * BM, n0 = tile_n * BN;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -410,7 +441,8 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_tile_direct_kernel(const __
                                                                           const float* __restrict__ bias,
                                                                           TC* __restrict__ C, int M, int N, int K,
                                                                           long long lda, long long ldc, int tiles_m,
-                                                                          int tiles_n, int vector_ok, int k_per_range,
+                                                                          int tiles_n, int group_m, int vector_ok,
+                                                                          int k_per_range,
                                                                           long long range_stride, TileNorm norm) {
   typedef __attribute__((address_space(3))) void* lds_ptr;
   const int k_begin = blockIdx.y * k_per_range, k_end = min(K, k_begin + k_per_range);
@@ -428,7 +460,8 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_tile_direct_kernel(const __
   const int per_xcd = (total + XCDS - 1) / XCDS;
   const int logical = (blockIdx.x % XCDS) * per_xcd + blockIdx.x / XCDS;
   if (logical >= total) return;
-  const int tile_n = logical / tiles_m, tile_m = logical % tiles_m;
+  int tile_m, tile_n;
+  tile_of(logical, tiles_m, tiles_n, group_m, &tile_m, &tile_n);
   const int m0 = tile_m * BM, n0 = tile_n * BN;
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -1687,6 +1720,8 @@ int launch_mid(const __bf16* A, const __bf16* W, const float* bias, TC* C, float
   return VK_UNSUPPORTED_SIZE;
 }
 
+int g_tile_group_m = 0;   // 0: chosen by shape; else the rows of tiles per block of tile_of, for measurements
+
 template <bool DIRECT, int BM, int BN, int WM, int WN, typename TC, bool ACC, bool GATED, int STAGES>
 constexpr auto tile_kernel() {
   if constexpr (DIRECT) return gemm_tile_direct_kernel<BM, BN, WM, WN, TC, ACC, GATED, STAGES>;
@@ -1704,6 +1739,10 @@ int launch_tile_as(const __bf16* A, const __bf16* W, const float* bias, TC* C, i
   const long long total = (long long)tiles_m * tiles_n;
   const long long grid = (total + XCDS - 1) / XCDS * XCDS;
   if (grid > 0x7fffffffLL) return VK_UNSUPPORTED_SIZE;
+  // the tiles that an XCD works on at one time: one per CU, or two where the stages' LDS lets two share a CU
+  const long long at_once = (long long)(compute_units() / XCDS) * (lds_bytes * 2 <= 160 * 1024 ? 2 : 1);
+  const int group_m = g_tile_group_m > 0 ? (g_tile_group_m < tiles_m ? g_tile_group_m : tiles_m)
+                                         : tile_group_rows(tiles_m, grid / XCDS < at_once ? grid / XCDS : at_once, BM, BN);
   if (ranges <= 1 || GATED) {
     static bool configured = false;
     auto kernel = tile_kernel<DIRECT, BM, BN, WM, WN, TC, ACC, GATED, STAGES>();
@@ -1712,8 +1751,8 @@ int launch_tile_as(const __bf16* A, const __bf16* W, const float* bias, TC* C, i
       if (e != hipSuccess) return (int)e;
       configured = true;
     }
-    kernel<<<(int)grid, WM * WN * 64, lds_bytes, s>>>(A, W, bias, C, M, N, K, lda, ldc, tiles_m, tiles_n, vector_ok, K,
-                                                      0, norm);
+    kernel<<<(int)grid, WM * WN * 64, lds_bytes, s>>>(A, W, bias, C, M, N, K, lda, ldc, tiles_m, tiles_n, group_m,
+                                                      vector_ok, K, 0, norm);
     VK_LAUNCH_CHECK();
     return 0;
   }
@@ -1729,8 +1768,8 @@ int launch_tile_as(const __bf16* A, const __bf16* W, const float* bias, TC* C, i
     const int k_per_range = ((K + ranges - 1) / ranges + BK - 1) / BK * BK;
     const int used = (K + k_per_range - 1) / k_per_range;
     kernel<<<dim3((unsigned)grid, used), WM * WN * 64, lds_bytes, s>>>(A, W, nullptr, partial, M, N, K, lda, N, tiles_m,
-                                                                       tiles_n, (N & 3) == 0 ? 1 : 0, k_per_range,
-                                                                       (long long)M * N, norm);
+                                                                       tiles_n, group_m, (N & 3) == 0 ? 1 : 0,
+                                                                       k_per_range, (long long)M * N, norm);
     VK_LAUNCH_CHECK();
     const long long threads = (long long)M * ((N + 3) / 4);
     gemm_reduce_kernel<TC, ACC><<<(int)((threads + 255) / 256), 256, 0, s>>>(partial, bias, C, M, N, ldc, used, vector_ok);
@@ -2211,6 +2250,13 @@ extern "C" int vk_gemm_bf16_gated_tile_scaled(const void* A, const void* W, void
   norm.eps = eps;
   return launch_tile<__bf16, false, true>((const __bf16*)A, (const __bf16*)W, nullptr, (__bf16*)C, M, N, K, lda, ldc, 0,
                                           nullptr, 0, (hipStream_t)stream, norm);
+}
+
+// For measurements: the rows of tiles per block of the tiled kernel's tile order (0: chosen by shape).
+extern "C" int vk_gemm_bf16_tile_group(int rows) {
+  if (rows < 0) return VK_BAD_ARGUMENT;
+  g_tile_group_m = rows;
+  return 0;
 }
 
 extern "C" int vk_gemm_bf16_tile_config(int tiling, int ranges, int stages) {

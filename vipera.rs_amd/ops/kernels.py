@@ -696,6 +696,12 @@ def gemm_bf16_force_tiling(tiling: int = -1, ranges: int = 1, stages: int = 0) -
     _status(fn(-1 if tiling < 0 else tiling, int(ranges), int(stages)), "gemm_bf16_force_tiling")
 
 
+def gemm_bf16_force_tile_group(rows: int = 0) -> None:
+    """For measurements: the tiled kernel walks its tiles in blocks of ``rows`` rows of tiles (0: chosen by shape)."""
+    fn = _fn("gemm_bf16", "vk_gemm_bf16_tile_group", [_i])
+    _status(fn(int(rows)), "gemm_bf16_force_tile_group")
+
+
 # ----------------------------------------------------------------------------------------------
 def attn_bf16_padded_width(head_dim: int) -> int:
     """The padded head width a matrix-core attention module is compiled for (a multiple of 32)."""
