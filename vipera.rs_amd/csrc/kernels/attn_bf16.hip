@@ -562,11 +562,24 @@ __global__ __launch_bounds__(SPLIT ? 2 * PT_THREADS : PT_THREADS) void attn_pref
   // work items as in attn_prefill_kernel: long ones first, paired with short ones on a CU (SPLIT: one
   // workgroup per CU, longest first)
   const int total = CHUNKED ? (int)gridDim.x / max_chunks : (int)gridDim.x, round = blockIdx.x / cus;
-  const int taken = (round >> 1) * cus + blockIdx.x % cus;
+  // Workgroups go to the XCDs in turn, and the query heads of one key head read the same K and V: of every 8 x
+  // group workgroups in a row the ones that land on one XCD take the heads of one group, so that the XCD's L2
+  // fetches those tiles once (with numbers in a row, every head of a group ran on another XCD). Every other run
+  // of 8 groups is dealt to the XCDs in the opposite order: the items come sorted by length, and dealt one way
+  // only the first XCDs would get the longer item of every run.
+  const int heads_per_key = heads / kv_heads;
+  auto by_xcd = [&](int number, int count) {
+    const int block = 8 * heads_per_key;
+    if (number >= count / block * block) return number;
+    const int within = number % block;
+    const int xcd = ((number / block) & 1) ? 7 - within % 8 : within % 8;
+    return number - within + xcd * heads_per_key + within / 8;
+  };
+  const int taken = (round >> 1) * cus + by_xcd((int)blockIdx.x % cus, min(cus, total - round * cus));
   // CHUNKED: the chunks of one (tile, head) are neighbours, the tiles that see most positions come first
   const int chunk = CHUNKED ? (int)blockIdx.x % max_chunks : 0;
   const int item = CHUNKED ? total - 1 - (int)blockIdx.x / max_chunks
-                           : SPLIT ? total - 1 - (int)blockIdx.x : (round & 1) ? taken : total - 1 - taken;
+                           : SPLIT ? total - 1 - by_xcd((int)blockIdx.x, total) : (round & 1) ? taken : total - 1 - taken;
   const int tile = item / heads;
   const int entry = tiles[2 * tile], tile_off = tiles[2 * tile + 1];
   const int h = item % heads, kvh = h / (heads / kv_heads);
