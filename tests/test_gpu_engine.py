@@ -250,7 +250,63 @@ def test_a_captured_step_of_many_requests_rotates_by_the_positions_of_each_repla
         assert torch.equal(outs[0], outs[1]), f"replay {step} differs from the eager step"
         for r in prompts:
             lengths[r] += 1
-    assert runners[1].graphs.replays == 6 and list(runners[1].graphs.graphs) == [(160, 256)]
+    assert runners[1].graphs.replays == 6 and [key[:2] for key in runners[1].graphs.graphs] == [(160, 256)]
+
+
+def test_captured_steps_of_every_fill_class_follow_the_eager_steps(tmp_path):
+    """64 requests under one context bucket of 1,024: first one long among short ones (a small share of the bucket
+    is filled: the graph's attention cuts the positions into shorter chunks), then all long (the full class).  Each
+    class has a graph of its own where the launches differ, and every replay follows the eager step, whose chunks
+    are chosen from the true lengths."""
+    from helpers import rel_err
+    from vipera_rs_amd.engine.batch import StepEntry
+    from vipera_rs_amd.engine.graphs import DecodeGraphs
+    from vipera_rs_amd.engine.runner import ModelRunner
+    config = dict(CONFIG_A, max_position_embeddings=1024)
+    folder = make_folder(tmp_path, config, 8, torch.bfloat16)
+    vocab, live = config["vocab_size"], 64
+    runners = [ModelRunner.from_folder(folder, dtype="bfloat16", block_size=16, num_blocks=live * 60, num_slots=live)
+               for _ in range(2)]
+    runners[1].graphs = DecodeGraphs(runners[1], 1024)
+    lengths = {r: 0 for r in range(live)}
+
+    def extend(request, count):
+        tokens = random_tokens(vocab, count, 1000 * request + lengths[request])
+        for runner in runners:
+            runner.cache.reserve(request, lengths[request], lengths[request] + count)
+            runner.step([StepEntry(request, lengths[request], tokens, [])])
+        lengths[request] += count
+
+    def decode(step):
+        outs = []
+        for runner in runners:
+            entries = []
+            for r in range(live):
+                runner.cache.reserve(r, lengths[r], lengths[r] + 1)
+                entries.append(StepEntry(r, lengths[r], [(5 * r + 11 * step) % vocab], [0]))
+            outs.append(runner.step(entries).float().cpu().numpy())
+            torch.cuda.synchronize()
+        for r in range(live):
+            lengths[r] += 1
+            assert rel_err(outs[1][r], outs[0][r]) < 1e-2, f"step {step}, request {r} of {lengths[r]} positions"
+
+    extend(0, 900)
+    for r in range(1, live):
+        extend(r, 20 + r % 41)
+    for step in range(3):
+        decode(step)
+    assert {key[2] for key in runners[1].graphs.graphs} == {2}
+    for r in range(1, live):
+        extend(r, 800 - lengths[r] + r % 7)
+    for step in range(3, 6):
+        decode(step)
+    graphs = runners[1].graphs
+    assert graphs.replays == 6 and set(graphs.graphs) == {(64, 1024, 2), (64, 1024, 0)}
+    assert graphs.graphs[(64, 1024, 2)].plans != graphs.graphs[(64, 1024, 0)].plans
+    assert graphs.graphs[(64, 1024, 2)].plans[0][:2] == (128, 8) and graphs.graphs[(64, 1024, 0)].plans[0][:2] == (256, 4)
+    # a class whose launches are another's shares that one's graph
+    made = graphs.capture_ahead(1, 256)
+    assert made == 1 and len({id(g) for key, g in graphs.graphs.items() if key[:2] == (1, 256)}) == 1
 
 
 # --- steps launched ahead of their tokens ---------------------------------------------------------------------------

@@ -106,6 +106,23 @@ def test_decode_attention_chunks():
     assert chunks <= 128 and chunk * chunks >= 1 << 20 and chunk % 32 == 0
 
 
+def test_decode_attention_counts_the_entries_by_the_positions_they_hold():
+    assert decode_chunking(4096, 8, 4, 1, 8 * 4096) == decode_chunking(4096, 8, 4, 1)      # all full: as without
+    assert decode_chunking(16384, 64, 4, 1, 301000) == (1024, 16)      # 64 requests that fill 18 %: no long chunks
+    assert decode_chunking(8192, 16, 4, 1, 70000) == (512, 16)         # as 9 full ones
+    assert decode_chunking(8192, 8, 4, 1, 8 * 4100) == (256, 32)       # a little past a context bucket's half
+    assert decode_chunking(4096, 8, 4, 1, 1) == decode_chunking(4096, 1, 4, 1)             # never fewer than one entry
+    assert decode_chunking(4096, 8, 4, 1, 10 ** 9) == decode_chunking(4096, 8, 4, 1)       # nor more than there are
+
+
+def test_a_captured_step_is_chosen_by_the_share_of_its_context_bucket_that_is_filled():
+    from vipera_rs_amd.engine.graphs import FILL_CLASSES, fill_class
+    assert FILL_CLASSES == (1.0, 0.5, 0.25)
+    assert fill_class(8 * 4096, 8, 4096) == 0 and fill_class(8 * 3000, 8, 4096) == 0
+    assert fill_class(8 * 4100, 8, 8192) == 1              # equal lengths just past a bucket's edge
+    assert fill_class(301000, 64, 16384) == 2 and fill_class(8, 8, 256) == 2
+
+
 def test_one_workgroup_takes_all_chunks_of_a_request_and_key_head_where_those_fill_the_gpu():
     from vipera_rs_amd.ops.attention import joins_decode_chunks
     assert joins_decode_chunks(4, 64, 4, 1, 256) and joins_decode_chunks(4, 128, 4, 1, 256)

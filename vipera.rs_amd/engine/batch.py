@@ -54,6 +54,9 @@ class StepBatch:
     token_source: Optional[torch.Tensor] = None    # [T] int32: -1, or the row of `sampled_tokens` that holds the token
     sampled_tokens: Optional[torch.Tensor] = None  # the sampler's output buffer on the device (set by the runner)
     shared: Dict[object, torch.Tensor] = field(default_factory=dict)  # what parts compute once per step for all layers
+    # launch decisions that depend on more than the step's shapes (on ``sum_decode_kv_len``), noted by whoever takes
+    # them: a captured step is shared between the cases in which they come out the same
+    launch_plans: List[tuple] = field(default_factory=list)
     # host copies, for launch decisions
     host_counts: List[int] = field(default_factory=list)
     host_first_pos: List[int] = field(default_factory=list)
@@ -65,6 +68,7 @@ class StepBatch:
     prefill_tile_tokens: int = TILE_TOKENS   # tokens of one entry of `prefill_tiles`
     num_decode_entries: int = 0
     max_decode_kv_len: int = 0
+    sum_decode_kv_len: int = 0     # positions that the single-token entries see, added up (a captured step: assumed)
     max_tile_reach: int = 0        # positions that the last token of the longest prompt tile sees (no window counted)
     sum_tile_reach: int = 0        # the same, added over the prompt tiles
 
@@ -85,6 +89,7 @@ class PackedStep:
     max_decode_kv_len: int
     max_tile_reach: int = 0
     sum_tile_reach: int = 0
+    sum_decode_kv_len: int = 0
 
     def flat(self) -> np.ndarray:
         return np.concatenate([s.reshape(-1) for s in self.sections]) if self.sections else np.zeros(0, np.int32)
@@ -162,6 +167,7 @@ def pack_entries(entries: Sequence[StepEntry], cache, vocab_size: int, min_table
     tiles: List[int] = [x for _, k, off in tile_list for x in (k, off)]
     tile_reach = [p + min(TILE_TOKENS, int(counts_all[k]) - off) for p, k, off in tile_list]  # positions a tile's last token sees
     max_decode_kv = max((int(kv_len[k]) for k in singles), default=0)
+    sum_decode_kv = sum(int(kv_len[k]) for k in singles)
 
     tables, widths = [], []
     requests = [e.request for e in entries]
@@ -189,7 +195,7 @@ def pack_entries(entries: Sequence[StepEntry], cache, vocab_size: int, min_table
                 sources]
     sections += tables
     return PackedStep(sections, widths, T, E, len(rows), counts_all, [int(v) for v in first], [int(v) for v in slots],
-                      int(kv_len.max()), max_decode_kv, max(tile_reach, default=0), sum(tile_reach))
+                      int(kv_len.max()), max_decode_kv, max(tile_reach, default=0), sum(tile_reach), sum_decode_kv)
 
 
 def batch_from_buffer(packed: PackedStep, dev: torch.Tensor) -> StepBatch:
@@ -211,7 +217,7 @@ def batch_from_buffer(packed: PackedStep, dev: torch.Tensor) -> StepBatch:
         max_count=max(packed.counts), max_kv_len=packed.max_kv_len, all_single=max(packed.counts) == 1,
         num_prefill_tiles=packed.sections[8].size // 2, num_decode_entries=packed.sections[9].size,
         max_decode_kv_len=packed.max_decode_kv_len, max_tile_reach=packed.max_tile_reach,
-        sum_tile_reach=packed.sum_tile_reach,
+        sum_tile_reach=packed.sum_tile_reach, sum_decode_kv_len=packed.sum_decode_kv_len,
     )
 
 

@@ -1,9 +1,14 @@
 """Captured decode steps: a step of single tokens replayed as one HIP graph.
 
 A decode step launches a few hundred small kernels; launched one by one from Python the host is
-slower than the GPU.  A graph of the step is captured once per (padded batch size, context bucket)
-and replayed with new metadata copied into its standing buffers.  The kernels, their order and their
-arithmetic are those of the eager step.  Nothing that clears memory is recorded into a graph.
+slower than the GPU.  A graph of the step is captured once per (padded batch size, context bucket,
+fill class) and replayed with new metadata copied into its standing buffers.  The kernels, their order and
+their arithmetic are those of the eager step.  Nothing that clears memory is recorded into a graph.
+
+The fill class says which share of batch size x context bucket the entries' positions take up: the launches
+of a step may depend on it (the attention over single tokens cuts the positions into shorter chunks where
+most entries are short), and a graph holds the launches of its capture.  Classes whose launches come out the
+same share one graph.
 
 A graph is warmed up and captured on a step of padding entries only (token 0 at position 0 on the scratch
 page and the scratch state row), so that a real step runs exactly once, as the graph's first replay: a
@@ -27,6 +32,15 @@ from .batch import PackedStep, StepEntry, batch_from_buffer, pack_entries
 # costs what 96 cost in every product (72 requests as 96 took 8.02 ms, as 80 they take 7.69).
 BATCH_BUCKETS = (1, 2, 4, 6, 8, 12, 16, 24, 32, 48, 64, 80, 96, 112, 128, 160, 192, 224, 256)
 
+# The shares of batch bucket x context bucket that a captured step's entries are taken to fill; a step replays the
+# graph of the nearest one (in ratio).
+FILL_CLASSES = (1.0, 0.5, 0.25)
+
+
+def fill_class(total_kv_len: int, batch_bucket: int, context_bucket: int) -> int:
+    share = total_kv_len / float(batch_bucket * context_bucket)
+    return 0 if share > 0.7 else 1 if share > 0.35 else 2
+
 
 def _bucket(value: int, buckets: Sequence[int]) -> Optional[int]:
     for b in buckets:
@@ -36,8 +50,9 @@ def _bucket(value: int, buckets: Sequence[int]) -> Optional[int]:
 
 
 class _Captured:
-    def __init__(self, graph, buffer, staging, batch, logits):
+    def __init__(self, graph, buffer, staging, batch, logits, plans):
         self.graph, self.buffer, self.staging, self.batch, self.logits = graph, buffer, staging, batch, logits
+        self.plans = plans  # the launch decisions that the capture's step noted
         self.turn = 0  # which of the two staging buffers the last step used
         self.fetched = [None, None]  # per staging buffer: the event after the GPU's last read of it
 
@@ -48,7 +63,7 @@ class DecodeGraphs:
     def __init__(self, runner, max_context: int):
         self.runner = runner
         self.max_context = max_context
-        self.graphs: Dict[Tuple[int, int], _Captured] = {}
+        self.graphs: Dict[Tuple[int, int, int], _Captured] = {}
         self.pool = None
         self.replays = 0
 
@@ -61,7 +76,7 @@ class DecodeGraphs:
     def wants(self, entries: Sequence[StepEntry]) -> bool:
         return (all(len(e.tokens) == 1 for e in entries) and _bucket(len(entries), BATCH_BUCKETS) is not None)
 
-    def _pack(self, entries, batch_bucket: int, context_bucket: int) -> PackedStep:
+    def _pack(self, entries, batch_bucket: int, context_bucket: int, fill: int) -> PackedStep:
         cache = self.runner.cache
         width = max((context_bucket + g.block_size - 1) // g.block_size for g in cache.groups) if cache.groups else 1
         packed = pack_entries(entries, cache, self.runner.vocab_size, min_table_width=width,
@@ -72,25 +87,31 @@ class DecodeGraphs:
         packed.num_logit_rows = batch_bucket
         packed.max_decode_kv_len = context_bucket
         packed.max_kv_len = context_bucket
+        packed.sum_decode_kv_len = max(batch_bucket, int(FILL_CLASSES[fill] * batch_bucket * context_bucket))
         return packed
 
-    def _capture(self, batch_bucket: int, context_bucket: int, words: int) -> _Captured:
-        """Warm up and capture the step of ``batch_bucket`` entries over ``context_bucket`` positions (on padding
-        entries only) and keep it; ``words``: the length of such a step's packed metadata."""
+    def _capture(self, batch_bucket: int, context_bucket: int, fill: int, words: int) -> _Captured:
+        """Warm up and capture the step of ``batch_bucket`` entries over ``context_bucket`` positions, filled as
+        class ``fill`` says (on padding entries only), and keep it; ``words``: the length of such a step's
+        packed metadata.  If the step's launches are those of another fill class's graph, that one is shared."""
         runner = self.runner
         device = runner.runtime.device
-        # two pinned staging buffers, used in turn: with steps launched ahead of their results, the copy of
-        # the step before may still be waiting in the stream when the next step is packed
-        staging = [torch.empty(words, dtype=torch.int32).pin_memory() for _ in range(2)]
-        buffer = torch.empty(words, dtype=torch.int32, device=device)
-        padding = self._pack([], batch_bucket, context_bucket)
-        staging[0].numpy()[:] = padding.flat()
-        buffer.copy_(staging[0], non_blocking=True)
+        padding = self._pack([], batch_bucket, context_bucket, fill)
+        buffer = torch.from_numpy(padding.flat()).to(device)
         batch = batch_from_buffer(padding, buffer)
         batch.sampled_tokens = runner.sampled_tokens
         # an eager run first: it loads every kernel module the step needs, outside of the capture
         runner.model.forward(batch, runner.storage)
         torch.cuda.synchronize(device)
+        plans = tuple(batch.launch_plans)
+        for other in range(len(FILL_CLASSES)):
+            same = self.graphs.get((batch_bucket, context_bucket, other))
+            if same is not None and same.plans == plans:
+                self.graphs[(batch_bucket, context_bucket, fill)] = same
+                return same
+        # two pinned staging buffers, used in turn: with steps launched ahead of their results, the copy of
+        # the step before may still be waiting in the stream when the next step is packed
+        staging = [torch.empty(words, dtype=torch.int32).pin_memory() for _ in range(2)]
         graph = torch.cuda.CUDAGraph()
         # No garbage collection while the stream is capturing: a collected object that holds pinned or
         # device memory, an event or another graph (an engine that is no longer used, say) would be
@@ -107,14 +128,15 @@ class DecodeGraphs:
                 gc.enable()
         if self.pool is None:
             self.pool = graph.pool()
-        captured = _Captured(graph, buffer, staging, batch, logits)
-        self.graphs[(batch_bucket, context_bucket)] = captured
+        captured = _Captured(graph, buffer, staging, batch, logits, plans)
+        self.graphs[(batch_bucket, context_bucket, fill)] = captured
         return captured
 
     def capture_ahead(self, max_batch: int, max_context: int) -> int:
         """Capture the steps of every batch bucket up to ``max_batch`` entries and every context bucket up to
-        ``max_context`` positions that are not captured yet, so that no step of a running engine has to (a
-        capture drains the stream and takes tens of milliseconds). Returns how many were captured."""
+        ``max_context`` positions that are not captured yet, in every fill class, so that no step of a running
+        engine has to (a capture drains the stream and takes tens of milliseconds). Returns how many were captured
+        (fill classes that share a graph count once)."""
         top_batch = _bucket(max(1, min(max_batch, BATCH_BUCKETS[-1])), BATCH_BUCKETS)
         top_context = self._context_bucket(max(1, min(max_context, self.max_context)))
         made = 0
@@ -123,10 +145,11 @@ class DecodeGraphs:
                 break
             context_bucket = 256
             while context_bucket <= top_context:
-                if (batch_bucket, context_bucket) not in self.graphs:
-                    words = self._pack([], batch_bucket, context_bucket).flat().size
-                    self._capture(batch_bucket, context_bucket, words)
-                    made += 1
+                for fill in range(len(FILL_CLASSES)):
+                    if (batch_bucket, context_bucket, fill) not in self.graphs:
+                        known = {id(g) for g in self.graphs.values()}
+                        words = self._pack([], batch_bucket, context_bucket, fill).flat().size
+                        made += id(self._capture(batch_bucket, context_bucket, fill, words)) not in known
                 context_bucket *= 2
         return made
 
@@ -136,12 +159,12 @@ class DecodeGraphs:
         batch_bucket = _bucket(len(entries), BATCH_BUCKETS)
         longest = max(e.start + 1 for e in entries)
         context_bucket = self._context_bucket(longest)
-        packed = self._pack(entries, batch_bucket, context_bucket)
+        fill = fill_class(sum(e.start + 1 for e in entries), batch_bucket, context_bucket)
+        packed = self._pack(entries, batch_bucket, context_bucket, fill)
         flat = packed.flat()
-        key = (batch_bucket, context_bucket)
-        captured = self.graphs.get(key)
+        captured = self.graphs.get((batch_bucket, context_bucket, fill))
         if captured is None:
-            captured = self._capture(batch_bucket, context_bucket, flat.size)
+            captured = self._capture(batch_bucket, context_bucket, fill, flat.size)
         captured.turn ^= 1
         staging = captured.staging[captured.turn]
         if captured.fetched[captured.turn] is not None:

@@ -131,6 +131,7 @@ class DecoderModel:
         # what parts share within a step is computed anew in every run: a run that is being captured into a graph
         # must launch it too, or the graph would replay with what an earlier run left
         batch.shared.clear()
+        batch.launch_plans.clear()
         x = self.embedding.embed(batch)
         tokens = x.shape[0]
         incoming = None

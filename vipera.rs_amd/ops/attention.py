@@ -19,13 +19,21 @@ DECODE_LONG_CHUNKS = (4096, 2048)   # taken where they still make DECODE_LONG_WA
 DECODE_LONG_WAVES = 2048
 
 
-def decode_chunking(max_kv_len: int, num_entries: int, kv_heads: int, head_blocks: int):
+def decode_chunking(max_kv_len: int, num_entries: int, kv_heads: int, head_blocks: int, total_kv_len: int = 0):
     """``(chunk, chunks)``: positions per chunk (a multiple of 32) and chunks that cover ``max_kv_len``.
 
     Chunks of 1,024 positions, or shorter while the waves are fewer than 512; with many requests at long contexts
     chunks of 2,048 or 4,096 where those still make 2,048 waves (a wave then streams longer for every merge: 64
     requests x 4 key heads at 32,768 positions read their 4.3 GB at 6.06 TB/s in chunks of 4,096, at 5.68 in chunks
-    of 1,024; with 1,024 waves chunks of 2,048 fall to 4.6 TB/s)."""
+    of 1,024; with 1,024 waves chunks of 2,048 fall to 4.6 TB/s).
+
+    The waves that count are those with positions to read: the chunks past a request's own length end at once.
+    ``total_kv_len``, the lengths of all entries added up, says how many there are: the entries count as
+    ``total_kv_len / max_kv_len`` full ones (64 requests of 384 to 8,448 positions, 301,000 together, under a
+    longest of 16,384: 147 us a layer in chunks of 1,024, 210 in the chunks of 2,048 that 64 full entries would
+    get; 16 such requests 31 us in chunks of 512, 36 in chunks of 1,024).  Zero: every entry counts as full."""
+    if total_kv_len > 0 and max_kv_len > 0:
+        num_entries = max(1, min(num_entries, -(-total_kv_len // max_kv_len)))
     pairs = num_entries * kv_heads * head_blocks
     for chunk in DECODE_LONG_CHUNKS:
         chunks = (max_kv_len + chunk - 1) // chunk
@@ -34,7 +42,7 @@ def decode_chunking(max_kv_len: int, num_entries: int, kv_heads: int, head_block
     chunk = 1024
     while chunk > DECODE_CHUNK_MIN:
         chunks = (max_kv_len + chunk - 1) // chunk
-        if num_entries * kv_heads * head_blocks * chunks >= DECODE_WAVES_WANTED:
+        if pairs * chunks >= DECODE_WAVES_WANTED:
             break
         chunk //= 2
     chunks = max(1, (max_kv_len + chunk - 1) // chunk)
@@ -116,9 +124,11 @@ def paged_attention(qkv, k_cache, v_cache, out, batch, table, heads, kv_heads, h
             group = heads // kv_heads
             visible = batch.max_decode_kv_len
             head_blocks = (group + 15) // 16
-            chunk, chunks = decode_chunking(visible, batch.num_decode_entries, kv_heads, head_blocks)
+            chunk, chunks = decode_chunking(visible, batch.num_decode_entries, kv_heads, head_blocks,
+                                            batch.sum_decode_kv_len)
             join = joins_decode_chunks(chunks, batch.num_decode_entries, kv_heads, head_blocks,
                                        kernels.compute_units(qkv.device))
+            batch.launch_plans.append((chunk, chunks, join))
             partial = None if join else torch.empty(batch.num_decode_entries * heads * chunks * (head_dim + 2),
                                                     dtype=torch.float32, device=qkv.device)
             kernels.attn_bf16_decode(qkv, k_cache, v_cache, out, partial, batch.decode_entries, batch.entry_start,
