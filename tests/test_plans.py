@@ -115,6 +115,22 @@ def test_decode_attention_counts_the_entries_by_the_positions_they_hold():
     assert decode_chunking(4096, 8, 4, 1, 10 ** 9) == decode_chunking(4096, 8, 4, 1)       # nor more than there are
 
 
+def test_decode_attention_chunks_cover_every_length_for_any_batch():
+    import random
+    rng = random.Random(5)
+    for _ in range(3000):
+        longest = rng.choice([1, 31, 32, 33, 100, 1000, 4096, 8191, 40000, rng.randrange(1, 1 << 21)])
+        entries = rng.choice([1, 2, 7, 8, 63, 64, 200, 256])
+        kv_heads, head_blocks = rng.choice([1, 2, 4, 8]), rng.choice([1, 2])
+        total = rng.choice([0, 1, longest, rng.randrange(1, entries * longest + 1), entries * longest, 10 * entries * longest])
+        chunk, chunks = decode_chunking(longest, entries, kv_heads, head_blocks, total)
+        assert chunk % 32 == 0 and chunk >= 128 and 1 <= chunks <= 128, (longest, entries, total)
+        assert chunk * chunks >= longest and chunk * (chunks - 1) < longest, (longest, entries, total)
+        # fewer positions in all never make the chunks longer
+        if total:
+            assert chunk <= decode_chunking(longest, entries, kv_heads, head_blocks)[0]
+
+
 def test_a_captured_step_is_chosen_by_the_share_of_its_context_bucket_that_is_filled():
     from vipera_rs_amd.engine.graphs import FILL_CLASSES, fill_class
     assert FILL_CLASSES == (1.0, 0.5, 0.25)
