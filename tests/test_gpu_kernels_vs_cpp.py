@@ -183,11 +183,14 @@ def test_the_first_norm_of_a_layer_split_between_the_layers(m, width, k_in, head
 
 
 @pytest.mark.parametrize("m,heads,kv_heads,hd,k,scaled", [(17, 5, 2, 48, 1024, False), (64, 4, 4, 128, 2048, True),
-                                                          (33, 7, 1, 64, 1536, True), (40, 3, 1, 16, 1024, False)])
+                                                          (33, 7, 1, 64, 1536, True), (40, 3, 1, 16, 1024, False),
+                                                          (8, 5, 2, 48, 1024, True), (16, 4, 4, 128, 2048, False),
+                                                          (3, 7, 1, 64, 1536, True), (1, 3, 1, 32, 1024, False)])
 def test_split_qkv_product_that_rotates_while_it_adds_its_ranges(m, heads, kv_heads, hd, k, scaled):
-    """17 to 64 tokens: K split over workgroups, and the kernel that adds the ranges divides by the norm (if scaled),
-    adds the bias, rotates and writes the cache. Beside its twin; and without the norm bit for bit what the split
-    product, its sum and the rotation kernel leave."""
+    """Up to 64 tokens (the widest models take this path from few tokens on; the norm's sums then come 16 to a
+    group, 64 past 16 tokens): K split over workgroups, and the kernel that adds the ranges divides by the norm (if
+    scaled), adds the bias, rotates and writes the cache. Beside its twin; and without the norm bit for bit what the
+    split product, its sum and the rotation kernel leave."""
     from vipera_rs_amd.ops import kernels
     bs, n = 8, (heads + 2 * kv_heads) * hd
     g = torch.Generator().manual_seed(m + n + k)
@@ -201,7 +204,7 @@ def test_split_qkv_product_that_rotates_while_it_adds_its_ranges(m, heads, kv_he
     table = torch.arange(entries * 70, dtype=torch.int32).view(entries, 70)
     k_cache = torch.full((entries * 70, kv_heads, bs, hd), 9.0, dtype=torch.bfloat16)
     v_cache = torch.full((entries * 70, kv_heads, hd, bs), 9.0, dtype=torch.bfloat16)
-    stride = 64
+    stride = kernels.follow_stride(m)
     sumsq = (torch.rand(3 * stride, generator=g) * k).float() if scaled else None
     partial = torch.empty(2 * 64 * n)
     args = [a, w, bias, torch.empty(m, n, dtype=torch.bfloat16), m, n, k, k, n, 2, 1, partial, partial.numel(), i32(positions), inv,

@@ -40,14 +40,17 @@ def test_real_layer_sizes_under_every_cut(real, dtype, tol):
 
 # hidden 896 is no multiple of 256 and has heads of width 64; rows of 2,048 values lie 4 KB apart, which the
 # weight-streaming kernels answer with a different first chunk for every workgroup
+# hidden 5,120: weights of 26 to 71 M elements, whose products split K over workgroups from few tokens on (q/k/v from
+# eleven, the output projection from seven, the down projection from the first)
 OTHER_WIDTHS = {
     "0.5b": dict(hidden_size=896, num_attention_heads=14, num_key_value_heads=2, intermediate_size=4864),
     "3b": dict(hidden_size=2048, num_attention_heads=16, num_key_value_heads=2, intermediate_size=11008),
+    "14b": dict(hidden_size=5120, num_attention_heads=40, num_key_value_heads=8, intermediate_size=13824),
 }
 
 
 @pytest.mark.parametrize("name", sorted(OTHER_WIDTHS))
-def test_the_layer_sizes_of_two_other_models_under_every_cut(tmp_path, name):
+def test_the_layer_sizes_of_other_models_under_every_cut(tmp_path, name):
     config = dict(CONFIG_7B_LAYER, **OTHER_WIDTHS[name])
     tokens = random_tokens(1000, 150, 31)
     folder = make_folder(tmp_path / name, config, 5, torch.bfloat16)
@@ -64,10 +67,12 @@ def _under_every_cut(folder, want, tokens, dtype, tol):
     whole = runner.step([StepEntry(0, 0, tokens, list(range(len(tokens))))]).cpu().numpy()
     assert rel_err(whole, want) < tol
     runner.cache.release(0)
-    # portions of changing size, then the last 20 tokens one by one, beside another request's portions
+    # portions of changing size beside another request's portions (steps of 87, 20, 19, 47, 28 and 11 tokens), alone
+    # (8, 12 and 4 tokens), then the last tokens one by one
     other = random_tokens(1000, 90, 22)
     rows, at, oat = [], 0, 0
-    sizes = [70, 3, 2, 40, 15]
+    sizes = [70, 3, 2, 30, 11, 6, 8, 12, 4]
+    assert len(tokens) - sum(sizes) >= 4
     for size in sizes + [1] * (len(tokens) - sum(sizes)):
         entries = []
         runner.cache.reserve(1, at, at + size)

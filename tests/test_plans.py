@@ -11,17 +11,19 @@ QKV_7B, O_7B, GATE_UP_7B, DOWN_7B, HEAD_7B = (4608, 3584), (3584, 3584), (37888,
 def test_few_tokens_stream_the_weights_with_k_split_inside_a_workgroup():
     for n, k in (QKV_7B, O_7B, DOWN_7B, HEAD_7B):
         assert streams_in_wave_order(1, n, k) and streams_in_wave_order(4, n, k)
-    assert streams_in_wave_order(16, *QKV_7B) and streams_in_wave_order(16, *O_7B)
-    assert streams_in_wave_order(8, *DOWN_7B)              # up to 8 tokens also with a long K: no second kernel for K ranges
-    assert streams_in_wave_order(8, 1536, 8960)
-    assert not streams_in_wave_order(9, *DOWN_7B)          # past 8 tokens activations are shared through LDS instead
+    assert streams_in_wave_order(16, *QKV_7B) and streams_in_wave_order(16, *O_7B)    # small weights: up to 16 tokens
+    assert streams_in_wave_order(16, *QKV_7B, rotates=True) and not streams_in_wave_order(17, *QKV_7B)
+    assert streams_in_wave_order(5, *DOWN_7B) and not streams_in_wave_order(6, *DOWN_7B)   # 68 M elements, few rows
+    assert streams_in_wave_order(8, 1536, 8960) and not streams_in_wave_order(9, 1536, 8960)   # small, with a long K
+    assert streams_in_wave_order(6, 2048, 11008) and not streams_in_wave_order(7, 2048, 11008)     # the 3B down projection
+    assert streams_in_wave_order(6, 5120, 5120) and not streams_in_wave_order(7, 5120, 5120)
     assert not streams_in_wave_order(1, 5120, 27648) and not streams_in_wave_order(8, 5120, 27648)   # the 32B down projection
-    assert streams_in_wave_order(1, 152064, 5120) and streams_in_wave_order(8, 5120, 5120)
-    # the 14B down projection: two rounds of small workgroups that would each read all activations
-    assert streams_in_wave_order(4, 5120, 13824) and not streams_in_wave_order(5, 5120, 13824)
-    assert streams_in_wave_order(8, 8192, 8192) and streams_in_wave_order(8, 10240, 8192)     # 72B: two whole rounds, or more
-    assert not streams_in_wave_order(8, *HEAD_7B)          # many rows: likewise
-    assert not streams_in_wave_order(17, *QKV_7B)
+    assert streams_in_wave_order(1, 152064, 5120) and not streams_in_wave_order(8, *HEAD_7B)      # many rows: up to 4
+    # 60 M elements and 4,096 rows or more: K goes over workgroups from the first token on
+    assert not streams_in_wave_order(1, 5120, 13824) and not streams_in_wave_order(1, 8192, 8192)
+    # q/k/v, whose second kernel costs more
+    assert streams_in_wave_order(3, 10240, 8192, rotates=True) and not streams_in_wave_order(4, 10240, 8192, rotates=True)
+    assert streams_in_wave_order(10, 7168, 5120, rotates=True) and not streams_in_wave_order(11, 7168, 5120, rotates=True)
 
 
 def test_the_lds_shared_product_splits_k_where_rows_are_few():
@@ -68,10 +70,13 @@ def test_the_gated_product_goes_resident_tiled_or_lds_shared():
     assert gated_plan(8, 4096, 1024, cus=256) != 0         # 128 pairs over 256 CUs: half of them would have none
 
 
-def test_q_k_v_of_17_to_64_tokens_rotates_in_the_kernel_that_adds_its_ranges():
+def test_q_k_v_rotates_in_the_kernel_that_adds_its_ranges_where_k_is_split():
     assert split_qkv_plan(64, *QKV_7B) == (3, 1) and split_qkv_plan(17, *QKV_7B) == (3, 1)
     assert split_qkv_plan(16, *QKV_7B) is None and split_qkv_plan(65, *QKV_7B) is None
     assert split_qkv_plan(32, 1024, 512) is None           # K too short to split
+    # the widest models split from few tokens on, in two ranges where the rows alone would fill the CUs
+    assert split_qkv_plan(8, 10240, 8192) == (2, 1) and split_qkv_plan(3, 10240, 8192) is None
+    assert split_qkv_plan(16, 7168, 5120) == (2, 1) and split_qkv_plan(8, 7168, 5120) is None
 
 
 def test_room_for_the_sums_of_squares():

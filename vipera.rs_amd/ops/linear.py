@@ -51,22 +51,43 @@ def mid_plan(m: int, n: int, k: int) -> Tuple[int, int]:
     return max(1, min(k // 512, 256 // row_blocks)), rows_per_wave
 
 
-def streams_in_wave_order(m: int, n: int, k: int, cus: int = 256) -> bool:
-    """Whether a bfloat16 product of ``m`` tokens runs on the kernel whose waves split K inside a workgroup: up to 4
-    tokens; up to 8 where the weight has few rows, also with a long K (every workgroup reads all activations,
-    but there is no second kernel that adds K ranges: the down projection at 8 tokens 30.2 against 28.2 + 4.9 us at
-    the 7B widths, 12.1 against 11.1 + 6.2 at the 1.5B widths); up to 16 with a short K as well.  Not for a weight
-    of few rows and more than 100 M elements, whose workgroups would each stream most of a megabyte through four
-    waves (the 32B down projection, 5,120 x 27,648: 62.2 us against 50.7 + 5 with K split over workgroups at one
-    token, 67.9 against 52.2 + 5 at eight).  Nor past 4 tokens for a long K whose 16-row workgroups are more than
-    one round over the ``cus`` CUs and less than two: the launch then makes two rounds of workgroups of ten rows or
-    so, each of which reads all activations, nearly as many bytes again as the weights (the 14B down projection,
-    5,120 x 13,824, at 8 tokens: 37.8 us against 29.7 + 2.5)."""
-    if n < 16_384 and n * k > 100_000_000:
+def streams_in_wave_order(m: int, n: int, k: int, rotates: bool = False) -> bool:
+    """Whether a bfloat16 product of ``m`` tokens runs on the kernel whose waves split K inside a workgroup (one
+    launch; every workgroup of 16 rows reads all activations) and not on the one that shares the activations through
+    LDS, splits K over workgroups and adds the ranges with a second kernel.  The first grows with the tokens, the
+    second has the second launch to pay, so each weight has a number of tokens up to which the first is chosen
+    (times in us of the product with what it fuses, the first kernel against the two, weights rotated so that none
+    stays cached):
+
+    * up to 4 tokens for a weight of 16,384 rows or more (the output matrix);
+    * never for a weight of fewer rows and more than 100 M elements, whose workgroups would each stream most of a
+      megabyte through four waves (the 32B down projection, 5,120 x 27,648: 57.1 against 52.8 at one token, 69.4
+      against 52.5 at eight);
+    * 60 M elements and more: never with 4,096 rows or more (8,192 x 8,192: 30.2 against 26.7 at one token, 32.4
+      against 26.5 at eight; 5,120 x 13,824: 29.6 against 28.5 and 38.1 against 29.1), up to 5 tokens with fewer
+      (the 7B down projection, 3,584 x 18,944: 25.9 against 27.7 at one, 28.3 against 27.9 at six, 30.2 against 28.0
+      at eight);
+    * 20 M elements and more: up to 6 (5,120 x 5,120: 13.5 against 14.0 at one token, 15.1 against 14.6 at six, 16.6
+      against 14.4 at eight; 2,048 x 11,008: 14.3 against 13.7 at four, 15.5 against 13.8 at eight);
+    * smaller weights: up to 8 with a long K (1,536 x 8,960: 12.7 against 13.1 at eight, 14.3 against 13.0 at
+      twelve), up to 16 with a short one (3,584 x 3,584: 11.0 against 12.9 at sixteen).
+
+    ``rotates``: the product is q/k/v, whose second kernel also rotates and writes the cache and costs 2 us more:
+    up to 3 tokens from 60 M elements on (10,240 x 8,192: 32.5 against 34.6 at one token, 34.9 against 34.2 at four,
+    39.3 against 34.8 at eight), up to 10 from 20 M on (7,168 x 5,120: 19.3 against 20.0 at eight, 24.6 against 20.6
+    at sixteen)."""
+    if n >= 16_384:
+        return m <= 4
+    elements = n * k
+    if elements > 100_000_000:
         return False
-    if m > 4 and k >= 8_192 and cus < (n + 15) // 16 < 2 * cus:
-        return False
-    return m <= 4 or (m <= 8 and n < 16_384) or (m <= 16 and n < 16_384 and k < 8_192)
+    if elements >= 60_000_000:
+        limit = 3 if rotates else 5 if n < 4_096 else 0
+    elif elements >= 20_000_000:
+        limit = 10 if rotates else 6
+    else:
+        limit = 8 if k >= 8_192 else 16
+    return m <= limit
 
 
 def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
@@ -105,11 +126,13 @@ def linear_follow(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor]
 
 def split_qkv_plan(m: int, n: int, k: int) -> Optional[Tuple[int, int]]:
     """``(ranges, tiles per wave)`` if a q/k/v product of ``m`` tokens runs with K split over workgroups, so that the
-    kernel that adds the ranges can also rotate and write the cache (17 to 64 tokens), else None."""
-    if m <= 16 or m > 64 or streams_in_wave_order(m, n, k):
+    kernel that adds the ranges can also rotate and write the cache (up to 64 tokens, where the product does not run
+    in wave order), else None."""
+    if m > 64 or streams_in_wave_order(m, n, k, rotates=True):
         return None
     ranges, rows_per_wave = mid_plan(m, n, k)
-    return (ranges, rows_per_wave) if ranges >= 2 and k // ranges >= 512 else None
+    ranges = max(ranges, 2)   # the second kernel is what rotates: two ranges where one would do (10,240 x 8,192)
+    return (ranges, rows_per_wave) if k // ranges >= 512 else None
 
 
 def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:

@@ -93,7 +93,7 @@ class Attention(Mixer):
 
     def _fused(self, tokens: int, position, batch) -> Optional[str]:
         """How product, rotation and cache write of a step of ``tokens`` run as one launch sequence without a
-        rotation kernel, if they do: "stream" (up to 16 tokens, one kernel) or "split" (17 to 64 tokens, K split
+        rotation kernel, if they do: "stream" (up to 16 tokens, one kernel) or "split" (up to 64 tokens, K split
         over workgroups and the kernel that adds the ranges rotates).  All bfloat16, a full rotation computed in the
         kernel (no table of the step's angles)."""
         fused = position.fused_rotary()
@@ -102,7 +102,7 @@ class Attention(Mixer):
                 and self.w_qkv.dtype == torch.bfloat16 and self.head_dim % 2 == 0 and k % 8 == 0
                 and position.step_angles(batch) is None):
             return None
-        if tokens <= 16 and streams_in_wave_order(tokens, n, k) and n * k * 2 < 2 ** 31:
+        if tokens <= 16 and streams_in_wave_order(tokens, n, k, rotates=True) and n * k * 2 < 2 ** 31:
             return "stream"
         if self.head_dim % 8 == 0 and split_qkv_plan(tokens, n, k) is not None:
             return "split"
