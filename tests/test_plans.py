@@ -152,6 +152,9 @@ def test_one_workgroup_takes_all_chunks_of_a_request_and_key_head_where_those_fi
     # a few more pairs than CUs: the CUs with two workgroups would set the time
     assert not joins_decode_chunks(4, 72, 4, 1, 256) and not joins_decode_chunks(4, 40, 8, 1, 256)
     assert not joins_decode_chunks(4, 96, 4, 1, 256) and joins_decode_chunks(4, 112, 4, 1, 256)
+    # heads wider than 128 keep a workgroup per chunk: one wave a SIMD, with room for their sums
+    assert joins_decode_chunks(4, 64, 4, 1, 256, 128) and joins_decode_chunks(4, 64, 4, 1, 256, 112)
+    assert not joins_decode_chunks(4, 64, 4, 1, 256, 160) and not joins_decode_chunks(4, 64, 4, 1, 256, 256)
 
 
 def test_prompt_tiles_are_halved_between_sixteen_waves_only_where_a_cu_would_be_left_with_one_workgroup():

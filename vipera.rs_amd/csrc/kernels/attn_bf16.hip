@@ -876,8 +876,15 @@ __global__ __launch_bounds__(256) void attn_prefill_merge_kernel(const float* __
 // For steps whose (entry, key head) pairs alone fill the GPU (64 requests x 4 key heads), where the chunks only
 // serve to keep several waves on a CU.
 constexpr int JOINED_WAVES = 8;
+// Waves per SIMD that the kernel's registers are sized for: two (256 registers a lane); with a head width of 256 the
+// output sums and the operands in flight take more than that and would spill some 400 values, so one.
+#if HDP > 128
+#define VK_DECODE_WAVES_PER_SIMD 1
+#else
+#define VK_DECODE_WAVES_PER_SIMD 2
+#endif
 template <bool REGS, bool JOINED>
-__global__ __launch_bounds__(JOINED ? JOINED_WAVES * 64 : 64) __attribute__((amdgpu_waves_per_eu(2))) void attn_decode_kernel(
+__global__ __launch_bounds__(JOINED ? JOINED_WAVES * 64 : 64) __attribute__((amdgpu_waves_per_eu(VK_DECODE_WAVES_PER_SIMD))) void attn_decode_kernel(
     const __bf16* __restrict__ q, long long q_stride, const __bf16* __restrict__ k_cache,
     const __bf16* __restrict__ v_cache, float* __restrict__ partial, __bf16* __restrict__ out,
     const int* __restrict__ entries, const int* __restrict__ entry_start, const int* __restrict__ entry_first_pos,

@@ -52,7 +52,8 @@ def decode_chunking(max_kv_len: int, num_entries: int, kv_heads: int, head_block
     return chunk, chunks
 
 
-def joins_decode_chunks(chunks: int, num_entries: int, kv_heads: int, head_blocks: int, cus: int) -> bool:
+def joins_decode_chunks(chunks: int, num_entries: int, kv_heads: int, head_blocks: int, cus: int,
+                        head_dim: int = 128) -> bool:
     """Whether one workgroup per (entry, key head) takes all chunks, a wave each, and merges them itself instead of
     a workgroup per chunk and a second kernel: where those pairs alone fill the GPU (64 requests x 4 key heads on 256
     CUs), so that the chunks only serve to keep several waves on a CU; the merge kernel and the chunks' round trip
@@ -63,6 +64,8 @@ def joins_decode_chunks(chunks: int, num_entries: int, kv_heads: int, head_block
     pairs = num_entries * kv_heads * head_blocks
     if cus < pairs < 1.55 * cus:
         return False
+    if kernels.attn_bf16_padded_width(head_dim) > 128:
+        return False    # eight waves a workgroup are two a SIMD: 256 registers each, which a wider head's sums overflow
     return chunks <= kernels.ATTN_DECODE_JOINED_CHUNKS and pairs >= 0.8 * cus
 
 
@@ -127,7 +130,7 @@ def paged_attention(qkv, k_cache, v_cache, out, batch, table, heads, kv_heads, h
             chunk, chunks = decode_chunking(visible, batch.num_decode_entries, kv_heads, head_blocks,
                                             batch.sum_decode_kv_len)
             join = joins_decode_chunks(chunks, batch.num_decode_entries, kv_heads, head_blocks,
-                                       kernels.compute_units(qkv.device))
+                                       kernels.compute_units(qkv.device), head_dim)
             batch.launch_plans.append((chunk, chunks, join))
             partial = None if join else torch.empty(batch.num_decode_entries * heads * chunks * (head_dim + 2),
                                                     dtype=torch.float32, device=qkv.device)
