@@ -139,7 +139,10 @@ class DecodeGraphs:
         (fill classes that share a graph count once)."""
         top_batch = _bucket(max(1, min(max_batch, BATCH_BUCKETS[-1])), BATCH_BUCKETS)
         top_context = self._context_bucket(max(1, min(max_context, self.max_context)))
-        made = 0
+        def distinct() -> int:
+            return len({id(captured) for captured in self.graphs.values()})
+
+        before = distinct()
         for batch_bucket in BATCH_BUCKETS:
             if batch_bucket > top_batch:
                 break
@@ -147,11 +150,10 @@ class DecodeGraphs:
             while context_bucket <= top_context:
                 for fill in range(len(FILL_CLASSES)):
                     if (batch_bucket, context_bucket, fill) not in self.graphs:
-                        known = {id(g) for g in self.graphs.values()}
                         words = self._pack([], batch_bucket, context_bucket, fill).flat().size
-                        made += id(self._capture(batch_bucket, context_bucket, fill, words)) not in known
+                        self._capture(batch_bucket, context_bucket, fill, words)
                 context_bucket *= 2
-        return made
+        return distinct() - before
 
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         """Logits ``[wanted, vocab]`` like the eager step; ``want`` of an entry is ``[]`` or ``[0]``."""
