@@ -46,6 +46,9 @@ OTHER_WIDTHS = {
     "0.5b": dict(hidden_size=896, num_attention_heads=14, num_key_value_heads=2, intermediate_size=4864),
     "3b": dict(hidden_size=2048, num_attention_heads=16, num_key_value_heads=2, intermediate_size=11008),
     "14b": dict(hidden_size=5120, num_attention_heads=40, num_key_value_heads=8, intermediate_size=13824),
+    # the attention of the 72B shape (q/k/v of 10,240 x 8,192 splits K from four tokens on, in two ranges that the
+    # rows alone would not ask for; the output projection from the first) with a small feed-forward
+    "72b attention": dict(hidden_size=8192, num_attention_heads=64, num_key_value_heads=8, intermediate_size=1024),
 }
 
 
